@@ -1,0 +1,231 @@
+/*
+ * oslo_hip.h -- C ABI of liboslo_hip.so: the fused non-GEMM transformer-layer
+ * kernels (LayerNorm / RMSNorm, scaled causal / padding-masked softmax,
+ * bias-GeLU, bias-dropout-add; forward and backward) for AMD gfx950.
+ *
+ * Conventions shared by every entry point
+ *   - All tensor arguments are raw DEVICE pointers to contiguous row-major
+ *     storage.  The library never allocates, frees or synchronises: the caller
+ *     owns every output and every workspace (sizes from oslo_workspace_bytes).
+ *   - `stream` is a hipStream_t passed as void* (NULL = the default stream).
+ *     Launches are asynchronous on that stream.
+ *   - Return value: OSLO_OK (0) or a negative OSLO_ERR_* code; the message
+ *     for the calling thread's last failure is oslo_hip_last_error().
+ *   - dtype arguments take OSLO_DTYPE_* values.  Accumulation is fp32.
+ *   - Element counts are 64-bit; a tensor may exceed 2^31 elements.
+ *
+ * Each declaration cites the interface of the reference (EleutherAI/oslo) it
+ * replaces; paths are relative to the reference's repository root.
+ */
+#ifndef OSLO_HIP_H
+#define OSLO_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define OSLO_HIP_ABI_VERSION 1
+
+#define OSLO_OK 0
+#define OSLO_ERR_INVALID_ARGUMENT (-1)
+#define OSLO_ERR_UNSUPPORTED (-2)
+#define OSLO_ERR_WORKSPACE (-3)
+#define OSLO_ERR_LAUNCH (-4)
+
+#define OSLO_DTYPE_F32 0
+#define OSLO_DTYPE_F16 1
+#define OSLO_DTYPE_BF16 2
+
+/* ops for oslo_workspace_bytes */
+#define OSLO_OP_LN_BWD 1
+#define OSLO_OP_RMS_BWD 2
+#define OSLO_OP_BIAS_GELU_BWD 3
+#define OSLO_OP_BIAS_DROPOUT_ADD_BWD 4
+
+/* ---- library state ----------------------------------------------------- */
+
+/* Message of the calling thread's most recent failing call ("" if none). */
+const char *oslo_hip_last_error(void);
+/* Architecture the device code was compiled for ("gfx950"). */
+const char *oslo_hip_arch(void);
+int oslo_hip_abi_version(void);
+
+/* Bytes of fp32 scratch the backward entry point `op` needs for an
+ * [n1, n2] problem (column-partial sums for the parameter gradients).
+ * Replaces the part_grad_gamma / part_grad_beta allocation inside
+ * oslo/torch/_C/csrc/fused_layer_norm.cu:831-833, moved to the caller. */
+int64_t oslo_workspace_bytes(int op, int64_t n1, int64_t n2);
+
+/* ---- LayerNorm / RMSNorm ----------------------------------------------- *
+ * x is [n1, n2] of dtype_in; y, gamma, beta have dtype_out; mean / invvar are
+ * fp32 [n1].  Allowed (dtype_in, dtype_out): (f32,f32) (f32,f16) (f32,bf16)
+ * (f16,f16) (bf16,bf16) -- the matrix of
+ * oslo/torch/_C/csrc/includes/type_shim.h:128-237 without fp64.
+ * gamma == NULL (then beta must be NULL too) selects the non-affine form.  */
+
+/* Replaces layer_norm_forward, layer_norm_forward_affine and
+ * layer_norm_forward_affine_mixed_dtypes
+ * (oslo/torch/_C/csrc/FusedLayerNormBinder.cpp:135-207, 404-417 ->
+ * cuda_layer_norm, fused_layer_norm.cu:771-788).
+ * y = (x - mean) * invvar * gamma + beta evaluated in fp32, rounded once.  */
+int oslo_ln_fwd(const void *x, const void *gamma, const void *beta, void *y,
+                float *mean, float *invvar, int64_t n1, int64_t n2, double eps,
+                int dtype_in, int dtype_out, void *stream);
+
+/* Replaces layer_norm_backward and layer_norm_backward_affine
+ * (FusedLayerNormBinder.cpp:221-266 -> cuda_layer_norm_gradient,
+ * fused_layer_norm.cu:908-935; three launches there, one pass + a finalize
+ * here).  dy, gamma, dgamma, dbeta have dtype_out; x, dx have dtype_in.
+ * dgamma / dbeta may be NULL only when gamma is NULL.                      */
+int oslo_ln_bwd(const void *dy, const void *x, const float *mean,
+                const float *invvar, const void *gamma, void *dx, void *dgamma,
+                void *dbeta, void *workspace, int64_t workspace_bytes,
+                int64_t n1, int64_t n2, int dtype_in, int dtype_out,
+                void *stream);
+
+/* Replaces rms_norm_forward, rms_norm_forward_affine and
+ * rms_norm_forward_affine_mixed_dtypes (FusedLayerNormBinder.cpp:285-358 ->
+ * cuda_rms_norm, fused_layer_norm.cu:790-806).
+ * y = gamma * round_out(x * invvar): the normalised value is rounded to
+ * dtype_out before the scale, as fused_layer_norm.cu:338 and
+ * oslo/torch/nn/modules/layer_norm.py:27-30 both do.                       */
+int oslo_rms_fwd(const void *x, const void *gamma, void *y, float *invvar,
+                 int64_t n1, int64_t n2, double eps, int dtype_in,
+                 int dtype_out, void *stream);
+
+/* Replaces rms_norm_backward and rms_norm_backward_affine
+ * (FusedLayerNormBinder.cpp:360-402 -> cuda_rms_norm_gradient,
+ * fused_layer_norm.cu:937-963).                                            */
+int oslo_rms_bwd(const void *dy, const void *x, const float *invvar,
+                 const void *gamma, void *dx, void *dgamma, void *workspace,
+                 int64_t workspace_bytes, int64_t n1, int64_t n2, int dtype_in,
+                 int dtype_out, void *stream);
+
+/* ---- scaled masked softmax --------------------------------------------- *
+ * Input, output and gradients share one dtype (f32, f16 or bf16).          */
+
+/* Replaces fused_scaled_upper_triang_masked_softmax_forward
+ * (oslo/torch/_C/csrc/FusedScaleMaskSoftmaxBinder.cpp:76-86, 122-124; the
+ * reference declares fwd_cuda but ships no definition).  x, y are
+ * [attn_batches, sq, sk]; key j of query i is visible when
+ * j <= i + (sk - sq); y = softmax(scale * x) over the visible keys, exact 0
+ * elsewhere -- the semantics of
+ * oslo/transformers/models/gpt2/modeling_gpt2.py:116-138.                  */
+int oslo_softmax_causal_fwd(const void *x, void *y, int64_t attn_batches,
+                            int64_t sq, int64_t sk, float scale, int dtype,
+                            void *stream);
+
+/* Replaces fused_scaled_upper_triang_masked_softmax_backward
+ * (FusedScaleMaskSoftmaxBinder.cpp:88-105, 125-127).
+ * dx = scale * y * (dy - sum_j dy_j y_j).  dx may alias dy.                */
+int oslo_softmax_causal_bwd(const void *dy, const void *y, void *dx,
+                            int64_t attn_batches, int64_t sq, int64_t sk,
+                            float scale, int dtype, void *stream);
+
+/* Replaces fused_scaled_masked_softmax_forward
+ * (FusedScaleMaskSoftmaxBinder.cpp:39-49, 112-114).  x, y are
+ * [b, np, sq, sk]; mask is uint8/bool [mask_b, 1, mask_sq, sk] with
+ * mask_b in {1, b} and mask_sq in {1, sq}; non-zero = masked out.  Masked
+ * keys get probability exactly 0 (the limit of the additive -10000 of
+ * oslo/transformers/models/bert/modeling_bert.py:298-306 and
+ * modeling_gpt2.py:573-581); a row whose keys are all masked becomes the
+ * uniform 1/sk that masked_fill(mask, -10000) followed by softmax gives.   */
+int oslo_softmax_masked_fwd(const void *x, const uint8_t *mask, void *y,
+                            int64_t b, int64_t np, int64_t sq, int64_t sk,
+                            int64_t mask_b, int64_t mask_sq, float scale,
+                            int dtype, void *stream);
+
+/* Replaces fused_scaled_masked_softmax_backward
+ * (FusedScaleMaskSoftmaxBinder.cpp:51-64, 115-117).  mask may be NULL (the
+ * reference signature has none); when given, loads of masked keys are
+ * skipped, which is valid because y is exactly 0 there unless the whole row
+ * is masked (such rows are then read in full).  dx may alias dy.           */
+int oslo_softmax_masked_bwd(const void *dy, const void *y, const uint8_t *mask,
+                            void *dx, int64_t b, int64_t np, int64_t sq,
+                            int64_t sk, int64_t mask_b, int64_t mask_sq,
+                            float scale, int dtype, void *stream);
+
+/* Replaces get_batch_per_block (FusedScaleMaskSoftmaxBinder.cpp:66-70,
+ * 118-121): softmax rows one workgroup of the masked kernel handles.  The
+ * kernels here have no divisibility requirement on it.  Negative on error. */
+int oslo_softmax_batch_per_block(int64_t sq, int64_t sk, int64_t b,
+                                 int64_t np);
+
+/* ---- bias-GeLU (tanh approximation) ------------------------------------ *
+ * x, y, g, dx are [rows, cols]; bias, dbias are [cols]; one dtype for all. */
+
+/* Replaces _fused_bias_gelu_fwb / _fused_gelu_fwb
+ * (oslo/torch/nn/modules/functional.py:23-25, 37-40), TorchScript there.
+ * bias == NULL gives plain GeLU.                                           */
+int oslo_bias_gelu_fwd(const void *x, const void *bias, void *y, int64_t rows,
+                       int64_t cols, int dtype, void *stream);
+
+/* Replaces _fused_bias_gelu_bwd / _fused_gelu_bwd (functional.py:28-34,
+ * 43-50) and the autograd sum-to-size that turns the full-size bias gradient
+ * of functional.py:84 into [cols]: dbias = column sum of dx, fused here.
+ * dbias may be NULL (then workspace may be NULL).                          */
+int oslo_bias_gelu_bwd(const void *g, const void *x, const void *bias,
+                       void *dx, void *dbias, void *workspace,
+                       int64_t workspace_bytes, int64_t rows, int64_t cols,
+                       int dtype, void *stream);
+
+/* ---- bias-dropout-add --------------------------------------------------- *
+ * Dropout mask: element i (row-major index) belongs to group i / 8; the
+ * group's four 32-bit words are Philox4x32-10 with key = seed and counter =
+ * (offset_lo, offset_hi, group_lo, group_hi); element i takes the 16-bit half
+ * ((i % 8) & 1) of word (i % 8) / 2 (low half first) and is KEPT when that
+ * value >= round(p * 65536).  Kept values are scaled by 1 / (1 - p).       */
+
+/* Replaces fused_bias_dropout (functional.py:295-298:
+ * F.dropout(x + bias, p, training)) plus the residual add its callers do
+ * next (oslo/transformers/models/gpt2/modeling_gpt2.py:300, 369, 396).
+ * out = keep * (x + bias) / (1 - p) + residual.  bias, residual, mask_out may
+ * each be NULL; p == 0 (or eval mode: pass p = 0) is the identity mask.
+ * mask_out, if given, receives the keep mask as one uint8 per element.     */
+int oslo_bias_dropout_add_fwd(const void *x, const void *bias,
+                              const void *residual, void *out,
+                              uint8_t *mask_out, int64_t rows, int64_t cols,
+                              float p, uint64_t seed, uint64_t offset,
+                              int dtype, void *stream);
+
+/* Backward of the above: dx = keep * g / (1 - p) with the mask regenerated
+ * from (seed, offset); dbias = column sum of dx (NULL to skip); the residual
+ * gradient is g itself.  dx may alias g.                                   */
+int oslo_bias_dropout_add_bwd(const void *g, void *dx, void *dbias,
+                              void *workspace, int64_t workspace_bytes,
+                              int64_t rows, int64_t cols, float p,
+                              uint64_t seed, uint64_t offset, int dtype,
+                              void *stream);
+
+/* ---- test and measurement hooks (no counterpart in the reference) ------ */
+
+/* Writes the keep mask (1 = kept) of n elements as uint8. */
+int oslo_philox_mask(uint8_t *mask_out, int64_t n, float p, uint64_t seed,
+                     uint64_t offset, void *stream);
+
+/* Raw Philox4x32-10 words: out[4*i .. 4*i+3] for counter
+ * (offset_lo, offset_hi, group_lo, group_hi), group = first_group + i.     */
+int oslo_philox_words(uint32_t *out, int64_t ngroups, int64_t first_group,
+                      uint64_t seed, uint64_t offset, void *stream);
+
+/* Plain device copy of `bytes` (multiple of 16) with the same 128-bit
+ * load/store path the kernels use; calibrates bandwidth and HBM counters. */
+int oslo_copy_probe(const void *src, void *dst, int64_t bytes, void *stream);
+
+/* Wavefront reduction self-test: out[0..3] = (sum, max, sum-of-pair a,
+ * sum-of-pair b) of lane-dependent values; the expected values are
+ * 2016, 63, 2016, 4032.                                                    */
+int oslo_wave_reduce_selftest(float *out4, void *stream);
+
+/* Overrides a launch heuristic (for tuning sweeps): key is one of
+ * "norm_fwd_vpl", "norm_bwd_vpl", "norm_bwd_blocks_per_cu",
+ * "softmax_rows_per_wave", "eltwise_unroll", "eltwise_rowgroups";
+ * value 0 restores the default.  Process-wide, not thread-safe.            */
+int oslo_tune(const char *key, int value);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* OSLO_HIP_H */

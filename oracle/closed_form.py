@@ -1,0 +1,248 @@
+"""numpy restatement of the hot path's arithmetic.  Test infrastructure only.
+
+Every function takes numpy arrays holding the operands' exact values (a bf16
+or fp16 tensor is passed as the float32/float64 array of its values), computes
+in ``acc`` precision (float64 unless stated) and, where ``out`` names a storage
+type, rounds the result to it once at the point where the fused kernel rounds.
+File:line citations are into the reference repository (EleutherAI/oslo).
+"""
+import numpy as np
+
+GELU_A = 0.79788456  # oslo/torch/nn/modules/functional.py:25
+GELU_B = 0.044715  # functional.py:25
+GELU_C = 0.1070322243  # functional.py:32
+
+
+# ---------------------------------------------------------------------------
+# storage-type rounding
+# ---------------------------------------------------------------------------
+def round_bf16(a):
+    """Round-to-nearest-even to bfloat16, returned as float32 values."""
+    a32 = np.ascontiguousarray(a, dtype=np.float32)
+    u = a32.view(np.uint32).astype(np.uint64)
+    bias = ((u >> 16) & 1) + 0x7FFF
+    r = ((u + bias) & 0xFFFF0000).astype(np.uint32)
+    out = r.view(np.float32).reshape(a32.shape).copy()
+    nan = np.isnan(a32)
+    if nan.any():
+        out[nan] = np.nan
+    return out
+
+
+def round_f16(a):
+    return np.asarray(a, dtype=np.float64).astype(np.float16).astype(np.float32)
+
+
+def round_to(a, out):
+    """out in {'f32', 'f16', 'bf16', 'f64'}: value after storing `a` as that type.
+
+    Rounding a float64 value to bf16/fp16 goes through float32 first, as the
+    kernels' fp32 arithmetic does; the double rounding differs from direct
+    rounding only for values within 2^-29 relative of a tie.
+    """
+    if out == "f64":
+        return np.asarray(a, dtype=np.float64)
+    if out == "f32":
+        return np.asarray(a, dtype=np.float64).astype(np.float32)
+    if out == "f16":
+        return round_f16(a)
+    if out == "bf16":
+        return round_bf16(np.asarray(a, dtype=np.float64).astype(np.float32))
+    raise ValueError(out)
+
+
+def ulp_of(out):
+    """Relative spacing (2^-mantissa_bits) of a storage type."""
+    return {"f32": 2.0 ** -23, "f16": 2.0 ** -10, "bf16": 2.0 ** -7, "f64": 2.0 ** -52}[out]
+
+
+# ---------------------------------------------------------------------------
+# softmax
+# ---------------------------------------------------------------------------
+def causal_hidden(sq, sk):
+    """True where key j is hidden from query i: j > i + (sk - sq).
+
+    The lower-triangular visibility of
+    oslo/transformers/models/gpt2/modeling_gpt2.py:126-132 (bias[..., sk-sq:sk, :sk]).
+    """
+    i = np.arange(sq)[:, None]
+    j = np.arange(sk)[None, :]
+    return j > i + (sk - sq)
+
+
+def softmax_masked_fwd(x, hidden, scale, out="f64", acc=np.float64):
+    """y = softmax(scale * x) over visible keys; hidden keys get exactly 0; a
+    row with no visible key becomes uniform 1/sk.
+
+    modeling_gpt2.py:116-138 (scale, where(causal, w, -1e4), softmax) and
+    oslo/transformers/models/bert/modeling_bert.py:298-306 (scale, additive
+    mask, softmax): exp(-1e4 - max) underflows to 0 in every storage type, so
+    the fill value is the limit "probability 0"; a fully hidden row is
+    softmax of a constant = uniform.  `hidden` broadcasts against `x`.
+    """
+    x = np.asarray(x, dtype=acc)
+    hidden = np.broadcast_to(np.asarray(hidden, dtype=bool), x.shape)
+    t = np.where(hidden, -np.inf, x * acc(scale))
+    m = t.max(axis=-1, keepdims=True)
+    empty = np.isneginf(m)
+    m = np.where(empty, 0.0, m)
+    e = np.exp(t - m)
+    s = e.sum(axis=-1, keepdims=True)
+    with np.errstate(invalid="ignore", divide="ignore"):
+        y = np.where(empty, acc(1.0) / x.shape[-1], e / np.where(empty, 1.0, s))
+    return round_to(y, out)
+
+
+def softmax_causal_fwd(x, scale, out="f64", acc=np.float64):
+    """x: [attn_batches, sq, sk]
+    (oslo/torch/_C/csrc/FusedScaleMaskSoftmaxBinder.cpp:76-86)."""
+    sq, sk = x.shape[-2], x.shape[-1]
+    return softmax_masked_fwd(x, causal_hidden(sq, sk), scale, out, acc)
+
+
+def softmax_bwd(dy, y, scale, out="f64", acc=np.float64):
+    """dx = scale * y * (dy - sum_j dy_j y_j)
+    (closed form also held by the reference's LightSeq test,
+    oslo/lightseq2/csrc/tests/cuda/test_kernel.py:361-368, there without scale)."""
+    dy = np.asarray(dy, dtype=acc)
+    y = np.asarray(y, dtype=acc)
+    s = (dy * y).sum(axis=-1, keepdims=True)
+    return round_to(acc(scale) * (y * (dy - s)), out)
+
+
+# ---------------------------------------------------------------------------
+# LayerNorm / RMSNorm
+# ---------------------------------------------------------------------------
+def layer_norm_fwd(x, gamma, beta, eps, out="f64", acc=np.float64):
+    """Returns (y, mean, invvar) over the last axis.
+
+    mean / biased variance / invvar = rsqrt(var + eps) as
+    oslo/torch/_C/csrc/fused_layer_norm.cu:310-359; y = (x - mean) * invvar
+    * gamma + beta evaluated in `acc` and rounded once, which is what
+    torch.nn.functional.layer_norm (the reference's CPU path,
+    oslo/torch/nn/modules/layer_norm.py:452-455) does for 16-bit tensors.
+    """
+    x = np.asarray(x, dtype=acc)
+    mean = x.mean(axis=-1, keepdims=True)
+    var = ((x - mean) ** 2).mean(axis=-1, keepdims=True)
+    invvar = 1.0 / np.sqrt(var + acc(eps))
+    y = (x - mean) * invvar
+    if gamma is not None:
+        y = y * np.asarray(gamma, dtype=acc) + np.asarray(beta, dtype=acc)
+    return round_to(y, out), mean[..., 0], invvar[..., 0]
+
+
+def layer_norm_bwd(dy, x, mean, invvar, gamma, out_dx="f64", out_param="f64", acc=np.float64):
+    """Returns (dx, dgamma, dbeta); fused_layer_norm.cu:594-741 (dx) and
+    :458-591 (dgamma = sum dy * xhat, dbeta = sum dy)."""
+    dy = np.asarray(dy, dtype=acc)
+    x = np.asarray(x, dtype=acc)
+    n2 = x.shape[-1]
+    mean = np.asarray(mean, dtype=acc)[..., None]
+    invvar = np.asarray(invvar, dtype=acc)[..., None]
+    xhat = (x - mean) * invvar
+    g = 1.0 if gamma is None else np.asarray(gamma, dtype=acc)
+    dyg = dy * g
+    s1 = dyg.sum(axis=-1, keepdims=True)
+    s2 = (dyg * xhat).sum(axis=-1, keepdims=True)
+    dx = (n2 * dyg - s1 - xhat * s2) * (invvar / n2)
+    if gamma is None:
+        return round_to(dx, out_dx), None, None
+    flat_dy = dy.reshape(-1, n2)
+    flat_xh = xhat.reshape(-1, n2)
+    dgamma = (flat_dy * flat_xh).sum(axis=0)
+    dbeta = flat_dy.sum(axis=0)
+    return round_to(dx, out_dx), round_to(dgamma, out_param), round_to(dbeta, out_param)
+
+
+def rms_norm_fwd(x, gamma, eps, out="f64", acc=np.float64):
+    """Returns (y, invvar).  invvar = rsqrt(mean(x^2) + eps); the normalised
+    value is rounded to the output type BEFORE the scale by gamma, then the
+    product is rounded again: layer_norm.py:20-30 (manual_rms_norm) and
+    fused_layer_norm.cu:338 agree on that order."""
+    x = np.asarray(x, dtype=acc)
+    invvar = 1.0 / np.sqrt((x * x).mean(axis=-1, keepdims=True) + acc(eps))
+    y = round_to(x * invvar, out)
+    if gamma is not None:
+        y = round_to(np.asarray(gamma, dtype=acc) * np.asarray(y, dtype=acc), out)
+    return y, invvar[..., 0]
+
+
+def rms_norm_bwd(dy, x, invvar, gamma, out_dx="f64", out_param="f64", acc=np.float64):
+    """Returns (dx, dgamma); fused_layer_norm.cu:594-741 with rms_only."""
+    dy = np.asarray(dy, dtype=acc)
+    x = np.asarray(x, dtype=acc)
+    n2 = x.shape[-1]
+    invvar = np.asarray(invvar, dtype=acc)[..., None]
+    xhat = x * invvar
+    g = 1.0 if gamma is None else np.asarray(gamma, dtype=acc)
+    dyg = dy * g
+    s2 = (dyg * xhat).sum(axis=-1, keepdims=True)
+    dx = (n2 * dyg - xhat * s2) * (invvar / n2)
+    if gamma is None:
+        return round_to(dx, out_dx), None
+    dgamma = (dy.reshape(-1, n2) * xhat.reshape(-1, n2)).sum(axis=0)
+    return round_to(dx, out_dx), round_to(dgamma, out_param)
+
+
+# ---------------------------------------------------------------------------
+# bias-GeLU
+# ---------------------------------------------------------------------------
+def bias_gelu_fwd(x, bias, out="f64", acc=np.float64):
+    """functional.py:37-40 (bias) / :23-25 (no bias), tanh approximation."""
+    u = np.asarray(x, dtype=acc)
+    if bias is not None:
+        u = u + np.asarray(bias, dtype=acc)
+    y = u * 0.5 * (1.0 + np.tanh(GELU_A * u * (1 + GELU_B * u * u)))
+    return round_to(y, out)
+
+
+def bias_gelu_bwd(g, x, bias, out="f64", acc=np.float64):
+    """Returns (dx, dbias).  functional.py:43-50; dbias is the column sum of dx
+    AS STORED (autograd sum-reduces the rounded full-size tensor that
+    functional.py:84 returns for the bias)."""
+    u = np.asarray(x, dtype=acc)
+    if bias is not None:
+        u = u + np.asarray(bias, dtype=acc)
+    t = np.tanh(GELU_A * u * (1 + GELU_B * u * u))
+    ff = 0.5 * u * ((1 - t * t) * (GELU_A + GELU_C * u * u)) + 0.5 * (1 + t)
+    dx = round_to(ff * np.asarray(g, dtype=acc), out)
+    if bias is None:
+        return dx, None
+    cols = dx.shape[-1]
+    dbias = np.asarray(dx, dtype=acc).reshape(-1, cols).sum(axis=0)
+    return dx, round_to(dbias, out)
+
+
+# ---------------------------------------------------------------------------
+# bias-dropout-add
+# ---------------------------------------------------------------------------
+def bias_dropout_add_fwd(x, bias, residual, keep, p, out="f64", acc=np.float64):
+    """out = keep * (x + bias) / (1 - p) + residual, rounded once.
+
+    functional.py:295-298 (F.dropout(x + bias, p, training)) followed by the
+    caller's residual add (modeling_gpt2.py:369, 396).  `keep` is the 0/1 mask
+    (None = keep everything, i.e. p == 0 or eval mode).
+    """
+    t = np.asarray(x, dtype=acc)
+    if bias is not None:
+        t = t + np.asarray(bias, dtype=acc)
+    if keep is not None:
+        scale = acc(np.float32(1.0) / (np.float32(1.0) - np.float32(p))) if p < 1.0 else acc(0.0)
+        t = np.where(np.asarray(keep, dtype=bool), t * scale, 0.0)
+    if residual is not None:
+        t = t + np.asarray(residual, dtype=acc)
+    return round_to(t, out)
+
+
+def bias_dropout_add_bwd(g, keep, p, out="f64", acc=np.float64):
+    """Returns (dx, dbias): dx = keep * g / (1 - p); dbias = column sum of dx as
+    stored; the residual's gradient is g itself."""
+    t = np.asarray(g, dtype=acc)
+    if keep is not None:
+        scale = acc(np.float32(1.0) / (np.float32(1.0) - np.float32(p))) if p < 1.0 else acc(0.0)
+        t = np.where(np.asarray(keep, dtype=bool), t * scale, 0.0)
+    dx = round_to(t, out)
+    cols = dx.shape[-1]
+    dbias = np.asarray(dx, dtype=acc).reshape(-1, cols).sum(axis=0)
+    return dx, round_to(dbias, out)

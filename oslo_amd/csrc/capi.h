@@ -1,0 +1,56 @@
+// Host-side helpers shared by the C-ABI entry points: error reporting,
+// argument checks, launch-heuristic knobs and cached device facts.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdarg.h>
+#include <stdint.h>
+#include <stdio.h>
+
+#include "../../include/oslo_hip.h"
+
+namespace oslo {
+
+// Records the calling thread's error message and returns `code`.
+int fail(int code, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
+
+// hipGetLastError() after a launch -> OSLO_OK or OSLO_ERR_LAUNCH.
+int check_launch(const char *what);
+
+// Number of compute units of the current device (cached per device id).
+int device_cu_count();
+
+// Launch-heuristic overrides set through oslo_tune(); 0 = use the default.
+struct Tuning {
+  int norm_fwd_vpl;
+  int norm_bwd_vpl;
+  int norm_bwd_blocks_per_cu;
+  int softmax_rows_per_wave;
+  int eltwise_unroll;
+  int eltwise_rowgroups;
+};
+extern Tuning g_tune;
+
+inline bool aligned16(const void *p) {
+  return (reinterpret_cast<uintptr_t>(p) & 15u) == 0;
+}
+
+inline bool valid_dtype(int d) {
+  return d == OSLO_DTYPE_F32 || d == OSLO_DTYPE_F16 || d == OSLO_DTYPE_BF16;
+}
+
+inline int dtype_size(int d) { return d == OSLO_DTYPE_F32 ? 4 : 2; }
+
+inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
+// Column-partial workspace layout shared by the backward kernels and the
+// finalize kernel: `narrays` fp32 arrays of [parts, cols].
+int64_t colsum_parts_norm(int64_t n1, int64_t n2);
+int64_t colsum_parts_eltwise(int64_t rows, int64_t cols);
+
+}  // namespace oslo
+
+#define OSLO_REQUIRE(cond, ...)                                       \
+  do {                                                                \
+    if (!(cond)) return ::oslo::fail(OSLO_ERR_INVALID_ARGUMENT, __VA_ARGS__); \
+  } while (0)

@@ -1,0 +1,734 @@
+// bias-GeLU (tanh approximation) and bias-dropout-add, forward and backward,
+// plus the Philox test hooks, for gfx950.
+//
+// Thread mapping (all kernels): a lane owns one chunk of 8 consecutive
+// columns; a wavefront spans 512 columns of one row; the four wavefronts of a
+// workgroup and the workgroups along grid.y stride over the rows, U rows per
+// step so that a lane keeps U independent 128-bit loads in flight.  The bias
+// chunk lives in registers for the whole kernel.  Backward kernels keep the
+// column sums of dx for their 8 columns in registers, fold the four
+// wavefronts through LDS and write one fp32 partial row per workgroup row
+// (grid.y of them); colsum_finalize_kernel reduces those deterministically.
+//
+// Formulas: oslo/torch/nn/modules/functional.py:23-50 (GeLU forward and
+// derivative with the constants 0.79788456, 0.044715, 0.1070322243),
+// :295-298 (dropout(x + bias)).
+#include "capi.h"
+#include "colsum.cuh"
+#include "common.cuh"
+
+namespace oslo {
+
+constexpr int kE = 8;  // chunk = dropout group = 8 elements for every dtype
+
+// -2 * log2(e) * 0.79788456 and that times 0.044715: exp(-2 z) = exp2(u * (K1 + K2 u^2))
+constexpr float kGeluK1 = -2.0f * 1.4426950408889634f * 0.79788456f;
+constexpr float kGeluK2 = kGeluK1 * 0.044715f;
+
+// gelu(u) = u * sigmoid(2 z), z = 0.79788456 u (1 + 0.044715 u^2); identical
+// to u * 0.5 * (1 + tanh z) without the cancellation of 1 + tanh for u << 0.
+__device__ __forceinline__ float gelu_fwd(float u) {
+  const float e = __builtin_amdgcn_exp2f(u * (kGeluK1 + kGeluK2 * u * u));
+  return u * __builtin_amdgcn_rcpf(1.0f + e);
+}
+
+// d gelu / du = 0.5 u (1 - t^2)(0.79788456 + 0.1070322243 u^2) + 0.5 (1 + t)
+// with t = tanh z; in terms of s = sigmoid(2 z), e = exp(-2 z):
+// 1 + t = 2 s and 1 - t^2 = 4 e s^2.
+__device__ __forceinline__ float gelu_bwd(float u) {
+  const float arg = fminf(u * (kGeluK1 + kGeluK2 * u * u), 80.0f);
+  const float e = __builtin_amdgcn_exp2f(arg);
+  const float s = __builtin_amdgcn_rcpf(1.0f + e);
+  return 2.0f * u * (e * s * s) * (0.79788456f + 0.1070322243f * u * u) + s;
+}
+
+struct EltGeom {
+  int64_t rows;
+  int64_t cols;
+  int nchunks;  // cols / 8
+};
+
+template <typename T, int U, bool HAS_BIAS>
+__global__ __launch_bounds__(256) void bias_gelu_fwd_kernel(
+    const T *__restrict__ x, const T *__restrict__ bias, T *__restrict__ y,
+    EltGeom g) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int cc = blockIdx.x * kWave + lane;
+  if (cc >= g.nchunks) return;
+  float b[kE];
+  if constexpr (HAS_BIAS) load_chunk<T, kE, false>(bias + (int64_t)cc * kE, b);
+  const int64_t rstride = (int64_t)gridDim.y * 4;
+  for (int64_t r0 = (int64_t)blockIdx.y * 4 + wave; r0 < g.rows;
+       r0 += rstride * U) {
+    float v[U][kE];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int64_t r = r0 + u * rstride;
+      if (r < g.rows) load_chunk<T, kE>(x + r * g.cols + (int64_t)cc * kE, v[u]);
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int64_t r = r0 + u * rstride;
+      if (r < g.rows) {
+        float o[kE];
+#pragma unroll
+        for (int e = 0; e < kE; ++e)
+          o[e] = gelu_fwd(HAS_BIAS ? v[u][e] + b[e] : v[u][e]);
+        store_chunk<T, kE>(y + r * g.cols + (int64_t)cc * kE, o);
+      }
+    }
+  }
+}
+
+// Folds the per-lane column sums of the four waves and writes the partial row
+// of this workgroup row.  acc is rounded-dx sums; sh is [4][64 * 8] floats.
+__device__ __forceinline__ void write_col_partials(const float *acc, float *sh,
+                                                   float *__restrict__ part,
+                                                   int64_t cols, int cc,
+                                                   int nchunks, int lane,
+                                                   int wave) {
+#pragma unroll
+  for (int e = 0; e < kE; ++e) sh[(wave * kE + e) * kWave + lane] = acc[e];
+  __syncthreads();
+  if (wave == 0 && cc < nchunks) {
+    float o[kE];
+#pragma unroll
+    for (int e = 0; e < kE; ++e) {
+      o[e] = (sh[(0 * kE + e) * kWave + lane] + sh[(1 * kE + e) * kWave + lane]) +
+             (sh[(2 * kE + e) * kWave + lane] + sh[(3 * kE + e) * kWave + lane]);
+    }
+    store_chunk<float, kE>(part + (int64_t)blockIdx.y * cols + (int64_t)cc * kE,
+                           o);
+  }
+}
+
+template <typename T, int U, bool HAS_BIAS>
+__global__ __launch_bounds__(256) void bias_gelu_bwd_kernel(
+    const T *__restrict__ gr, const T *__restrict__ x,
+    const T *__restrict__ bias, T *__restrict__ dx, float *__restrict__ part,
+    EltGeom g) {
+  __shared__ float sh[4 * kE * kWave];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int cc = blockIdx.x * kWave + lane;
+  const bool cvalid = cc < g.nchunks;
+  float b[kE], acc[kE];
+#pragma unroll
+  for (int e = 0; e < kE; ++e) {
+    b[e] = 0.f;
+    acc[e] = 0.f;
+  }
+  if (cvalid) {
+    if constexpr (HAS_BIAS) load_chunk<T, kE, false>(bias + (int64_t)cc * kE, b);
+    const int64_t rstride = (int64_t)gridDim.y * 4;
+    for (int64_t r0 = (int64_t)blockIdx.y * 4 + wave; r0 < g.rows;
+         r0 += rstride * U) {
+      float v[U][kE], gv[U][kE];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int64_t r = r0 + u * rstride;
+        if (r < g.rows) {
+          load_chunk<T, kE>(x + r * g.cols + (int64_t)cc * kE, v[u]);
+          load_chunk<T, kE>(gr + r * g.cols + (int64_t)cc * kE, gv[u]);
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int64_t r = r0 + u * rstride;
+        if (r < g.rows) {
+          float o[kE];
+#pragma unroll
+          for (int e = 0; e < kE; ++e) {
+            o[e] = gelu_bwd(v[u][e] + b[e]) * gv[u][e];
+            acc[e] += io<T>::round(o[e]);  // sum of dx as stored
+          }
+          store_chunk<T, kE>(dx + r * g.cols + (int64_t)cc * kE, o);
+        }
+      }
+    }
+  }
+  if (part != nullptr)
+    write_col_partials(acc, sh, part, g.cols, cc, g.nchunks, lane, wave);
+}
+
+// ---------------------------------------------------------------------------
+// bias-dropout-add
+// ---------------------------------------------------------------------------
+struct DropArgs {
+  uint64_t seed, offset;
+  uint32_t threshold;  // keep when the 16-bit draw >= threshold
+  float scale;         // 1 / (1 - p), 0 when p >= 1
+};
+
+template <typename T, int U, bool HAS_BIAS, bool HAS_RES, bool DROP>
+__global__ __launch_bounds__(256) void bias_dropout_add_fwd_kernel(
+    const T *__restrict__ x, const T *__restrict__ bias,
+    const T *__restrict__ res, T *__restrict__ out,
+    uint8_t *__restrict__ mask_out, EltGeom g, DropArgs d) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int cc = blockIdx.x * kWave + lane;
+  if (cc >= g.nchunks) return;
+  float b[kE];
+  if constexpr (HAS_BIAS) load_chunk<T, kE, false>(bias + (int64_t)cc * kE, b);
+  const int64_t rstride = (int64_t)gridDim.y * 4;
+  for (int64_t r0 = (int64_t)blockIdx.y * 4 + wave; r0 < g.rows;
+       r0 += rstride * U) {
+    float v[U][kE], rv[U][kE];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int64_t r = r0 + u * rstride;
+      if (r < g.rows) {
+        load_chunk<T, kE>(x + r * g.cols + (int64_t)cc * kE, v[u]);
+        if constexpr (HAS_RES)
+          load_chunk<T, kE>(res + r * g.cols + (int64_t)cc * kE, rv[u]);
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int64_t r = r0 + u * rstride;
+      if (r < g.rows) {
+        uint32_t keep = 0xffu;
+        if constexpr (DROP)
+          keep = dropout_keep_bits((uint64_t)r * (uint64_t)g.nchunks + cc,
+                                   d.seed, d.offset, d.threshold);
+        float o[kE];
+#pragma unroll
+        for (int e = 0; e < kE; ++e) {
+          float t = HAS_BIAS ? v[u][e] + b[e] : v[u][e];
+          if constexpr (DROP) t = (keep >> e) & 1u ? t * d.scale : 0.f;
+          o[e] = HAS_RES ? t + rv[u][e] : t;
+        }
+        store_chunk<T, kE>(out + r * g.cols + (int64_t)cc * kE, o);
+        if (mask_out != nullptr) {
+          u32x2 m;
+          m.x = m.y = 0;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            m.x |= ((keep >> e) & 1u) << (8 * e);
+            m.y |= ((keep >> (4 + e)) & 1u) << (8 * e);
+          }
+          *reinterpret_cast<u32x2 *>(mask_out + r * g.cols + (int64_t)cc * kE) = m;
+        }
+      }
+    }
+  }
+}
+
+template <typename T, int U, bool DROP>
+__global__ __launch_bounds__(256) void bias_dropout_add_bwd_kernel(
+    const T *__restrict__ gr, T *__restrict__ dx, float *__restrict__ part,
+    EltGeom g, DropArgs d) {
+  __shared__ float sh[4 * kE * kWave];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int cc = blockIdx.x * kWave + lane;
+  const bool cvalid = cc < g.nchunks;
+  float acc[kE];
+#pragma unroll
+  for (int e = 0; e < kE; ++e) acc[e] = 0.f;
+  if (cvalid) {
+    const int64_t rstride = (int64_t)gridDim.y * 4;
+    for (int64_t r0 = (int64_t)blockIdx.y * 4 + wave; r0 < g.rows;
+         r0 += rstride * U) {
+      float gv[U][kE];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int64_t r = r0 + u * rstride;
+        if (r < g.rows)
+          load_chunk<T, kE>(gr + r * g.cols + (int64_t)cc * kE, gv[u]);
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int64_t r = r0 + u * rstride;
+        if (r < g.rows) {
+          uint32_t keep = 0xffu;
+          if constexpr (DROP)
+            keep = dropout_keep_bits((uint64_t)r * (uint64_t)g.nchunks + cc,
+                                     d.seed, d.offset, d.threshold);
+          float o[kE];
+#pragma unroll
+          for (int e = 0; e < kE; ++e) {
+            float t = gv[u][e];
+            if constexpr (DROP) t = (keep >> e) & 1u ? t * d.scale : 0.f;
+            o[e] = t;
+            acc[e] += io<T>::round(t);
+          }
+          if (dx != nullptr)
+            store_chunk<T, kE>(dx + r * g.cols + (int64_t)cc * kE, o);
+        }
+      }
+    }
+  }
+  if (part != nullptr)
+    write_col_partials(acc, sh, part, g.cols, cc, g.nchunks, lane, wave);
+}
+
+// ---------------------------------------------------------------------------
+// generic (cols not a multiple of 8, or unaligned pointers): one thread per
+// element, grid-stride; the mask is the same function of the element index.
+// ---------------------------------------------------------------------------
+__device__ __forceinline__ bool keep_element(int64_t i, const DropArgs &d) {
+  const uint32_t bits =
+      dropout_keep_bits((uint64_t)i >> 3, d.seed, d.offset, d.threshold);
+  return (bits >> (i & 7)) & 1u;
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void bias_gelu_fwd_generic_kernel(
+    const T *__restrict__ x, const T *__restrict__ bias, T *__restrict__ y,
+    int64_t n, int64_t cols) {
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n;
+       i += (int64_t)gridDim.x * 256) {
+    float u = io<T>::from_scalar(x[i]);
+    if (bias) u += io<T>::from_scalar(bias[i % cols]);
+    y[i] = io<T>::to_scalar(gelu_fwd(u));
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void bias_gelu_bwd_generic_kernel(
+    const T *__restrict__ gr, const T *__restrict__ x,
+    const T *__restrict__ bias, T *__restrict__ dx, int64_t n, int64_t cols) {
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n;
+       i += (int64_t)gridDim.x * 256) {
+    float u = io<T>::from_scalar(x[i]);
+    if (bias) u += io<T>::from_scalar(bias[i % cols]);
+    dx[i] = io<T>::to_scalar(gelu_bwd(u) * io<T>::from_scalar(gr[i]));
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void bias_dropout_add_fwd_generic_kernel(
+    const T *__restrict__ x, const T *__restrict__ bias,
+    const T *__restrict__ res, T *__restrict__ out,
+    uint8_t *__restrict__ mask_out, int64_t n, int64_t cols, DropArgs d,
+    bool drop) {
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n;
+       i += (int64_t)gridDim.x * 256) {
+    float t = io<T>::from_scalar(x[i]);
+    if (bias) t += io<T>::from_scalar(bias[i % cols]);
+    const bool keep = drop ? keep_element(i, d) : true;
+    if (drop) t = keep ? t * d.scale : 0.f;
+    if (res) t += io<T>::from_scalar(res[i]);
+    out[i] = io<T>::to_scalar(t);
+    if (mask_out) mask_out[i] = keep ? 1 : 0;
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void bias_dropout_add_bwd_generic_kernel(
+    const T *__restrict__ gr, T *__restrict__ dx, int64_t n, DropArgs d,
+    bool drop) {
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n;
+       i += (int64_t)gridDim.x * 256) {
+    float t = io<T>::from_scalar(gr[i]);
+    if (drop) t = keep_element(i, d) ? t * d.scale : 0.f;
+    dx[i] = io<T>::to_scalar(t);
+  }
+}
+
+// Column sum of an already stored [rows, cols] tensor (generic path only).
+template <typename T>
+__global__ __launch_bounds__(256) void colsum_generic_kernel(
+    const T *__restrict__ a, T *__restrict__ out, int64_t rows, int64_t cols) {
+  const int64_t col = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (col >= cols) return;
+  float s = 0.f;
+  for (int64_t r = 0; r < rows; ++r) s += io<T>::from_scalar(a[r * cols + col]);
+  out[col] = io<T>::to_scalar(s);
+}
+
+__global__ __launch_bounds__(256) void philox_mask_kernel(
+    uint8_t *__restrict__ mask_out, int64_t n, DropArgs d) {
+  const int64_t ngroups = (n + 7) / 8;
+  for (int64_t grp = (int64_t)blockIdx.x * 256 + threadIdx.x; grp < ngroups;
+       grp += (int64_t)gridDim.x * 256) {
+    const uint32_t keep =
+        dropout_keep_bits((uint64_t)grp, d.seed, d.offset, d.threshold);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const int64_t i = grp * 8 + e;
+      if (i < n) mask_out[i] = (keep >> e) & 1u;
+    }
+  }
+}
+
+__global__ __launch_bounds__(256) void philox_words_kernel(
+    uint32_t *__restrict__ out, int64_t ngroups, int64_t first_group,
+    uint64_t seed, uint64_t offset) {
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < ngroups;
+       i += (int64_t)gridDim.x * 256) {
+    const uint64_t grp = (uint64_t)(first_group + i);
+    const Philox4 r = philox4x32_10((uint32_t)offset, (uint32_t)(offset >> 32),
+                                    (uint32_t)grp, (uint32_t)(grp >> 32),
+                                    (uint32_t)seed, (uint32_t)(seed >> 32));
+    out[4 * i + 0] = r.x;
+    out[4 * i + 1] = r.y;
+    out[4 * i + 2] = r.z;
+    out[4 * i + 3] = r.w;
+  }
+}
+
+__global__ __launch_bounds__(256) void copy_probe_kernel(
+    const u32x4 *__restrict__ src, u32x4 *__restrict__ dst, int64_t nvec) {
+  const int64_t stride = (int64_t)gridDim.x * 256;
+  int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  for (; i + 3 * stride < nvec; i += 4 * stride) {
+    u32x4 a = ld16_stream(src + i), b = ld16_stream(src + i + stride);
+    u32x4 c = ld16_stream(src + i + 2 * stride),
+          e = ld16_stream(src + i + 3 * stride);
+    st16_stream(dst + i, a);
+    st16_stream(dst + i + stride, b);
+    st16_stream(dst + i + 2 * stride, c);
+    st16_stream(dst + i + 3 * stride, e);
+  }
+  for (; i < nvec; i += stride) st16_stream(dst + i, ld16_stream(src + i));
+}
+
+__global__ __launch_bounds__(64) void wave_reduce_selftest_kernel(float *out) {
+  const int lane = threadIdx.x;
+  const float s = wave_sum((float)lane);
+  const float m = wave_max((float)((lane * 37) % 64));
+  float a = (float)lane, b = (float)(2 * lane);
+  a = wave_sum(a);
+  b = wave_sum(b);
+  if (lane == 17) {
+    out[0] = s;
+    out[1] = m;
+    out[2] = a;
+    out[3] = b;
+  }
+}
+
+// ---------------------------------------------------------------------------
+// host side
+// ---------------------------------------------------------------------------
+int64_t colsum_parts_eltwise(int64_t rows, int64_t cols) {
+  const int64_t col_tiles = ceil_div(ceil_div(cols, kE), kWave);
+  int64_t target = g_tune.eltwise_rowgroups > 0
+                       ? g_tune.eltwise_rowgroups
+                       : ceil_div((int64_t)device_cu_count() * 8, col_tiles);
+  const int64_t maxp = ceil_div(rows, 4);
+  if (target > maxp) target = maxp;
+  if (target < 1) target = 1;
+  if (target > 65535) target = 65535;
+  return target;
+}
+
+static inline int eltwise_unroll() {
+  const int u = g_tune.eltwise_unroll;
+  return u == 1 || u == 2 || u == 4 ? u : 4;
+}
+
+static inline dim3 eltwise_grid(const EltGeom &g) {
+  return dim3((unsigned)ceil_div(g.nchunks, kWave),
+              (unsigned)colsum_parts_eltwise(g.rows, g.cols));
+}
+
+static inline int64_t flat_grid(int64_t n) {
+  int64_t grid = ceil_div(n, 256);
+  const int64_t cap = (int64_t)device_cu_count() * 32;
+  return grid < cap ? (grid < 1 ? 1 : grid) : cap;
+}
+
+static DropArgs make_drop(float p, uint64_t seed, uint64_t offset) {
+  DropArgs d;
+  d.seed = seed;
+  d.offset = offset;
+  double t = (double)p * 65536.0 + 0.5;
+  d.threshold = t >= 65536.0 ? 65536u : (uint32_t)t;
+  d.scale = p < 1.0f ? 1.0f / (1.0f - p) : 0.f;
+  return d;
+}
+
+#define OSLO_ELT_U(U_, ...)  \
+  do {                       \
+    switch (U_) {            \
+      case 1: { constexpr int U = 1; __VA_ARGS__; } break; \
+      case 2: { constexpr int U = 2; __VA_ARGS__; } break; \
+      default: { constexpr int U = 4; __VA_ARGS__; } break; \
+    }                        \
+  } while (0)
+
+template <typename T>
+static int run_bias_gelu_fwd(const void *x, const void *bias, void *y,
+                             int64_t rows, int64_t cols, hipStream_t st) {
+  const bool vec_ok = cols % kE == 0 && aligned16(x) && aligned16(y) &&
+                      aligned16(bias) && cols / kE <= 0x7fffffff;
+  if (!vec_ok) {
+    const int64_t n = rows * cols;
+    bias_gelu_fwd_generic_kernel<T><<<dim3((unsigned)flat_grid(n)), 256, 0, st>>>(
+        (const T *)x, (const T *)bias, (T *)y, n, cols);
+    return check_launch("bias_gelu_fwd_generic_kernel");
+  }
+  EltGeom g{rows, cols, (int)(cols / kE)};
+  const dim3 grid = eltwise_grid(g);
+  OSLO_ELT_U(eltwise_unroll(), {
+    if (bias)
+      bias_gelu_fwd_kernel<T, U, true><<<grid, 256, 0, st>>>(
+          (const T *)x, (const T *)bias, (T *)y, g);
+    else
+      bias_gelu_fwd_kernel<T, U, false><<<grid, 256, 0, st>>>(
+          (const T *)x, nullptr, (T *)y, g);
+  });
+  return check_launch("bias_gelu_fwd_kernel");
+}
+
+template <typename T>
+static int run_bias_gelu_bwd(const void *gr, const void *x, const void *bias,
+                             void *dx, void *dbias, void *ws, int64_t ws_bytes,
+                             int64_t rows, int64_t cols, hipStream_t st) {
+  const bool vec_ok = cols % kE == 0 && aligned16(x) && aligned16(gr) &&
+                      aligned16(dx) && aligned16(bias) && aligned16(ws) &&
+                      cols / kE <= 0x7fffffff;
+  if (!vec_ok) {
+    const int64_t n = rows * cols;
+    bias_gelu_bwd_generic_kernel<T><<<dim3((unsigned)flat_grid(n)), 256, 0, st>>>(
+        (const T *)gr, (const T *)x, (const T *)bias, (T *)dx, n, cols);
+    int rc = check_launch("bias_gelu_bwd_generic_kernel");
+    if (rc != OSLO_OK || dbias == nullptr) return rc;
+    colsum_generic_kernel<T><<<dim3((unsigned)ceil_div(cols, 256)), 256, 0, st>>>(
+        (const T *)dx, (T *)dbias, rows, cols);
+    return check_launch("colsum_generic_kernel");
+  }
+  EltGeom g{rows, cols, (int)(cols / kE)};
+  const dim3 grid = eltwise_grid(g);
+  float *part = nullptr;
+  if (dbias != nullptr) {
+    const int64_t need = (int64_t)grid.y * cols * (int64_t)sizeof(float);
+    if (ws == nullptr || ws_bytes < need)
+      return fail(OSLO_ERR_WORKSPACE,
+                  "bias_gelu bwd: workspace of %lld bytes needed, %lld given",
+                  (long long)need, (long long)ws_bytes);
+    part = (float *)ws;
+  }
+  OSLO_ELT_U(eltwise_unroll() > 2 ? 2 : eltwise_unroll(), {
+    if (bias)
+      bias_gelu_bwd_kernel<T, U, true><<<grid, 256, 0, st>>>(
+          (const T *)gr, (const T *)x, (const T *)bias, (T *)dx, part, g);
+    else
+      bias_gelu_bwd_kernel<T, U, false><<<grid, 256, 0, st>>>(
+          (const T *)gr, (const T *)x, nullptr, (T *)dx, part, g);
+  });
+  int rc = check_launch("bias_gelu_bwd_kernel");
+  if (rc != OSLO_OK || dbias == nullptr) return rc;
+  return launch_colsum_finalize<T>(part, grid.y, cols, dbias, nullptr, st);
+}
+
+template <typename T>
+static int run_bda_fwd(const void *x, const void *bias, const void *res,
+                       void *out, uint8_t *mask_out, int64_t rows, int64_t cols,
+                       float p, uint64_t seed, uint64_t offset,
+                       hipStream_t st) {
+  const DropArgs d = make_drop(p, seed, offset);
+  const bool drop = p > 0.f;
+  const bool vec_ok = cols % kE == 0 && aligned16(x) && aligned16(out) &&
+                      aligned16(bias) && aligned16(res) &&
+                      (reinterpret_cast<uintptr_t>(mask_out) & 7u) == 0 &&
+                      cols / kE <= 0x7fffffff;
+  if (!vec_ok) {
+    const int64_t n = rows * cols;
+    bias_dropout_add_fwd_generic_kernel<T>
+        <<<dim3((unsigned)flat_grid(n)), 256, 0, st>>>(
+            (const T *)x, (const T *)bias, (const T *)res, (T *)out, mask_out,
+            n, cols, d, drop);
+    return check_launch("bias_dropout_add_fwd_generic_kernel");
+  }
+  EltGeom g{rows, cols, (int)(cols / kE)};
+  const dim3 grid = eltwise_grid(g);
+#define OSLO_BDA_FWD(HB, HR, DR)                                            \
+  bias_dropout_add_fwd_kernel<T, U, HB, HR, DR><<<grid, 256, 0, st>>>(      \
+      (const T *)x, (const T *)bias, (const T *)res, (T *)out, mask_out, g, d)
+  OSLO_ELT_U(eltwise_unroll() > 2 ? 2 : eltwise_unroll(), {
+    const int key = (bias ? 4 : 0) | (res ? 2 : 0) | (drop ? 1 : 0);
+    switch (key) {
+      case 0: OSLO_BDA_FWD(false, false, false); break;
+      case 1: OSLO_BDA_FWD(false, false, true); break;
+      case 2: OSLO_BDA_FWD(false, true, false); break;
+      case 3: OSLO_BDA_FWD(false, true, true); break;
+      case 4: OSLO_BDA_FWD(true, false, false); break;
+      case 5: OSLO_BDA_FWD(true, false, true); break;
+      case 6: OSLO_BDA_FWD(true, true, false); break;
+      default: OSLO_BDA_FWD(true, true, true); break;
+    }
+  });
+#undef OSLO_BDA_FWD
+  return check_launch("bias_dropout_add_fwd_kernel");
+}
+
+template <typename T>
+static int run_bda_bwd(const void *gr, void *dx, void *dbias, void *ws,
+                       int64_t ws_bytes, int64_t rows, int64_t cols, float p,
+                       uint64_t seed, uint64_t offset, hipStream_t st) {
+  const DropArgs d = make_drop(p, seed, offset);
+  const bool drop = p > 0.f;
+  const bool vec_ok = cols % kE == 0 && aligned16(gr) && aligned16(dx) &&
+                      aligned16(ws) && cols / kE <= 0x7fffffff;
+  if (!vec_ok) {
+    OSLO_REQUIRE(dx != nullptr,
+                 "bias_dropout_add bwd: dx required for this shape/alignment");
+    const int64_t n = rows * cols;
+    bias_dropout_add_bwd_generic_kernel<T>
+        <<<dim3((unsigned)flat_grid(n)), 256, 0, st>>>((const T *)gr, (T *)dx,
+                                                       n, d, drop);
+    int rc = check_launch("bias_dropout_add_bwd_generic_kernel");
+    if (rc != OSLO_OK || dbias == nullptr) return rc;
+    colsum_generic_kernel<T><<<dim3((unsigned)ceil_div(cols, 256)), 256, 0, st>>>(
+        (const T *)dx, (T *)dbias, rows, cols);
+    return check_launch("colsum_generic_kernel");
+  }
+  EltGeom g{rows, cols, (int)(cols / kE)};
+  const dim3 grid = eltwise_grid(g);
+  float *part = nullptr;
+  if (dbias != nullptr) {
+    const int64_t need = (int64_t)grid.y * cols * (int64_t)sizeof(float);
+    if (ws == nullptr || ws_bytes < need)
+      return fail(OSLO_ERR_WORKSPACE,
+                  "bias_dropout_add bwd: workspace of %lld bytes needed, %lld "
+                  "given",
+                  (long long)need, (long long)ws_bytes);
+    part = (float *)ws;
+  }
+  OSLO_ELT_U(eltwise_unroll(), {
+    if (drop)
+      bias_dropout_add_bwd_kernel<T, U, true><<<grid, 256, 0, st>>>(
+          (const T *)gr, (T *)dx, part, g, d);
+    else
+      bias_dropout_add_bwd_kernel<T, U, false><<<grid, 256, 0, st>>>(
+          (const T *)gr, (T *)dx, part, g, d);
+  });
+  int rc = check_launch("bias_dropout_add_bwd_kernel");
+  if (rc != OSLO_OK || dbias == nullptr) return rc;
+  return launch_colsum_finalize<T>(part, grid.y, cols, dbias, nullptr, st);
+}
+
+#define OSLO_ELT_DISPATCH(dtype, FN, ...)                      \
+  do {                                                         \
+    if (dtype == OSLO_DTYPE_F32) return FN<float>(__VA_ARGS__); \
+    if (dtype == OSLO_DTYPE_F16) return FN<_Float16>(__VA_ARGS__); \
+    return FN<__bf16>(__VA_ARGS__);                            \
+  } while (0)
+
+static int check_elt(const char *what, int64_t rows, int64_t cols, int dtype) {
+  if (!valid_dtype(dtype))
+    return fail(OSLO_ERR_INVALID_ARGUMENT, "%s: unknown dtype %d", what, dtype);
+  if (rows < 0 || cols < 1)
+    return fail(OSLO_ERR_INVALID_ARGUMENT, "%s: bad shape [%lld, %lld]", what,
+                (long long)rows, (long long)cols);
+  return OSLO_OK;
+}
+
+// Zero parameter gradient for an empty batch (P = 0 partial rows).
+template <typename T>
+static int zero_vector(void *out, int64_t cols, hipStream_t st) {
+  return launch_colsum_finalize<T>(nullptr, 0, cols, out, nullptr, st);
+}
+
+}  // namespace oslo
+
+extern "C" {
+
+using namespace oslo;
+
+int oslo_bias_gelu_fwd(const void *x, const void *bias, void *y, int64_t rows,
+                       int64_t cols, int dtype, void *stream) {
+  int rc = check_elt("bias_gelu fwd", rows, cols, dtype);
+  if (rc != OSLO_OK) return rc;
+  if (rows == 0) return OSLO_OK;
+  OSLO_REQUIRE(x && y, "bias_gelu fwd: null tensor pointer");
+  OSLO_ELT_DISPATCH(dtype, run_bias_gelu_fwd, x, bias, y, rows, cols,
+                    (hipStream_t)stream);
+}
+
+int oslo_bias_gelu_bwd(const void *g, const void *x, const void *bias,
+                       void *dx, void *dbias, void *workspace,
+                       int64_t workspace_bytes, int64_t rows, int64_t cols,
+                       int dtype, void *stream) {
+  int rc = check_elt("bias_gelu bwd", rows, cols, dtype);
+  if (rc != OSLO_OK) return rc;
+  if (rows == 0) {
+    if (dbias) OSLO_ELT_DISPATCH(dtype, zero_vector, dbias, cols, (hipStream_t)stream);
+    return OSLO_OK;
+  }
+  OSLO_REQUIRE(g && x && dx, "bias_gelu bwd: null tensor pointer");
+  OSLO_ELT_DISPATCH(dtype, run_bias_gelu_bwd, g, x, bias, dx, dbias, workspace,
+                    workspace_bytes, rows, cols, (hipStream_t)stream);
+}
+
+int oslo_bias_dropout_add_fwd(const void *x, const void *bias,
+                              const void *residual, void *out,
+                              uint8_t *mask_out, int64_t rows, int64_t cols,
+                              float p, uint64_t seed, uint64_t offset,
+                              int dtype, void *stream) {
+  int rc = check_elt("bias_dropout_add fwd", rows, cols, dtype);
+  if (rc != OSLO_OK) return rc;
+  OSLO_REQUIRE(p >= 0.f && p <= 1.f, "bias_dropout_add fwd: p = %f not in [0, 1]",
+               (double)p);
+  if (rows == 0) return OSLO_OK;
+  OSLO_REQUIRE(x && out, "bias_dropout_add fwd: null tensor pointer");
+  OSLO_ELT_DISPATCH(dtype, run_bda_fwd, x, bias, residual, out, mask_out, rows,
+                    cols, p, seed, offset, (hipStream_t)stream);
+}
+
+int oslo_bias_dropout_add_bwd(const void *g, void *dx, void *dbias,
+                              void *workspace, int64_t workspace_bytes,
+                              int64_t rows, int64_t cols, float p,
+                              uint64_t seed, uint64_t offset, int dtype,
+                              void *stream) {
+  int rc = check_elt("bias_dropout_add bwd", rows, cols, dtype);
+  if (rc != OSLO_OK) return rc;
+  OSLO_REQUIRE(p >= 0.f && p <= 1.f, "bias_dropout_add bwd: p = %f not in [0, 1]",
+               (double)p);
+  if (rows == 0) {
+    if (dbias) OSLO_ELT_DISPATCH(dtype, zero_vector, dbias, cols, (hipStream_t)stream);
+    return OSLO_OK;
+  }
+  OSLO_REQUIRE(g != nullptr, "bias_dropout_add bwd: null gradient pointer");
+  OSLO_REQUIRE(dx != nullptr || dbias != nullptr,
+               "bias_dropout_add bwd: nothing to compute");
+  OSLO_ELT_DISPATCH(dtype, run_bda_bwd, g, dx, dbias, workspace,
+                    workspace_bytes, rows, cols, p, seed, offset,
+                    (hipStream_t)stream);
+}
+
+int oslo_philox_mask(uint8_t *mask_out, int64_t n, float p, uint64_t seed,
+                     uint64_t offset, void *stream) {
+  OSLO_REQUIRE(n >= 0 && p >= 0.f && p <= 1.f, "philox_mask: bad arguments");
+  if (n == 0) return OSLO_OK;
+  OSLO_REQUIRE(mask_out != nullptr, "philox_mask: null output");
+  philox_mask_kernel<<<dim3((unsigned)flat_grid((n + 7) / 8)), 256, 0,
+                       (hipStream_t)stream>>>(mask_out, n,
+                                              make_drop(p, seed, offset));
+  return check_launch("philox_mask_kernel");
+}
+
+int oslo_philox_words(uint32_t *out, int64_t ngroups, int64_t first_group,
+                      uint64_t seed, uint64_t offset, void *stream) {
+  OSLO_REQUIRE(ngroups >= 0, "philox_words: bad arguments");
+  if (ngroups == 0) return OSLO_OK;
+  OSLO_REQUIRE(out != nullptr, "philox_words: null output");
+  philox_words_kernel<<<dim3((unsigned)flat_grid(ngroups)), 256, 0,
+                        (hipStream_t)stream>>>(out, ngroups, first_group, seed,
+                                               offset);
+  return check_launch("philox_words_kernel");
+}
+
+int oslo_copy_probe(const void *src, void *dst, int64_t bytes, void *stream) {
+  OSLO_REQUIRE(bytes >= 0 && bytes % 16 == 0 && aligned16(src) && aligned16(dst),
+               "copy_probe: bytes must be a multiple of 16 and pointers "
+               "16-byte aligned");
+  if (bytes == 0) return OSLO_OK;
+  const int64_t nvec = bytes / 16;
+  int64_t grid = ceil_div(nvec, 256 * 4);
+  const int64_t cap = (int64_t)device_cu_count() * 16;
+  if (grid > cap) grid = cap;
+  copy_probe_kernel<<<dim3((unsigned)grid), 256, 0, (hipStream_t)stream>>>(
+      (const u32x4 *)src, (u32x4 *)dst, nvec);
+  return check_launch("copy_probe_kernel");
+}
+
+int oslo_wave_reduce_selftest(float *out4, void *stream) {
+  OSLO_REQUIRE(out4 != nullptr, "wave_reduce_selftest: null output");
+  wave_reduce_selftest_kernel<<<1, 64, 0, (hipStream_t)stream>>>(out4);
+  return check_launch("wave_reduce_selftest_kernel");
+}
+
+}  // extern "C"

@@ -1,0 +1,770 @@
+// LayerNorm / RMSNorm forward and backward for gfx950.
+//
+// Register-resident path (rows of up to 64 * 16 * 8 chunks): a row is split
+// over `wpr` consecutive wavefronts, every lane holds VPL chunks of E
+// elements in registers, so x (and dy) are read from HBM exactly once.
+// Statistics are the exact two-pass form of Welford/Chan for resident data:
+// mean first, then the sum of squared deviations, both reduced with DPP
+// inside a wave and through LDS across the waves of a row.
+//
+// Backward is a single pass over dy and x: persistent workgroups stride over
+// the rows, keep the per-column partial sums of dgamma / dbeta in registers
+// for the columns their lanes own, and write one fp32 partial row per
+// workgroup; a small finalize kernel reduces the partial rows in a fixed
+// order (deterministic, no atomics).
+//
+// Formulas follow oslo/torch/_C/csrc/fused_layer_norm.cu:310-359 (forward)
+// and :594-741 (grad input), :458-591 (grad gamma/beta) of the reference.
+#include "capi.h"
+#include "common.cuh"
+#include "colsum.cuh"
+
+namespace oslo {
+
+// ---------------------------------------------------------------------------
+// helpers
+// ---------------------------------------------------------------------------
+// Two simultaneous row sums sharing one barrier.  red is [2][16] floats.
+__device__ __forceinline__ void row_sum2(float &a, float &b, float *red,
+                                         int wave, int first, int wpr,
+                                         int lane) {
+  a = wave_sum(a);
+  b = wave_sum(b);
+  if (wpr > 1) {
+    if (lane == 0) {
+      red[wave] = a;
+      red[16 + wave] = b;
+    }
+    __syncthreads();
+    float ra = red[first], rb = red[16 + first];
+    for (int w = 1; w < wpr; ++w) {
+      ra += red[first + w];
+      rb += red[16 + first + w];
+    }
+    a = ra;
+    b = rb;
+  }
+}
+
+__device__ __forceinline__ float row_sum1(float a, float *red, int wave,
+                                          int first, int wpr, int lane) {
+  a = wave_sum(a);
+  if (wpr > 1) {
+    if (lane == 0) red[wave] = a;
+    __syncthreads();
+    float ra = red[first];
+    for (int w = 1; w < wpr; ++w) ra += red[first + w];
+    a = ra;
+  }
+  return a;
+}
+
+// ---------------------------------------------------------------------------
+// forward, register-resident
+// ---------------------------------------------------------------------------
+template <typename T, typename V, int VPL, bool RMS, int MAXT>
+__global__ __launch_bounds__(MAXT) void norm_fwd_reg_kernel(
+    const T *__restrict__ x, const V *__restrict__ gamma,
+    const V *__restrict__ beta, V *__restrict__ y, float *__restrict__ mean,
+    float *__restrict__ invvar, int64_t n1, int n2, float eps, int wpr,
+    int rpb) {
+  constexpr int E = chunk_elems<T, V>::value;
+  __shared__ float red[2][16];
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int rslot = wave / wpr;
+  const int first = rslot * wpr;
+  const int nchunks = n2 / E;
+  const int cstride = kWave * wpr;
+  const int c0 = (wave - first) * kWave + lane;
+  const float fn = (float)n2;
+  int parity = 0;
+
+  for (int64_t base = (int64_t)blockIdx.x * rpb; base < n1;
+       base += (int64_t)gridDim.x * rpb) {
+    const int64_t row = base + rslot;
+    const bool rvalid = row < n1;
+    const T *xr = x + row * n2;
+    float v[VPL][E];
+#pragma unroll
+    for (int k = 0; k < VPL; ++k) {
+      const int c = c0 + k * cstride;
+      if (rvalid && c < nchunks) {
+        load_chunk<T, E>(xr + (int64_t)c * E, v[k]);
+      } else {
+#pragma unroll
+        for (int e = 0; e < E; ++e) v[k][e] = 0.f;
+      }
+    }
+
+    float mu = 0.f, q = 0.f;
+    if constexpr (!RMS) {
+      float s = 0.f;
+#pragma unroll
+      for (int k = 0; k < VPL; ++k)
+#pragma unroll
+        for (int e = 0; e < E; ++e) s += v[k][e];
+      s = row_sum1(s, red[0], wave, first, wpr, lane);
+      mu = s / fn;
+#pragma unroll
+      for (int k = 0; k < VPL; ++k) {
+        const int c = c0 + k * cstride;
+        if (c < nchunks) {
+#pragma unroll
+          for (int e = 0; e < E; ++e) {
+            const float d = v[k][e] - mu;
+            q += d * d;
+          }
+        }
+      }
+      q = row_sum1(q, red[1], wave, first, wpr, lane);
+    } else {
+#pragma unroll
+      for (int k = 0; k < VPL; ++k)
+#pragma unroll
+        for (int e = 0; e < E; ++e) q += v[k][e] * v[k][e];
+      q = row_sum1(q, red[parity], wave, first, wpr, lane);
+      parity ^= 1;
+    }
+    const float rs = 1.0f / sqrtf(q / fn + eps);
+
+    if (rvalid) {
+      V *yr = y + row * n2;
+#pragma unroll
+      for (int k = 0; k < VPL; ++k) {
+        const int c = c0 + k * cstride;
+        if (c < nchunks) {
+          float o[E];
+          if constexpr (!RMS) {
+#pragma unroll
+            for (int e = 0; e < E; ++e) o[e] = (v[k][e] - mu) * rs;
+            if (gamma != nullptr) {
+              float g[E], b[E];
+              load_chunk<V, E, false>(gamma + (int64_t)c * E, g);
+              load_chunk<V, E, false>(beta + (int64_t)c * E, b);
+#pragma unroll
+              for (int e = 0; e < E; ++e) o[e] = o[e] * g[e] + b[e];
+            }
+          } else {
+#pragma unroll
+            for (int e = 0; e < E; ++e) o[e] = io<V>::round(v[k][e] * rs);
+            if (gamma != nullptr) {
+              float g[E];
+              load_chunk<V, E, false>(gamma + (int64_t)c * E, g);
+#pragma unroll
+              for (int e = 0; e < E; ++e) o[e] = g[e] * o[e];
+            }
+          }
+          store_chunk<V, E>(yr + (int64_t)c * E, o);
+        }
+      }
+      if (c0 == 0) {
+        if constexpr (!RMS) mean[row] = mu;
+        invvar[row] = rs;
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// forward, generic (any n2, any alignment): one 256-thread workgroup per row,
+// streaming Welford per thread merged with Chan's formula; second pass
+// re-reads the row (L2-resident).
+// ---------------------------------------------------------------------------
+struct Wf {
+  float n, mu, m2;
+};
+__device__ __forceinline__ Wf wf_merge(Wf a, Wf b) {
+  const float n = a.n + b.n;
+  if (n == 0.f) return Wf{0.f, 0.f, 0.f};
+  const float d = b.mu - a.mu;
+  const float fb = b.n / n;
+  return Wf{n, a.mu + d * fb, a.m2 + b.m2 + d * d * a.n * fb};
+}
+
+template <typename T, typename V, bool RMS>
+__global__ __launch_bounds__(256) void norm_fwd_generic_kernel(
+    const T *__restrict__ x, const V *__restrict__ gamma,
+    const V *__restrict__ beta, V *__restrict__ y, float *__restrict__ mean,
+    float *__restrict__ invvar, int64_t n1, int64_t n2, float eps) {
+  __shared__ float sh[3][4];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  for (int64_t row = blockIdx.x; row < n1; row += gridDim.x) {
+    const T *xr = x + row * n2;
+    Wf w{0.f, 0.f, 0.f};
+    for (int64_t i = tid; i < n2; i += 256) {
+      const float v = io<T>::from_scalar(xr[i]);
+      if constexpr (RMS) {
+        w.m2 += v * v;
+      } else {
+        w.n += 1.f;
+        const float d = v - w.mu;
+        w.mu += d / w.n;
+        w.m2 += d * (v - w.mu);
+      }
+    }
+#pragma unroll
+    for (int m = 1; m < 64; m <<= 1) {
+      Wf o{__shfl_xor(w.n, m, 64), __shfl_xor(w.mu, m, 64),
+           __shfl_xor(w.m2, m, 64)};
+      if constexpr (RMS)
+        w.m2 += o.m2;
+      else
+        w = wf_merge(w, o);
+    }
+    if (lane == 0) {
+      sh[0][wave] = w.n;
+      sh[1][wave] = w.mu;
+      sh[2][wave] = w.m2;
+    }
+    __syncthreads();
+    Wf t{sh[0][0], sh[1][0], sh[2][0]};
+    for (int k = 1; k < 4; ++k) {
+      Wf o{sh[0][k], sh[1][k], sh[2][k]};
+      if constexpr (RMS)
+        t.m2 += o.m2;
+      else
+        t = wf_merge(t, o);
+    }
+    __syncthreads();
+    const float mu = RMS ? 0.f : t.mu;
+    const float rs = 1.0f / sqrtf(t.m2 / (float)n2 + eps);
+    V *yr = y + row * n2;
+    for (int64_t i = tid; i < n2; i += 256) {
+      const float v = io<T>::from_scalar(xr[i]);
+      float o;
+      if constexpr (!RMS) {
+        o = (v - mu) * rs;
+        if (gamma != nullptr)
+          o = o * io<V>::from_scalar(gamma[i]) + io<V>::from_scalar(beta[i]);
+      } else {
+        o = io<V>::round(v * rs);
+        if (gamma != nullptr) o = io<V>::from_scalar(gamma[i]) * o;
+      }
+      yr[i] = io<V>::to_scalar(o);
+    }
+    if (tid == 0) {
+      if constexpr (!RMS) mean[row] = mu;
+      invvar[row] = rs;
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// backward, register-resident, single pass
+// ---------------------------------------------------------------------------
+template <typename T, typename V, int VPL, bool RMS>
+__global__ __launch_bounds__(1024) void norm_bwd_reg_kernel(
+    const V *__restrict__ dy, const T *__restrict__ x,
+    const float *__restrict__ mean, const float *__restrict__ invvar,
+    const V *__restrict__ gamma, T *__restrict__ dx, float *__restrict__ part,
+    int64_t n1, int n2, int wpr, int rpb) {
+  constexpr int E = chunk_elems<T, V>::value;
+  extern __shared__ float xslot[];  // [n2] when rpb > 1
+  __shared__ float red[2][32];
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int rslot = wave / wpr;
+  const int first = rslot * wpr;
+  const int nchunks = n2 / E;
+  const int cstride = kWave * wpr;
+  const int c0 = (wave - first) * kWave + lane;
+  const float fn = (float)n2;
+  const bool affine = gamma != nullptr;
+
+  float gm[VPL][E], acc_g[VPL][E], acc_b[VPL][E];
+#pragma unroll
+  for (int k = 0; k < VPL; ++k) {
+    const int c = c0 + k * cstride;
+    if (affine && c < nchunks) {
+      load_chunk<V, E, false>(gamma + (int64_t)c * E, gm[k]);
+    } else {
+#pragma unroll
+      for (int e = 0; e < E; ++e) gm[k][e] = 1.f;
+    }
+#pragma unroll
+    for (int e = 0; e < E; ++e) {
+      acc_g[k][e] = 0.f;
+      acc_b[k][e] = 0.f;
+    }
+  }
+
+  int parity = 0;
+  for (int64_t base = (int64_t)blockIdx.x * rpb; base < n1;
+       base += (int64_t)gridDim.x * rpb) {
+    const int64_t row = base + rslot;
+    const bool rvalid = row < n1;
+    const V *dyr = dy + row * n2;
+    const T *xr = x + row * n2;
+    float d[VPL][E], xh[VPL][E];
+#pragma unroll
+    for (int k = 0; k < VPL; ++k) {
+      const int c = c0 + k * cstride;
+      if (rvalid && c < nchunks) {
+        load_chunk<V, E>(dyr + (int64_t)c * E, d[k]);
+        load_chunk<T, E>(xr + (int64_t)c * E, xh[k]);
+      } else {
+#pragma unroll
+        for (int e = 0; e < E; ++e) {
+          d[k][e] = 0.f;
+          xh[k][e] = 0.f;
+        }
+      }
+    }
+    float mu = 0.f, rs = 0.f;
+    if (rvalid) {
+      if constexpr (!RMS) mu = mean[row];
+      rs = invvar[row];
+    }
+    float s1 = 0.f, s2 = 0.f;
+#pragma unroll
+    for (int k = 0; k < VPL; ++k) {
+#pragma unroll
+      for (int e = 0; e < E; ++e) {
+        const float h = (xh[k][e] - mu) * rs;  // normalised input
+        const float dg = d[k][e] * gm[k][e];
+        xh[k][e] = h;
+        s1 += dg;
+        s2 += dg * h;
+        acc_g[k][e] += d[k][e] * h;
+        acc_b[k][e] += d[k][e];
+      }
+    }
+    if constexpr (RMS) {
+      s2 = row_sum1(s2, red[parity], wave, first, wpr, lane);
+      s1 = 0.f;
+    } else {
+      row_sum2(s1, s2, red[parity], wave, first, wpr, lane);
+    }
+    parity ^= 1;
+    const float term = rs / fn;
+    if (rvalid) {
+      T *dxr = dx + row * n2;
+#pragma unroll
+      for (int k = 0; k < VPL; ++k) {
+        const int c = c0 + k * cstride;
+        if (c < nchunks) {
+          float o[E];
+#pragma unroll
+          for (int e = 0; e < E; ++e) {
+            float f = fn * d[k][e] * gm[k][e];
+            f -= s1;
+            f -= xh[k][e] * s2;
+            o[e] = f * term;
+          }
+          store_chunk<T, E>(dxr + (int64_t)c * E, o);
+        }
+      }
+    }
+  }
+
+  if (part == nullptr) return;  // uniform: no parameter gradients wanted
+
+  // Fold the row slots of this workgroup into slot 0, one slot at a time.
+  constexpr int NARR = RMS ? 1 : 2;
+#pragma unroll
+  for (int a = 0; a < NARR; ++a) {
+    for (int s = 1; s < rpb; ++s) {
+      __syncthreads();
+      if (rslot == s) {
+#pragma unroll
+        for (int k = 0; k < VPL; ++k) {
+          const int c = c0 + k * cstride;
+          if (c < nchunks) {
+#pragma unroll
+            for (int e = 0; e < E; ++e)
+              xslot[c * E + e] = a == 0 ? acc_g[k][e] : acc_b[k][e];
+          }
+        }
+      }
+      __syncthreads();
+      if (rslot == 0) {
+#pragma unroll
+        for (int k = 0; k < VPL; ++k) {
+          const int c = c0 + k * cstride;
+          if (c < nchunks) {
+#pragma unroll
+            for (int e = 0; e < E; ++e) {
+              if (a == 0)
+                acc_g[k][e] += xslot[c * E + e];
+              else
+                acc_b[k][e] += xslot[c * E + e];
+            }
+          }
+        }
+      }
+    }
+  }
+  if (rslot == 0) {
+    const int64_t P = gridDim.x;
+#pragma unroll
+    for (int a = 0; a < NARR; ++a) {
+      float *prow = part + ((int64_t)a * P + blockIdx.x) * n2;
+#pragma unroll
+      for (int k = 0; k < VPL; ++k) {
+        const int c = c0 + k * cstride;
+        if (c < nchunks)
+          store_chunk<float, E>(prow + (int64_t)c * E,
+                                a == 0 ? acc_g[k] : acc_b[k]);
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// backward, generic: dx per row by one workgroup (two passes over the row),
+// parameter gradients by one thread per column walking all rows.
+// ---------------------------------------------------------------------------
+template <typename T, typename V, bool RMS>
+__global__ __launch_bounds__(256) void norm_bwd_dx_generic_kernel(
+    const V *__restrict__ dy, const T *__restrict__ x,
+    const float *__restrict__ mean, const float *__restrict__ invvar,
+    const V *__restrict__ gamma, T *__restrict__ dx, int64_t n1, int64_t n2) {
+  __shared__ float sh[2][4];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  for (int64_t row = blockIdx.x; row < n1; row += gridDim.x) {
+    const V *dyr = dy + row * n2;
+    const T *xr = x + row * n2;
+    const float mu = RMS ? 0.f : mean[row];
+    const float rs = invvar[row];
+    float s1 = 0.f, s2 = 0.f;
+    for (int64_t i = tid; i < n2; i += 256) {
+      const float g = gamma ? io<V>::from_scalar(gamma[i]) : 1.f;
+      const float dg = io<V>::from_scalar(dyr[i]) * g;
+      const float h = (io<T>::from_scalar(xr[i]) - mu) * rs;
+      s1 += dg;
+      s2 += dg * h;
+    }
+    s1 = wave_sum(s1);
+    s2 = wave_sum(s2);
+    if (lane == 0) {
+      sh[0][wave] = s1;
+      sh[1][wave] = s2;
+    }
+    __syncthreads();
+    s1 = (sh[0][0] + sh[0][1]) + (sh[0][2] + sh[0][3]);
+    s2 = (sh[1][0] + sh[1][1]) + (sh[1][2] + sh[1][3]);
+    __syncthreads();
+    if constexpr (RMS) s1 = 0.f;
+    const float fn = (float)n2;
+    const float term = rs / fn;
+    T *dxr = dx + row * n2;
+    for (int64_t i = tid; i < n2; i += 256) {
+      const float g = gamma ? io<V>::from_scalar(gamma[i]) : 1.f;
+      const float h = (io<T>::from_scalar(xr[i]) - mu) * rs;
+      float f = fn * io<V>::from_scalar(dyr[i]) * g;
+      f -= s1;
+      f -= h * s2;
+      dxr[i] = io<T>::to_scalar(f * term);
+    }
+  }
+}
+
+template <typename T, typename V, bool RMS>
+__global__ __launch_bounds__(256) void norm_bwd_param_generic_kernel(
+    const V *__restrict__ dy, const T *__restrict__ x,
+    const float *__restrict__ mean, const float *__restrict__ invvar,
+    V *__restrict__ dgamma, V *__restrict__ dbeta, int64_t n1, int64_t n2) {
+  const int64_t col = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (col >= n2) return;
+  float ag = 0.f, ab = 0.f;
+  for (int64_t row = 0; row < n1; ++row) {
+    const float mu = RMS ? 0.f : mean[row];
+    const float d = io<V>::from_scalar(dy[row * n2 + col]);
+    ag += d * (io<T>::from_scalar(x[row * n2 + col]) - mu) * invvar[row];
+    ab += d;
+  }
+  dgamma[col] = io<V>::to_scalar(ag);
+  if constexpr (!RMS) dbeta[col] = io<V>::to_scalar(ab);
+}
+
+// ---------------------------------------------------------------------------
+// host side
+// ---------------------------------------------------------------------------
+struct RowSplit {
+  int vpl;  // chunks per lane (template value)
+  int wpr;  // waves per row
+  int rpb;  // rows per workgroup iteration
+  bool ok;
+};
+
+// Splits a row of `nchunks` chunks over waves so that a lane holds at most
+// `cap` chunks; `allowed` lists the instantiated VPL values (ascending).
+static RowSplit split_row(int64_t nchunks, int cap, const int *allowed,
+                          int nallowed, int min_waves) {
+  RowSplit r{0, 1, 1, false};
+  if (nchunks <= 0) return r;
+  int64_t wpr = ceil_div(nchunks, (int64_t)kWave * cap);
+  if (wpr > 16) return r;
+  int64_t vpl = ceil_div(nchunks, kWave * wpr);
+  for (int i = 0; i < nallowed; ++i) {
+    if (allowed[i] >= vpl) {
+      r.vpl = allowed[i];
+      r.wpr = (int)wpr;
+      int rpb = min_waves / r.wpr;
+      if (rpb < 1) rpb = 1;
+      while (rpb * r.wpr > 16) --rpb;
+      r.rpb = rpb;
+      r.ok = true;
+      return r;
+    }
+  }
+  return r;
+}
+
+int64_t colsum_parts_norm(int64_t n1, int64_t n2) {
+  (void)n2;
+  int bpc = g_tune.norm_bwd_blocks_per_cu > 0 ? g_tune.norm_bwd_blocks_per_cu : 1;
+  int64_t p = (int64_t)device_cu_count() * bpc;
+  if (p > n1) p = n1;
+  if (p < 1) p = 1;
+  return p;
+}
+
+template <typename T, typename V, bool RMS>
+static int launch_norm_fwd(const void *x, const void *gamma, const void *beta,
+                           void *y, float *mean, float *invvar, int64_t n1,
+                           int64_t n2, float eps, hipStream_t st) {
+  constexpr int E = chunk_elems<T, V>::value;
+  const bool vec_ok = n2 % E == 0 && aligned16(x) && aligned16(y) &&
+                      aligned16(gamma) && aligned16(beta) &&
+                      n2 <= (int64_t)kWave * 16 * 8 * E;
+  static const int kVpl[] = {1, 2, 4, 8};
+  RowSplit sp{0, 1, 1, false};
+  if (vec_ok) {
+    const int cap = g_tune.norm_fwd_vpl > 0 ? g_tune.norm_fwd_vpl : 4;
+    sp = split_row(n2 / E, cap > 8 ? 8 : cap, kVpl, 4, 4);
+    // more than 32 resident elements per lane only fit the register budget
+    // of a workgroup of at most 256 threads
+    if (sp.ok && sp.wpr * sp.rpb > 4 && sp.vpl * E > 32)
+      sp = split_row(n2 / E, 32 / E, kVpl, 4, 4);
+  }
+  if (!sp.ok) {
+    int64_t grid = n1 < 65535 * 16 ? n1 : 65535 * 16;
+    norm_fwd_generic_kernel<T, V, RMS><<<dim3((unsigned)grid), 256, 0, st>>>(
+        (const T *)x, (const V *)gamma, (const V *)beta, (V *)y, mean, invvar,
+        n1, n2, eps);
+    return check_launch("norm_fwd_generic_kernel");
+  }
+  const int threads = kWave * sp.wpr * sp.rpb;
+  int64_t grid = ceil_div(n1, sp.rpb);
+  const int64_t maxgrid = (int64_t)device_cu_count() * 64;
+  if (grid > maxgrid) grid = maxgrid;
+#define OSLO_FWD_CASE(VPL)                                                  \
+  case VPL:                                                                 \
+    if (threads <= 256)                                                     \
+      norm_fwd_reg_kernel<T, V, VPL, RMS, 256>                              \
+          <<<dim3((unsigned)grid), threads, 0, st>>>(                       \
+              (const T *)x, (const V *)gamma, (const V *)beta, (V *)y,      \
+              mean, invvar, n1, (int)n2, eps, sp.wpr, sp.rpb);              \
+    else if constexpr (VPL * E <= 32)                                       \
+      norm_fwd_reg_kernel<T, V, VPL, RMS, 1024>                             \
+          <<<dim3((unsigned)grid), threads, 0, st>>>(                       \
+              (const T *)x, (const V *)gamma, (const V *)beta, (V *)y,      \
+              mean, invvar, n1, (int)n2, eps, sp.wpr, sp.rpb);              \
+    else                                                                    \
+      return fail(OSLO_ERR_UNSUPPORTED,                                     \
+                  "norm fwd: vpl=%d needs a workgroup of at most 256 "      \
+                  "threads", VPL);                                          \
+    break;
+  switch (sp.vpl) {
+    OSLO_FWD_CASE(1)
+    OSLO_FWD_CASE(2)
+    OSLO_FWD_CASE(4)
+    OSLO_FWD_CASE(8)
+    default:
+      return fail(OSLO_ERR_UNSUPPORTED, "norm fwd: no kernel for vpl=%d", sp.vpl);
+  }
+#undef OSLO_FWD_CASE
+  return check_launch("norm_fwd_reg_kernel");
+}
+
+template <typename T, typename V, bool RMS>
+static int launch_norm_bwd(const void *dy, const void *x, const float *mean,
+                           const float *invvar, const void *gamma, void *dx,
+                           void *dgamma, void *dbeta, void *ws,
+                           int64_t ws_bytes, int64_t n1, int64_t n2,
+                           hipStream_t st) {
+  constexpr int E = chunk_elems<T, V>::value;
+  constexpr int NARR = RMS ? 1 : 2;
+  const bool want_params = dgamma != nullptr;
+  const bool vec_ok = n2 % E == 0 && aligned16(dy) && aligned16(x) &&
+                      aligned16(dx) && aligned16(gamma) && aligned16(ws) &&
+                      n2 <= (int64_t)kWave * 16 * (16 / E) * E;
+  // at most 16 elements per lane: 5 register arrays of that size stay
+  // below the 128-VGPR budget of a 1024-thread workgroup
+  static const int kVpl8[] = {1, 2};
+  static const int kVpl4[] = {1, 2, 4};
+  RowSplit sp{0, 1, 1, false};
+  if (vec_ok) {
+    int cap = g_tune.norm_bwd_vpl > 0 ? g_tune.norm_bwd_vpl : 16 / E;
+    if (cap > 16 / E) cap = 16 / E;
+    sp = split_row(n2 / E, cap, E == 8 ? kVpl8 : kVpl4, E == 8 ? 2 : 3, 16);
+  }
+  if (!sp.ok) {
+    int64_t grid = n1 < 65535 * 16 ? n1 : 65535 * 16;
+    norm_bwd_dx_generic_kernel<T, V, RMS><<<dim3((unsigned)grid), 256, 0, st>>>(
+        (const V *)dy, (const T *)x, mean, invvar, (const V *)gamma, (T *)dx,
+        n1, n2);
+    int rc = check_launch("norm_bwd_dx_generic_kernel");
+    if (rc != OSLO_OK || !want_params) return rc;
+    norm_bwd_param_generic_kernel<T, V, RMS>
+        <<<dim3((unsigned)ceil_div(n2, 256)), 256, 0, st>>>(
+            (const V *)dy, (const T *)x, mean, invvar, (V *)dgamma,
+            (V *)dbeta, n1, n2);
+    return check_launch("norm_bwd_param_generic_kernel");
+  }
+  int64_t P = colsum_parts_norm(n1, n2);
+  if (P > ceil_div(n1, sp.rpb)) P = ceil_div(n1, sp.rpb);
+  float *part = nullptr;
+  if (want_params) {
+    const int64_t need = (int64_t)NARR * P * n2 * (int64_t)sizeof(float);
+    if (ws == nullptr || ws_bytes < need)
+      return fail(OSLO_ERR_WORKSPACE,
+                  "norm bwd: workspace of %lld bytes needed, %lld given",
+                  (long long)need, (long long)ws_bytes);
+    part = (float *)ws;
+  }
+  const int threads = kWave * sp.wpr * sp.rpb;
+  const size_t lds = sp.rpb > 1 ? (size_t)n2 * sizeof(float) : 0;
+#define OSLO_BWD_CASE(VPL)                                                   \
+  case VPL:                                                                  \
+    if constexpr (VPL * E <= 16)                                             \
+      norm_bwd_reg_kernel<T, V, VPL, RMS>                                    \
+          <<<dim3((unsigned)P), threads, lds, st>>>(                         \
+              (const V *)dy, (const T *)x, mean, invvar, (const V *)gamma,   \
+              (T *)dx, part, n1, (int)n2, sp.wpr, sp.rpb);                   \
+    break;
+  switch (sp.vpl) {
+    OSLO_BWD_CASE(1)
+    OSLO_BWD_CASE(2)
+    OSLO_BWD_CASE(4)
+    default:
+      return fail(OSLO_ERR_UNSUPPORTED, "norm bwd: no kernel for vpl=%d", sp.vpl);
+  }
+#undef OSLO_BWD_CASE
+  int rc = check_launch("norm_bwd_reg_kernel");
+  if (rc != OSLO_OK || !want_params) return rc;
+  return launch_colsum_finalize<V>(part, P, n2, dgamma, RMS ? nullptr : dbeta,
+                                   st);
+}
+
+static int check_norm_dtypes(int din, int dout) {
+  if (!valid_dtype(din) || !valid_dtype(dout))
+    return fail(OSLO_ERR_INVALID_ARGUMENT, "unknown dtype (%d, %d)", din, dout);
+  if (din != OSLO_DTYPE_F32 && din != dout)
+    return fail(OSLO_ERR_UNSUPPORTED,
+                "dtype pair (in=%d, out=%d) unsupported: a 16-bit input "
+                "requires the same output type",
+                din, dout);
+  return OSLO_OK;
+}
+
+// Expands to a call of FN<T, V, RMS> for the allowed dtype pairs.
+#define OSLO_NORM_DISPATCH(din, dout, RMS, FN, ...)                          \
+  do {                                                                       \
+    if (din == OSLO_DTYPE_F32 && dout == OSLO_DTYPE_F32)                     \
+      return FN<float, float, RMS>(__VA_ARGS__);                             \
+    if (din == OSLO_DTYPE_F32 && dout == OSLO_DTYPE_F16)                     \
+      return FN<float, _Float16, RMS>(__VA_ARGS__);                          \
+    if (din == OSLO_DTYPE_F32 && dout == OSLO_DTYPE_BF16)                    \
+      return FN<float, __bf16, RMS>(__VA_ARGS__);                            \
+    if (din == OSLO_DTYPE_F16) return FN<_Float16, _Float16, RMS>(__VA_ARGS__); \
+    return FN<__bf16, __bf16, RMS>(__VA_ARGS__);                             \
+  } while (0)
+
+static int norm_fwd_entry(bool rms, const void *x, const void *gamma,
+                          const void *beta, void *y, float *mean,
+                          float *invvar, int64_t n1, int64_t n2, double eps,
+                          int din, int dout, void *stream) {
+  int rc = check_norm_dtypes(din, dout);
+  if (rc != OSLO_OK) return rc;
+  OSLO_REQUIRE(n1 >= 0 && n2 >= 1, "norm fwd: bad shape [%lld, %lld]",
+               (long long)n1, (long long)n2);
+  OSLO_REQUIRE(n2 <= 0x7fffffff, "norm fwd: n2 too large");
+  if (n1 == 0) return OSLO_OK;
+  OSLO_REQUIRE(x && y && invvar, "norm fwd: null tensor pointer");
+  OSLO_REQUIRE(rms || mean, "layer norm fwd: null mean pointer");
+  OSLO_REQUIRE(rms || (gamma == nullptr) == (beta == nullptr),
+               "layer norm fwd: gamma and beta must both be given or both be "
+               "NULL");
+  hipStream_t st = (hipStream_t)stream;
+  if (rms)
+    OSLO_NORM_DISPATCH(din, dout, true, launch_norm_fwd, x, gamma, nullptr, y,
+                       nullptr, invvar, n1, n2, (float)eps, st);
+  OSLO_NORM_DISPATCH(din, dout, false, launch_norm_fwd, x, gamma, beta, y,
+                     mean, invvar, n1, n2, (float)eps, st);
+}
+
+static int norm_bwd_entry(bool rms, const void *dy, const void *x,
+                          const float *mean, const float *invvar,
+                          const void *gamma, void *dx, void *dgamma,
+                          void *dbeta, void *ws, int64_t ws_bytes, int64_t n1,
+                          int64_t n2, int din, int dout, void *stream) {
+  int rc = check_norm_dtypes(din, dout);
+  if (rc != OSLO_OK) return rc;
+  OSLO_REQUIRE(n1 >= 0 && n2 >= 1, "norm bwd: bad shape [%lld, %lld]",
+               (long long)n1, (long long)n2);
+  OSLO_REQUIRE(n2 <= 0x7fffffff, "norm bwd: n2 too large");
+  OSLO_REQUIRE(gamma != nullptr || dgamma == nullptr,
+               "norm bwd: dgamma requested without gamma");
+  OSLO_REQUIRE(rms || (dgamma == nullptr) == (dbeta == nullptr),
+               "layer norm bwd: dgamma and dbeta must both be given or both be "
+               "NULL");
+  if (n1 == 0) {
+    // an empty batch still defines zero parameter gradients
+    hipStream_t st0 = (hipStream_t)stream;
+    if (dgamma)
+      (void)hipMemsetAsync(dgamma, 0, (size_t)n2 * dtype_size(dout), st0);
+    if (dbeta)
+      (void)hipMemsetAsync(dbeta, 0, (size_t)n2 * dtype_size(dout), st0);
+    return OSLO_OK;
+  }
+  OSLO_REQUIRE(dy && x && invvar && dx, "norm bwd: null tensor pointer");
+  OSLO_REQUIRE(rms || mean, "layer norm bwd: null mean pointer");
+  hipStream_t st = (hipStream_t)stream;
+  if (rms)
+    OSLO_NORM_DISPATCH(din, dout, true, launch_norm_bwd, dy, x, nullptr, invvar,
+                       gamma, dx, dgamma, nullptr, ws, ws_bytes, n1, n2, st);
+  OSLO_NORM_DISPATCH(din, dout, false, launch_norm_bwd, dy, x, mean, invvar,
+                     gamma, dx, dgamma, dbeta, ws, ws_bytes, n1, n2, st);
+}
+
+}  // namespace oslo
+
+extern "C" {
+
+int oslo_ln_fwd(const void *x, const void *gamma, const void *beta, void *y,
+                float *mean, float *invvar, int64_t n1, int64_t n2, double eps,
+                int dtype_in, int dtype_out, void *stream) {
+  return oslo::norm_fwd_entry(false, x, gamma, beta, y, mean, invvar, n1, n2,
+                              eps, dtype_in, dtype_out, stream);
+}
+
+int oslo_rms_fwd(const void *x, const void *gamma, void *y, float *invvar,
+                 int64_t n1, int64_t n2, double eps, int dtype_in,
+                 int dtype_out, void *stream) {
+  return oslo::norm_fwd_entry(true, x, gamma, nullptr, y, nullptr, invvar, n1,
+                              n2, eps, dtype_in, dtype_out, stream);
+}
+
+int oslo_ln_bwd(const void *dy, const void *x, const float *mean,
+                const float *invvar, const void *gamma, void *dx, void *dgamma,
+                void *dbeta, void *workspace, int64_t workspace_bytes,
+                int64_t n1, int64_t n2, int dtype_in, int dtype_out,
+                void *stream) {
+  return oslo::norm_bwd_entry(false, dy, x, mean, invvar, gamma, dx, dgamma,
+                              dbeta, workspace, workspace_bytes, n1, n2,
+                              dtype_in, dtype_out, stream);
+}
+
+int oslo_rms_bwd(const void *dy, const void *x, const float *invvar,
+                 const void *gamma, void *dx, void *dgamma, void *workspace,
+                 int64_t workspace_bytes, int64_t n1, int64_t n2, int dtype_in,
+                 int dtype_out, void *stream) {
+  return oslo::norm_bwd_entry(true, dy, x, nullptr, invvar, gamma, dx, dgamma,
+                              nullptr, workspace, workspace_bytes, n1, n2,
+                              dtype_in, dtype_out, stream);
+}
+
+}  // extern "C"

@@ -1,0 +1,657 @@
+// Scaled causal (upper-triangular) and padding-masked softmax, forward and
+// backward, for gfx950.
+//
+// A row of sk keys is held in registers by `wpr` wavefronts (one wavefront
+// for sk <= 64 * VPL * E); a wavefront processes RPW rows at once so that
+// short rows still keep several 128-bit loads in flight per lane.  Keys that
+// are masked out are never loaded: the causal kernels stop at the diagonal,
+// the masked kernels read the mask bytes of a chunk first and skip the chunk
+// when all of them are set.  Probabilities of masked keys are written as
+// exact zeros.
+//
+// Semantics: oslo/transformers/models/gpt2/modeling_gpt2.py:116-138 (causal),
+// oslo/transformers/models/bert/modeling_bert.py:298-306 (additive padding
+// mask); entry-point shapes follow
+// oslo/torch/_C/csrc/FusedScaleMaskSoftmaxBinder.cpp:39-105.
+#include "capi.h"
+#include "common.cuh"
+
+namespace oslo {
+
+constexpr int kModeCausal = 0;
+constexpr int kModeMasked = 1;
+constexpr int kModeDense = 2;  // backward without a mask
+
+constexpr float kLog2e = 1.4426950408889634f;
+
+struct SoftmaxGeom {
+  int64_t rows;     // total softmax rows
+  int sq, sk;
+  int np;           // heads (masked mode)
+  int mask_b_stride_rows;  // mask rows per batch entry: mask_sq, or 0 if mask_b == 1
+  int mask_per_query;      // 1 if mask_sq == sq else 0
+  int wpr, rpb;     // waves per row, rows per workgroup pass (without RPW)
+};
+
+__device__ __forceinline__ float row_reduce_sum(float a, float *red, int wave,
+                                                int first, int wpr, int lane) {
+  a = wave_sum(a);
+  if (wpr > 1) {
+    if (lane == 0) red[wave] = a;
+    __syncthreads();
+    float r = red[first];
+    for (int w = 1; w < wpr; ++w) r += red[first + w];
+    a = r;
+  }
+  return a;
+}
+__device__ __forceinline__ float row_reduce_max(float a, float *red, int wave,
+                                                int first, int wpr, int lane) {
+  a = wave_max(a);
+  if (wpr > 1) {
+    if (lane == 0) red[wave] = a;
+    __syncthreads();
+    float r = red[first];
+    for (int w = 1; w < wpr; ++w) r = fmaxf(r, red[first + w]);
+    a = r;
+  }
+  return a;
+}
+
+// Mask bytes of one chunk -> bit e set when key e of the chunk is masked out.
+template <int E>
+__device__ __forceinline__ uint32_t load_mask_bits(const uint8_t *p) {
+  uint32_t bits = 0;
+  if constexpr (E == 8) {
+    const u32x2 m = *reinterpret_cast<const u32x2 *>(p);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      bits |= ((m.x >> (8 * e)) & 0xffu) ? (1u << e) : 0u;
+      bits |= ((m.y >> (8 * e)) & 0xffu) ? (1u << (4 + e)) : 0u;
+    }
+  } else {
+    const uint32_t m = *reinterpret_cast<const uint32_t *>(p);
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+      bits |= ((m >> (8 * e)) & 0xffu) ? (1u << e) : 0u;
+  }
+  return bits;
+}
+
+// Row bookkeeping shared by forward and backward.  Rows are numbered so that
+// a workgroup's rows are consecutive; in causal mode the order inside an
+// attention batch is reversed (long rows first) so the tail of the launch
+// consists of the cheap rows.
+template <int MODE>
+__device__ __forceinline__ void row_setup(const SoftmaxGeom &g, int64_t r,
+                                          const uint8_t *mask, int64_t &row,
+                                          int &visible,
+                                          const uint8_t *&mrow) {
+  mrow = nullptr;
+  visible = g.sk;
+  row = r;
+  if constexpr (MODE == kModeCausal) {
+    const int64_t batch = r / g.sq;
+    const int qi = g.sq - 1 - (int)(r - batch * g.sq);
+    row = batch * g.sq + qi;
+    int v = qi + 1 + (g.sk - g.sq);
+    visible = v < 0 ? 0 : (v > g.sk ? g.sk : v);
+  } else if constexpr (MODE == kModeMasked) {
+    const int64_t bh = r / g.sq;
+    const int qi = (int)(r - bh * g.sq);
+    const int64_t bi = bh / g.np;
+    const int64_t mr =
+        bi * g.mask_b_stride_rows + (g.mask_per_query ? qi : 0);
+    mrow = mask + mr * g.sk;
+  }
+}
+
+template <typename T, int VPL, int RPW, int MODE>
+__global__ __launch_bounds__(1024) void softmax_fwd_kernel(
+    const T *__restrict__ x, const uint8_t *__restrict__ mask,
+    T *__restrict__ y, SoftmaxGeom g, float scale) {
+  constexpr int E = io<T>::EPV;
+  __shared__ float red[2][16];
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int rslot = wave / g.wpr;
+  const int first = rslot * g.wpr;
+  const int nchunks = g.sk / E;
+  const int cstride = kWave * g.wpr;
+  const int c0 = (wave - first) * kWave + lane;
+  const float ninf = -__builtin_inff();
+
+  const int64_t rbase =
+      ((int64_t)blockIdx.x * g.rpb + rslot) * RPW;  // first row of this wave
+
+  float v[RPW][VPL][E];
+  uint32_t mbits[RPW][VPL];  // bit e set: key masked out
+  int64_t row[RPW];
+  bool rvalid[RPW];
+
+#pragma unroll
+  for (int j = 0; j < RPW; ++j) {
+    const int64_t r = rbase + j;
+    rvalid[j] = r < g.rows;
+    int visible = 0;
+    const uint8_t *mrow = nullptr;
+    row[j] = 0;
+    if (rvalid[j]) row_setup<MODE>(g, r, mask, row[j], visible, mrow);
+#pragma unroll
+    for (int k = 0; k < VPL; ++k) {
+      const int c = c0 + k * cstride;
+      uint32_t mb = (1u << E) - 1u;
+      if (rvalid[j] && c < nchunks) {
+        if constexpr (MODE == kModeCausal) {
+          const int left = visible - c * E;  // visible keys in this chunk
+          mb = left >= E ? 0u : (left <= 0 ? mb : (mb & ~((1u << left) - 1u)));
+        } else {
+          mb = load_mask_bits<E>(mrow + (int64_t)c * E);
+        }
+      }
+      mbits[j][k] = mb;
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < RPW; ++j) {
+    const T *xr = x + row[j] * g.sk;
+#pragma unroll
+    for (int k = 0; k < VPL; ++k) {
+      const int c = c0 + k * cstride;
+      if (mbits[j][k] != (1u << E) - 1u) {
+        load_chunk<T, E>(xr + (int64_t)c * E, v[j][k]);
+      } else {
+#pragma unroll
+        for (int e = 0; e < E; ++e) v[j][k][e] = 0.f;
+      }
+    }
+  }
+
+  float mx[RPW];
+#pragma unroll
+  for (int j = 0; j < RPW; ++j) {
+    float m = ninf;
+#pragma unroll
+    for (int k = 0; k < VPL; ++k)
+#pragma unroll
+      for (int e = 0; e < E; ++e) {
+        const float t = (mbits[j][k] >> e) & 1u ? ninf : v[j][k][e] * scale;
+        v[j][k][e] = t;
+        m = fmaxf(m, t);
+      }
+    mx[j] = m;
+  }
+#pragma unroll
+  for (int j = 0; j < RPW; ++j)
+    mx[j] = row_reduce_max(mx[j], red[0], wave, first, g.wpr, lane);
+  // (one barrier separates the two LDS areas; RPW > 1 implies wpr == 1,
+  //  where LDS is not used at all)
+
+  float sm[RPW];
+#pragma unroll
+  for (int j = 0; j < RPW; ++j) {
+    float s = 0.f;
+    const float off = mx[j] == ninf ? 0.f : mx[j];
+#pragma unroll
+    for (int k = 0; k < VPL; ++k)
+#pragma unroll
+      for (int e = 0; e < E; ++e) {
+        const float p = __builtin_amdgcn_exp2f((v[j][k][e] - off) * kLog2e);
+        v[j][k][e] = p;  // exp2(-inf) == 0 for masked keys
+        s += p;
+      }
+    sm[j] = s;
+  }
+#pragma unroll
+  for (int j = 0; j < RPW; ++j)
+    sm[j] = row_reduce_sum(sm[j], red[1], wave, first, g.wpr, lane);
+
+#pragma unroll
+  for (int j = 0; j < RPW; ++j) {
+    if (!rvalid[j]) continue;
+    // a row without any visible key: uniform distribution, as softmax of a
+    // constant fill value gives
+    const bool empty = mx[j] == ninf;
+    const float inv = empty ? 0.f : 1.0f / sm[j];
+    const float fill = empty ? 1.0f / (float)g.sk : 0.f;
+    T *yr = y + row[j] * g.sk;
+#pragma unroll
+    for (int k = 0; k < VPL; ++k) {
+      const int c = c0 + k * cstride;
+      if (c < nchunks) {
+        float o[E];
+#pragma unroll
+        for (int e = 0; e < E; ++e) o[e] = v[j][k][e] * inv + fill;
+        store_chunk<T, E>(yr + (int64_t)c * E, o);
+      }
+    }
+  }
+}
+
+template <typename T, int VPL, int RPW, int MODE>
+__global__ __launch_bounds__(1024) void softmax_bwd_kernel(
+    const T *__restrict__ dy, const T *__restrict__ y,
+    const uint8_t *__restrict__ mask, T *__restrict__ dx, SoftmaxGeom g,
+    float scale) {
+  constexpr int E = io<T>::EPV;
+  constexpr uint32_t kAll = (1u << E) - 1u;
+  __shared__ float red[2][16];
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int rslot = wave / g.wpr;
+  const int first = rslot * g.wpr;
+  const int nchunks = g.sk / E;
+  const int cstride = kWave * g.wpr;
+  const int c0 = (wave - first) * kWave + lane;
+
+  const int64_t rbase = ((int64_t)blockIdx.x * g.rpb + rslot) * RPW;
+
+  float yv[RPW][VPL][E], gv[RPW][VPL][E];
+  bool skip[RPW][VPL];
+  int64_t row[RPW];
+  bool rvalid[RPW];
+
+#pragma unroll
+  for (int j = 0; j < RPW; ++j) {
+    const int64_t r = rbase + j;
+    rvalid[j] = r < g.rows;
+    int visible = 0;
+    const uint8_t *mrow = nullptr;
+    row[j] = 0;
+    if (rvalid[j]) row_setup<MODE>(g, r, mask, row[j], visible, mrow);
+    float anyvis = 0.f;
+#pragma unroll
+    for (int k = 0; k < VPL; ++k) {
+      const int c = c0 + k * cstride;
+      bool sk_ = true;
+      if (rvalid[j] && c < nchunks) {
+        if constexpr (MODE == kModeCausal) {
+          sk_ = visible - c * E <= 0;
+        } else if constexpr (MODE == kModeMasked) {
+          sk_ = load_mask_bits<E>(mrow + (int64_t)c * E) == kAll;
+        } else {
+          sk_ = false;
+        }
+      }
+      skip[j][k] = sk_;
+      if (!sk_) anyvis = 1.f;
+    }
+    if constexpr (MODE != kModeDense) {
+      // a row with no visible key holds the uniform distribution: read it all
+      anyvis = row_reduce_max(anyvis, red[0], wave, first, g.wpr, lane);
+      if (g.wpr > 1) __syncthreads();
+      if (anyvis == 0.f) {
+#pragma unroll
+        for (int k = 0; k < VPL; ++k)
+          skip[j][k] = !(rvalid[j] && c0 + k * cstride < nchunks);
+      }
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < RPW; ++j) {
+    const T *yr = y + row[j] * g.sk;
+    const T *gr = dy + row[j] * g.sk;
+#pragma unroll
+    for (int k = 0; k < VPL; ++k) {
+      const int c = c0 + k * cstride;
+      if (!skip[j][k]) {
+        load_chunk<T, E>(yr + (int64_t)c * E, yv[j][k]);
+        load_chunk<T, E>(gr + (int64_t)c * E, gv[j][k]);
+      } else {
+#pragma unroll
+        for (int e = 0; e < E; ++e) {
+          yv[j][k][e] = 0.f;
+          gv[j][k][e] = 0.f;
+        }
+      }
+    }
+  }
+  float s[RPW];
+#pragma unroll
+  for (int j = 0; j < RPW; ++j) {
+    float a = 0.f;
+#pragma unroll
+    for (int k = 0; k < VPL; ++k)
+#pragma unroll
+      for (int e = 0; e < E; ++e) a += yv[j][k][e] * gv[j][k][e];
+    s[j] = a;
+  }
+#pragma unroll
+  for (int j = 0; j < RPW; ++j)
+    s[j] = row_reduce_sum(s[j], red[1], wave, first, g.wpr, lane);
+
+#pragma unroll
+  for (int j = 0; j < RPW; ++j) {
+    if (!rvalid[j]) continue;
+    T *dxr = dx + row[j] * g.sk;
+#pragma unroll
+    for (int k = 0; k < VPL; ++k) {
+      const int c = c0 + k * cstride;
+      if (c < nchunks) {
+        float o[E];
+#pragma unroll
+        for (int e = 0; e < E; ++e)
+          o[e] = scale * (yv[j][k][e] * (gv[j][k][e] - s[j]));
+        store_chunk<T, E>(dxr + (int64_t)c * E, o);
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// generic kernels: any sk / alignment; one 256-thread workgroup per row,
+// three passes over the (L2-resident) row.
+// ---------------------------------------------------------------------------
+__device__ __forceinline__ float block_reduce_256(float v, float *sh, bool is_max) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  v = is_max ? wave_max(v) : wave_sum(v);
+  __syncthreads();
+  if (lane == 0) sh[wave] = v;
+  __syncthreads();
+  return is_max ? fmaxf(fmaxf(sh[0], sh[1]), fmaxf(sh[2], sh[3]))
+                : (sh[0] + sh[1]) + (sh[2] + sh[3]);
+}
+
+template <typename T, int MODE>
+__global__ __launch_bounds__(256) void softmax_fwd_generic_kernel(
+    const T *__restrict__ x, const uint8_t *__restrict__ mask,
+    T *__restrict__ y, SoftmaxGeom g, float scale) {
+  __shared__ float sh[4];
+  const float ninf = -__builtin_inff();
+  for (int64_t r = blockIdx.x; r < g.rows; r += gridDim.x) {
+    int64_t row;
+    int visible;
+    const uint8_t *mrow;
+    row_setup<MODE>(g, r, mask, row, visible, mrow);
+    const T *xr = x + row * g.sk;
+    T *yr = y + row * g.sk;
+    float m = ninf;
+    for (int i = threadIdx.x; i < g.sk; i += 256) {
+      const bool hidden = MODE == kModeCausal ? i >= visible : mrow[i] != 0;
+      if (!hidden) m = fmaxf(m, io<T>::from_scalar(xr[i]) * scale);
+    }
+    m = block_reduce_256(m, sh, true);
+    const bool empty = m == ninf;
+    float s = 0.f;
+    for (int i = threadIdx.x; i < g.sk; i += 256) {
+      const bool hidden = MODE == kModeCausal ? i >= visible : mrow[i] != 0;
+      if (!hidden)
+        s += __builtin_amdgcn_exp2f((io<T>::from_scalar(xr[i]) * scale - m) *
+                                    kLog2e);
+    }
+    s = block_reduce_256(s, sh, false);
+    const float inv = empty ? 0.f : 1.0f / s;
+    const float fill = empty ? 1.0f / (float)g.sk : 0.f;
+    for (int i = threadIdx.x; i < g.sk; i += 256) {
+      const bool hidden = MODE == kModeCausal ? i >= visible : mrow[i] != 0;
+      float p = 0.f;
+      if (!hidden)
+        p = __builtin_amdgcn_exp2f((io<T>::from_scalar(xr[i]) * scale - m) *
+                                   kLog2e);
+      yr[i] = io<T>::to_scalar(p * inv + fill);
+    }
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void softmax_bwd_generic_kernel(
+    const T *__restrict__ dy, const T *__restrict__ y, T *__restrict__ dx,
+    int64_t rows, int sk, float scale) {
+  __shared__ float sh[4];
+  for (int64_t r = blockIdx.x; r < rows; r += gridDim.x) {
+    const T *yr = y + r * sk;
+    const T *gr = dy + r * sk;
+    T *dxr = dx + r * sk;
+    float s = 0.f;
+    for (int i = threadIdx.x; i < sk; i += 256)
+      s += io<T>::from_scalar(yr[i]) * io<T>::from_scalar(gr[i]);
+    s = block_reduce_256(s, sh, false);
+    for (int i = threadIdx.x; i < sk; i += 256) {
+      const float yy = io<T>::from_scalar(yr[i]);
+      dxr[i] = io<T>::to_scalar(scale * (yy * (io<T>::from_scalar(gr[i]) - s)));
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// host side
+// ---------------------------------------------------------------------------
+struct SoftmaxPlan {
+  int vpl, rpw, wpr, rpb;
+  bool ok;
+};
+
+// max_elems: elements of one operand a lane may hold (register budget).
+static SoftmaxPlan plan_softmax(int64_t sk, int E, int max_elems) {
+  SoftmaxPlan p{0, 1, 1, 1, false};
+  if (sk % E != 0) return p;
+  const int64_t nchunks = sk / E;
+  const int maxvpl = max_elems / E;  // 8 or 4 for 16-bit types, 16 or 8 for fp32
+  int64_t wpr = ceil_div(nchunks, (int64_t)kWave * (maxvpl > 8 ? 8 : maxvpl));
+  if (wpr > 16) return p;
+  const int64_t need = ceil_div(nchunks, kWave * wpr);
+  int vpl = need <= 1 ? 1 : need <= 2 ? 2 : need <= 4 ? 4 : 8;
+  int rpw = 1;
+  if (wpr == 1) {
+    // aim at 32 resident elements per lane per operand
+    int want = g_tune.softmax_rows_per_wave > 0 ? g_tune.softmax_rows_per_wave
+                                                : 32 / (vpl * E);
+    rpw = want >= 4 ? 4 : (want >= 2 ? 2 : 1);
+    while (rpw > 1 && (rpw * vpl * E > max_elems || rpw * vpl > 8)) rpw >>= 1;
+  }
+  p.vpl = vpl;
+  p.rpw = rpw;
+  p.wpr = (int)wpr;
+  p.rpb = wpr >= 4 ? 1 : (int)(4 / wpr);
+  while (p.rpb * p.wpr > 16) --p.rpb;
+  p.ok = true;
+  return p;
+}
+
+constexpr int kFwdMaxElems = 64;  // one operand resident
+constexpr int kBwdMaxElems = 32;  // two operands resident
+
+#define OSLO_SM_CASES(LAUNCH)        \
+  if (pl.vpl == 1 && pl.rpw == 1) {  \
+    LAUNCH(1, 1);                    \
+  } else if (pl.vpl == 1 && pl.rpw == 2) { \
+    LAUNCH(1, 2);                    \
+  } else if (pl.vpl == 1 && pl.rpw == 4) { \
+    LAUNCH(1, 4);                    \
+  } else if (pl.vpl == 2 && pl.rpw == 1) { \
+    LAUNCH(2, 1);                    \
+  } else if (pl.vpl == 2 && pl.rpw == 2) { \
+    LAUNCH(2, 2);                    \
+  } else if (pl.vpl == 2 && pl.rpw == 4) { \
+    LAUNCH(2, 4);                    \
+  } else if (pl.vpl == 4 && pl.rpw == 1) { \
+    LAUNCH(4, 1);                    \
+  } else if (pl.vpl == 4 && pl.rpw == 2) { \
+    LAUNCH(4, 2);                    \
+  } else {                           \
+    LAUNCH(8, 1);                    \
+  }
+
+template <typename T, int MODE>
+static int launch_softmax_fwd(const void *x, const uint8_t *mask, void *y,
+                              SoftmaxGeom g, float scale, hipStream_t st) {
+  constexpr int E = io<T>::EPV;
+  SoftmaxPlan pl = plan_softmax(g.sk, E, kFwdMaxElems);
+  const bool vec_ok = pl.ok && aligned16(x) && aligned16(y) &&
+                      (MODE != kModeMasked ||
+                       (reinterpret_cast<uintptr_t>(mask) % E) == 0);
+  if (!vec_ok) {
+    const int64_t grid = g.rows < (int64_t)device_cu_count() * 32
+                             ? g.rows
+                             : (int64_t)device_cu_count() * 32;
+    softmax_fwd_generic_kernel<T, MODE><<<dim3((unsigned)grid), 256, 0, st>>>(
+        (const T *)x, mask, (T *)y, g, scale);
+    return check_launch("softmax_fwd_generic_kernel");
+  }
+  g.wpr = pl.wpr;
+  g.rpb = pl.rpb;
+  const int threads = kWave * pl.wpr * pl.rpb;
+  const int64_t grid = ceil_div(g.rows, (int64_t)pl.rpb * pl.rpw);
+  OSLO_REQUIRE(grid <= 0x7fffffff, "softmax fwd: too many rows");
+#define OSLO_SM_FWD(VPL, RPW)                              \
+  if constexpr (VPL * RPW * E <= kFwdMaxElems)             \
+    softmax_fwd_kernel<T, VPL, RPW, MODE>                  \
+        <<<dim3((unsigned)grid), threads, 0, st>>>(        \
+            (const T *)x, mask, (T *)y, g, scale)
+  OSLO_SM_CASES(OSLO_SM_FWD)
+#undef OSLO_SM_FWD
+  return check_launch("softmax_fwd_kernel");
+}
+
+template <typename T, int MODE>
+static int launch_softmax_bwd(const void *dy, const void *y,
+                              const uint8_t *mask, void *dx, SoftmaxGeom g,
+                              float scale, hipStream_t st) {
+  constexpr int E = io<T>::EPV;
+  SoftmaxPlan pl = plan_softmax(g.sk, E, kBwdMaxElems);
+  const bool vec_ok = pl.ok && aligned16(dy) && aligned16(y) &&
+                      aligned16(dx) &&
+                      (MODE != kModeMasked ||
+                       (reinterpret_cast<uintptr_t>(mask) % E) == 0);
+  if (!vec_ok) {
+    const int64_t grid = g.rows < (int64_t)device_cu_count() * 32
+                             ? g.rows
+                             : (int64_t)device_cu_count() * 32;
+    softmax_bwd_generic_kernel<T><<<dim3((unsigned)grid), 256, 0, st>>>(
+        (const T *)dy, (const T *)y, (T *)dx, g.rows, g.sk, scale);
+    return check_launch("softmax_bwd_generic_kernel");
+  }
+  g.wpr = pl.wpr;
+  g.rpb = pl.rpb;
+  const int threads = kWave * pl.wpr * pl.rpb;
+  const int64_t grid = ceil_div(g.rows, (int64_t)pl.rpb * pl.rpw);
+  OSLO_REQUIRE(grid <= 0x7fffffff, "softmax bwd: too many rows");
+#define OSLO_SM_BWD(VPL, RPW)                              \
+  if constexpr (VPL * RPW * E <= kBwdMaxElems)             \
+    softmax_bwd_kernel<T, VPL, RPW, MODE>                  \
+        <<<dim3((unsigned)grid), threads, 0, st>>>(        \
+            (const T *)dy, (const T *)y, mask, (T *)dx, g, scale)
+  OSLO_SM_CASES(OSLO_SM_BWD)
+#undef OSLO_SM_BWD
+  return check_launch("softmax_bwd_kernel");
+}
+
+#define OSLO_SM_DISPATCH(dtype, MODE, FN, ...)                       \
+  do {                                                               \
+    if (dtype == OSLO_DTYPE_F32) return FN<float, MODE>(__VA_ARGS__); \
+    if (dtype == OSLO_DTYPE_F16) return FN<_Float16, MODE>(__VA_ARGS__); \
+    return FN<__bf16, MODE>(__VA_ARGS__);                            \
+  } while (0)
+
+static int check_softmax_shape(const char *what, int64_t rows_outer, int64_t sq,
+                               int64_t sk, int dtype) {
+  if (!valid_dtype(dtype))
+    return fail(OSLO_ERR_INVALID_ARGUMENT, "%s: unknown dtype %d", what, dtype);
+  if (rows_outer < 0 || sq < 0 || sk < 1 || sq > 0x7fffffff || sk > 0x7fffffff)
+    return fail(OSLO_ERR_INVALID_ARGUMENT, "%s: bad shape [%lld, %lld, %lld]",
+                what, (long long)rows_outer, (long long)sq, (long long)sk);
+  return OSLO_OK;
+}
+
+}  // namespace oslo
+
+extern "C" {
+
+using namespace oslo;
+
+int oslo_softmax_causal_fwd(const void *x, void *y, int64_t attn_batches,
+                            int64_t sq, int64_t sk, float scale, int dtype,
+                            void *stream) {
+  int rc = check_softmax_shape("softmax causal fwd", attn_batches, sq, sk, dtype);
+  if (rc != OSLO_OK) return rc;
+  if (attn_batches * sq == 0) return OSLO_OK;
+  OSLO_REQUIRE(x && y, "softmax causal fwd: null tensor pointer");
+  SoftmaxGeom g{attn_batches * sq, (int)sq, (int)sk, 1, 0, 0, 1, 1};
+  OSLO_SM_DISPATCH(dtype, kModeCausal, launch_softmax_fwd, x, nullptr, y, g,
+                   scale, (hipStream_t)stream);
+}
+
+int oslo_softmax_causal_bwd(const void *dy, const void *y, void *dx,
+                            int64_t attn_batches, int64_t sq, int64_t sk,
+                            float scale, int dtype, void *stream) {
+  int rc = check_softmax_shape("softmax causal bwd", attn_batches, sq, sk, dtype);
+  if (rc != OSLO_OK) return rc;
+  if (attn_batches * sq == 0) return OSLO_OK;
+  OSLO_REQUIRE(dy && y && dx, "softmax causal bwd: null tensor pointer");
+  SoftmaxGeom g{attn_batches * sq, (int)sq, (int)sk, 1, 0, 0, 1, 1};
+  OSLO_SM_DISPATCH(dtype, kModeCausal, launch_softmax_bwd, dy, y, nullptr, dx,
+                   g, scale, (hipStream_t)stream);
+}
+
+static int masked_geom(const char *what, int64_t b, int64_t np, int64_t sq,
+                       int64_t sk, int64_t mask_b, int64_t mask_sq,
+                       SoftmaxGeom *g) {
+  if (b < 0 || np < 0 || np > 0x7fffffff)
+    return fail(OSLO_ERR_INVALID_ARGUMENT, "%s: bad batch/head count", what);
+  if (!(mask_b == 1 || mask_b == b) || !(mask_sq == 1 || mask_sq == sq))
+    return fail(OSLO_ERR_INVALID_ARGUMENT,
+                "%s: mask shape [%lld,1,%lld,%lld] does not broadcast to "
+                "[%lld,%lld,%lld,%lld]",
+                what, (long long)mask_b, (long long)mask_sq, (long long)sk,
+                (long long)b, (long long)np, (long long)sq, (long long)sk);
+  *g = SoftmaxGeom{b * np * sq,
+                   (int)sq,
+                   (int)sk,
+                   (int)(np > 0 ? np : 1),
+                   (int)(mask_b == 1 ? 0 : mask_sq),
+                   (int)(mask_sq == sq && sq != 1 ? 1 : 0),
+                   1,
+                   1};
+  return OSLO_OK;
+}
+
+int oslo_softmax_masked_fwd(const void *x, const uint8_t *mask, void *y,
+                            int64_t b, int64_t np, int64_t sq, int64_t sk,
+                            int64_t mask_b, int64_t mask_sq, float scale,
+                            int dtype, void *stream) {
+  int rc = check_softmax_shape("softmax masked fwd", b, sq, sk, dtype);
+  if (rc != OSLO_OK) return rc;
+  SoftmaxGeom g;
+  rc = masked_geom("softmax masked fwd", b, np, sq, sk, mask_b, mask_sq, &g);
+  if (rc != OSLO_OK) return rc;
+  if (g.rows == 0) return OSLO_OK;
+  OSLO_REQUIRE(x && y && mask, "softmax masked fwd: null tensor pointer");
+  OSLO_SM_DISPATCH(dtype, kModeMasked, launch_softmax_fwd, x, mask, y, g, scale,
+                   (hipStream_t)stream);
+}
+
+int oslo_softmax_masked_bwd(const void *dy, const void *y, const uint8_t *mask,
+                            void *dx, int64_t b, int64_t np, int64_t sq,
+                            int64_t sk, int64_t mask_b, int64_t mask_sq,
+                            float scale, int dtype, void *stream) {
+  int rc = check_softmax_shape("softmax masked bwd", b, sq, sk, dtype);
+  if (rc != OSLO_OK) return rc;
+  SoftmaxGeom g;
+  if (mask == nullptr) {
+    mask_b = 1;
+    mask_sq = 1;
+  }
+  rc = masked_geom("softmax masked bwd", b, np, sq, sk, mask_b, mask_sq, &g);
+  if (rc != OSLO_OK) return rc;
+  if (g.rows == 0) return OSLO_OK;
+  OSLO_REQUIRE(dy && y && dx, "softmax masked bwd: null tensor pointer");
+  if (mask == nullptr)
+    OSLO_SM_DISPATCH(dtype, kModeDense, launch_softmax_bwd, dy, y, nullptr, dx,
+                     g, scale, (hipStream_t)stream);
+  OSLO_SM_DISPATCH(dtype, kModeMasked, launch_softmax_bwd, dy, y, mask, dx, g,
+                   scale, (hipStream_t)stream);
+}
+
+int oslo_softmax_batch_per_block(int64_t sq, int64_t sk, int64_t b,
+                                 int64_t np) {
+  if (sq < 1 || sk < 1 || b < 1 || np < 1)
+    return fail(OSLO_ERR_INVALID_ARGUMENT,
+                "softmax_batch_per_block: bad shape");
+  // rows per workgroup of the 16-bit masked kernel (the reference's shim only
+  // admits fp16 / bf16); rows that do not vectorise run one row per workgroup
+  SoftmaxPlan pl = plan_softmax(sk, 8, kFwdMaxElems);
+  if (!pl.ok) return 1;
+  return pl.rpb * pl.rpw;
+}
+
+}  // extern "C"

@@ -1,0 +1,642 @@
+"""Loader and thin bindings for ``liboslo_hip.so`` (the C ABI in ``include/oslo_hip.h``).
+
+Mirrors the role of the reference's ``oslo/torch/_C/__init__.py``: lazily
+obtained kernel objects (``get_layernorm_kernel()`` at ``_C/__init__.py:193-206``
+there) whose methods have the signatures of the reference's pybind modules
+(``FusedLayerNormBinder.cpp:404-424``, ``FusedScaleMaskSoftmaxBinder.cpp:111-127``).
+Instead of JIT-compiling CUDA through ``torch.utils.cpp_extension`` the shared
+library is built ahead of time by ``hipcc`` for gfx950 and bound with ctypes;
+tensors cross the boundary as raw device pointers and every output and
+workspace is allocated here, by torch's caching allocator.
+
+A missing or unloadable library raises ``EnvironmentError`` (the reference's
+exception type, ``_C/__init__.py:200-204``); there is no fallback for GPU
+tensors.
+"""
+import ctypes
+import os
+import subprocess
+import threading
+
+import torch
+
+_CSRC_DIR = os.path.normpath(
+    os.path.join(os.path.dirname(os.path.abspath(__file__)), "..", "..", "csrc")
+)
+LIBRARY_PATH = os.path.join(_CSRC_DIR, "liboslo_hip.so")
+
+OSLO_OP_LN_BWD = 1
+OSLO_OP_RMS_BWD = 2
+OSLO_OP_BIAS_GELU_BWD = 3
+OSLO_OP_BIAS_DROPOUT_ADD_BWD = 4
+
+ABI_VERSION = 1
+
+_DTYPE_CODE = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}
+
+_lib = None
+_lib_lock = threading.Lock()
+
+_p = ctypes.c_void_p
+_i64 = ctypes.c_int64
+_u64 = ctypes.c_uint64
+_int = ctypes.c_int
+_f32 = ctypes.c_float
+_f64 = ctypes.c_double
+
+# name -> (restype, argtypes); one entry per declaration in include/oslo_hip.h
+_SIGNATURES = {
+    "oslo_hip_last_error": (ctypes.c_char_p, []),
+    "oslo_hip_arch": (ctypes.c_char_p, []),
+    "oslo_hip_abi_version": (_int, []),
+    "oslo_workspace_bytes": (_i64, [_int, _i64, _i64]),
+    "oslo_ln_fwd": (_int, [_p, _p, _p, _p, _p, _p, _i64, _i64, _f64, _int, _int, _p]),
+    "oslo_ln_bwd": (
+        _int,
+        [_p, _p, _p, _p, _p, _p, _p, _p, _p, _i64, _i64, _i64, _int, _int, _p],
+    ),
+    "oslo_rms_fwd": (_int, [_p, _p, _p, _p, _i64, _i64, _f64, _int, _int, _p]),
+    "oslo_rms_bwd": (
+        _int,
+        [_p, _p, _p, _p, _p, _p, _p, _i64, _i64, _i64, _int, _int, _p],
+    ),
+    "oslo_softmax_causal_fwd": (_int, [_p, _p, _i64, _i64, _i64, _f32, _int, _p]),
+    "oslo_softmax_causal_bwd": (_int, [_p, _p, _p, _i64, _i64, _i64, _f32, _int, _p]),
+    "oslo_softmax_masked_fwd": (
+        _int,
+        [_p, _p, _p, _i64, _i64, _i64, _i64, _i64, _i64, _f32, _int, _p],
+    ),
+    "oslo_softmax_masked_bwd": (
+        _int,
+        [_p, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _i64, _f32, _int, _p],
+    ),
+    "oslo_softmax_batch_per_block": (_int, [_i64, _i64, _i64, _i64]),
+    "oslo_bias_gelu_fwd": (_int, [_p, _p, _p, _i64, _i64, _int, _p]),
+    "oslo_bias_gelu_bwd": (_int, [_p, _p, _p, _p, _p, _p, _i64, _i64, _i64, _int, _p]),
+    "oslo_bias_dropout_add_fwd": (
+        _int,
+        [_p, _p, _p, _p, _p, _i64, _i64, _f32, _u64, _u64, _int, _p],
+    ),
+    "oslo_bias_dropout_add_bwd": (
+        _int,
+        [_p, _p, _p, _p, _i64, _i64, _i64, _f32, _u64, _u64, _int, _p],
+    ),
+    "oslo_philox_mask": (_int, [_p, _i64, _f32, _u64, _u64, _p]),
+    "oslo_philox_words": (_int, [_p, _i64, _i64, _u64, _u64, _p]),
+    "oslo_copy_probe": (_int, [_p, _p, _i64, _p]),
+    "oslo_wave_reduce_selftest": (_int, [_p, _p]),
+    "oslo_tune": (_int, [ctypes.c_char_p, _int]),
+}
+
+EXPORTED_SYMBOLS = tuple(_SIGNATURES)
+
+
+def build_library(force=False):
+    """Compiles ``liboslo_hip.so`` in place with hipcc (``make`` in ``csrc``)."""
+    cmd = ["make", "-C", _CSRC_DIR, "-j8"]
+    if force:
+        subprocess.run(["make", "-C", _CSRC_DIR, "clean"], check=True,
+                       stdout=subprocess.DEVNULL)
+    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if proc.returncode != 0:
+        raise EnvironmentError(
+            "Failed compiling the HIP kernels for gfx950 (%s):\n%s"
+            % (" ".join(cmd), proc.stdout[-4000:])
+        )
+    return LIBRARY_PATH
+
+
+def load_library():
+    """Returns the ctypes handle, loading (and if absent, building) the library."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    with _lib_lock:
+        if _lib is not None:
+            return _lib
+        if not os.path.exists(LIBRARY_PATH):
+            build_library()
+        try:
+            lib = ctypes.CDLL(LIBRARY_PATH)
+            for name, (restype, argtypes) in _SIGNATURES.items():
+                fn = getattr(lib, name)
+                fn.restype = restype
+                fn.argtypes = argtypes
+            if lib.oslo_hip_abi_version() != ABI_VERSION:
+                raise OSError(
+                    "ABI version %d, expected %d"
+                    % (lib.oslo_hip_abi_version(), ABI_VERSION)
+                )
+        except (OSError, AttributeError) as exc:
+            raise EnvironmentError(
+                "Failed loading the HIP kernels (%s): %s. Rebuild with "
+                "`make -C %s`." % (LIBRARY_PATH, exc, _CSRC_DIR)
+            ) from exc
+        _lib = lib
+    return _lib
+
+
+def _check(rc, lib):
+    if rc != 0:
+        raise RuntimeError(lib.oslo_hip_last_error().decode("utf-8", "replace"))
+
+
+def _ptr(t):
+    return None if t is None else t.data_ptr()
+
+
+def _stream(t):
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def _dtype_code(t, what):
+    try:
+        return _DTYPE_CODE[t.dtype]
+    except KeyError:
+        raise RuntimeError(
+            "%s: dtype %s is not supported by the HIP kernels "
+            "(float32, float16 and bfloat16 are)" % (what, t.dtype)
+        ) from None
+
+
+def _check_input(t, name):
+    # CHECK_INPUT of FusedLayerNormBinder.cpp:8-14
+    if not t.is_cuda:
+        raise RuntimeError("%s must be a CUDA tensor" % name)
+    if not t.is_contiguous():
+        raise RuntimeError("%s must be contiguous" % name)
+
+
+def _workspace(lib, op, n1, n2, device):
+    nbytes = lib.oslo_workspace_bytes(op, n1, n2)
+    if nbytes < 0:
+        _check(int(nbytes), lib)
+    return torch.empty(max(int(nbytes), 16), dtype=torch.uint8, device=device), int(nbytes)
+
+
+def tune(key, value):
+    """Overrides a launch heuristic of the library (0 restores the default)."""
+    lib = load_library()
+    _check(lib.oslo_tune(key.encode(), int(value)), lib)
+
+
+# ---------------------------------------------------------------------------
+# LayerNorm / RMSNorm
+# ---------------------------------------------------------------------------
+def _compute_n1_n2(input, normalized_shape):
+    # check_args / compute_n1_n2 of FusedLayerNormBinder.cpp:19-36, 59-93
+    normalized_shape = tuple(int(s) for s in normalized_shape)
+    if len(normalized_shape) < 1:
+        raise RuntimeError(
+            "Expected normalized_shape to be at least 1-dimensional, i.e., "
+            "containing at least one element, but got normalized_shape=%s"
+            % (list(normalized_shape),)
+        )
+    nd = len(normalized_shape)
+    if input.dim() < nd or tuple(input.shape[input.dim() - nd:]) != normalized_shape:
+        raise RuntimeError(
+            "Given normalized_shape=%s, expected input with shape [*, %s], but got "
+            "input of size%s"
+            % (
+                list(normalized_shape),
+                ", ".join(str(s) for s in normalized_shape),
+                list(input.shape),
+            )
+        )
+    n2 = 1
+    for s in normalized_shape:
+        n2 *= s
+    n1 = input.numel() // n2 if n2 > 0 else 0
+    return n1, n2
+
+
+def _check_param(p, normalized_shape, name):
+    if p is not None and tuple(p.shape) != tuple(int(s) for s in normalized_shape):
+        raise RuntimeError(
+            "%s of shape %s does not match normalized_shape=%s"
+            % (name, list(p.shape), list(normalized_shape))
+        )
+
+
+class _LayerNormKernel:
+    """The ten functions of the reference's ``oslo_fused_layer_norm`` module."""
+
+    def __init__(self, lib):
+        self._lib = lib
+
+    # -- forward ----------------------------------------------------------
+    def _forward(self, rms, input, normalized_shape, gamma, beta, eps, out_dtype):
+        lib = self._lib
+        _check_input(input, "input")
+        n1, n2 = _compute_n1_n2(input, normalized_shape)
+        if gamma is not None:
+            _check_param(gamma, normalized_shape, "gamma")
+            _check_param(beta, normalized_shape, "beta")
+        din = _dtype_code(input, "input")
+        output = torch.empty_like(input, dtype=out_dtype)
+        dout = _dtype_code(output, "output")
+        for name, t in (("gamma", gamma), ("beta", beta)):
+            if t is not None:
+                _check_input(t, name)
+                if t.dtype != out_dtype:
+                    raise RuntimeError(
+                        "%s has dtype %s but the output dtype is %s"
+                        % (name, t.dtype, out_dtype)
+                    )
+        invvar = torch.empty(n1, dtype=torch.float32, device=input.device)
+        with torch.cuda.device_of(input):
+            if rms:
+                rc = lib.oslo_rms_fwd(
+                    _ptr(input), _ptr(gamma), _ptr(output), _ptr(invvar),
+                    n1, n2, float(eps), din, dout, _stream(input),
+                )
+                _check(rc, lib)
+                return [output, invvar]
+            mean = torch.empty(n1, dtype=torch.float32, device=input.device)
+            rc = lib.oslo_ln_fwd(
+                _ptr(input), _ptr(gamma), _ptr(beta), _ptr(output), _ptr(mean),
+                _ptr(invvar), n1, n2, float(eps), din, dout, _stream(input),
+            )
+            _check(rc, lib)
+        return [output, mean, invvar]
+
+    def layer_norm_forward(self, input, normalized_shape, eps):
+        return self._forward(False, input, normalized_shape, None, None, eps, input.dtype)
+
+    def layer_norm_forward_affine(self, input, normalized_shape, gamma, beta, eps):
+        return self._forward(False, input, normalized_shape, gamma, beta, eps, input.dtype)
+
+    def layer_norm_forward_affine_mixed_dtypes(self, input, normalized_shape, gamma, beta, eps):
+        return self._forward(False, input, normalized_shape, gamma, beta, eps, gamma.dtype)
+
+    def rms_norm_forward(self, input, normalized_shape, eps):
+        return self._forward(True, input, normalized_shape, None, None, eps, input.dtype)
+
+    def rms_norm_forward_affine(self, input, normalized_shape, gamma, eps):
+        return self._forward(True, input, normalized_shape, gamma, None, eps, input.dtype)
+
+    def rms_norm_forward_affine_mixed_dtypes(self, input, normalized_shape, gamma, eps):
+        return self._forward(True, input, normalized_shape, gamma, None, eps, gamma.dtype)
+
+    # -- backward ---------------------------------------------------------
+    def _backward(self, rms, dout, mean, invvar, input, normalized_shape, gamma, beta):
+        lib = self._lib
+        for name, t in (("dout", dout), ("invvar", invvar), ("input", input)):
+            _check_input(t, name)
+        if not rms:
+            _check_input(mean, "mean")
+        n1, n2 = _compute_n1_n2(input, normalized_shape)
+        if dout.shape != input.shape:
+            raise RuntimeError(
+                "dout of size %s does not match input of size %s"
+                % (list(dout.shape), list(input.shape))
+            )
+        din = _dtype_code(input, "input")
+        dcode = _dtype_code(dout, "dout")
+        grad_input = torch.empty_like(input)
+        grad_gamma = grad_beta = None
+        ws, ws_bytes = None, 0
+        if gamma is not None:
+            _check_input(gamma, "gamma")
+            _check_param(gamma, normalized_shape, "gamma")
+            if gamma.dtype != dout.dtype:
+                raise RuntimeError(
+                    "gamma has dtype %s but dout has dtype %s" % (gamma.dtype, dout.dtype)
+                )
+            grad_gamma = torch.empty_like(gamma)
+            if not rms:
+                grad_beta = torch.empty_like(beta if beta is not None else gamma)
+            ws, ws_bytes = _workspace(
+                lib, OSLO_OP_RMS_BWD if rms else OSLO_OP_LN_BWD, n1, n2, input.device
+            )
+        with torch.cuda.device_of(input):
+            if rms:
+                rc = lib.oslo_rms_bwd(
+                    _ptr(dout), _ptr(input), _ptr(invvar), _ptr(gamma), _ptr(grad_input),
+                    _ptr(grad_gamma), _ptr(ws), ws_bytes, n1, n2, din, dcode,
+                    _stream(input),
+                )
+            else:
+                rc = lib.oslo_ln_bwd(
+                    _ptr(dout), _ptr(input), _ptr(mean), _ptr(invvar), _ptr(gamma),
+                    _ptr(grad_input), _ptr(grad_gamma), _ptr(grad_beta), _ptr(ws),
+                    ws_bytes, n1, n2, din, dcode, _stream(input),
+                )
+            _check(rc, lib)
+        return grad_input, grad_gamma, grad_beta
+
+    def layer_norm_backward(self, dout, mean, invvar, input, normalized_shape, eps):
+        return self._backward(False, dout, mean, invvar, input, normalized_shape, None, None)[0]
+
+    def layer_norm_backward_affine(
+        self, dout, mean, invvar, input, normalized_shape, gamma, beta, eps
+    ):
+        return list(
+            self._backward(False, dout, mean, invvar, input, normalized_shape, gamma, beta)
+        )
+
+    def rms_norm_backward(self, dout, invvar, input, normalized_shape, eps):
+        return self._backward(True, dout, None, invvar, input, normalized_shape, None, None)[0]
+
+    def rms_norm_backward_affine(self, dout, invvar, input, normalized_shape, gamma, eps):
+        gi, gg, _ = self._backward(
+            True, dout, None, invvar, input, normalized_shape, gamma, None
+        )
+        return [gi, gg]
+
+
+# ---------------------------------------------------------------------------
+# scaled masked softmax
+# ---------------------------------------------------------------------------
+class _SoftmaxKernel:
+    """The five functions of ``FusedScaleMaskSoftmaxBinder.cpp:111-127``.
+
+    The reference admits fp16 / bf16 only (``:42-44, 84-86``); fp32 is accepted
+    here as well.  ``fused_scaled_masked_softmax_backward`` takes an optional
+    ``mask`` (not in the reference signature) that lets the kernel skip loads
+    of masked keys.
+    """
+
+    def __init__(self, lib):
+        self._lib = lib
+
+    @staticmethod
+    def _mask_u8(mask):
+        if mask.dtype == torch.bool:
+            return mask.contiguous().view(torch.uint8)
+        if mask.dtype == torch.uint8:
+            return mask.contiguous()
+        return (mask != 0).contiguous().view(torch.uint8)
+
+    def fused_scaled_masked_softmax_forward(self, input, mask, scale_factor):
+        lib = self._lib
+        if input.dim() != 4:
+            raise RuntimeError("expected 4D tensor")
+        if mask.dim() != 4:
+            raise RuntimeError("expected 4D tensor")
+        _check_input(input, "input")
+        b, np_, sq, sk = input.shape
+        mb, mh, msq, msk = mask.shape
+        if mh != 1 or msk != sk or mb not in (1, b) or msq not in (1, sq):
+            raise RuntimeError(
+                "mask of size %s does not broadcast to [%d, 1, %d, %d]"
+                % (list(mask.shape), b, sq, sk)
+            )
+        m8 = self._mask_u8(mask)
+        out = torch.empty_like(input)
+        with torch.cuda.device_of(input):
+            rc = lib.oslo_softmax_masked_fwd(
+                _ptr(input), _ptr(m8), _ptr(out), b, np_, sq, sk, mb, msq,
+                float(scale_factor), _dtype_code(input, "input"), _stream(input),
+            )
+            _check(rc, lib)
+        return out
+
+    def fused_scaled_masked_softmax_backward(
+        self, output_grads, softmax_results, scale_factor, mask=None, inplace=False
+    ):
+        lib = self._lib
+        if output_grads.dim() != 4 or softmax_results.dim() != 4:
+            raise RuntimeError("expected 4D tensor")
+        _check_input(output_grads, "output_grads")
+        _check_input(softmax_results, "softmax_results")
+        if output_grads.dtype != softmax_results.dtype:
+            raise RuntimeError("output_grads and softmax_results differ in dtype")
+        b, np_, sq, sk = softmax_results.shape
+        mb = msq = 1
+        m8 = None
+        if mask is not None:
+            mb, _, msq, _ = mask.shape
+            m8 = self._mask_u8(mask)
+        # inplace=True overwrites output_grads, as the kernel this shim was
+        # written for does
+        grad_input = output_grads if inplace else torch.empty_like(output_grads)
+        with torch.cuda.device_of(output_grads):
+            rc = lib.oslo_softmax_masked_bwd(
+                _ptr(output_grads), _ptr(softmax_results), _ptr(m8), _ptr(grad_input),
+                b, np_, sq, sk, mb, msq, float(scale_factor),
+                _dtype_code(output_grads, "output_grads"), _stream(output_grads),
+            )
+            _check(rc, lib)
+        return grad_input
+
+    def get_batch_per_block(self, query_seq_len, key_seq_len, batches, attn_heads):
+        lib = self._lib
+        rc = lib.oslo_softmax_batch_per_block(
+            int(query_seq_len), int(key_seq_len), int(batches), int(attn_heads)
+        )
+        if rc < 0:
+            _check(rc, lib)
+        return int(rc)
+
+    def fused_scaled_upper_triang_masked_softmax_forward(self, input, scale_factor):
+        lib = self._lib
+        if input.dim() != 3:
+            raise RuntimeError("expected 3D tensor")
+        _check_input(input, "input")
+        ab, sq, sk = input.shape
+        out = torch.empty_like(input)
+        with torch.cuda.device_of(input):
+            rc = lib.oslo_softmax_causal_fwd(
+                _ptr(input), _ptr(out), ab, sq, sk, float(scale_factor),
+                _dtype_code(input, "input"), _stream(input),
+            )
+            _check(rc, lib)
+        return out
+
+    def fused_scaled_upper_triang_masked_softmax_backward(
+        self, output_grads, softmax_results, scale_factor, inplace=False
+    ):
+        lib = self._lib
+        if output_grads.dim() != 3 or softmax_results.dim() != 3:
+            raise RuntimeError("expected 3D tensor")
+        _check_input(output_grads, "output_grads")
+        _check_input(softmax_results, "softmax_results")
+        if output_grads.dtype != softmax_results.dtype:
+            raise RuntimeError("output_grads and softmax_results differ in dtype")
+        ab, sq, sk = softmax_results.shape
+        grad_input = output_grads if inplace else torch.empty_like(output_grads)
+        with torch.cuda.device_of(output_grads):
+            rc = lib.oslo_softmax_causal_bwd(
+                _ptr(output_grads), _ptr(softmax_results), _ptr(grad_input), ab, sq, sk,
+                float(scale_factor), _dtype_code(output_grads, "output_grads"),
+                _stream(output_grads),
+            )
+            _check(rc, lib)
+        return grad_input
+
+
+# ---------------------------------------------------------------------------
+# bias-GeLU and bias-dropout-add (TorchScript in the reference,
+# oslo/torch/nn/modules/functional.py:23-50, 295-298; native here)
+# ---------------------------------------------------------------------------
+def _rows_cols(x, bias):
+    cols = x.shape[-1] if x.dim() > 0 else 1
+    if bias is not None:
+        if bias.dim() != 1 or bias.shape[0] != cols:
+            raise RuntimeError(
+                "bias of size %s does not match the last dimension of input of size %s"
+                % (list(bias.shape), list(x.shape))
+            )
+    rows = x.numel() // cols if cols > 0 else 0
+    return rows, cols
+
+
+class _FusedElementwiseKernel:
+    def __init__(self, lib):
+        self._lib = lib
+
+    def bias_gelu_forward(self, input, bias):
+        lib = self._lib
+        _check_input(input, "input")
+        if bias is not None:
+            _check_input(bias, "bias")
+            if bias.dtype != input.dtype:
+                raise RuntimeError("bias and input differ in dtype")
+        rows, cols = _rows_cols(input, bias)
+        out = torch.empty_like(input)
+        with torch.cuda.device_of(input):
+            rc = lib.oslo_bias_gelu_fwd(
+                _ptr(input), _ptr(bias), _ptr(out), rows, cols,
+                _dtype_code(input, "input"), _stream(input),
+            )
+            _check(rc, lib)
+        return out
+
+    def bias_gelu_backward(self, grad_output, input, bias, need_bias_grad=True):
+        lib = self._lib
+        _check_input(grad_output, "grad_output")
+        _check_input(input, "input")
+        if grad_output.dtype != input.dtype or grad_output.shape != input.shape:
+            raise RuntimeError("grad_output does not match input")
+        rows, cols = _rows_cols(input, bias)
+        grad_input = torch.empty_like(input)
+        grad_bias = None
+        ws, ws_bytes = None, 0
+        if bias is not None and need_bias_grad:
+            grad_bias = torch.empty_like(bias)
+            ws, ws_bytes = _workspace(lib, OSLO_OP_BIAS_GELU_BWD, rows, cols, input.device)
+        with torch.cuda.device_of(input):
+            rc = lib.oslo_bias_gelu_bwd(
+                _ptr(grad_output), _ptr(input), _ptr(bias), _ptr(grad_input),
+                _ptr(grad_bias), _ptr(ws), ws_bytes, rows, cols,
+                _dtype_code(input, "input"), _stream(input),
+            )
+            _check(rc, lib)
+        return grad_input, grad_bias
+
+    def bias_dropout_add_forward(
+        self, input, bias, residual, p, seed, offset, out=None, return_mask=False
+    ):
+        lib = self._lib
+        _check_input(input, "input")
+        for name, t in (("bias", bias), ("residual", residual)):
+            if t is not None:
+                _check_input(t, name)
+                if t.dtype != input.dtype:
+                    raise RuntimeError("%s and input differ in dtype" % name)
+        if residual is not None and residual.shape != input.shape:
+            raise RuntimeError("residual does not match input")
+        rows, cols = _rows_cols(input, bias)
+        if out is None:
+            out = torch.empty_like(input)
+        mask = (
+            torch.empty(input.shape, dtype=torch.uint8, device=input.device)
+            if return_mask
+            else None
+        )
+        with torch.cuda.device_of(input):
+            rc = lib.oslo_bias_dropout_add_fwd(
+                _ptr(input), _ptr(bias), _ptr(residual), _ptr(out), _ptr(mask),
+                rows, cols, float(p), int(seed), int(offset),
+                _dtype_code(input, "input"), _stream(input),
+            )
+            _check(rc, lib)
+        return (out, mask) if return_mask else out
+
+    def bias_dropout_add_backward(
+        self, grad_output, p, seed, offset, need_input_grad=True, need_bias_grad=True
+    ):
+        lib = self._lib
+        _check_input(grad_output, "grad_output")
+        cols = grad_output.shape[-1]
+        rows = grad_output.numel() // cols if cols > 0 else 0
+        grad_input = torch.empty_like(grad_output) if need_input_grad else None
+        grad_bias = None
+        ws, ws_bytes = None, 0
+        if need_bias_grad:
+            grad_bias = torch.empty(cols, dtype=grad_output.dtype, device=grad_output.device)
+            ws, ws_bytes = _workspace(
+                lib, OSLO_OP_BIAS_DROPOUT_ADD_BWD, rows, cols, grad_output.device
+            )
+        if grad_input is None and grad_bias is None:
+            return None, None
+        with torch.cuda.device_of(grad_output):
+            rc = lib.oslo_bias_dropout_add_bwd(
+                _ptr(grad_output), _ptr(grad_input), _ptr(grad_bias), _ptr(ws), ws_bytes,
+                rows, cols, float(p), int(seed), int(offset),
+                _dtype_code(grad_output, "grad_output"), _stream(grad_output),
+            )
+            _check(rc, lib)
+        return grad_input, grad_bias
+
+    def philox_mask(self, n, p, seed, offset, device):
+        lib = self._lib
+        mask = torch.empty(int(n), dtype=torch.uint8, device=device)
+        with torch.cuda.device(mask.device):
+            rc = lib.oslo_philox_mask(
+                _ptr(mask), int(n), float(p), int(seed), int(offset), _stream(mask)
+            )
+            _check(rc, lib)
+        return mask
+
+    def philox_words(self, ngroups, first_group, seed, offset, device):
+        lib = self._lib
+        out = torch.empty(int(ngroups) * 4, dtype=torch.int32, device=device)
+        with torch.cuda.device(out.device):
+            rc = lib.oslo_philox_words(
+                _ptr(out), int(ngroups), int(first_group), int(seed), int(offset),
+                _stream(out),
+            )
+            _check(rc, lib)
+        return out
+
+    def copy_probe(self, src, dst):
+        lib = self._lib
+        nbytes = src.numel() * src.element_size()
+        with torch.cuda.device_of(src):
+            _check(lib.oslo_copy_probe(_ptr(src), _ptr(dst), nbytes, _stream(src)), lib)
+        return dst
+
+    def wave_reduce_selftest(self, device):
+        lib = self._lib
+        out = torch.zeros(4, dtype=torch.float32, device=device)
+        with torch.cuda.device(out.device):
+            _check(lib.oslo_wave_reduce_selftest(_ptr(out), _stream(out)), lib)
+        return out
+
+
+_layernorm_kernel = None
+_softmax_kernel = None
+_elementwise_kernel = None
+
+
+def get_layernorm_kernel():
+    global _layernorm_kernel
+    if _layernorm_kernel is None:
+        _layernorm_kernel = _LayerNormKernel(load_library())
+    return _layernorm_kernel
+
+
+def get_softmax_kernel():
+    global _softmax_kernel
+    if _softmax_kernel is None:
+        _softmax_kernel = _SoftmaxKernel(load_library())
+    return _softmax_kernel
+
+
+def get_fused_elementwise_kernel():
+    global _elementwise_kernel
+    if _elementwise_kernel is None:
+        _elementwise_kernel = _FusedElementwiseKernel(load_library())
+    return _elementwise_kernel

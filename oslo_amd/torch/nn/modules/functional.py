@@ -1,0 +1,414 @@
+"""Autograd Functions and user functions of the fused non-GEMM ops.
+
+Same names, argument order and defaults as the reference's
+``oslo/torch/nn/modules/functional.py`` (Functions ``:53-230``, user functions
+``:249-298``).  GPU tensors go to the HIP kernels through
+``oslo_amd.torch._C``; CPU tensors take the same plain-torch formulas the
+reference evaluates there (its TorchScript bodies ``:23-50, 295-298`` and the
+module fallbacks ``layer_norm.py:17-30, 452-455``).
+"""
+import torch
+from torch import Tensor
+from torch.nn import functional as F
+
+from oslo_amd.torch._C import (
+    get_fused_elementwise_kernel,
+    get_layernorm_kernel,
+    get_softmax_kernel,
+)
+
+"""
+Autograd Functions
+"""
+
+
+def _cast_if_autocast_enabled(*args):
+    # functional.py:16-20 of the reference, with the torch.amp spellings
+    if not torch.is_autocast_enabled("cuda"):
+        return args
+    dtype = torch.get_autocast_dtype("cuda")
+
+    def cast(a):
+        if isinstance(a, torch.Tensor) and a.is_floating_point() and a.is_cuda:
+            return a.to(dtype)
+        return a
+
+    return tuple(cast(a) for a in args)
+
+
+def _gelu_fwd_torch(x):
+    # functional.py:23-25
+    return x * 0.5 * (1.0 + torch.tanh(0.79788456 * x * (1 + 0.044715 * x * x)))
+
+
+def _gelu_bwd_torch(g, x):
+    # functional.py:28-34
+    tanh_out = torch.tanh(0.79788456 * x * (1 + 0.044715 * x * x))
+    ff = 0.5 * x * (
+        (1 - tanh_out * tanh_out) * (0.79788456 + 0.1070322243 * x * x)
+    ) + 0.5 * (1 + tanh_out)
+    return ff * g
+
+
+class _FusedGeLUFunction(torch.autograd.Function):
+    """
+    Kernel fusion function: GeLU
+    """
+
+    @staticmethod
+    def forward(ctx, input):
+        ctx.input_tensor = input
+        if not input.is_cuda:
+            return _gelu_fwd_torch(input)
+        return get_fused_elementwise_kernel().bias_gelu_forward(input.contiguous(), None)
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        input = ctx.input_tensor
+        if not input.is_cuda:
+            return _gelu_bwd_torch(grad_output, input)
+        grad_input, _ = get_fused_elementwise_kernel().bias_gelu_backward(
+            grad_output.contiguous(), input.contiguous(), None
+        )
+        return grad_input
+
+
+class _FusedBiasGeLUFunction(torch.autograd.Function):
+    """
+    Kernel fusion function: Bias + GeLU
+    """
+
+    @staticmethod
+    def forward(ctx, input, bias):
+        ctx.save_for_backward(input, bias)
+        if not input.is_cuda:
+            return _gelu_fwd_torch(input + bias)
+        return get_fused_elementwise_kernel().bias_gelu_forward(
+            input.contiguous(), bias.contiguous()
+        )
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        input, bias = ctx.saved_tensors
+        if not input.is_cuda:
+            # the reference returns the full-size tensor twice and lets autograd
+            # sum it down to the bias shape (functional.py:80-84)
+            tmp = _gelu_bwd_torch(grad_output, input + bias)
+            return tmp, tmp
+        grad_input, grad_bias = get_fused_elementwise_kernel().bias_gelu_backward(
+            grad_output.contiguous(),
+            input.contiguous(),
+            bias.contiguous(),
+            need_bias_grad=ctx.needs_input_grad[1],
+        )
+        return grad_input, grad_bias
+
+
+class _FusedBiasDropoutAddFunction(torch.autograd.Function):
+    """
+    Kernel fusion function: Bias + Dropout (+ residual add)
+
+    The keep mask is a pure function of (seed, offset, element index) and is
+    regenerated in backward, never stored.
+    """
+
+    @staticmethod
+    def forward(ctx, input, bias, residual, p, seed, offset, inplace):
+        kernel = get_fused_elementwise_kernel()
+        input_ = input.contiguous()
+        out = kernel.bias_dropout_add_forward(
+            input_,
+            None if bias is None else bias.contiguous(),
+            None if residual is None else residual.contiguous(),
+            p,
+            seed,
+            offset,
+            out=input_ if (inplace and input_ is input) else None,
+        )
+        if inplace and input_ is input:
+            ctx.mark_dirty(input)
+        ctx.p, ctx.seed, ctx.offset = p, seed, offset
+        ctx.has_bias = bias is not None
+        ctx.has_residual = residual is not None
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        grad_output = grad_output.contiguous()
+        need_x = ctx.needs_input_grad[0]
+        need_b = ctx.has_bias and ctx.needs_input_grad[1]
+        need_r = ctx.has_residual and ctx.needs_input_grad[2]
+        grad_input, grad_bias = get_fused_elementwise_kernel().bias_dropout_add_backward(
+            grad_output, ctx.p, ctx.seed, ctx.offset,
+            need_input_grad=need_x, need_bias_grad=need_b,
+        )
+        return grad_input, grad_bias, (grad_output if need_r else None), None, None, None, None
+
+
+def _next_philox_state(device):
+    """(seed, offset) from torch's generator of `device`; advances the offset."""
+    index = device.index if device.index is not None else torch.cuda.current_device()
+    gen = torch.cuda.default_generators[index]
+    seed = gen.initial_seed()
+    offset = gen.get_offset()
+    gen.set_offset(offset + 4)
+    return seed, offset
+
+
+def _norm_forward(ctx, rms, mixed, input, weight, bias, normalized_shape, eps):
+    """Shared forward of the six norm Functions: contiguous operands in, stats
+    saved for backward (mean only for LayerNorm)."""
+    kernel = get_layernorm_kernel()
+    ctx.normalized_shape = normalized_shape
+    ctx.eps = eps
+    ctx.rms = rms
+    ctx.affine = weight is not None
+    x = input.contiguous()
+    if not ctx.affine:
+        fwd = kernel.rms_norm_forward if rms else kernel.layer_norm_forward
+        output, *stats = fwd(x, normalized_shape, eps)
+        ctx.save_for_backward(x, *stats)
+        return output
+    w = weight.contiguous()
+    if rms:
+        fwd = (
+            kernel.rms_norm_forward_affine_mixed_dtypes
+            if mixed
+            else kernel.rms_norm_forward_affine
+        )
+        output, invvar = fwd(x, normalized_shape, w, eps)
+        ctx.save_for_backward(x, w, invvar)
+        return output
+    b = bias.contiguous()
+    fwd = (
+        kernel.layer_norm_forward_affine_mixed_dtypes
+        if mixed
+        else kernel.layer_norm_forward_affine
+    )
+    output, mean, invvar = fwd(x, normalized_shape, w, b, eps)
+    ctx.save_for_backward(x, w, b, mean, invvar)
+    return output
+
+
+def _norm_backward(ctx, grad_output):
+    """Shared backward: returns (grad_input, grad_weight, grad_bias); the last
+    two are None where the variant has no such parameter."""
+    kernel = get_layernorm_kernel()
+    g = grad_output.contiguous()
+    shape, eps = ctx.normalized_shape, ctx.eps
+    saved = ctx.saved_tensors
+    if not ctx.affine:
+        if ctx.rms:
+            x, invvar = saved
+            return kernel.rms_norm_backward(g, invvar, x, shape, eps), None, None
+        x, mean, invvar = saved
+        return kernel.layer_norm_backward(g, mean, invvar, x, shape, eps), None, None
+    if ctx.rms:
+        x, w, invvar = saved
+        gi, gw = kernel.rms_norm_backward_affine(g, invvar, x, shape, w, eps)
+        return gi, gw, None
+    x, w, b, mean, invvar = saved
+    gi, gw, gb = kernel.layer_norm_backward_affine(g, mean, invvar, x, shape, w, b, eps)
+    return gi, gw, gb
+
+
+class _FusedLayerNormAffineFunction(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, input, weight, bias, normalized_shape, eps):
+        return _norm_forward(ctx, False, False, input, weight, bias, normalized_shape, eps)
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        gi, gw, gb = _norm_backward(ctx, grad_output)
+        return gi, gw, gb, None, None
+
+
+class _FusedRMSNormAffineFunction(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, input, weight, normalized_shape, eps):
+        return _norm_forward(ctx, True, False, input, weight, None, normalized_shape, eps)
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        gi, gw, _ = _norm_backward(ctx, grad_output)
+        return gi, gw, None, None
+
+
+class _FusedLayerNormAffineMixedDtypesFunction(_FusedLayerNormAffineFunction):
+    # output in the parameters' dtype; backward inherited
+    @staticmethod
+    def forward(ctx, input, weight, bias, normalized_shape, eps):
+        return _norm_forward(ctx, False, True, input, weight, bias, normalized_shape, eps)
+
+
+class _FusedRMSNormAffineMixedDtypesFunction(_FusedRMSNormAffineFunction):
+    @staticmethod
+    def forward(ctx, input, weight, normalized_shape, eps):
+        return _norm_forward(ctx, True, True, input, weight, None, normalized_shape, eps)
+
+
+class _FusedLayerNormFunction(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, input, normalized_shape, eps):
+        return _norm_forward(ctx, False, False, input, None, None, normalized_shape, eps)
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        return _norm_backward(ctx, grad_output)[0], None, None
+
+
+class _FusedRMSNormFunction(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, input, normalized_shape, eps):
+        return _norm_forward(ctx, True, False, input, None, None, normalized_shape, eps)
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        return _norm_backward(ctx, grad_output)[0], None, None
+
+
+class _ScaledUpperTriangMaskedSoftmax(torch.autograd.Function):
+    """
+    Fused: scale -> causal (upper-triangular) mask -> softmax, on
+    [attn_batches, sq, sk] (FusedScaleMaskSoftmaxBinder.cpp:76-105).
+    Saves the output only; backward is scale * y * (g - sum(g * y)).
+    """
+
+    @staticmethod
+    def forward(ctx, inputs, scale):
+        scale = float(scale)
+        softmax_results = (
+            get_softmax_kernel().fused_scaled_upper_triang_masked_softmax_forward(
+                inputs.contiguous(), scale
+            )
+        )
+        ctx.scale = scale
+        ctx.save_for_backward(softmax_results)
+        return softmax_results
+
+    @staticmethod
+    def backward(ctx, output_grads):
+        (softmax_results,) = ctx.saved_tensors
+        input_grads = (
+            get_softmax_kernel().fused_scaled_upper_triang_masked_softmax_backward(
+                output_grads.contiguous(), softmax_results, ctx.scale
+            )
+        )
+        return input_grads, None
+
+
+class _ScaledMaskedSoftmax(torch.autograd.Function):
+    """
+    Fused: scale -> padding mask -> softmax, on [b, np, sq, sk] with a
+    [b or 1, 1, sq or 1, sk] mask, True = masked out
+    (FusedScaleMaskSoftmaxBinder.cpp:39-70).
+    """
+
+    @staticmethod
+    def forward(ctx, inputs, mask, scale):
+        scale = float(scale)
+        softmax_results = get_softmax_kernel().fused_scaled_masked_softmax_forward(
+            inputs.contiguous(), mask, scale
+        )
+        ctx.scale = scale
+        ctx.save_for_backward(softmax_results, mask)
+        return softmax_results
+
+    @staticmethod
+    def backward(ctx, output_grads):
+        softmax_results, mask = ctx.saved_tensors
+        input_grads = get_softmax_kernel().fused_scaled_masked_softmax_backward(
+            output_grads.contiguous(), softmax_results, ctx.scale, mask=mask
+        )
+        return input_grads, None, None
+
+
+"""
+User Functions
+"""
+
+
+def fused_layer_norm_affine(input, weight, bias, normalized_shape, eps=1e-6):
+    args = _cast_if_autocast_enabled(input, weight, bias, normalized_shape, eps)
+    with torch.amp.autocast("cuda", enabled=False):
+        return _FusedLayerNormAffineFunction.apply(*args)
+
+
+def fused_layer_norm(input, normalized_shape, eps=1e-6):
+    args = _cast_if_autocast_enabled(input, normalized_shape, eps)
+    with torch.amp.autocast("cuda", enabled=False):
+        return _FusedLayerNormFunction.apply(*args)
+
+
+def mixed_dtype_fused_layer_norm_affine(
+    input, weight, bias, normalized_shape, eps=1e-6
+):
+    args = _cast_if_autocast_enabled(input, weight, bias, normalized_shape, eps)
+    with torch.amp.autocast("cuda", enabled=False):
+        return _FusedLayerNormAffineMixedDtypesFunction.apply(*args)
+
+
+def fused_rms_norm_affine(input, weight, normalized_shape, eps=1e-6):
+    args = _cast_if_autocast_enabled(input, weight, normalized_shape, eps)
+    with torch.amp.autocast("cuda", enabled=False):
+        return _FusedRMSNormAffineFunction.apply(*args)
+
+
+def fused_rms_norm(input, normalized_shape, eps=1e-6):
+    args = _cast_if_autocast_enabled(input, normalized_shape, eps)
+    with torch.amp.autocast("cuda", enabled=False):
+        return _FusedRMSNormFunction.apply(*args)
+
+
+def mixed_dtype_fused_rms_norm_affine(input, weight, normalized_shape, eps=1e-6):
+    args = _cast_if_autocast_enabled(input, weight, normalized_shape, eps)
+    with torch.amp.autocast("cuda", enabled=False):
+        return _FusedRMSNormAffineMixedDtypesFunction.apply(*args)
+
+
+def fused_gelu(x):
+    return _FusedGeLUFunction.apply(x)
+
+
+def fused_bias_gelu(x, bias):
+    return _FusedBiasGeLUFunction.apply(x, bias)
+
+
+def fused_bias_dropout(x, bias, p, training, inplace):
+    # type: (Tensor, Tensor, float, bool, bool) -> Tensor
+    if not x.is_cuda:
+        return F.dropout(x + bias, p=p, training=training, inplace=inplace)
+    return fused_bias_dropout_add(x, bias, None, p, training, inplace)
+
+
+def fused_bias_dropout_add(x, bias, residual, p, training, inplace=False):
+    """dropout(x + bias) + residual in one kernel.
+
+    The reference fuses only ``dropout(x + bias)`` (functional.py:295-298) and
+    its callers add the residual next (modeling_gpt2.py:300, 369); passing the
+    residual here folds that add into the same pass.  ``bias`` and ``residual``
+    may be None.
+    """
+    if p < 0.0 or p > 1.0:
+        raise ValueError(
+            "dropout probability has to be between 0 and 1, but got {}".format(p)
+        )
+    if not x.is_cuda:
+        y = x if bias is None else x + bias
+        y = F.dropout(y, p=p, training=training, inplace=inplace and bias is None)
+        return y if residual is None else y + residual
+    p_eff = float(p) if training else 0.0
+    seed, offset = _next_philox_state(x.device) if p_eff > 0.0 else (0, 0)
+    return _FusedBiasDropoutAddFunction.apply(
+        x, bias, residual, p_eff, seed, offset, bool(inplace)
+    )
+
+
+def scaled_upper_triang_masked_softmax(input, scale=1.0):
+    """softmax(scale * input) under a causal mask; input is [attn_batches, sq, sk]."""
+    return _ScaledUpperTriangMaskedSoftmax.apply(input, scale)
+
+
+def scaled_masked_softmax(input, mask, scale=1.0):
+    """softmax(scale * input) with `mask` (True = masked out); input is [b, np, sq, sk]."""
+    return _ScaledMaskedSoftmax.apply(input, mask, scale)

@@ -1,0 +1,86 @@
+"""Shared helpers of the test-suite: seeded inputs and the parity metrics.
+
+Parity metrics (the tolerances the tests state):
+  fp32 outputs   |a - t| <= 1e-5 * |t| + atol, t = float64 oracle, atol a small
+                 multiple of the output scale for values that cancel to ~0.
+  16-bit outputs (1) against the float64 oracle rounded once to the storage
+                 type: at least 99.8 % of the elements bit-identical and no
+                 element further than 1 ulp; (2) relative L2 error against the
+                 unrounded float64 oracle <= 2e-3.
+                 (A per-element 2e-3 bound is not meaningful for bf16, whose
+                 half-ulp is 3.9e-3: two correct roundings of values 1e-7
+                 apart can differ by a full ulp.)
+"""
+import numpy as np
+import torch
+
+NP_NAME = {torch.float32: "f32", torch.float16: "f16", torch.bfloat16: "bf16"}
+
+
+def randn(shape, dtype, seed, std=1.0, mean=0.0):
+    """Seeded N(mean, std) drawn on the CPU in fp32, then cast to `dtype`."""
+    g = torch.Generator().manual_seed(seed)
+    t = torch.randn(shape, generator=g, dtype=torch.float32) * std + mean
+    return t.to(dtype)
+
+
+def f64(t):
+    """Exact values of a tensor as a float64 numpy array."""
+    return t.detach().to("cpu").to(torch.float64).numpy()
+
+
+def _ordered_int(t):
+    if t.dtype == torch.float32:
+        i = t.contiguous().view(torch.int32).to(torch.int64)
+        mag = 0x7FFFFFFF
+    else:
+        i = t.contiguous().view(torch.int16).to(torch.int64)
+        mag = 0x7FFF
+    return torch.where(i >= 0, i, -(i & mag))
+
+
+def ulp_distance(a, b):
+    """Elementwise distance in units of the storage type's spacing."""
+    assert a.dtype == b.dtype and a.shape == b.shape
+    return (_ordered_int(a.cpu()) - _ordered_int(b.cpu())).abs()
+
+
+def rel_l2(actual64, truth64):
+    num = np.linalg.norm((actual64 - truth64).ravel())
+    den = np.linalg.norm(truth64.ravel())
+    return float(num / den) if den > 0 else float(num)
+
+
+def check_lowp(actual, truth64, what, min_exact=0.998, max_ulp=1, l2_tol=2e-3):
+    """16-bit parity (see module docstring).  `actual` is a torch tensor of the
+    storage dtype, `truth64` the float64 oracle (unrounded)."""
+    actual = actual.detach().cpu()
+    expect = torch.from_numpy(np.asarray(truth64, dtype=np.float64)).to(torch.float32).to(actual.dtype)
+    expect = expect.reshape(actual.shape)
+    assert torch.isfinite(actual.float()).all(), what + ": non-finite output"
+    d = ulp_distance(actual, expect)
+    exact = float((d == 0).double().mean())
+    worst = int(d.max()) if d.numel() else 0
+    l2 = rel_l2(f64(actual), np.asarray(truth64, dtype=np.float64).reshape(actual.shape))
+    assert worst <= max_ulp, "%s: %d ulp off the rounded oracle (exact %.5f)" % (what, worst, exact)
+    assert exact >= min_exact, "%s: only %.5f bit-identical" % (what, exact)
+    assert l2 <= l2_tol, "%s: relative L2 error %.3e > %.1e" % (what, l2, l2_tol)
+    return exact, worst, l2
+
+
+def check_f32(actual, truth64, what, rtol=1e-5, atol=1e-6):
+    a = f64(actual)
+    t = np.asarray(truth64, dtype=np.float64).reshape(a.shape)
+    assert np.isfinite(a).all(), what + ": non-finite output"
+    err = np.abs(a - t)
+    bound = rtol * np.abs(t) + atol
+    bad = err > bound
+    assert not bad.any(), "%s: %d elements off, worst |err| %.3e at |t| %.3e" % (
+        what, int(bad.sum()), float(err[bad].max()), float(np.abs(t)[bad][err[bad].argmax()]))
+    return float((err / (np.abs(t) + atol / rtol)).max())
+
+
+def check(actual, truth64, what, atol=1e-6, **kw):
+    if actual.dtype == torch.float32:
+        return check_f32(actual, truth64, what, atol=atol)
+    return check_lowp(actual, truth64, what, **kw)

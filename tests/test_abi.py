@@ -1,0 +1,78 @@
+"""The C-ABI library loads on a machine without a GPU and exports every symbol
+that include/oslo_hip.h declares; argument validation that needs no device is
+exercised too (no kernel is launched here)."""
+import ctypes
+import os
+import re
+
+import pytest
+
+from oslo_amd.torch import _C
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_symbols():
+    text = open(os.path.join(ROOT, "include", "oslo_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(oslo_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_and_loader_agree():
+    assert declared_symbols() == sorted(_C.EXPORTED_SYMBOLS)
+
+
+def test_library_exports_every_declared_symbol():
+    lib = _C.load_library()
+    for name in declared_symbols():
+        assert hasattr(lib, name), name
+    assert lib.oslo_hip_arch() == b"gfx950"
+    assert lib.oslo_hip_abi_version() == _C.ABI_VERSION
+
+
+def test_workspace_bytes_and_errors():
+    lib = _C.load_library()
+    assert lib.oslo_workspace_bytes(_C.OSLO_OP_LN_BWD, 0, 128) == 0
+    ln = lib.oslo_workspace_bytes(_C.OSLO_OP_LN_BWD, 4096, 1024)
+    rms = lib.oslo_workspace_bytes(_C.OSLO_OP_RMS_BWD, 4096, 1024)
+    assert ln == 2 * rms and rms % (1024 * 4) == 0 and rms > 0
+    assert lib.oslo_workspace_bytes(_C.OSLO_OP_BIAS_GELU_BWD, 100, 64) > 0
+    assert lib.oslo_workspace_bytes(99, 4, 4) < 0
+    assert b"unknown op" in lib.oslo_hip_last_error()
+
+
+def test_invalid_arguments_are_rejected_before_any_launch():
+    lib = _C.load_library()
+    # unsupported dtype pair: fp16 input with bf16 output
+    rc = lib.oslo_ln_fwd(None, None, None, None, None, None, 4, 8, 1e-5, 1, 2, None)
+    assert rc == -2 and b"dtype pair" in lib.oslo_hip_last_error()
+    rc = lib.oslo_ln_fwd(None, None, None, None, None, None, 4, 8, 1e-5, 7, 0, None)
+    assert rc == -1
+    rc = lib.oslo_softmax_causal_fwd(None, None, 2, 4, 0, 1.0, 0, None)
+    assert rc == -1 and b"bad shape" in lib.oslo_hip_last_error()
+    rc = lib.oslo_softmax_masked_fwd(None, None, None, 2, 2, 4, 8, 3, 1, 1.0, 0, None)
+    assert rc == -1 and b"broadcast" in lib.oslo_hip_last_error()
+    rc = lib.oslo_bias_dropout_add_fwd(None, None, None, None, None, 4, 8, 1.5, 0, 0, 0, None)
+    assert rc == -1 and b"not in [0, 1]" in lib.oslo_hip_last_error()
+    rc = lib.oslo_copy_probe(None, None, 24, None)
+    assert rc == -1
+    assert lib.oslo_tune(b"no_such_knob", 1) == -1
+    assert lib.oslo_tune(b"norm_fwd_vpl", 0) == 0
+    # empty problems succeed without touching any pointer
+    assert lib.oslo_ln_fwd(None, None, None, None, None, None, 0, 8, 1e-5, 0, 0, None) == 0
+    assert lib.oslo_bias_gelu_fwd(None, None, None, 0, 8, 2, None) == 0
+
+
+def test_batch_per_block():
+    lib = _C.load_library()
+    assert lib.oslo_softmax_batch_per_block(1024, 1024, 16, 16) >= 1
+    assert lib.oslo_softmax_batch_per_block(0, 8, 1, 1) < 0
+
+
+def test_missing_library_raises_environment_error(monkeypatch, tmp_path):
+    monkeypatch.setattr(_C, "_lib", None)
+    bogus = tmp_path / "liboslo_hip.so"
+    bogus.write_bytes(b"not an ELF file")
+    monkeypatch.setattr(_C, "LIBRARY_PATH", str(bogus))
+    with pytest.raises(EnvironmentError):
+        _C.load_library()

@@ -1,0 +1,288 @@
+"""Pins the numpy oracle (oracle/closed_form.py) without a GPU: against torch's
+library routines and autograd in float64, against finite differences, and
+against the invariants the mathematics fixes.  Each check is chosen so that a
+dropped term, a wrong sign or a transposed operand fails it."""
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle import closed_form as cf
+from oracle import torch_path as tp
+
+
+def rng(seed):
+    return np.random.default_rng(seed)
+
+
+# ---------------------------------------------------------------- rounding
+def test_round_bf16_matches_torch():
+    a = rng(0).standard_normal(100000).astype(np.float32) * 37.0
+    a[:8] = [0.0, -0.0, 1.0, 1.00390625, 1.001953125, 1.005859375, 3.0e38, 1e-40]
+    got = cf.round_bf16(a)
+    want = torch.from_numpy(a).to(torch.bfloat16).to(torch.float32).numpy()
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+def test_round_f16_matches_torch():
+    a = rng(1).standard_normal(100000).astype(np.float32) * 11.0
+    got = cf.round_f16(a)
+    want = torch.from_numpy(a).to(torch.float16).to(torch.float32).numpy()
+    assert np.array_equal(got, want)
+
+
+# ---------------------------------------------------------------- softmax
+@pytest.mark.parametrize("sq,sk", [(1, 1), (5, 5), (3, 7), (7, 3), (16, 16)])
+def test_causal_softmax_vs_torch_where_chain(sq, sk):
+    x = rng(2).standard_normal((3, sq, sk))
+    y = cf.softmax_causal_fwd(x, 0.37)
+    ref = tp.causal_softmax(torch.from_numpy(x), 0.37).numpy() if sq <= sk else None
+    if ref is not None:
+        # the -1e4 fill of the reference underflows to exactly 0 in the softmax
+        assert np.allclose(y, ref, rtol=1e-12, atol=0)
+        assert np.array_equal(y == 0, ref == 0)
+    hidden = cf.causal_hidden(sq, sk)
+    rows_visible = (~hidden).sum(-1)
+    # hidden keys are exactly 0 in every row that sees at least one key
+    assert np.all(y[:, hidden & (rows_visible > 0)[:, None]] == 0)
+    assert np.allclose(y.sum(-1)[:, rows_visible > 0], 1.0, atol=1e-14)
+    # query i sees exactly i + 1 + (sk - sq) keys
+    want_nz = np.clip(np.arange(sq) + 1 + (sk - sq), 0, sk)
+    got_nz = (y[0] > 0).sum(-1)
+    assert np.array_equal(got_nz[want_nz > 0], want_nz[want_nz > 0])
+    # no visible key: uniform
+    assert np.allclose(y[:, want_nz == 0], 1.0 / sk)
+    if sq == sk:
+        assert np.all(y[:, 0, 0] == 1.0)
+
+
+def test_masked_softmax_vs_torch_additive_mask():
+    b, h, sq, sk = 3, 2, 4, 12
+    x = rng(3).standard_normal((b, h, sq, sk)) * 2
+    valid = np.array([12, 5, 1])
+    pad = np.arange(sk)[None, :] >= valid[:, None]
+    y = cf.softmax_masked_fwd(x, pad[:, None, None, :], 0.125)
+    ref = tp.padding_softmax(torch.from_numpy(x), torch.from_numpy(pad), 0.125).numpy()
+    assert np.allclose(y, ref, rtol=1e-12, atol=0)
+    assert np.all(y[np.broadcast_to(pad[:, None, None, :], y.shape)] == 0)
+    # masked_fill(-inf) variant (DistilBERT) is the same function
+    t = torch.from_numpy(x * 0.125).masked_fill(torch.from_numpy(pad)[:, None, None, :], -np.inf)
+    assert np.allclose(y, torch.softmax(t, -1).numpy(), rtol=1e-12, atol=0)
+
+
+def test_masked_softmax_fully_masked_row_is_uniform():
+    x = rng(4).standard_normal((1, 1, 2, 8))
+    hidden = np.zeros((1, 1, 2, 8), dtype=bool)
+    hidden[0, 0, 1, :] = True
+    y = cf.softmax_masked_fwd(x, hidden, 1.0)
+    assert np.allclose(y[0, 0, 1], 1 / 8)
+    t = torch.from_numpy(x).masked_fill(torch.from_numpy(hidden), -10000.0)
+    assert np.allclose(y, torch.softmax(t, -1).numpy(), rtol=1e-12)
+
+
+def test_softmax_shift_invariance_and_scale():
+    x = rng(5).standard_normal((2, 6, 6))
+    a = cf.softmax_causal_fwd(x, 0.5)
+    b = cf.softmax_causal_fwd(x + 3.25, 0.5)
+    assert np.allclose(a, b, rtol=1e-12, atol=1e-16)
+    c = cf.softmax_causal_fwd(2 * x, 0.25)
+    assert np.allclose(a, c, rtol=1e-12, atol=1e-16)
+
+
+def test_softmax_bwd_vs_autograd_and_row_sum():
+    x = torch.from_numpy(rng(6).standard_normal((2, 5, 9))).requires_grad_()
+    g = torch.from_numpy(rng(7).standard_normal((2, 5, 9)))
+    scale = 0.3
+    y = tp.causal_softmax(x, scale)
+    y.backward(g)
+    dx = cf.softmax_bwd(g.numpy(), y.detach().numpy(), scale)
+    assert np.allclose(dx, x.grad.numpy(), rtol=1e-10, atol=1e-14)
+    assert np.allclose(dx.sum(-1), 0, atol=1e-14)
+    # dropping the scale or the row sum must be visible
+    assert not np.allclose(cf.softmax_bwd(g.numpy(), y.detach().numpy(), 1.0), x.grad.numpy())
+
+
+# ---------------------------------------------------------------- norms
+@pytest.mark.parametrize("n2", [1, 7, 64, 513])
+def test_layer_norm_fwd_bwd_vs_torch_fp64(n2):
+    r = rng(8 + n2)
+    x = torch.from_numpy(r.standard_normal((6, n2)) * 1.7 + 0.4).requires_grad_()
+    w = torch.from_numpy(1 + 0.1 * r.standard_normal(n2)).requires_grad_()
+    b = torch.from_numpy(0.1 * r.standard_normal(n2)).requires_grad_()
+    g = torch.from_numpy(r.standard_normal((6, n2)))
+    eps = 1e-5
+    y = F.layer_norm(x, (n2,), w, b, eps)
+    y.backward(g)
+    oy, mean, invvar = cf.layer_norm_fwd(x.detach().numpy(), w.detach().numpy(), b.detach().numpy(), eps)
+    assert np.allclose(oy, y.detach().numpy(), rtol=1e-11, atol=1e-13)
+    assert np.allclose(mean, x.detach().numpy().mean(-1))
+    assert np.allclose(invvar, 1 / np.sqrt(x.detach().numpy().var(-1) + eps))
+    dx, dg, db = cf.layer_norm_bwd(g.numpy(), x.detach().numpy(), mean, invvar, w.detach().numpy())
+    assert np.allclose(dx, x.grad.numpy(), rtol=1e-9, atol=1e-11)
+    assert np.allclose(dg, w.grad.numpy(), rtol=1e-10, atol=1e-12)
+    assert np.allclose(db, b.grad.numpy(), rtol=1e-10, atol=1e-12)
+    assert np.allclose(db, g.numpy().sum(0))
+
+
+def test_layer_norm_invariants():
+    r = rng(20)
+    x = r.standard_normal((5, 96)) * 3 + 1
+    g = r.standard_normal((5, 96))
+    eps = 1e-5
+    y, mean, invvar = cf.layer_norm_fwd(x, None, None, eps)
+    assert np.allclose(y.mean(-1), 0, atol=1e-14)
+    var = x.var(-1)
+    assert np.allclose(y.var(-1), var / (var + eps), rtol=1e-12)
+    dx, dg, db = cf.layer_norm_bwd(g, x, mean, invvar, None)
+    assert dg is None and db is None
+    assert np.allclose(dx.sum(-1), 0, atol=1e-13)
+    # sum(dx * xhat) vanishes up to the factor eps / (var + eps) ~ 1e-6
+    assert np.allclose((dx * y).sum(-1), 0, atol=1e-4)
+    dx0, _, _ = cf.layer_norm_bwd(g, x, mean, 1 / np.sqrt(x.var(-1)), None)
+    y0 = (x - x.mean(-1, keepdims=True)) / np.sqrt(x.var(-1, keepdims=True))
+    assert np.allclose((dx0 * y0).sum(-1), 0, atol=1e-12)
+
+
+@pytest.mark.parametrize("n2", [1, 8, 200])
+def test_rms_norm_fwd_bwd_vs_autograd_fp64(n2):
+    r = rng(30 + n2)
+    x = torch.from_numpy(r.standard_normal((4, n2)) + 0.3).requires_grad_()
+    w = torch.from_numpy(1 + 0.1 * r.standard_normal(n2)).requires_grad_()
+    g = torch.from_numpy(r.standard_normal((4, n2)))
+    eps = 1e-6
+    # manual_rms_norm takes the variance in fp32 whatever the input type
+    # (layer_norm.py:20), so the reference path itself pins only ~1e-7; the
+    # same formula without that cast pins the rest of the digits
+    y = w * (x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps))
+    y.backward(g)
+    oy, invvar = cf.rms_norm_fwd(x.detach().numpy(), w.detach().numpy(), eps)
+    assert np.allclose(oy, y.detach().numpy(), rtol=1e-12, atol=1e-14)
+    assert np.allclose(oy, tp.rms_norm(x.detach(), w.detach(), eps).numpy(), rtol=1e-6)
+    dx, dg = cf.rms_norm_bwd(g.numpy(), x.detach().numpy(), invvar, w.detach().numpy())
+    assert np.allclose(dx, x.grad.numpy(), rtol=1e-9, atol=1e-12)
+    assert np.allclose(dg, w.grad.numpy(), rtol=1e-10, atol=1e-12)
+    xhat = x.detach().numpy() * invvar[:, None]
+    dx0, _ = cf.rms_norm_bwd(g.numpy(), x.detach().numpy(), invvar, None)
+    if n2 > 1:
+        # exact only for eps -> 0; eps = 1e-6 leaves a 1e-6-relative residue
+        assert np.allclose((dx0 * xhat).sum(-1), 0, atol=1e-4)
+
+
+def test_rms_norm_rounding_order_matches_reference_cpu_path_bf16():
+    """manual_rms_norm rounds x * rsqrt(var) to bf16 and then gamma * that to
+    bf16 again; the oracle must reproduce those two roundings bit for bit."""
+    g = torch.Generator().manual_seed(5)
+    x = torch.randn(64, 256, generator=g).to(torch.bfloat16)
+    w = (1 + 0.02 * torch.randn(256, generator=g)).to(torch.bfloat16)
+    ref = tp.rms_norm(x, w, 1e-5)
+    assert ref.dtype == torch.bfloat16
+    oy, _ = cf.rms_norm_fwd(x.double().numpy(), w.double().numpy(), 1e-5, out="bf16")
+    same = np.mean(oy == ref.float().numpy())
+    # torch evaluates x * rsqrt(var) in fp32, the oracle in fp64: a handful of
+    # values that sit on a bf16 tie may differ
+    assert same > 0.9995, same
+    single = cf.round_to(
+        w.double().numpy() * (x.double().numpy() * cf.rms_norm_fwd(x.double().numpy(), None, 1e-5)[1][:, None]),
+        "bf16",
+    )
+    assert np.mean(single == ref.float().numpy()) < 0.99  # single rounding is measurably different
+
+
+def test_layer_norm_single_rounding_matches_torch_cpu_bf16():
+    g = torch.Generator().manual_seed(6)
+    x = torch.randn(64, 512, generator=g).to(torch.bfloat16)
+    w = (1 + 0.02 * torch.randn(512, generator=g)).to(torch.bfloat16)
+    b = (0.02 * torch.randn(512, generator=g)).to(torch.bfloat16)
+    ref = tp.layer_norm(x, w, b, 1e-5)
+    oy, _, _ = cf.layer_norm_fwd(x.double().numpy(), w.double().numpy(), b.double().numpy(), 1e-5, out="bf16")
+    assert np.mean(oy == ref.float().numpy()) > 0.999
+
+
+# ---------------------------------------------------------------- bias-GeLU
+def test_bias_gelu_vs_torch_tanh_gelu_fp64():
+    r = rng(40)
+    x = torch.from_numpy(r.standard_normal((7, 24)) * 3).requires_grad_()
+    b = torch.from_numpy(0.2 * r.standard_normal(24)).requires_grad_()
+    g = torch.from_numpy(r.standard_normal((7, 24)))
+    y = F.gelu(x + b, approximate="tanh")
+    y.backward(g)
+    oy = cf.bias_gelu_fwd(x.detach().numpy(), b.detach().numpy())
+    # 0.79788456 is sqrt(2/pi) to fp32 precision: agreement to ~1e-8, not 1e-16
+    assert np.allclose(oy, y.detach().numpy(), rtol=2e-7, atol=1e-8)
+    dx, db = cf.bias_gelu_bwd(g.numpy(), x.detach().numpy(), b.detach().numpy())
+    assert np.allclose(dx, x.grad.numpy(), rtol=2e-6, atol=1e-7)
+    assert np.allclose(db, b.grad.numpy(), rtol=2e-6, atol=1e-6)
+    # the explicit derivative of the reference equals autograd of its forward
+    x2 = x.detach().clone().requires_grad_()
+    tp.bias_gelu(x2, b.detach()).backward(g)
+    assert np.allclose(dx, x2.grad.numpy(), rtol=1e-7, atol=1e-9)
+    assert np.allclose(tp.bias_gelu_grad(g, x.detach(), b.detach()).numpy(), dx, rtol=1e-12, atol=1e-14)
+
+
+def test_gelu_special_values():
+    u = np.array([0.0, 1.5, -1.5, 30.0, -30.0])
+    y = cf.bias_gelu_fwd(u, None)
+    assert y[0] == 0
+    assert np.isclose(y[1] - y[2], 1.5, rtol=1e-14)  # gelu(u) - gelu(-u) = u
+    assert y[3] == 30.0 and abs(y[4]) == 0.0
+    d, _ = cf.bias_gelu_bwd(np.ones(5), u, None)
+    assert d[0] == 0.5 and d[3] == 1.0 and abs(d[4]) == 0.0
+    eps = 1e-6
+    fd = (cf.bias_gelu_fwd(u + eps, None) - cf.bias_gelu_fwd(u - eps, None)) / (2 * eps)
+    assert np.allclose(d, fd, atol=1e-8)
+
+
+def test_constants():
+    assert np.float32(cf.GELU_A) == np.float32(np.sqrt(2 / np.pi))
+    assert np.isclose(cf.GELU_C, 3 * cf.GELU_B * cf.GELU_A, rtol=1e-9)
+
+
+# ---------------------------------------------------------------- bias-dropout-add
+def test_bias_dropout_add_identity_and_scaling():
+    r = rng(50)
+    x, res = r.standard_normal((6, 16)), r.standard_normal((6, 16))
+    b = r.standard_normal(16)
+    out = cf.bias_dropout_add_fwd(x, b, res, None, 0.0)
+    assert np.array_equal(out, x + b + res)
+    keep = r.random((6, 16)) > 0.3
+    out = cf.bias_dropout_add_fwd(x, b, None, keep, 0.3)
+    scale = float(np.float32(1) / (np.float32(1) - np.float32(0.3)))
+    assert np.array_equal(out[~keep], np.zeros((~keep).sum()))
+    assert np.allclose(out[keep], ((x + b) * scale)[keep], rtol=1e-15)
+    ref = tp.bias_dropout_add(torch.from_numpy(x), torch.from_numpy(b), torch.from_numpy(res), 0.3, True,
+                              keep=torch.from_numpy(keep))
+    assert np.allclose(cf.bias_dropout_add_fwd(x, b, res, keep, 0.3), ref.numpy(), rtol=3e-7, atol=3e-7)
+
+
+def test_bias_dropout_add_bwd_vs_autograd():
+    r = rng(51)
+    x = torch.from_numpy(r.standard_normal((5, 8))).requires_grad_()
+    b = torch.from_numpy(r.standard_normal(8)).requires_grad_()
+    res = torch.from_numpy(r.standard_normal((5, 8))).requires_grad_()
+    keep = torch.from_numpy(r.random((5, 8)) > 0.25)
+    g = torch.from_numpy(r.standard_normal((5, 8)))
+    tp.bias_dropout_add(x, b, res, 0.25, True, keep=keep).backward(g)
+    dx, db = cf.bias_dropout_add_bwd(g.numpy(), keep.numpy(), 0.25)
+    assert np.allclose(dx, x.grad.numpy(), rtol=1e-7)
+    assert np.allclose(db, b.grad.numpy(), rtol=1e-7)
+    assert np.array_equal(res.grad.numpy(), g.numpy())
+
+
+def test_autograd_sums_full_size_bias_grad():
+    """The reference returns a [rows, cols] gradient for the [cols] bias
+    (functional.py:84); autograd reduces it to the column sum."""
+
+    class Fn(torch.autograd.Function):
+        @staticmethod
+        def forward(ctx, x, b):
+            return x + b
+
+        @staticmethod
+        def backward(ctx, g):
+            return g, g
+
+    x = torch.randn(5, 3, dtype=torch.float64, requires_grad=True)
+    b = torch.randn(3, dtype=torch.float64, requires_grad=True)
+    g = torch.randn(5, 3, dtype=torch.float64)
+    Fn.apply(x, b).backward(g)
+    assert torch.allclose(b.grad, g.sum(0))
