@@ -1,0 +1,456 @@
+#!/usr/bin/env python3
+"""Benchmark of the fused non-GEMM kernels on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+Headline workload (BASELINE.json configs[1]): LayerNorm and RMSNorm forward +
+backward on a bf16 [16384, 4096] activation.  One step = LN fwd, LN bwd, RMS
+fwd, RMS bwd over one batch, called through the C ABI with every buffer
+resident in HBM and pre-allocated; buffer sets rotate so the 256 MB Infinity
+Cache cannot serve the reads.  `value` = algorithmic bytes of a step (10 T,
+T = 134.2 MB) / wall time per step.
+
+Prints ONE JSON line.  Beside the contract's keys it carries
+  roofline      the dominant launch (LN backward), timed with events on the
+                launch stream inside the timed region,
+  cpu_baseline  the reference's unfused torch path (oracle/torch_path.py) on
+                the host cores, same workload,
+  kernels       achieved GB/s and fraction of the 8 TB/s HBM peak for every
+                fused kernel of BASELINE.json's five configurations.
+"""
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published
+METRIC = "achieved HBM GB/s (% of MI355X peak) per fused fwd+bwd kernel; speedup vs CPU path"
+
+F32, F16, BF16 = 0, 1, 2
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--table-iters", type=int, default=20, help="launches per kernel in the per-kernel table (0 = skip)")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-reps", type=int, default=3)
+    return ap.parse_args()
+
+
+class Lib:
+    """Raw C-ABI calls on pre-allocated tensors (no allocation per call)."""
+
+    def __init__(self, torch, _C):
+        self.torch = torch
+        self.lib = _C.load_library()
+        self._C = _C
+
+    def stream(self):
+        return self.torch.cuda.current_stream().cuda_stream
+
+    def ok(self, rc):
+        if rc != 0:
+            raise RuntimeError(self.lib.oslo_hip_last_error().decode())
+
+    def ws(self, op, n1, n2, device):
+        nbytes = int(self.lib.oslo_workspace_bytes(op, n1, n2))
+        return self.torch.empty(max(nbytes, 16), dtype=self.torch.uint8, device=device), nbytes
+
+
+def p(t):
+    return None if t is None else t.data_ptr()
+
+
+def time_launches(torch, fn, iters, nsets):
+    """Average duration in ms of fn(i % nsets), events on the current stream."""
+    for i in range(min(3, iters)):
+        fn(i % nsets)
+    torch.cuda.synchronize()
+    e0 = torch.cuda.Event(enable_timing=True)
+    e1 = torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for i in range(iters):
+        fn(i % nsets)
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / iters
+
+
+def norm_buffers(torch, dev, n1, n2, nsets, seed):
+    g = torch.Generator(device=dev).manual_seed(seed)
+    sets = []
+    for _ in range(nsets):
+        s = {
+            "x": torch.randn(n1, n2, generator=g, device=dev).to(torch.bfloat16),
+            "dy": torch.randn(n1, n2, generator=g, device=dev).to(torch.bfloat16),
+            "y": torch.empty(n1, n2, device=dev, dtype=torch.bfloat16),
+            "dx": torch.empty(n1, n2, device=dev, dtype=torch.bfloat16),
+            "mean": torch.empty(n1, device=dev, dtype=torch.float32),
+            "invvar": torch.empty(n1, device=dev, dtype=torch.float32),
+        }
+        sets.append(s)
+    gamma = (1 + 0.02 * torch.randn(n2, generator=g, device=dev)).to(torch.bfloat16)
+    beta = (0.02 * torch.randn(n2, generator=g, device=dev)).to(torch.bfloat16)
+    dgamma = torch.empty_like(gamma)
+    dbeta = torch.empty_like(beta)
+    return sets, gamma, beta, dgamma, dbeta
+
+
+def make_norm_calls(L, dev, n1, n2, nsets, seed=0):
+    torch = L.torch
+    lib = L.lib
+    sets, gamma, beta, dgamma, dbeta = norm_buffers(torch, dev, n1, n2, nsets, seed)
+    ws_ln, ws_ln_bytes = L.ws(L._C.OSLO_OP_LN_BWD, n1, n2, dev)
+    ws_rms, ws_rms_bytes = L.ws(L._C.OSLO_OP_RMS_BWD, n1, n2, dev)
+    keep = (sets, gamma, beta, dgamma, dbeta, ws_ln, ws_rms)
+
+    def ln_fwd(i):
+        s = sets[i]
+        L.ok(lib.oslo_ln_fwd(p(s["x"]), p(gamma), p(beta), p(s["y"]), p(s["mean"]), p(s["invvar"]),
+                             n1, n2, 1e-5, BF16, BF16, L.stream()))
+
+    def ln_bwd(i):
+        s = sets[i]
+        L.ok(lib.oslo_ln_bwd(p(s["dy"]), p(s["x"]), p(s["mean"]), p(s["invvar"]), p(gamma), p(s["dx"]),
+                             p(dgamma), p(dbeta), p(ws_ln), ws_ln_bytes, n1, n2, BF16, BF16, L.stream()))
+
+    def rms_fwd(i):
+        s = sets[i]
+        L.ok(lib.oslo_rms_fwd(p(s["x"]), p(gamma), p(s["y"]), p(s["invvar"]), n1, n2, 1e-5, BF16, BF16,
+                              L.stream()))
+
+    def rms_bwd(i):
+        s = sets[i]
+        L.ok(lib.oslo_rms_bwd(p(s["dy"]), p(s["x"]), p(s["invvar"]), p(gamma), p(s["dx"]), p(dgamma),
+                              p(ws_rms), ws_rms_bytes, n1, n2, BF16, BF16, L.stream()))
+
+    return {"ln_fwd": ln_fwd, "ln_bwd": ln_bwd, "rms_fwd": rms_fwd, "rms_bwd": rms_bwd, "_keep": keep}
+
+
+def table_row(name, cfg, shape, dtype, nbytes, ms):
+    gbps = nbytes / (ms * 1e-3) / 1e9
+    return {
+        "kernel": name, "config": cfg, "shape": shape, "io_dtype": dtype,
+        "algorithmic_MB": round(nbytes / 1e6, 1), "us": round(ms * 1e3, 2),
+        "GBps": round(gbps, 1), "frac_of_peak": round(gbps / HBM_PEAK_GBPS, 4),
+    }
+
+
+def nsets_for(total_bytes_per_set):
+    """Enough rotating sets that consecutive launches cannot hit in the 256 MB cache."""
+    return max(1, min(8, math.ceil(1.0e9 / max(total_bytes_per_set, 1))))
+
+
+def kernel_table(L, dev, iters):
+    """Every fused kernel at the shapes of BASELINE.json's five configurations."""
+    torch = L.torch
+    lib = L.lib
+    rows = []
+
+    def timed(fn, nsets):
+        return time_launches(torch, fn, iters, nsets)
+
+    # ---- LayerNorm / RMSNorm: cfg2 and cfg5 ----
+    for cfg, n1, n2 in (("cfg2", 16384, 4096), ("cfg5", 8192, 6144)):
+        T = n1 * n2 * 2
+        ns = nsets_for(4 * T)
+        calls = make_norm_calls(L, dev, n1, n2, ns, seed=1)
+        for name, mult in (("ln_fwd", 2), ("ln_bwd", 3), ("rms_fwd", 2), ("rms_bwd", 3)):
+            if cfg == "cfg5" and name.startswith("rms"):
+                continue
+            if name.endswith("bwd"):
+                calls[name.replace("bwd", "fwd")](0)
+                for i in range(ns):
+                    calls[name.replace("bwd", "fwd")](i)
+            rows.append(table_row(name, cfg, [n1, n2], "bf16", mult * T, timed(calls[name], ns)))
+        del calls
+        torch.cuda.empty_cache()
+
+    # ---- causal softmax: cfg1 (fp32) and cfg5 (bf16) ----
+    for cfg, ab, s, tdt, code, esz, scale in (
+        ("cfg1", 48, 512, torch.float32, F32, 4, 0.125),
+        ("cfg5", 256, 2048, torch.bfloat16, BF16, 2, 1.0 / math.sqrt(96.0)),
+    ):
+        T = ab * s * s * esz
+        f = (s + 1) / (2.0 * s)
+        ns = nsets_for(4 * T)
+        g = torch.Generator(device=dev).manual_seed(2)
+        bufs = []
+        for _ in range(ns):
+            x = torch.randn(ab, s, s, generator=g, device=dev).to(tdt)
+            dy = torch.randn(ab, s, s, generator=g, device=dev).to(tdt)
+            bufs.append((x, torch.empty_like(x), dy, torch.empty_like(x)))
+
+        def fwd(i):
+            x, y, dy, dx = bufs[i]
+            L.ok(lib.oslo_softmax_causal_fwd(p(x), p(y), ab, s, s, scale, code, L.stream()))
+
+        def bwd(i):
+            x, y, dy, dx = bufs[i]
+            L.ok(lib.oslo_softmax_causal_bwd(p(dy), p(y), p(dx), ab, s, s, scale, code, L.stream()))
+
+        rows.append(table_row("softmax_causal_fwd", cfg, [ab, s, s], str(tdt).split(".")[-1], (1 + f) * T, timed(fwd, ns)))
+        rows.append(table_row("softmax_causal_bwd", cfg, [ab, s, s], str(tdt).split(".")[-1], (1 + 2 * f) * T, timed(bwd, ns)))
+        del bufs
+        torch.cuda.empty_cache()
+
+    # ---- padding-masked softmax: cfg3 ----
+    b, h, s = 16, 16, 1024
+    T = b * h * s * s * 2
+    g = torch.Generator(device=dev).manual_seed(3)
+    valid = torch.randint(256, 1025, (b,), generator=torch.Generator().manual_seed(3))
+    r = float(valid.double().mean()) / s
+    mask = (torch.arange(s)[None, :] >= valid[:, None]).view(b, 1, 1, s).to(dev).view(torch.uint8)
+    ns = 2
+    bufs = []
+    for _ in range(ns):
+        x = (2 * torch.randn(b, h, s, s, generator=g, device=dev)).to(torch.float16)
+        dy = torch.randn(b, h, s, s, generator=g, device=dev).to(torch.float16)
+        bufs.append((x, torch.empty_like(x), dy, torch.empty_like(x)))
+
+    def mfwd(i):
+        x, y, dy, dx = bufs[i]
+        L.ok(lib.oslo_softmax_masked_fwd(p(x), p(mask), p(y), b, h, s, s, b, 1, 0.125, F16, L.stream()))
+
+    def mbwd(i):
+        x, y, dy, dx = bufs[i]
+        L.ok(lib.oslo_softmax_masked_bwd(p(dy), p(y), p(mask), p(dx), b, h, s, s, b, 1, 0.125, F16, L.stream()))
+
+    row = table_row("softmax_masked_fwd", "cfg3", [b, h, s, s], "float16", (r + 1) * T, timed(mfwd, ns))
+    row["valid_fraction"] = round(r, 4)
+    row["dense_equiv_GBps"] = round(2 * T / (row["us"] * 1e-6) / 1e9, 1)
+    rows.append(row)
+    row = table_row("softmax_masked_bwd", "cfg3", [b, h, s, s], "float16", (2 * r + 1) * T, timed(mbwd, ns))
+    row["valid_fraction"] = round(r, 4)
+    row["dense_equiv_GBps"] = round(3 * T / (row["us"] * 1e-6) / 1e9, 1)
+    rows.append(row)
+    del bufs
+    torch.cuda.empty_cache()
+
+    # ---- bias-GeLU: cfg4 and cfg5 ----
+    for cfg, n1, n2 in (("cfg4", 16384, 16384), ("cfg5", 8192, 24576)):
+        T = n1 * n2 * 2
+        ns = nsets_for(4 * T)
+        g = torch.Generator(device=dev).manual_seed(4)
+        bias = (0.02 * torch.randn(n2, generator=g, device=dev)).to(torch.bfloat16)
+        dbias = torch.empty_like(bias)
+        ws, wsb = L.ws(L._C.OSLO_OP_BIAS_GELU_BWD, n1, n2, dev)
+        bufs = []
+        for _ in range(ns):
+            x = torch.randn(n1, n2, generator=g, device=dev).to(torch.bfloat16)
+            gg = torch.randn(n1, n2, generator=g, device=dev).to(torch.bfloat16)
+            bufs.append((x, torch.empty_like(x), gg, torch.empty_like(x)))
+
+        def gfwd(i):
+            x, y, gg, dx = bufs[i]
+            L.ok(lib.oslo_bias_gelu_fwd(p(x), p(bias), p(y), n1, n2, BF16, L.stream()))
+
+        def gbwd(i):
+            x, y, gg, dx = bufs[i]
+            L.ok(lib.oslo_bias_gelu_bwd(p(gg), p(x), p(bias), p(dx), p(dbias), p(ws), wsb, n1, n2, BF16, L.stream()))
+
+        rows.append(table_row("bias_gelu_fwd", cfg, [n1, n2], "bf16", 2 * T, timed(gfwd, ns)))
+        rows.append(table_row("bias_gelu_bwd", cfg, [n1, n2], "bf16", 3 * T, timed(gbwd, ns)))
+        del bufs
+        torch.cuda.empty_cache()
+
+    # ---- bias-dropout-add: cfg4 (p = 0.1 and p = 0) and cfg5 ----
+    for cfg, n1, n2, pdrop in (("cfg4", 16384, 4096, 0.1), ("cfg4", 16384, 4096, 0.0), ("cfg5", 8192, 6144, 0.1)):
+        T = n1 * n2 * 2
+        ns = nsets_for(5 * T)
+        g = torch.Generator(device=dev).manual_seed(5)
+        bias = (0.02 * torch.randn(n2, generator=g, device=dev)).to(torch.bfloat16)
+        dbias = torch.empty_like(bias)
+        ws, wsb = L.ws(L._C.OSLO_OP_BIAS_DROPOUT_ADD_BWD, n1, n2, dev)
+        bufs = []
+        for _ in range(ns):
+            x = torch.randn(n1, n2, generator=g, device=dev).to(torch.bfloat16)
+            res = torch.randn(n1, n2, generator=g, device=dev).to(torch.bfloat16)
+            gg = torch.randn(n1, n2, generator=g, device=dev).to(torch.bfloat16)
+            bufs.append((x, res, torch.empty_like(x), gg, torch.empty_like(x)))
+
+        def dfwd(i):
+            x, res, out, gg, dx = bufs[i]
+            L.ok(lib.oslo_bias_dropout_add_fwd(p(x), p(bias), p(res), p(out), None, n1, n2, pdrop, 1234, 0, BF16,
+                                               L.stream()))
+
+        def dbwd(i):
+            x, res, out, gg, dx = bufs[i]
+            L.ok(lib.oslo_bias_dropout_add_bwd(p(gg), p(dx), p(dbias), p(ws), wsb, n1, n2, pdrop, 1234, 0, BF16,
+                                               L.stream()))
+
+        tag = "p=%.1f" % pdrop
+        r1 = table_row("bias_dropout_add_fwd", cfg, [n1, n2], "bf16", 3 * T, timed(dfwd, ns))
+        r2 = table_row("bias_dropout_add_bwd", cfg, [n1, n2], "bf16", 2 * T, timed(dbwd, ns))
+        r1["p"] = r2["p"] = pdrop
+        rows += [r1, r2]
+        del bufs
+        torch.cuda.empty_cache()
+
+    # ---- plain copy with the same load/store path: the practical ceiling ----
+    nbytes = 1 << 30
+    src = [torch.empty(nbytes, dtype=torch.uint8, device=dev) for _ in range(2)]
+    dst = [torch.empty(nbytes, dtype=torch.uint8, device=dev) for _ in range(2)]
+    for s_ in src:
+        s_.fill_(1)
+
+    def cp(i):
+        L.ok(lib.oslo_copy_probe(p(src[i]), p(dst[i]), nbytes, L.stream()))
+
+    rows.append(table_row("copy_probe", "-", [nbytes], "u8", 2 * nbytes, timed(cp, 2)))
+    return rows
+
+
+def cpu_baseline(n1, n2, reps):
+    """The reference's unfused torch path on the host cores, same workload."""
+    import torch
+
+    from oracle import torch_path as tp
+
+    threads = min(os.cpu_count() or 1, 16)
+    torch.set_num_threads(threads)
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(n1, n2, generator=g).to(torch.bfloat16)
+    dy = torch.randn(n1, n2, generator=g).to(torch.bfloat16)
+    gamma = (1 + 0.02 * torch.randn(n2, generator=g)).to(torch.bfloat16)
+    beta = (0.02 * torch.randn(n2, generator=g)).to(torch.bfloat16)
+
+    def step():
+        xr = x.clone().requires_grad_()
+        w, b = gamma.clone().requires_grad_(), beta.clone().requires_grad_()
+        tp.layer_norm(xr, w, b, 1e-5).backward(dy)
+        xr = x.clone().requires_grad_()
+        w = gamma.clone().requires_grad_()
+        tp.rms_norm(xr, w, 1e-5).backward(dy)
+
+    step()
+    times = []
+    for _ in range(reps):
+        t0 = time.perf_counter()
+        step()
+        times.append(time.perf_counter() - t0)
+    times.sort()
+    med = times[len(times) // 2]
+    nbytes = 10 * n1 * n2 * 2
+    return {
+        "value": round(nbytes / med / 1e9, 3),
+        "unit": "GB/s",
+        "cores": threads,
+        "kind": "port",
+        "sample": "full workload [%d,%d] bf16, LN+RMS fwd+bwd via torch CPU ops (F.layer_norm, manual_rms_norm, autograd), "
+                  "median of %d reps, %.2f s each" % (n1, n2, reps, med),
+        "ms_per_step": round(med * 1e3, 1),
+    }
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        sys.stderr.write(
+            "bench.py: this build measures one GPU only (the path has no collectives); "
+            "run with --gpus 1.\n"
+        )
+        sys.exit(2)
+
+    import torch
+
+    from oslo_amd.torch import _C
+
+    if not torch.cuda.is_available():
+        sys.stderr.write("bench.py: no GPU visible\n")
+        sys.exit(1)
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    L = Lib(torch, _C)
+
+    n1, n2 = 16384, 4096
+    T = n1 * n2 * 2
+    nsets = 4
+    calls = make_norm_calls(L, dev, n1, n2, nsets, seed=0)
+
+    def step(i):
+        k = i % nsets
+        calls["ln_fwd"](k)
+        calls["ln_bwd"](k)
+        calls["rms_fwd"](k)
+        calls["rms_bwd"](k)
+
+    for i in range(args.warmup):
+        step(i)
+    torch.cuda.synchronize()
+
+    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        k = i % nsets
+        calls["ln_fwd"](k)
+        ev[i][0].record()
+        calls["ln_bwd"](k)
+        ev[i][1].record()
+        calls["rms_fwd"](k)
+        calls["rms_bwd"](k)
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+
+    ms_per_step = (t1 - t0) * 1e3 / args.steps
+    step_bytes = 10 * T
+    value = step_bytes / (ms_per_step * 1e-3) / 1e9
+    bwd_ms = sum(a.elapsed_time(b) for a, b in ev) / len(ev)
+    achieved = 3 * T / (bwd_ms * 1e-3) / 1e9
+
+    out = {
+        "metric": METRIC,
+        "value": round(value, 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {
+            "workload": "BASELINE.json configs[1]: LayerNorm + RMSNorm fwd+bwd, bf16 [16384,4096], eps 1e-5; "
+                        "step = ln_fwd, ln_bwd, rms_fwd, rms_bwd",
+            "io_dtype": "bf16",
+            "algorithmic_MB_per_step": round(step_bytes / 1e6, 1),
+            "rotating_buffer_sets": nsets,
+        },
+        "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBPS, 2),
+        "roofline": {
+            "kernel": "oslo_ln_bwd = norm_bwd_reg_kernel + colsum_finalize_kernel",
+            "bound": "hbm",
+            "achieved": round(achieved, 1),
+            "peak": HBM_PEAK_GBPS,
+            "unit": "GB/s",
+            "frac": round(achieved / HBM_PEAK_GBPS, 4),
+            "traffic": None,
+            "algorithmic_MB_per_launch": round(3 * T / 1e6, 1),
+            "avg_us": round(bwd_ms * 1e3, 2),
+        },
+    }
+    del calls
+    torch.cuda.empty_cache()
+
+    if args.table_iters > 0:
+        out["kernels"] = kernel_table(L, dev, args.table_iters)
+    if not args.no_cpu_baseline:
+        cb = cpu_baseline(n1, n2, args.cpu_reps)
+        cb["speedup_gpu_over_cpu"] = round(value / cb["value"], 1) if cb["value"] > 0 else None
+        out["cpu_baseline"] = cb
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

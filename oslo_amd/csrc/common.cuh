@@ -95,7 +95,10 @@ template <> struct io<_Float16> {
   static __device__ __forceinline__ void unpack(u32x4 r, float *f) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      f16x2 h = __builtin_bit_cast(f16x2, r[i]);
+      // copy the element first: a bit_cast straight from the vector-element
+      // lvalue r[i] reads element 0 with this compiler
+      const uint32_t w = r[i];
+      f16x2 h = __builtin_bit_cast(f16x2, w);
       f[2 * i] = static_cast<float>(h.x);
       f[2 * i + 1] = static_cast<float>(h.y);
     }

@@ -325,6 +325,24 @@ __global__ __launch_bounds__(256) void bias_dropout_add_bwd_generic_kernel(
   }
 }
 
+// dbias alone on the generic path: one thread per column walks the rows and
+// sums the values dx would hold, without storing them.
+template <typename T>
+__global__ __launch_bounds__(256) void bias_dropout_add_dbias_generic_kernel(
+    const T *__restrict__ gr, T *__restrict__ dbias, int64_t rows,
+    int64_t cols, DropArgs d, bool drop) {
+  const int64_t col = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (col >= cols) return;
+  float s = 0.f;
+  for (int64_t r = 0; r < rows; ++r) {
+    const int64_t i = r * cols + col;
+    float t = io<T>::from_scalar(gr[i]);
+    if (drop) t = keep_element(i, d) ? t * d.scale : 0.f;
+    s += io<T>::round(t);
+  }
+  dbias[col] = io<T>::to_scalar(s);
+}
+
 // Column sum of an already stored [rows, cols] tensor (generic path only).
 template <typename T>
 __global__ __launch_bounds__(256) void colsum_generic_kernel(
@@ -563,8 +581,12 @@ static int run_bda_bwd(const void *gr, void *dx, void *dbias, void *ws,
   const bool vec_ok = cols % kE == 0 && aligned16(gr) && aligned16(dx) &&
                       aligned16(ws) && cols / kE <= 0x7fffffff;
   if (!vec_ok) {
-    OSLO_REQUIRE(dx != nullptr,
-                 "bias_dropout_add bwd: dx required for this shape/alignment");
+    if (dx == nullptr) {
+      bias_dropout_add_dbias_generic_kernel<T>
+          <<<dim3((unsigned)ceil_div(cols, 256)), 256, 0, st>>>(
+              (const T *)gr, (T *)dbias, rows, cols, d, drop);
+      return check_launch("bias_dropout_add_dbias_generic_kernel");
+    }
     const int64_t n = rows * cols;
     bias_dropout_add_bwd_generic_kernel<T>
         <<<dim3((unsigned)flat_grid(n)), 256, 0, st>>>((const T *)gr, (T *)dx,

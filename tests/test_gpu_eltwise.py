@@ -1,0 +1,156 @@
+"""bias-GeLU and bias-dropout-add forward and backward on the GPU, through the
+C ABI, against the float64 oracle; dropout masks bit-exact against the integer
+Philox oracle."""
+import numpy as np
+import pytest
+import torch
+
+from helpers import check, f64, randn
+from oracle import closed_form as cf
+from oracle import philox
+from oracle import torch_path as tp
+from oslo_amd.torch import _C
+
+pytestmark = pytest.mark.gpu
+
+F32, F16, BF16 = torch.float32, torch.float16, torch.bfloat16
+
+SHAPES = [
+    # (rows, cols, dtype)
+    (64, 4096, BF16),
+    (37, 1024, BF16),     # ragged row count
+    (16, 16384, BF16),
+    (5, 768, F16),        # column tiles partly empty
+    (300, 512, F32),
+    (1, 8, BF16),
+    (1000, 24, F32),
+    (9, 100, F16),        # cols % 8 != 0: scalar kernels
+    (7, 1, F32),
+    (2051, 64, BF16),
+]
+
+
+@pytest.mark.parametrize("rows,cols,dtype", SHAPES)
+@pytest.mark.parametrize("with_bias", [True, False])
+def test_bias_gelu(device, rows, cols, dtype, with_bias):
+    x = randn((rows, cols), dtype, seed=rows + cols, std=1.5)
+    bias = randn((cols,), dtype, seed=rows + cols + 1, std=0.3) if with_bias else None
+    g = randn((rows, cols), dtype, seed=rows + cols + 2)
+    k = _C.get_fused_elementwise_kernel()
+    bd = bias.to(device) if with_bias else None
+    y = k.bias_gelu_forward(x.to(device), bd)
+    oy = cf.bias_gelu_fwd(f64(x), f64(bias) if with_bias else None)
+    check(y, oy, "bias_gelu fwd", atol=1e-6)
+    dx, db = k.bias_gelu_backward(g.to(device), x.to(device), bd)
+    odx, _ = cf.bias_gelu_bwd(f64(g), f64(x), f64(bias) if with_bias else None)
+    check(dx, odx, "bias_gelu bwd dx", atol=1e-6)
+    if with_bias:
+        # dbias = column sum of dx as stored
+        want = f64(dx).sum(0)
+        check(db, want, "bias_gelu dbias", atol=1e-5 * np.sqrt(rows) + 1e-6, min_exact=0.97)
+    else:
+        assert db is None
+
+
+def test_gelu_extreme_inputs(device):
+    k = _C.get_fused_elementwise_kernel()
+    # tiny and moderate inputs: relative accuracy down to the smallest values
+    small = [0.0, -0.0, 1e-30, -1e-30, 1e-10, -1e-10, 0.5, -0.5, 3.0, -3.0, 5.0, -5.0]
+    x = torch.tensor(small * 4 + [0.0] * 16, dtype=F32).view(1, -1)
+    y = k.bias_gelu_forward(x.to(device), None)
+    check(y, cf.bias_gelu_fwd(f64(x), None), "gelu small inputs", atol=1e-37)
+    # large inputs: gelu(u) -> u or -> 0.  The float64 tanh form itself loses
+    # 1 + tanh(z) to cancellation below ~1e-16 * |u|, hence the absolute floor
+    big = [9.0, -9.0, 30.0, -30.0, 100.0, -100.0, 1e4, -1e4]
+    x = torch.tensor(big * 8, dtype=F32).view(1, -1)
+    y = k.bias_gelu_forward(x.to(device), None)
+    check(y, cf.bias_gelu_fwd(f64(x), None), "gelu large inputs", atol=1e-14)
+    assert (y.cpu()[0, 1::2].abs() < 1e-20).all()
+    both = torch.tensor((small + big) * 4, dtype=F32).view(1, -1)
+    dx, _ = k.bias_gelu_backward(torch.ones_like(both).to(device), both.to(device), None)
+    check(dx, cf.bias_gelu_bwd(np.ones_like(f64(both)), f64(both), None)[0], "gelu' extremes", atol=1e-7)
+    assert torch.isfinite(dx).all()
+
+
+def test_bias_gelu_matches_reference_formulas_fp32(device):
+    x = randn((128, 1024), F32, seed=3, std=2.0)
+    b = randn((1024,), F32, seed=4, std=0.02)
+    g = randn((128, 1024), F32, seed=5)
+    k = _C.get_fused_elementwise_kernel()
+    y = k.bias_gelu_forward(x.to(device), b.to(device))
+    dx, db = k.bias_gelu_backward(g.to(device), x.to(device), b.to(device))
+    check(y, f64(tp.bias_gelu(x.double(), b.double())), "vs functional.py:37-40", atol=1e-6)
+    ref_dx = tp.bias_gelu_grad(g.double(), x.double(), b.double())
+    check(dx, f64(ref_dx), "vs functional.py:43-50", atol=1e-6)
+    check(db, f64(ref_dx.sum(0)), "dbias vs autograd reduction", atol=2e-4)
+
+
+@pytest.mark.parametrize("rows,cols,dtype", SHAPES)
+@pytest.mark.parametrize("p", [0.0, 0.1, 0.5])
+@pytest.mark.parametrize("parts", ["bias+res", "bias", "res", "none"])
+def test_bias_dropout_add(device, rows, cols, dtype, p, parts):
+    if parts != "bias+res" and (rows, cols) not in [(64, 4096), (9, 100), (5, 768)]:
+        pytest.skip("operand subsets are covered on three shapes")
+    seed, offset = 1234, 8
+    x = randn((rows, cols), dtype, seed=rows + cols, std=1.0)
+    bias = randn((cols,), dtype, seed=1, std=0.02) if "bias" in parts else None
+    res = randn((rows, cols), dtype, seed=2) if "res" in parts else None
+    g = randn((rows, cols), dtype, seed=3)
+    k = _C.get_fused_elementwise_kernel()
+    dev = lambda t: None if t is None else t.to(device)
+    out, mask = k.bias_dropout_add_forward(dev(x), dev(bias), dev(res), p, seed, offset, return_mask=True)
+    keep = philox.keep_mask(rows * cols, p, seed, offset).reshape(rows, cols)
+    assert np.array_equal(mask.cpu().numpy(), keep), "dropout mask differs from the Philox oracle"
+    want = cf.bias_dropout_add_fwd(
+        f64(x), None if bias is None else f64(bias), None if res is None else f64(res),
+        keep if p > 0 else None, p,
+    )
+    if p == 0.0:
+        # exactness: fp32 arithmetic on <= 3 operands of <= 24 significant bits,
+        # rounded once -> bit-identical to the oracle
+        check(out, want, "bda fwd p=0", atol=0 if dtype != F32 else 1e-7, min_exact=1.0, max_ulp=0)
+    else:
+        check(out, want, "bda fwd", atol=1e-6)
+    # same call without the mask output gives the same values
+    out2 = k.bias_dropout_add_forward(dev(x), dev(bias), dev(res), p, seed, offset)
+    assert torch.equal(out, out2)
+
+    dx, db = k.bias_dropout_add_backward(dev(g), p, seed, offset)
+    odx, _ = cf.bias_dropout_add_bwd(f64(g), keep if p > 0 else None, p)
+    check(dx, odx, "bda bwd dx", atol=1e-6)
+    if p == 0.0:
+        assert torch.equal(dx.cpu(), g)
+    check(db, f64(dx).sum(0), "bda dbias", atol=1e-5 * np.sqrt(rows) + 1e-6, min_exact=0.97)
+    # dbias alone (dx not wanted)
+    _, db2 = k.bias_dropout_add_backward(dev(g), p, seed, offset, need_input_grad=False)
+    assert torch.equal(db, db2)
+
+
+def test_dropout_mask_is_a_function_of_seed_offset_only(device):
+    k = _C.get_fused_elementwise_kernel()
+    x = randn((64, 512), BF16, 1).to(device)
+    _, m1 = k.bias_dropout_add_forward(x, None, None, 0.3, 7, 0, return_mask=True)
+    _, m2 = k.bias_dropout_add_forward(x.float(), None, None, 0.3, 7, 0, return_mask=True)
+    _, m3 = k.bias_dropout_add_forward(x, None, None, 0.3, 7, 4, return_mask=True)
+    _, m4 = k.bias_dropout_add_forward(x, None, None, 0.3, 8, 0, return_mask=True)
+    assert torch.equal(m1, m2)          # independent of dtype / vector width
+    assert not torch.equal(m1, m3) and not torch.equal(m1, m4)
+    flat = k.philox_mask(64 * 512, 0.3, 7, 0, device)
+    assert torch.equal(m1.view(-1), flat)
+    rate = m1.float().mean().item()
+    assert abs(rate - 0.7) < 5 * (0.21 / (64 * 512)) ** 0.5 + 1e-4
+
+
+def test_argument_checks(device):
+    k = _C.get_fused_elementwise_kernel()
+    x = torch.zeros(4, 16, device=device)
+    with pytest.raises(RuntimeError, match="bias"):
+        k.bias_gelu_forward(x, torch.zeros(8, device=device))
+    with pytest.raises(RuntimeError, match="dtype"):
+        k.bias_gelu_forward(x, torch.zeros(16, device=device, dtype=F16))
+    with pytest.raises(RuntimeError, match="not in"):
+        k.bias_dropout_add_forward(x, None, None, 1.5, 0, 0)
+    out = k.bias_dropout_add_forward(x + 1, None, None, 1.0, 0, 0)
+    assert (out == 0).all()
+    y = k.bias_gelu_forward(torch.zeros(0, 16, device=device), None)
+    assert y.shape == (0, 16)

@@ -1,0 +1,159 @@
+"""Scaled causal / padding-masked softmax forward and backward on the GPU,
+through the C ABI, against the float64 oracle and the reference's unfused torch
+chain on identical seeded inputs.  Masked probabilities must be exact zeros."""
+import numpy as np
+import pytest
+import torch
+
+from helpers import check, f64, randn
+from oracle import closed_form as cf
+from oracle import torch_path as tp
+from oslo_amd.torch import _C
+
+pytestmark = pytest.mark.gpu
+
+F32, F16, BF16 = torch.float32, torch.float16, torch.bfloat16
+
+CAUSAL_CASES = [
+    # (attn_batches, sq, sk, dtype, scale)
+    (6, 512, 512, F32, 0.125),      # config-1 row shape
+    (3, 128, 128, F32, 0.125),
+    (5, 64, 64, BF16, 0.3),
+    (2, 2048, 2048, BF16, 0.10206207),  # config-5 row shape
+    (2, 1024, 1024, F16, 0.125),
+    (3, 37, 64, F16, 0.5),          # sq != sk (sub-sequence of queries)
+    (3, 64, 40, BF16, 0.5),         # sq > sk: the first queries see no key
+    (1, 8, 4096, BF16, 1.0),        # 8 chunks per lane
+    (1, 4, 16384, F16, 1.0),        # several waves per row
+    (2, 33, 33, F32, 0.7),          # odd length: scalar kernel
+    (2, 9, 100000, BF16, 1.0),      # beyond the register path
+    (1, 1, 8, F32, 2.0),
+]
+
+
+@pytest.mark.parametrize("ab,sq,sk,dtype,scale", CAUSAL_CASES)
+def test_causal(device, ab, sq, sk, dtype, scale):
+    x = randn((ab, sq, sk), dtype, seed=sq + sk)
+    dy = randn((ab, sq, sk), dtype, seed=sq + sk + 1)
+    k = _C.get_softmax_kernel()
+    y = k.fused_scaled_upper_triang_masked_softmax_forward(x.to(device), scale)
+    oy = cf.softmax_causal_fwd(f64(x), scale)
+    check(y, oy, "causal fwd", atol=1e-9)
+    hidden = torch.from_numpy(cf.causal_hidden(sq, sk))
+    has_visible = (~hidden).any(-1)
+    ycpu = y.cpu()
+    assert (ycpu[:, hidden & has_visible[:, None]] == 0).all(), "hidden keys must be exactly 0"
+    # backward from the kernel's own output (what autograd saves)
+    dx = k.fused_scaled_upper_triang_masked_softmax_backward(dy.to(device), y, scale)
+    odx = cf.softmax_bwd(f64(dy), f64(y), scale)
+    check(dx, odx, "causal bwd", atol=1e-7)
+    assert (dx.cpu()[:, hidden & has_visible[:, None]] == 0).all()
+    # in-place variant writes the same values over dy
+    g = dy.to(device).clone()
+    out = k.fused_scaled_upper_triang_masked_softmax_backward(g, y, scale, inplace=True)
+    assert out.data_ptr() == g.data_ptr() and torch.equal(out, dx)
+
+
+def test_causal_fp32_matches_reference_chain(device):
+    """Config-1 semantics: fp32, scale 0.125, -1e4 fill (modeling_gpt2.py:116-138)."""
+    x = randn((2, 3, 256, 256), F32, seed=1)
+    g = randn((2, 3, 256, 256), F32, seed=2)
+    xr = x.clone().requires_grad_()
+    ref = tp.causal_softmax(xr, 0.125)
+    ref.backward(g)
+    k = _C.get_softmax_kernel()
+    y = k.fused_scaled_upper_triang_masked_softmax_forward(x.view(6, 256, 256).to(device), 0.125)
+    dx = k.fused_scaled_upper_triang_masked_softmax_backward(g.view(6, 256, 256).to(device), y, 0.125)
+    check(y.view_as(x), f64(ref), "causal fwd vs torch chain", atol=1e-9)
+    check(dx.view_as(x), f64(xr.grad), "causal bwd vs torch chain", atol=1e-7)
+
+
+MASKED_CASES = [
+    # (b, np, sq, sk, dtype, scale, mask kind)
+    (3, 2, 64, 1024, F16, 0.125, "padding"),    # config-3 row shape, [b,1,1,sk] mask
+    (2, 2, 128, 128, BF16, 0.125, "padding"),
+    (2, 3, 16, 512, F32, 0.125, "padding"),
+    (2, 2, 32, 256, F16, 0.25, "full"),          # [b,1,sq,sk] arbitrary mask
+    (2, 2, 32, 256, BF16, 0.25, "shared"),       # [1,1,sq,sk]
+    (1, 2, 8, 4096, BF16, 1.0, "padding"),
+    (1, 1, 4, 16384, F16, 1.0, "padding"),
+    (2, 1, 5, 37, F32, 0.5, "full"),             # scalar kernel
+    (2, 2, 16, 64, F16, 1.0, "rows_fully_masked"),
+    (2, 2, 16, 64, BF16, 1.0, "none_masked"),
+]
+
+
+def make_mask(kind, b, sq, sk, seed):
+    r = np.random.default_rng(seed)
+    if kind == "padding":
+        valid = r.integers(max(1, sk // 4), sk + 1, size=b)
+        valid[0] = sk
+        return torch.from_numpy(np.arange(sk)[None, :] >= valid[:, None]).view(b, 1, 1, sk)
+    if kind == "full":
+        m = r.random((b, 1, sq, sk)) < 0.4
+        m[..., 0] = False
+        return torch.from_numpy(m)
+    if kind == "shared":
+        m = r.random((1, 1, sq, sk)) < 0.4
+        m[..., 0] = False
+        return torch.from_numpy(m)
+    if kind == "rows_fully_masked":
+        m = r.random((b, 1, sq, sk)) < 0.3
+        m[:, :, ::3, :] = True
+        return torch.from_numpy(m)
+    return torch.zeros(b, 1, 1, sk, dtype=torch.bool)
+
+
+@pytest.mark.parametrize("b,np_,sq,sk,dtype,scale,kind", MASKED_CASES)
+def test_masked(device, b, np_, sq, sk, dtype, scale, kind):
+    x = randn((b, np_, sq, sk), dtype, seed=sk + sq, std=2.0)
+    dy = randn((b, np_, sq, sk), dtype, seed=sk + sq + 1)
+    mask = make_mask(kind, b, sq, sk, seed=sk)
+    k = _C.get_softmax_kernel()
+    y = k.fused_scaled_masked_softmax_forward(x.to(device), mask.to(device), scale)
+    oy = cf.softmax_masked_fwd(f64(x), mask.numpy(), scale)
+    check(y, oy, "masked fwd", atol=1e-9)
+    full = mask.expand(b, np_, sq, sk)
+    row_has_visible = (~full).any(-1, keepdim=True).expand_as(full)
+    assert (y.cpu()[full & row_has_visible] == 0).all()
+    odx = cf.softmax_bwd(f64(dy), f64(y), scale)
+    # with the mask (masked loads skipped) and without it (dense read): same result
+    dx_m = k.fused_scaled_masked_softmax_backward(dy.to(device), y, scale, mask=mask.to(device))
+    dx_d = k.fused_scaled_masked_softmax_backward(dy.to(device), y, scale)
+    check(dx_m, odx, "masked bwd (mask given)", atol=1e-7)
+    check(dx_d, odx, "masked bwd (dense)", atol=1e-7)
+    assert torch.equal(dx_m, dx_d)
+
+
+def test_padding_fp16_matches_reference_chain(device):
+    """Config-3 semantics against the unfused fp16 chain of the reference
+    (modeling_bert.py:298-306).  The chain rounds scale * x and the sum with the
+    mask to fp16 before the softmax; scale = 0.125 is exact, so the two paths
+    agree to the final rounding."""
+    b, h, sq, sk = 2, 2, 64, 512
+    x = randn((b, h, sq, sk), F16, seed=5, std=2.0)
+    valid = torch.tensor([512, 300])
+    pad = torch.arange(sk)[None, :] >= valid[:, None]
+    ref = tp.padding_softmax(x, pad, 0.125)
+    k = _C.get_softmax_kernel()
+    y = k.fused_scaled_masked_softmax_forward(x.to(device), pad.view(b, 1, 1, sk).to(device), 0.125)
+    assert (y.cpu() == ref).double().mean() > 0.999
+    assert (y.cpu().float() - ref.float()).abs().max() <= 2.0 ** -10
+
+
+def test_mask_dtypes_and_argument_checks(device):
+    k = _C.get_softmax_kernel()
+    x = randn((2, 2, 8, 64), F16, 1).to(device)
+    m_bool = torch.zeros(2, 1, 1, 64, dtype=torch.bool, device=device)
+    m_bool[1, ..., 40:] = True
+    a = k.fused_scaled_masked_softmax_forward(x, m_bool, 1.0)
+    b = k.fused_scaled_masked_softmax_forward(x, m_bool.to(torch.uint8), 1.0)
+    c = k.fused_scaled_masked_softmax_forward(x, m_bool.to(torch.float16), 1.0)
+    assert torch.equal(a, b) and torch.equal(a, c)
+    with pytest.raises(RuntimeError, match="4D"):
+        k.fused_scaled_masked_softmax_forward(x[0], m_bool, 1.0)
+    with pytest.raises(RuntimeError, match="3D"):
+        k.fused_scaled_upper_triang_masked_softmax_forward(x, 1.0)
+    with pytest.raises(RuntimeError, match="broadcast"):
+        k.fused_scaled_masked_softmax_forward(x, m_bool[:, :, :, :32], 1.0)
+    assert k.get_batch_per_block(1024, 1024, 16, 16) >= 1
