@@ -28,6 +28,9 @@ struct Tuning {
   int softmax_rows_per_wave;
   int eltwise_unroll;
   int eltwise_rowgroups;
+  int eltwise_fwd_steps;
+  int norm_bwd_waves;
+  int norm_fwd_waves;
 };
 extern Tuning g_tune;
 

@@ -37,7 +37,7 @@ int device_cu_count() {
   return cached[dev];
 }
 
-Tuning g_tune = {0, 0, 0, 0, 0, 0};
+Tuning g_tune = {0, 0, 0, 0, 0, 0, 0, 0, 0};
 
 }  // namespace oslo
 
@@ -83,6 +83,9 @@ int oslo_tune(const char *key, int value) {
       {"softmax_rows_per_wave", &oslo::g_tune.softmax_rows_per_wave},
       {"eltwise_unroll", &oslo::g_tune.eltwise_unroll},
       {"eltwise_rowgroups", &oslo::g_tune.eltwise_rowgroups},
+      {"eltwise_fwd_steps", &oslo::g_tune.eltwise_fwd_steps},
+      {"norm_bwd_waves", &oslo::g_tune.norm_bwd_waves},
+      {"norm_fwd_waves", &oslo::g_tune.norm_fwd_waves},
   };
   for (const Entry &e : table) {
     if (strcmp(e.name, key) == 0) {

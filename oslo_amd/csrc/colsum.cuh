@@ -7,52 +7,63 @@
 
 namespace oslo {
 
-// Reduces fp32 partial rows part[a][0..P) [cols] (a < narr) to out_a[cols] in
-// dtype V.  Workgroup = 8 column quads x 32 partial-row slices; cols % 4 == 0.
+// Reduces fp32 partial rows part[a][0..P)[cols] to out_a[cols] in dtype V;
+// blockIdx.y selects the array a.  A workgroup owns 32 columns: 8 column quads
+// times 128 slices of the partial rows, so that for the usual P of a few
+// hundred every thread issues all its loads at once; the slices are then
+// folded through LDS in a fixed order.  cols % 4 == 0.
 template <typename V>
-__global__ __launch_bounds__(256) void colsum_finalize_kernel(
+__global__ __launch_bounds__(1024) void colsum_finalize_kernel(
     const float *__restrict__ part, int64_t P, int64_t cols,
     V *__restrict__ out0, V *__restrict__ out1) {
-  __shared__ float sh[32][33];
+  __shared__ float sh[128][33];
+  __shared__ float sh2[8][33];
   const int tid = threadIdx.x;
   const int cq = tid & 7, ps = tid >> 3;
   const int64_t col = ((int64_t)blockIdx.x * 8 + cq) * 4;
-  const int narr = out1 != nullptr ? 2 : 1;
-  for (int a = 0; a < narr; ++a) {
-    float acc[4] = {0.f, 0.f, 0.f, 0.f};
-    if (col < cols) {
-      const float *base = part + (int64_t)a * P * cols + col;
+  const int a = blockIdx.y;
+  float acc[4] = {0.f, 0.f, 0.f, 0.f};
+  if (col < cols) {
+    const float *base = part + (int64_t)a * P * cols + col;
 #pragma unroll 4
-      for (int64_t p = ps; p < P; p += 32) {
-        float t[4];
-        io<float>::unpack(ld16_cached(base + p * cols), t);
+    for (int64_t p = ps; p < P; p += 128) {
+      float t[4];
+      io<float>::unpack(ld16_cached(base + p * cols), t);
 #pragma unroll
-        for (int e = 0; e < 4; ++e) acc[e] += t[e];
-      }
+      for (int e = 0; e < 4; ++e) acc[e] += t[e];
     }
-    __syncthreads();
+  }
 #pragma unroll
-    for (int e = 0; e < 4; ++e) sh[ps][cq * 4 + e] = acc[e];
-    __syncthreads();
-    if (tid < 32) {
-      float s = 0.f;
+  for (int e = 0; e < 4; ++e) sh[ps][cq * 4 + e] = acc[e];
+  __syncthreads();
+  if (tid < 256) {
+    const int g = tid >> 5, c = tid & 31;
+    float s = 0.f;
 #pragma unroll
-      for (int p = 0; p < 32; ++p) s += sh[p][tid];
-      const int64_t oc = (int64_t)blockIdx.x * 32 + tid;
-      if (oc < cols) {
-        V *o = a == 0 ? out0 : out1;
-        o[oc] = io<V>::to_scalar(s);
-      }
+    for (int i = 0; i < 16; ++i) s += sh[g * 16 + i][c];
+    sh2[g][c] = s;
+  }
+  __syncthreads();
+  if (tid < 32) {
+    float s = 0.f;
+#pragma unroll
+    for (int g = 0; g < 8; ++g) s += sh2[g][tid];
+    const int64_t oc = (int64_t)blockIdx.x * 32 + tid;
+    if (oc < cols) {
+      V *o = a == 0 ? out0 : out1;
+      o[oc] = io<V>::to_scalar(s);
     }
   }
 }
 
 template <typename V>
-static inline int launch_colsum_finalize(const float *part, int64_t P, int64_t cols,
-                                  void *out0, void *out1, hipStream_t st) {
+static inline int launch_colsum_finalize(const float *part, int64_t P,
+                                         int64_t cols, void *out0, void *out1,
+                                         hipStream_t st) {
   const int64_t grid = ceil_div(cols, 32);
-  colsum_finalize_kernel<V><<<dim3((unsigned)grid), 256, 0, st>>>(
-      part, P, cols, (V *)out0, (V *)out1);
+  colsum_finalize_kernel<V>
+      <<<dim3((unsigned)grid, out1 != nullptr ? 2 : 1), 1024, 0, st>>>(
+          part, P, cols, (V *)out0, (V *)out1);
   return check_launch("colsum_finalize_kernel");
 }
 

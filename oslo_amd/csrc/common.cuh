@@ -148,6 +148,29 @@ __device__ __forceinline__ void store_chunk(T *p, const float *f) {
     st16_stream(p + v * io<T>::EPV, io<T>::pack(f + v * io<T>::EPV));
 }
 
+// A chunk kept in its packed storage form, for loads issued one iteration
+// ahead of their use (software prefetch): E * sizeof(T) / 4 registers.
+template <typename T, int E> struct RawChunk {
+  static constexpr int NV = E * (int)sizeof(T) / 16;
+  u32x4 r[NV];
+  __device__ __forceinline__ void load(const T *p) {
+#pragma unroll
+    for (int v = 0; v < NV; ++v) r[v] = ld16_stream(p + v * io<T>::EPV);
+  }
+  __device__ __forceinline__ void load_cached(const T *p) {
+#pragma unroll
+    for (int v = 0; v < NV; ++v) r[v] = ld16_cached(p + v * io<T>::EPV);
+  }
+  __device__ __forceinline__ void zero() {
+#pragma unroll
+    for (int v = 0; v < NV; ++v) r[v] = u32x4{0u, 0u, 0u, 0u};
+  }
+  __device__ __forceinline__ void unpack(float *f) const {
+#pragma unroll
+    for (int v = 0; v < NV; ++v) io<T>::unpack(r[v], f + v * io<T>::EPV);
+  }
+};
+
 template <typename A, typename B> struct chunk_elems {
   static constexpr int value =
       16 / (int)(sizeof(A) < sizeof(B) ? sizeof(A) : sizeof(B));
@@ -198,6 +221,90 @@ __device__ __forceinline__ float wave_sum(float v) {
 }
 __device__ __forceinline__ float wave_max(float v) {
   return wave_allreduce<OpMax>(v);
+}
+
+// Welford partial statistics of a set of values: count, mean, and the sum of
+// squared deviations from that mean.  chan_merge combines two disjoint sets
+// (Chan, Golub, LeVeque 1979), as cuChanOnlineSum does in the reference
+// (oslo/torch/_C/csrc/fused_layer_norm.cu:22-38).
+struct Welford {
+  float n, mean, m2;
+};
+
+__device__ __forceinline__ Welford chan_merge(Welford a, Welford b) {
+  const float n = a.n + b.n;
+  const float r = n > 0.f ? b.n * __builtin_amdgcn_rcpf(n) : 0.f;
+  const float d = b.mean - a.mean;
+  Welford o;
+  o.n = n;
+  o.mean = a.mean + d * r;
+  o.m2 = a.m2 + b.m2 + d * d * (a.n * r);
+  return o;
+}
+
+template <int CTRL> __device__ __forceinline__ Welford dpp_welford(Welford v) {
+  Welford o;
+  o.n = dpp_mov<CTRL>(v.n);
+  o.mean = dpp_mov<CTRL>(v.mean);
+  o.m2 = dpp_mov<CTRL>(v.m2);
+  return o;
+}
+
+// All-reduce of Welford partials over the wave: four DPP butterfly steps
+// inside each row of 16 lanes, then the four row results (read from lanes 0,
+// 16, 32, 48) are merged in a fixed order, so every lane returns the same bits.
+__device__ __forceinline__ Welford wave_welford(Welford v) {
+  v = chan_merge(v, dpp_welford<kDppQuadSwap1>(v));
+  v = chan_merge(v, dpp_welford<kDppQuadSwap2>(v));
+  v = chan_merge(v, dpp_welford<kDppRowHalfMirror>(v));
+  v = chan_merge(v, dpp_welford<kDppRowMirror>(v));
+  Welford r[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    r[i].n = readlane(v.n, 16 * i);
+    r[i].mean = readlane(v.mean, 16 * i);
+    r[i].m2 = readlane(v.m2, 16 * i);
+  }
+  return chan_merge(chan_merge(r[0], r[1]), chan_merge(r[2], r[3]));
+}
+
+// The same all-reduce when every lane holds the same number of values
+// (`per_lane`): the merge of two equal-sized sets needs no division and is
+// symmetric, mean = (ma + mb) / 2, M2 = M2a + M2b + (mb - ma)^2 * n / 2.
+__device__ __forceinline__ void merge_equal(float &mean, float &m2, float omean,
+                                            float om2, float n_each) {
+  const float d = omean - mean;
+  mean = 0.5f * (mean + omean);
+  m2 = (m2 + om2) + d * d * (0.5f * n_each);
+}
+
+__device__ __forceinline__ Welford wave_welford_equal(float mean, float m2,
+                                                      float per_lane) {
+  merge_equal(mean, m2, dpp_mov<kDppQuadSwap1>(mean),
+              dpp_mov<kDppQuadSwap1>(m2), per_lane);
+  merge_equal(mean, m2, dpp_mov<kDppQuadSwap2>(mean),
+              dpp_mov<kDppQuadSwap2>(m2), 2.f * per_lane);
+  merge_equal(mean, m2, dpp_mov<kDppRowHalfMirror>(mean),
+              dpp_mov<kDppRowHalfMirror>(m2), 4.f * per_lane);
+  merge_equal(mean, m2, dpp_mov<kDppRowMirror>(mean),
+              dpp_mov<kDppRowMirror>(m2), 8.f * per_lane);
+  float ma = readlane(mean, 0), qa = readlane(m2, 0);
+  float mb = readlane(mean, 32), qb = readlane(m2, 32);
+  merge_equal(ma, qa, readlane(mean, 16), readlane(m2, 16), 16.f * per_lane);
+  merge_equal(mb, qb, readlane(mean, 48), readlane(m2, 48), 16.f * per_lane);
+  merge_equal(ma, qa, mb, qb, 32.f * per_lane);
+  Welford w;
+  w.n = 64.f * per_lane;
+  w.mean = ma;
+  w.m2 = qa;
+  return w;
+}
+
+// 1 / sqrt(a): hardware estimate plus one Newton step (error below 1 ulp).
+__device__ __forceinline__ float rsqrt_refined(float a) {
+  float y = __builtin_amdgcn_rsqf(a);
+  const float h = 0.5f * a * y;
+  return fmaf(y, 0.5f - h * y, y);
 }
 
 // Reduction over the WPR consecutive waves that share one row.  `red` is LDS

@@ -1,14 +1,16 @@
 // bias-GeLU (tanh approximation) and bias-dropout-add, forward and backward,
 // plus the Philox test hooks, for gfx950.
 //
-// Thread mapping (all kernels): a lane owns one chunk of 8 consecutive
-// columns; a wavefront spans 512 columns of one row; the four wavefronts of a
-// workgroup and the workgroups along grid.y stride over the rows, U rows per
-// step so that a lane keeps U independent 128-bit loads in flight.  The bias
-// chunk lives in registers for the whole kernel.  Backward kernels keep the
-// column sums of dx for their 8 columns in registers, fold the four
-// wavefronts through LDS and write one fp32 partial row per workgroup row
-// (grid.y of them); colsum_finalize_kernel reduces those deterministically.
+// Thread mapping (all vector kernels): a lane owns one chunk of 8 consecutive
+// columns.  A 256-thread workgroup is tx lanes wide (64, 128 or 256: up to
+// 2048 columns, one contiguous 4 KB piece of a row) and ty = 256 / tx rows
+// tall, and walks a band of consecutive rows, U row-steps at a time so that a
+// lane keeps U independent 128-bit loads in flight.  Workgroups are numbered
+// column tile first, then band, so the launch sweeps memory front to back.
+// Forward kernels use short bands (one step); backward kernels use longer
+// bands, keep the column sums of dx for their 8 columns in registers, fold the
+// ty rows through LDS and write one fp32 partial row per band, which
+// colsum_finalize_kernel reduces deterministically.
 //
 // Formulas: oslo/torch/nn/modules/functional.py:23-50 (GeLU forward and
 // derivative with the constants 0.79788456, 0.044715, 0.1070322243),
@@ -46,59 +48,81 @@ struct EltGeom {
   int64_t rows;
   int64_t cols;
   int nchunks;  // cols / 8
+  int tx;       // lanes along the columns per workgroup: 64, 128 or 256
+  int ty;       // 256 / tx rows side by side
+  int tiles;    // column tiles = ceil(nchunks / tx)
+  int64_t slots;  // workgroups per column tile; slot s visits row steps
+                  // s, s + slots, s + 2 slots, ... of ty * U rows each
 };
+
+// Position of this thread: column chunk cc (may be >= nchunks), its row
+// inside a step and the slot of its workgroup.  All workgroups advance through
+// the rows together, so at any time the launch touches one compact window of
+// memory that moves front to back.
+struct EltPos {
+  int cc, ry;
+  int64_t slot;
+};
+__device__ __forceinline__ EltPos elt_pos(const EltGeom &g) {
+  const int64_t b = blockIdx.x;
+  EltPos p;
+  p.slot = b / g.tiles;
+  p.cc = (int)(b - p.slot * g.tiles) * g.tx + (int)(threadIdx.x % g.tx);
+  p.ry = threadIdx.x / g.tx;
+  return p;
+}
 
 template <typename T, int U, bool HAS_BIAS>
 __global__ __launch_bounds__(256) void bias_gelu_fwd_kernel(
     const T *__restrict__ x, const T *__restrict__ bias, T *__restrict__ y,
     EltGeom g) {
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int cc = blockIdx.x * kWave + lane;
-  if (cc >= g.nchunks) return;
+  const EltPos ps = elt_pos(g);
+  if (ps.cc >= g.nchunks) return;
   float b[kE];
-  if constexpr (HAS_BIAS) load_chunk<T, kE, false>(bias + (int64_t)cc * kE, b);
-  const int64_t rstride = (int64_t)gridDim.y * 4;
-  for (int64_t r0 = (int64_t)blockIdx.y * 4 + wave; r0 < g.rows;
-       r0 += rstride * U) {
+  if constexpr (HAS_BIAS) load_chunk<T, kE, false>(bias + (int64_t)ps.cc * kE, b);
+  const int64_t coff = (int64_t)ps.cc * kE;
+  for (int64_t r0 = ps.slot * g.ty * U + ps.ry; r0 < g.rows;
+       r0 += g.slots * g.ty * U) {
     float v[U][kE];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      const int64_t r = r0 + u * rstride;
-      if (r < g.rows) load_chunk<T, kE>(x + r * g.cols + (int64_t)cc * kE, v[u]);
+      const int64_t r = r0 + u * g.ty;
+      if (r < g.rows) load_chunk<T, kE>(x + r * g.cols + coff, v[u]);
     }
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      const int64_t r = r0 + u * rstride;
+      const int64_t r = r0 + u * g.ty;
       if (r < g.rows) {
         float o[kE];
 #pragma unroll
         for (int e = 0; e < kE; ++e)
           o[e] = gelu_fwd(HAS_BIAS ? v[u][e] + b[e] : v[u][e]);
-        store_chunk<T, kE>(y + r * g.cols + (int64_t)cc * kE, o);
+        store_chunk<T, kE>(y + r * g.cols + coff, o);
       }
     }
   }
 }
 
-// Folds the per-lane column sums of the four waves and writes the partial row
-// of this workgroup row.  acc is rounded-dx sums; sh is [4][64 * 8] floats.
+// Folds the per-lane column sums of the ty rows of the workgroup and writes
+// the partial row of this slot.  sh is [ty][8][tx] floats (8 KB).
 __device__ __forceinline__ void write_col_partials(const float *acc, float *sh,
                                                    float *__restrict__ part,
-                                                   int64_t cols, int cc,
-                                                   int nchunks, int lane,
-                                                   int wave) {
+                                                   const EltGeom &g,
+                                                   const EltPos &ps) {
+  const int cx = threadIdx.x % g.tx;
+  const int ry = threadIdx.x / g.tx;
 #pragma unroll
-  for (int e = 0; e < kE; ++e) sh[(wave * kE + e) * kWave + lane] = acc[e];
+  for (int e = 0; e < kE; ++e) sh[(ry * kE + e) * g.tx + cx] = acc[e];
   __syncthreads();
-  if (wave == 0 && cc < nchunks) {
+  if (ry == 0 && ps.cc < g.nchunks) {
     float o[kE];
 #pragma unroll
     for (int e = 0; e < kE; ++e) {
-      o[e] = (sh[(0 * kE + e) * kWave + lane] + sh[(1 * kE + e) * kWave + lane]) +
-             (sh[(2 * kE + e) * kWave + lane] + sh[(3 * kE + e) * kWave + lane]);
+      float s = sh[e * g.tx + cx];
+      for (int q = 1; q < g.ty; ++q) s += sh[(q * kE + e) * g.tx + cx];
+      o[e] = s;
     }
-    store_chunk<float, kE>(part + (int64_t)blockIdx.y * cols + (int64_t)cc * kE,
-                           o);
+    store_chunk<float, kE>(part + ps.slot * g.cols + (int64_t)ps.cc * kE, o);
   }
 }
 
@@ -107,33 +131,31 @@ __global__ __launch_bounds__(256) void bias_gelu_bwd_kernel(
     const T *__restrict__ gr, const T *__restrict__ x,
     const T *__restrict__ bias, T *__restrict__ dx, float *__restrict__ part,
     EltGeom g) {
-  __shared__ float sh[4 * kE * kWave];
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int cc = blockIdx.x * kWave + lane;
-  const bool cvalid = cc < g.nchunks;
+  __shared__ float sh[256 * kE];
+  const EltPos ps = elt_pos(g);
   float b[kE], acc[kE];
 #pragma unroll
   for (int e = 0; e < kE; ++e) {
     b[e] = 0.f;
     acc[e] = 0.f;
   }
-  if (cvalid) {
-    if constexpr (HAS_BIAS) load_chunk<T, kE, false>(bias + (int64_t)cc * kE, b);
-    const int64_t rstride = (int64_t)gridDim.y * 4;
-    for (int64_t r0 = (int64_t)blockIdx.y * 4 + wave; r0 < g.rows;
-         r0 += rstride * U) {
+  if (ps.cc < g.nchunks) {
+    if constexpr (HAS_BIAS) load_chunk<T, kE, false>(bias + (int64_t)ps.cc * kE, b);
+    const int64_t coff = (int64_t)ps.cc * kE;
+    for (int64_t r0 = ps.slot * g.ty * U + ps.ry; r0 < g.rows;
+       r0 += g.slots * g.ty * U) {
       float v[U][kE], gv[U][kE];
 #pragma unroll
       for (int u = 0; u < U; ++u) {
-        const int64_t r = r0 + u * rstride;
+        const int64_t r = r0 + u * g.ty;
         if (r < g.rows) {
-          load_chunk<T, kE>(x + r * g.cols + (int64_t)cc * kE, v[u]);
-          load_chunk<T, kE>(gr + r * g.cols + (int64_t)cc * kE, gv[u]);
+          load_chunk<T, kE>(x + r * g.cols + coff, v[u]);
+          load_chunk<T, kE>(gr + r * g.cols + coff, gv[u]);
         }
       }
 #pragma unroll
       for (int u = 0; u < U; ++u) {
-        const int64_t r = r0 + u * rstride;
+        const int64_t r = r0 + u * g.ty;
         if (r < g.rows) {
           float o[kE];
 #pragma unroll
@@ -141,13 +163,12 @@ __global__ __launch_bounds__(256) void bias_gelu_bwd_kernel(
             o[e] = gelu_bwd(v[u][e] + b[e]) * gv[u][e];
             acc[e] += io<T>::round(o[e]);  // sum of dx as stored
           }
-          store_chunk<T, kE>(dx + r * g.cols + (int64_t)cc * kE, o);
+          store_chunk<T, kE>(dx + r * g.cols + coff, o);
         }
       }
     }
   }
-  if (part != nullptr)
-    write_col_partials(acc, sh, part, g.cols, cc, g.nchunks, lane, wave);
+  if (part != nullptr) write_col_partials(acc, sh, part, g, ps);
 }
 
 // ---------------------------------------------------------------------------
@@ -164,31 +185,29 @@ __global__ __launch_bounds__(256) void bias_dropout_add_fwd_kernel(
     const T *__restrict__ x, const T *__restrict__ bias,
     const T *__restrict__ res, T *__restrict__ out,
     uint8_t *__restrict__ mask_out, EltGeom g, DropArgs d) {
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int cc = blockIdx.x * kWave + lane;
-  if (cc >= g.nchunks) return;
+  const EltPos ps = elt_pos(g);
+  if (ps.cc >= g.nchunks) return;
   float b[kE];
-  if constexpr (HAS_BIAS) load_chunk<T, kE, false>(bias + (int64_t)cc * kE, b);
-  const int64_t rstride = (int64_t)gridDim.y * 4;
-  for (int64_t r0 = (int64_t)blockIdx.y * 4 + wave; r0 < g.rows;
-       r0 += rstride * U) {
+  if constexpr (HAS_BIAS) load_chunk<T, kE, false>(bias + (int64_t)ps.cc * kE, b);
+  const int64_t coff = (int64_t)ps.cc * kE;
+  for (int64_t r0 = ps.slot * g.ty * U + ps.ry; r0 < g.rows;
+       r0 += g.slots * g.ty * U) {
     float v[U][kE], rv[U][kE];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      const int64_t r = r0 + u * rstride;
+      const int64_t r = r0 + u * g.ty;
       if (r < g.rows) {
-        load_chunk<T, kE>(x + r * g.cols + (int64_t)cc * kE, v[u]);
-        if constexpr (HAS_RES)
-          load_chunk<T, kE>(res + r * g.cols + (int64_t)cc * kE, rv[u]);
+        load_chunk<T, kE>(x + r * g.cols + coff, v[u]);
+        if constexpr (HAS_RES) load_chunk<T, kE>(res + r * g.cols + coff, rv[u]);
       }
     }
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      const int64_t r = r0 + u * rstride;
+      const int64_t r = r0 + u * g.ty;
       if (r < g.rows) {
         uint32_t keep = 0xffu;
         if constexpr (DROP)
-          keep = dropout_keep_bits((uint64_t)r * (uint64_t)g.nchunks + cc,
+          keep = dropout_keep_bits((uint64_t)r * (uint64_t)g.nchunks + ps.cc,
                                    d.seed, d.offset, d.threshold);
         float o[kE];
 #pragma unroll
@@ -197,7 +216,7 @@ __global__ __launch_bounds__(256) void bias_dropout_add_fwd_kernel(
           if constexpr (DROP) t = (keep >> e) & 1u ? t * d.scale : 0.f;
           o[e] = HAS_RES ? t + rv[u][e] : t;
         }
-        store_chunk<T, kE>(out + r * g.cols + (int64_t)cc * kE, o);
+        store_chunk<T, kE>(out + r * g.cols + coff, o);
         if (mask_out != nullptr) {
           u32x2 m;
           m.x = m.y = 0;
@@ -206,7 +225,7 @@ __global__ __launch_bounds__(256) void bias_dropout_add_fwd_kernel(
             m.x |= ((keep >> e) & 1u) << (8 * e);
             m.y |= ((keep >> (4 + e)) & 1u) << (8 * e);
           }
-          *reinterpret_cast<u32x2 *>(mask_out + r * g.cols + (int64_t)cc * kE) = m;
+          *reinterpret_cast<u32x2 *>(mask_out + r * g.cols + coff) = m;
         }
       }
     }
@@ -217,31 +236,28 @@ template <typename T, int U, bool DROP>
 __global__ __launch_bounds__(256) void bias_dropout_add_bwd_kernel(
     const T *__restrict__ gr, T *__restrict__ dx, float *__restrict__ part,
     EltGeom g, DropArgs d) {
-  __shared__ float sh[4 * kE * kWave];
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int cc = blockIdx.x * kWave + lane;
-  const bool cvalid = cc < g.nchunks;
+  __shared__ float sh[256 * kE];
+  const EltPos ps = elt_pos(g);
   float acc[kE];
 #pragma unroll
   for (int e = 0; e < kE; ++e) acc[e] = 0.f;
-  if (cvalid) {
-    const int64_t rstride = (int64_t)gridDim.y * 4;
-    for (int64_t r0 = (int64_t)blockIdx.y * 4 + wave; r0 < g.rows;
-         r0 += rstride * U) {
+  if (ps.cc < g.nchunks) {
+    const int64_t coff = (int64_t)ps.cc * kE;
+    for (int64_t r0 = ps.slot * g.ty * U + ps.ry; r0 < g.rows;
+       r0 += g.slots * g.ty * U) {
       float gv[U][kE];
 #pragma unroll
       for (int u = 0; u < U; ++u) {
-        const int64_t r = r0 + u * rstride;
-        if (r < g.rows)
-          load_chunk<T, kE>(gr + r * g.cols + (int64_t)cc * kE, gv[u]);
+        const int64_t r = r0 + u * g.ty;
+        if (r < g.rows) load_chunk<T, kE>(gr + r * g.cols + coff, gv[u]);
       }
 #pragma unroll
       for (int u = 0; u < U; ++u) {
-        const int64_t r = r0 + u * rstride;
+        const int64_t r = r0 + u * g.ty;
         if (r < g.rows) {
           uint32_t keep = 0xffu;
           if constexpr (DROP)
-            keep = dropout_keep_bits((uint64_t)r * (uint64_t)g.nchunks + cc,
+            keep = dropout_keep_bits((uint64_t)r * (uint64_t)g.nchunks + ps.cc,
                                      d.seed, d.offset, d.threshold);
           float o[kE];
 #pragma unroll
@@ -251,14 +267,12 @@ __global__ __launch_bounds__(256) void bias_dropout_add_bwd_kernel(
             o[e] = t;
             acc[e] += io<T>::round(t);
           }
-          if (dx != nullptr)
-            store_chunk<T, kE>(dx + r * g.cols + (int64_t)cc * kE, o);
+          if (dx != nullptr) store_chunk<T, kE>(dx + r * g.cols + coff, o);
         }
       }
     }
   }
-  if (part != nullptr)
-    write_col_partials(acc, sh, part, g.cols, cc, g.nchunks, lane, wave);
+  if (part != nullptr) write_col_partials(acc, sh, part, g, ps);
 }
 
 // ---------------------------------------------------------------------------
@@ -419,26 +433,60 @@ __global__ __launch_bounds__(64) void wave_reduce_selftest_kernel(float *out) {
 // ---------------------------------------------------------------------------
 // host side
 // ---------------------------------------------------------------------------
-int64_t colsum_parts_eltwise(int64_t rows, int64_t cols) {
-  const int64_t col_tiles = ceil_div(ceil_div(cols, kE), kWave);
-  int64_t target = g_tune.eltwise_rowgroups > 0
-                       ? g_tune.eltwise_rowgroups
-                       : ceil_div((int64_t)device_cu_count() * 8, col_tiles);
-  const int64_t maxp = ceil_div(rows, 4);
-  if (target > maxp) target = maxp;
-  if (target < 1) target = 1;
-  if (target > 65535) target = 65535;
-  return target;
-}
-
-static inline int eltwise_unroll() {
+static inline int eltwise_unroll(int dflt) {
   const int u = g_tune.eltwise_unroll;
-  return u == 1 || u == 2 || u == 4 ? u : 4;
+  return u == 1 || u == 2 || u == 4 ? u : dflt;
 }
 
-static inline dim3 eltwise_grid(const EltGeom &g) {
-  return dim3((unsigned)ceil_div(g.nchunks, kWave),
-              (unsigned)colsum_parts_eltwise(g.rows, g.cols));
+// Tile shape for `cols`: tx lanes wide (power of two, 64..256), ty rows tall.
+static inline void eltwise_tile(int64_t cols, int *tx, int *ty, int *tiles) {
+  const int64_t nchunks = ceil_div(cols, kE);
+  int t = 64;
+  while (t < 256 && t < nchunks) t *= 2;
+  *tx = t;
+  *ty = 256 / t;
+  *tiles = (int)ceil_div(nchunks, t);
+}
+
+// Backward: workgroups per column tile = fp32 partial rows.  Enough workgroups
+// for about three per CU (measured best on MI355X: the workgroups advance
+// through the rows in step and each lane keeps several loads in flight), so
+// the partial rows stay around one percent of the tensor traffic.
+int64_t colsum_parts_eltwise(int64_t rows, int64_t cols) {
+  int tx, ty, tiles;
+  eltwise_tile(cols, &tx, &ty, &tiles);
+  int64_t parts = g_tune.eltwise_rowgroups > 0
+                      ? g_tune.eltwise_rowgroups
+                      : ceil_div((int64_t)device_cu_count() * 3, tiles);
+  const int64_t min_band =
+      g_tune.eltwise_rowgroups > 0 ? ty : (16 > ty ? 16 : ty);
+  const int64_t maxp = ceil_div(rows, min_band);
+  if (parts > maxp) parts = maxp;
+  if (parts < 1) parts = 1;
+  return parts;
+}
+
+static inline EltGeom eltwise_geom_bwd(int64_t rows, int64_t cols, int unroll) {
+  EltGeom g;
+  g.rows = rows;
+  g.cols = cols;
+  g.nchunks = (int)(cols / kE);
+  eltwise_tile(cols, &g.tx, &g.ty, &g.tiles);
+  const int64_t nsteps = ceil_div(rows, (int64_t)g.ty * unroll);
+  g.slots = colsum_parts_eltwise(rows, cols);
+  if (g.slots > nsteps) g.slots = nsteps;
+  return g;
+}
+
+static inline EltGeom eltwise_geom_fwd(int64_t rows, int64_t cols, int unroll) {
+  EltGeom g;
+  g.rows = rows;
+  g.cols = cols;
+  g.nchunks = (int)(cols / kE);
+  eltwise_tile(cols, &g.tx, &g.ty, &g.tiles);
+  const int steps = g_tune.eltwise_fwd_steps > 0 ? g_tune.eltwise_fwd_steps : 1;
+  g.slots = ceil_div(ceil_div(rows, (int64_t)g.ty * unroll), steps);
+  return g;
 }
 
 static inline int64_t flat_grid(int64_t n) {
@@ -477,9 +525,12 @@ static int run_bias_gelu_fwd(const void *x, const void *bias, void *y,
         (const T *)x, (const T *)bias, (T *)y, n, cols);
     return check_launch("bias_gelu_fwd_generic_kernel");
   }
-  EltGeom g{rows, cols, (int)(cols / kE)};
-  const dim3 grid = eltwise_grid(g);
-  OSLO_ELT_U(eltwise_unroll(), {
+  const int unroll = eltwise_unroll(2);
+  const EltGeom g = eltwise_geom_fwd(rows, cols, unroll);
+  const int64_t nblocks = g.slots * g.tiles;
+  OSLO_REQUIRE(nblocks <= 0x7fffffff, "bias_gelu fwd: too many workgroups");
+  const dim3 grid((unsigned)nblocks);
+  OSLO_ELT_U(unroll, {
     if (bias)
       bias_gelu_fwd_kernel<T, U, true><<<grid, 256, 0, st>>>(
           (const T *)x, (const T *)bias, (T *)y, g);
@@ -507,18 +558,22 @@ static int run_bias_gelu_bwd(const void *gr, const void *x, const void *bias,
         (const T *)dx, (T *)dbias, rows, cols);
     return check_launch("colsum_generic_kernel");
   }
-  EltGeom g{rows, cols, (int)(cols / kE)};
-  const dim3 grid = eltwise_grid(g);
+  const int unroll = eltwise_unroll(2) > 2 ? 2 : eltwise_unroll(2);
+  const EltGeom g = eltwise_geom_bwd(rows, cols, unroll);
+  const int64_t parts = g.slots;
+  const int64_t nblocks = parts * g.tiles;
+  OSLO_REQUIRE(nblocks <= 0x7fffffff, "bias_gelu bwd: too many workgroups");
+  const dim3 grid((unsigned)nblocks);
   float *part = nullptr;
   if (dbias != nullptr) {
-    const int64_t need = (int64_t)grid.y * cols * (int64_t)sizeof(float);
+    const int64_t need = parts * cols * (int64_t)sizeof(float);
     if (ws == nullptr || ws_bytes < need)
       return fail(OSLO_ERR_WORKSPACE,
                   "bias_gelu bwd: workspace of %lld bytes needed, %lld given",
                   (long long)need, (long long)ws_bytes);
     part = (float *)ws;
   }
-  OSLO_ELT_U(eltwise_unroll() > 2 ? 2 : eltwise_unroll(), {
+  OSLO_ELT_U(unroll, {
     if (bias)
       bias_gelu_bwd_kernel<T, U, true><<<grid, 256, 0, st>>>(
           (const T *)gr, (const T *)x, (const T *)bias, (T *)dx, part, g);
@@ -528,7 +583,7 @@ static int run_bias_gelu_bwd(const void *gr, const void *x, const void *bias,
   });
   int rc = check_launch("bias_gelu_bwd_kernel");
   if (rc != OSLO_OK || dbias == nullptr) return rc;
-  return launch_colsum_finalize<T>(part, grid.y, cols, dbias, nullptr, st);
+  return launch_colsum_finalize<T>(part, parts, cols, dbias, nullptr, st);
 }
 
 template <typename T>
@@ -550,12 +605,15 @@ static int run_bda_fwd(const void *x, const void *bias, const void *res,
             n, cols, d, drop);
     return check_launch("bias_dropout_add_fwd_generic_kernel");
   }
-  EltGeom g{rows, cols, (int)(cols / kE)};
-  const dim3 grid = eltwise_grid(g);
+  const int unroll = eltwise_unroll(2) > 2 ? 2 : eltwise_unroll(2);
+  const EltGeom g = eltwise_geom_fwd(rows, cols, unroll);
+  const int64_t nblocks = g.slots * g.tiles;
+  OSLO_REQUIRE(nblocks <= 0x7fffffff, "bias_dropout_add fwd: too many workgroups");
+  const dim3 grid((unsigned)nblocks);
 #define OSLO_BDA_FWD(HB, HR, DR)                                            \
   bias_dropout_add_fwd_kernel<T, U, HB, HR, DR><<<grid, 256, 0, st>>>(      \
       (const T *)x, (const T *)bias, (const T *)res, (T *)out, mask_out, g, d)
-  OSLO_ELT_U(eltwise_unroll() > 2 ? 2 : eltwise_unroll(), {
+  OSLO_ELT_U(unroll, {
     const int key = (bias ? 4 : 0) | (res ? 2 : 0) | (drop ? 1 : 0);
     switch (key) {
       case 0: OSLO_BDA_FWD(false, false, false); break;
@@ -597,11 +655,15 @@ static int run_bda_bwd(const void *gr, void *dx, void *dbias, void *ws,
         (const T *)dx, (T *)dbias, rows, cols);
     return check_launch("colsum_generic_kernel");
   }
-  EltGeom g{rows, cols, (int)(cols / kE)};
-  const dim3 grid = eltwise_grid(g);
+  const int unroll = eltwise_unroll(4);
+  const EltGeom g = eltwise_geom_bwd(rows, cols, unroll);
+  const int64_t parts = g.slots;
+  const int64_t nblocks = parts * g.tiles;
+  OSLO_REQUIRE(nblocks <= 0x7fffffff, "bias_dropout_add bwd: too many workgroups");
+  const dim3 grid((unsigned)nblocks);
   float *part = nullptr;
   if (dbias != nullptr) {
-    const int64_t need = (int64_t)grid.y * cols * (int64_t)sizeof(float);
+    const int64_t need = parts * cols * (int64_t)sizeof(float);
     if (ws == nullptr || ws_bytes < need)
       return fail(OSLO_ERR_WORKSPACE,
                   "bias_dropout_add bwd: workspace of %lld bytes needed, %lld "
@@ -609,7 +671,7 @@ static int run_bda_bwd(const void *gr, void *dx, void *dbias, void *ws,
                   (long long)need, (long long)ws_bytes);
     part = (float *)ws;
   }
-  OSLO_ELT_U(eltwise_unroll(), {
+  OSLO_ELT_U(unroll, {
     if (drop)
       bias_dropout_add_bwd_kernel<T, U, true><<<grid, 256, 0, st>>>(
           (const T *)gr, (T *)dx, part, g, d);
@@ -619,7 +681,7 @@ static int run_bda_bwd(const void *gr, void *dx, void *dbias, void *ws,
   });
   int rc = check_launch("bias_dropout_add_bwd_kernel");
   if (rc != OSLO_OK || dbias == nullptr) return rc;
-  return launch_colsum_finalize<T>(part, grid.y, cols, dbias, nullptr, st);
+  return launch_colsum_finalize<T>(part, parts, cols, dbias, nullptr, st);
 }
 
 #define OSLO_ELT_DISPATCH(dtype, FN, ...)                      \

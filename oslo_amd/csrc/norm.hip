@@ -59,19 +59,47 @@ __device__ __forceinline__ float row_sum1(float a, float *red, int wave,
   return a;
 }
 
+// Welford partials of equal size (every lane holds w.n values) merged over
+// the wave and then over the wpr waves of a row.  red holds two areas of 48
+// floats; `parity` alternates between them from one call to the next so that
+// a single barrier per call suffices.
+__device__ __forceinline__ Welford row_welford(Welford w, float *red, int wave,
+                                               int first, int wpr, int lane,
+                                               int parity) {
+  w = wave_welford_equal(w.mean, w.m2, w.n);
+  if (wpr > 1) {
+    float *area = red + parity * 48;
+    if (lane == 0) {
+      area[wave] = w.mean;
+      area[16 + wave] = w.m2;
+    }
+    __syncthreads();
+    Welford t{w.n, area[first], area[16 + first]};
+    for (int k = 1; k < wpr; ++k) {
+      const Welford o{w.n, area[first + k], area[16 + first + k]};
+      t = chan_merge(t, o);
+    }
+    w = t;
+  }
+  return w;
+}
+
 // ---------------------------------------------------------------------------
 // forward, register-resident
 // ---------------------------------------------------------------------------
-template <typename T, typename V, int VPL, bool RMS, int MAXT>
+// EVEN: every lane holds exactly VPL chunks of its row (no column guards;
+// LayerNorm then merges equal-sized Welford partials).
+template <typename T, typename V, int VPL, bool RMS, bool EVEN, int MAXT>
 __global__ __launch_bounds__(MAXT) void norm_fwd_reg_kernel(
     const T *__restrict__ x, const V *__restrict__ gamma,
     const V *__restrict__ beta, V *__restrict__ y, float *__restrict__ mean,
     float *__restrict__ invvar, int64_t n1, int n2, float eps, int wpr,
     int rpb) {
   constexpr int E = chunk_elems<T, V>::value;
-  __shared__ float red[2][16];
+  __shared__ float red[2][48];
   const int lane = threadIdx.x & 63;
-  const int wave = threadIdx.x >> 6;
+  // the wave index is uniform: keep it (and the row arithmetic) in scalar registers
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int rslot = wave / wpr;
   const int first = rslot * wpr;
   const int nchunks = n2 / E;
@@ -84,12 +112,13 @@ __global__ __launch_bounds__(MAXT) void norm_fwd_reg_kernel(
        base += (int64_t)gridDim.x * rpb) {
     const int64_t row = base + rslot;
     const bool rvalid = row < n1;
-    const T *xr = x + row * n2;
+    // a slot past the last row re-reads row n1 - 1 and stores nothing
+    const T *xr = x + (rvalid ? row : n1 - 1) * n2;
     float v[VPL][E];
 #pragma unroll
     for (int k = 0; k < VPL; ++k) {
       const int c = c0 + k * cstride;
-      if (rvalid && c < nchunks) {
+      if (EVEN || c < nchunks) {
         load_chunk<T, E>(xr + (int64_t)c * E, v[k]);
       } else {
 #pragma unroll
@@ -97,19 +126,57 @@ __global__ __launch_bounds__(MAXT) void norm_fwd_reg_kernel(
       }
     }
 
+    // the affine parameters of this lane's columns: requested now, used last
+    RawChunk<V, E> graw[VPL], braw[VPL];
+    if (gamma != nullptr) {
+#pragma unroll
+      for (int k = 0; k < VPL; ++k) {
+        const int c = c0 + k * cstride;
+        if (c < nchunks) {
+          graw[k].load_cached(gamma + (int64_t)c * E);
+          if constexpr (!RMS) braw[k].load_cached(beta + (int64_t)c * E);
+        }
+      }
+    }
+
     float mu = 0.f, q = 0.f;
-    if constexpr (!RMS) {
+    if constexpr (!RMS && EVEN) {
+      // Welford / Chan: exact mean and sum of squared deviations of the
+      // lane's own (register-resident) elements, then pairwise merges of the
+      // equal-sized (mean, M2) partials across lanes and waves: one barrier.
       float s = 0.f;
 #pragma unroll
       for (int k = 0; k < VPL; ++k)
 #pragma unroll
         for (int e = 0; e < E; ++e) s += v[k][e];
-      s = row_sum1(s, red[0], wave, first, wpr, lane);
+      Welford w;
+      w.n = (float)(VPL * E);
+      w.mean = s * (1.0f / (float)(VPL * E));
+      w.m2 = 0.f;
+#pragma unroll
+      for (int k = 0; k < VPL; ++k)
+#pragma unroll
+        for (int e = 0; e < E; ++e) {
+          const float d = v[k][e] - w.mean;
+          w.m2 += d * d;
+        }
+      w = row_welford(w, &red[0][0], wave, first, wpr, lane, parity);
+      parity ^= 1;
+      mu = w.mean;
+      q = w.m2;
+    } else if constexpr (!RMS) {
+      // ragged rows: the two-pass form, mean first, then the squared
+      // deviations of the valid elements
+      float s = 0.f;
+#pragma unroll
+      for (int k = 0; k < VPL; ++k)
+#pragma unroll
+        for (int e = 0; e < E; ++e) s += v[k][e];
+      s = row_sum1(s, &red[0][0], wave, first, wpr, lane);
       mu = s / fn;
 #pragma unroll
       for (int k = 0; k < VPL; ++k) {
-        const int c = c0 + k * cstride;
-        if (c < nchunks) {
+        if (c0 + k * cstride < nchunks) {
 #pragma unroll
           for (int e = 0; e < E; ++e) {
             const float d = v[k][e] - mu;
@@ -117,7 +184,7 @@ __global__ __launch_bounds__(MAXT) void norm_fwd_reg_kernel(
           }
         }
       }
-      q = row_sum1(q, red[1], wave, first, wpr, lane);
+      q = row_sum1(q, &red[1][0], wave, first, wpr, lane);
     } else {
 #pragma unroll
       for (int k = 0; k < VPL; ++k)
@@ -126,7 +193,7 @@ __global__ __launch_bounds__(MAXT) void norm_fwd_reg_kernel(
       q = row_sum1(q, red[parity], wave, first, wpr, lane);
       parity ^= 1;
     }
-    const float rs = 1.0f / sqrtf(q / fn + eps);
+    const float rs = rsqrt_refined(q / fn + eps);
 
     if (rvalid) {
       V *yr = y + row * n2;
@@ -140,8 +207,8 @@ __global__ __launch_bounds__(MAXT) void norm_fwd_reg_kernel(
             for (int e = 0; e < E; ++e) o[e] = (v[k][e] - mu) * rs;
             if (gamma != nullptr) {
               float g[E], b[E];
-              load_chunk<V, E, false>(gamma + (int64_t)c * E, g);
-              load_chunk<V, E, false>(beta + (int64_t)c * E, b);
+              graw[k].unpack(g);
+              braw[k].unpack(b);
 #pragma unroll
               for (int e = 0; e < E; ++e) o[e] = o[e] * g[e] + b[e];
             }
@@ -150,7 +217,7 @@ __global__ __launch_bounds__(MAXT) void norm_fwd_reg_kernel(
             for (int e = 0; e < E; ++e) o[e] = io<V>::round(v[k][e] * rs);
             if (gamma != nullptr) {
               float g[E];
-              load_chunk<V, E, false>(gamma + (int64_t)c * E, g);
+              graw[k].unpack(g);
 #pragma unroll
               for (int e = 0; e < E; ++e) o[e] = g[e] * o[e];
             }
@@ -253,7 +320,8 @@ __global__ __launch_bounds__(256) void norm_fwd_generic_kernel(
 // ---------------------------------------------------------------------------
 // backward, register-resident, single pass
 // ---------------------------------------------------------------------------
-template <typename T, typename V, int VPL, bool RMS>
+// EVEN: every lane holds exactly VPL chunks of its row (no column guards).
+template <typename T, typename V, int VPL, bool RMS, bool EVEN>
 __global__ __launch_bounds__(1024) void norm_bwd_reg_kernel(
     const V *__restrict__ dy, const T *__restrict__ x,
     const float *__restrict__ mean, const float *__restrict__ invvar,
@@ -263,7 +331,8 @@ __global__ __launch_bounds__(1024) void norm_bwd_reg_kernel(
   extern __shared__ float xslot[];  // [n2] when rpb > 1
   __shared__ float red[2][32];
   const int lane = threadIdx.x & 63;
-  const int wave = threadIdx.x >> 6;
+  // the wave index is uniform: keep it (and the row arithmetic) in scalar registers
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int rslot = wave / wpr;
   const int first = rslot * wpr;
   const int nchunks = n2 / E;
@@ -272,16 +341,16 @@ __global__ __launch_bounds__(1024) void norm_bwd_reg_kernel(
   const float fn = (float)n2;
   const bool affine = gamma != nullptr;
 
-  float gm[VPL][E], acc_g[VPL][E], acc_b[VPL][E];
+  // gamma stays packed (half the registers) and is unpacked once per row
+  RawChunk<V, E> gmraw[VPL];
+  float acc_g[VPL][E], acc_b[VPL][E];
 #pragma unroll
   for (int k = 0; k < VPL; ++k) {
     const int c = c0 + k * cstride;
-    if (affine && c < nchunks) {
-      load_chunk<V, E, false>(gamma + (int64_t)c * E, gm[k]);
-    } else {
-#pragma unroll
-      for (int e = 0; e < E; ++e) gm[k][e] = 1.f;
-    }
+    if (affine && c < nchunks)
+      gmraw[k].load_cached(gamma + (int64_t)c * E);
+    else
+      gmraw[k].zero();
 #pragma unroll
     for (int e = 0; e < E; ++e) {
       acc_g[k][e] = 0.f;
@@ -289,45 +358,67 @@ __global__ __launch_bounds__(1024) void norm_bwd_reg_kernel(
     }
   }
 
+  // The loads of a row are issued one iteration ahead, in packed form, so
+  // that they are in flight while the previous row is reduced and stored.
+  RawChunk<V, E> nd[VPL];
+  RawChunk<T, E> nx[VPL];
+  float nmu = 0.f, nrs = 0.f;
+  const int64_t rstride = (int64_t)gridDim.x * rpb;
+  // A slot past the last row re-reads row n1 - 1 (its results are discarded),
+  // which keeps the loads unconditional.
+#define OSLO_FETCH_ROW(BASE)                                       \
+  do {                                                             \
+    int64_t frow = (BASE) + rslot;                                 \
+    frow = frow < n1 ? frow : n1 - 1;                              \
+    _Pragma("unroll") for (int k = 0; k < VPL; ++k) {              \
+      const int c = c0 + k * cstride;                              \
+      if (EVEN || c < nchunks) {                                   \
+        nd[k].load(dy + frow * n2 + (int64_t)c * E);               \
+        nx[k].load(x + frow * n2 + (int64_t)c * E);                \
+      } else {                                                     \
+        nd[k].zero();                                              \
+        nx[k].zero();                                              \
+      }                                                            \
+    }                                                              \
+    if constexpr (!RMS) nmu = mean[frow];                          \
+    nrs = invvar[frow];                                            \
+  } while (0)
+
+  OSLO_FETCH_ROW((int64_t)blockIdx.x * rpb);
   int parity = 0;
-  for (int64_t base = (int64_t)blockIdx.x * rpb; base < n1;
-       base += (int64_t)gridDim.x * rpb) {
+  for (int64_t base = (int64_t)blockIdx.x * rpb; base < n1; base += rstride) {
     const int64_t row = base + rslot;
     const bool rvalid = row < n1;
-    const V *dyr = dy + row * n2;
-    const T *xr = x + row * n2;
     float d[VPL][E], xh[VPL][E];
 #pragma unroll
     for (int k = 0; k < VPL; ++k) {
-      const int c = c0 + k * cstride;
-      if (rvalid && c < nchunks) {
-        load_chunk<V, E>(dyr + (int64_t)c * E, d[k]);
-        load_chunk<T, E>(xr + (int64_t)c * E, xh[k]);
-      } else {
+      nd[k].unpack(d[k]);
+      nx[k].unpack(xh[k]);
+    }
+    if (!rvalid) {  // wave-uniform: a slot past the end contributes nothing
 #pragma unroll
-        for (int e = 0; e < E; ++e) {
-          d[k][e] = 0.f;
-          xh[k][e] = 0.f;
-        }
-      }
+      for (int k = 0; k < VPL; ++k)
+#pragma unroll
+        for (int e = 0; e < E; ++e) d[k][e] = 0.f;
     }
-    float mu = 0.f, rs = 0.f;
-    if (rvalid) {
-      if constexpr (!RMS) mu = mean[row];
-      rs = invvar[row];
-    }
+    const float mu = nmu, rs = nrs;
+    OSLO_FETCH_ROW(base + rstride);
     float s1 = 0.f, s2 = 0.f;
 #pragma unroll
     for (int k = 0; k < VPL; ++k) {
+      float gm[E];
+      gmraw[k].unpack(gm);
 #pragma unroll
       for (int e = 0; e < E; ++e) {
-        const float h = (xh[k][e] - mu) * rs;  // normalised input
-        const float dg = d[k][e] * gm[k][e];
+        // normalised input; subtract first: exact when x is close to the mean
+        const float h = (xh[k][e] - mu) * rs;
+        const float dg = affine ? d[k][e] * gm[e] : d[k][e];
         xh[k][e] = h;
         s1 += dg;
         s2 += dg * h;
         acc_g[k][e] += d[k][e] * h;
         acc_b[k][e] += d[k][e];
+        d[k][e] = dg;  // only dy * gamma is needed from here on
       }
     }
     if constexpr (RMS) {
@@ -337,21 +428,20 @@ __global__ __launch_bounds__(1024) void norm_bwd_reg_kernel(
       row_sum2(s1, s2, red[parity], wave, first, wpr, lane);
     }
     parity ^= 1;
+    // dx = invvar / n2 * (n2 * dy * gamma - s1 - xhat * s2), regrouped as
+    // invvar * (dy * gamma) - b1 - c2 * xhat
     const float term = rs / fn;
+    const float b1 = term * s1, c2 = term * s2;
     if (rvalid) {
       T *dxr = dx + row * n2;
 #pragma unroll
       for (int k = 0; k < VPL; ++k) {
         const int c = c0 + k * cstride;
-        if (c < nchunks) {
+        if (EVEN || c < nchunks) {
           float o[E];
 #pragma unroll
-          for (int e = 0; e < E; ++e) {
-            float f = fn * d[k][e] * gm[k][e];
-            f -= s1;
-            f -= xh[k][e] * s2;
-            o[e] = f * term;
-          }
+          for (int e = 0; e < E; ++e)
+            o[e] = fmaf(-c2, xh[k][e], fmaf(rs, d[k][e], -b1));
           store_chunk<T, E>(dxr + (int64_t)c * E, o);
         }
       }
@@ -532,12 +622,14 @@ static int launch_norm_fwd(const void *x, const void *gamma, const void *beta,
   static const int kVpl[] = {1, 2, 4, 8};
   RowSplit sp{0, 1, 1, false};
   if (vec_ok) {
+    // up to four chunks per lane measured fastest on MI355X
     const int cap = g_tune.norm_fwd_vpl > 0 ? g_tune.norm_fwd_vpl : 4;
-    sp = split_row(n2 / E, cap > 8 ? 8 : cap, kVpl, 4, 4);
+    const int waves = g_tune.norm_fwd_waves > 0 ? g_tune.norm_fwd_waves : 4;
+    sp = split_row(n2 / E, cap > 8 ? 8 : cap, kVpl, 4, waves);
     // more than 32 resident elements per lane only fit the register budget
     // of a workgroup of at most 256 threads
     if (sp.ok && sp.wpr * sp.rpb > 4 && sp.vpl * E > 32)
-      sp = split_row(n2 / E, 32 / E, kVpl, 4, 4);
+      sp = split_row(n2 / E, 32 / E, kVpl, 4, waves);
   }
   if (!sp.ok) {
     int64_t grid = n1 < 65535 * 16 ? n1 : 65535 * 16;
@@ -547,21 +639,35 @@ static int launch_norm_fwd(const void *x, const void *gamma, const void *beta,
     return check_launch("norm_fwd_generic_kernel");
   }
   const int threads = kWave * sp.wpr * sp.rpb;
+  // every lane holds exactly vpl chunks: LayerNorm takes the Welford path
+  const bool even = (n2 / E) == (int64_t)sp.vpl * kWave * sp.wpr;
   int64_t grid = ceil_div(n1, sp.rpb);
   const int64_t maxgrid = (int64_t)device_cu_count() * 64;
   if (grid > maxgrid) grid = maxgrid;
 #define OSLO_FWD_CASE(VPL)                                                  \
   case VPL:                                                                 \
-    if (threads <= 256)                                                     \
-      norm_fwd_reg_kernel<T, V, VPL, RMS, 256>                              \
+    if (threads <= 256 && even)                                             \
+      norm_fwd_reg_kernel<T, V, VPL, RMS, true, 256>                        \
           <<<dim3((unsigned)grid), threads, 0, st>>>(                       \
               (const T *)x, (const V *)gamma, (const V *)beta, (V *)y,      \
               mean, invvar, n1, (int)n2, eps, sp.wpr, sp.rpb);              \
-    else if constexpr (VPL * E <= 32)                                       \
-      norm_fwd_reg_kernel<T, V, VPL, RMS, 1024>                             \
+    else if (threads <= 256)                                                \
+      norm_fwd_reg_kernel<T, V, VPL, RMS, false, 256>                       \
           <<<dim3((unsigned)grid), threads, 0, st>>>(                       \
               (const T *)x, (const V *)gamma, (const V *)beta, (V *)y,      \
               mean, invvar, n1, (int)n2, eps, sp.wpr, sp.rpb);              \
+    else if constexpr (VPL * E <= 32) {                                     \
+      if (even)                                                             \
+        norm_fwd_reg_kernel<T, V, VPL, RMS, true, 1024>                     \
+            <<<dim3((unsigned)grid), threads, 0, st>>>(                     \
+                (const T *)x, (const V *)gamma, (const V *)beta, (V *)y,    \
+                mean, invvar, n1, (int)n2, eps, sp.wpr, sp.rpb);            \
+      else                                                                  \
+        norm_fwd_reg_kernel<T, V, VPL, RMS, false, 1024>                    \
+            <<<dim3((unsigned)grid), threads, 0, st>>>(                     \
+                (const T *)x, (const V *)gamma, (const V *)beta, (V *)y,    \
+                mean, invvar, n1, (int)n2, eps, sp.wpr, sp.rpb);            \
+    }                                                                       \
     else                                                                    \
       return fail(OSLO_ERR_UNSUPPORTED,                                     \
                   "norm fwd: vpl=%d needs a workgroup of at most 256 "      \
@@ -597,9 +703,22 @@ static int launch_norm_bwd(const void *dy, const void *x, const float *mean,
   static const int kVpl4[] = {1, 2, 4};
   RowSplit sp{0, 1, 1, false};
   if (vec_ok) {
-    int cap = g_tune.norm_bwd_vpl > 0 ? g_tune.norm_bwd_vpl : 16 / E;
-    if (cap > 16 / E) cap = 16 / E;
-    sp = split_row(n2 / E, cap, E == 8 ? kVpl8 : kVpl4, E == 8 ? 2 : 3, 16);
+    const int *allowed = E == 8 ? kVpl8 : kVpl4;
+    const int nallowed = E == 8 ? 2 : 3;
+    const int waves = g_tune.norm_bwd_waves > 0 ? g_tune.norm_bwd_waves : 16;
+    if (g_tune.norm_bwd_vpl > 0) {
+      int cap = g_tune.norm_bwd_vpl;
+      if (cap > 16 / E) cap = 16 / E;
+      sp = split_row(n2 / E, cap, allowed, nallowed, waves);
+    } else {
+      // measured best on MI355X: 8 elements per lane as long as a workgroup
+      // still holds two rows, else 16 elements per lane
+      sp = split_row(n2 / E, 8 / E, allowed, nallowed, waves);
+      if (!sp.ok || sp.rpb < 2) {
+        const RowSplit wide = split_row(n2 / E, 16 / E, allowed, nallowed, waves);
+        if (wide.ok) sp = wide;
+      }
+    }
   }
   if (!sp.ok) {
     int64_t grid = n1 < 65535 * 16 ? n1 : 65535 * 16;
@@ -627,13 +746,21 @@ static int launch_norm_bwd(const void *dy, const void *x, const float *mean,
   }
   const int threads = kWave * sp.wpr * sp.rpb;
   const size_t lds = sp.rpb > 1 ? (size_t)n2 * sizeof(float) : 0;
-#define OSLO_BWD_CASE(VPL)                                                   \
+  const bool even = (n2 / E) == (int64_t)sp.vpl * kWave * sp.wpr;
+#define OSLO_BWD_CASE(VPL)                                                  \
   case VPL:                                                                  \
-    if constexpr (VPL * E <= 16)                                             \
-      norm_bwd_reg_kernel<T, V, VPL, RMS>                                    \
-          <<<dim3((unsigned)P), threads, lds, st>>>(                         \
-              (const V *)dy, (const T *)x, mean, invvar, (const V *)gamma,   \
-              (T *)dx, part, n1, (int)n2, sp.wpr, sp.rpb);                   \
+    if constexpr (VPL * E <= 16) {                                           \
+      if (even)                                                              \
+        norm_bwd_reg_kernel<T, V, VPL, RMS, true>                            \
+            <<<dim3((unsigned)P), threads, lds, st>>>(                       \
+                (const V *)dy, (const T *)x, mean, invvar, (const V *)gamma, \
+                (T *)dx, part, n1, (int)n2, sp.wpr, sp.rpb);                 \
+      else                                                                   \
+        norm_bwd_reg_kernel<T, V, VPL, RMS, false>                           \
+            <<<dim3((unsigned)P), threads, lds, st>>>(                       \
+                (const V *)dy, (const T *)x, mean, invvar, (const V *)gamma, \
+                (T *)dx, part, n1, (int)n2, sp.wpr, sp.rpb);                 \
+    }                                                                        \
     break;
   switch (sp.vpl) {
     OSLO_BWD_CASE(1)

@@ -111,9 +111,11 @@ __global__ __launch_bounds__(1024) void softmax_fwd_kernel(
     const T *__restrict__ x, const uint8_t *__restrict__ mask,
     T *__restrict__ y, SoftmaxGeom g, float scale) {
   constexpr int E = io<T>::EPV;
+  constexpr uint32_t kAll = (1u << E) - 1u;
   __shared__ float red[2][16];
   const int lane = threadIdx.x & 63;
-  const int wave = threadIdx.x >> 6;
+  // the wave index is uniform: keep it (and the row arithmetic) in scalar registers
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int rslot = wave / g.wpr;
   const int first = rslot * g.wpr;
   const int nchunks = g.sk / E;
@@ -167,18 +169,43 @@ __global__ __launch_bounds__(1024) void softmax_fwd_kernel(
     }
   }
 
+  // Wave-uniform shortcuts: where no lane of the wave sees a key of chunk
+  // slot (j, k) the arithmetic is skipped altogether; where every lane sees
+  // all its keys the per-element mask selects are skipped.  The logits are
+  // kept in the log2 domain, t = x * (scale * log2 e), so exp is one exp2.
+  bool none_visible[RPW][VPL], all_visible[RPW][VPL];
+#pragma unroll
+  for (int j = 0; j < RPW; ++j)
+#pragma unroll
+    for (int k = 0; k < VPL; ++k) {
+      none_visible[j][k] = __builtin_amdgcn_ballot_w64(mbits[j][k] != kAll) == 0;
+      all_visible[j][k] = __builtin_amdgcn_ballot_w64(mbits[j][k] != 0u) == 0;
+    }
+  const float c2 = scale * kLog2e;
+
   float mx[RPW];
 #pragma unroll
   for (int j = 0; j < RPW; ++j) {
     float m = ninf;
 #pragma unroll
-    for (int k = 0; k < VPL; ++k)
+    for (int k = 0; k < VPL; ++k) {
+      if (none_visible[j][k]) continue;
+      if (all_visible[j][k]) {
 #pragma unroll
-      for (int e = 0; e < E; ++e) {
-        const float t = (mbits[j][k] >> e) & 1u ? ninf : v[j][k][e] * scale;
-        v[j][k][e] = t;
-        m = fmaxf(m, t);
+        for (int e = 0; e < E; ++e) {
+          const float t = v[j][k][e] * c2;
+          v[j][k][e] = t;
+          m = fmaxf(m, t);
+        }
+      } else {
+#pragma unroll
+        for (int e = 0; e < E; ++e) {
+          const float t = (mbits[j][k] >> e) & 1u ? ninf : v[j][k][e] * c2;
+          v[j][k][e] = t;
+          m = fmaxf(m, t);
+        }
       }
+    }
     mx[j] = m;
   }
 #pragma unroll
@@ -193,13 +220,15 @@ __global__ __launch_bounds__(1024) void softmax_fwd_kernel(
     float s = 0.f;
     const float off = mx[j] == ninf ? 0.f : mx[j];
 #pragma unroll
-    for (int k = 0; k < VPL; ++k)
+    for (int k = 0; k < VPL; ++k) {
+      if (none_visible[j][k]) continue;
 #pragma unroll
       for (int e = 0; e < E; ++e) {
-        const float p = __builtin_amdgcn_exp2f((v[j][k][e] - off) * kLog2e);
+        const float p = __builtin_amdgcn_exp2f(v[j][k][e] - off);
         v[j][k][e] = p;  // exp2(-inf) == 0 for masked keys
         s += p;
       }
+    }
     sm[j] = s;
   }
 #pragma unroll
@@ -220,8 +249,13 @@ __global__ __launch_bounds__(1024) void softmax_fwd_kernel(
       const int c = c0 + k * cstride;
       if (c < nchunks) {
         float o[E];
+        if (none_visible[j][k]) {
 #pragma unroll
-        for (int e = 0; e < E; ++e) o[e] = v[j][k][e] * inv + fill;
+          for (int e = 0; e < E; ++e) o[e] = fill;
+        } else {
+#pragma unroll
+          for (int e = 0; e < E; ++e) o[e] = v[j][k][e] * inv + fill;
+        }
         store_chunk<T, E>(yr + (int64_t)c * E, o);
       }
     }
@@ -237,7 +271,8 @@ __global__ __launch_bounds__(1024) void softmax_bwd_kernel(
   constexpr uint32_t kAll = (1u << E) - 1u;
   __shared__ float red[2][16];
   const int lane = threadIdx.x & 63;
-  const int wave = threadIdx.x >> 6;
+  // the wave index is uniform: keep it (and the row arithmetic) in scalar registers
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int rslot = wave / g.wpr;
   const int first = rslot * g.wpr;
   const int nchunks = g.sk / E;
@@ -306,14 +341,24 @@ __global__ __launch_bounds__(1024) void softmax_bwd_kernel(
       }
     }
   }
+  // wave-uniform: no lane of the wave loaded chunk slot (j, k) -> no arithmetic
+  bool none_loaded[RPW][VPL];
+#pragma unroll
+  for (int j = 0; j < RPW; ++j)
+#pragma unroll
+    for (int k = 0; k < VPL; ++k)
+      none_loaded[j][k] = __builtin_amdgcn_ballot_w64(!skip[j][k]) == 0;
+
   float s[RPW];
 #pragma unroll
   for (int j = 0; j < RPW; ++j) {
     float a = 0.f;
 #pragma unroll
-    for (int k = 0; k < VPL; ++k)
+    for (int k = 0; k < VPL; ++k) {
+      if (none_loaded[j][k]) continue;
 #pragma unroll
       for (int e = 0; e < E; ++e) a += yv[j][k][e] * gv[j][k][e];
+    }
     s[j] = a;
   }
 #pragma unroll
@@ -329,9 +374,14 @@ __global__ __launch_bounds__(1024) void softmax_bwd_kernel(
       const int c = c0 + k * cstride;
       if (c < nchunks) {
         float o[E];
+        if (none_loaded[j][k]) {
 #pragma unroll
-        for (int e = 0; e < E; ++e)
-          o[e] = scale * (yv[j][k][e] * (gv[j][k][e] - s[j]));
+          for (int e = 0; e < E; ++e) o[e] = 0.f;
+        } else {
+#pragma unroll
+          for (int e = 0; e < E; ++e)
+            o[e] = scale * (yv[j][k][e] * (gv[j][k][e] - s[j]));
+        }
         store_chunk<T, E>(dxr + (int64_t)c * E, o);
       }
     }
@@ -422,7 +472,8 @@ struct SoftmaxPlan {
 };
 
 // max_elems: elements of one operand a lane may hold (register budget).
-static SoftmaxPlan plan_softmax(int64_t sk, int E, int max_elems) {
+static SoftmaxPlan plan_softmax(int64_t sk, int E, int max_elems,
+                                int default_rpw) {
   SoftmaxPlan p{0, 1, 1, 1, false};
   if (sk % E != 0) return p;
   const int64_t nchunks = sk / E;
@@ -433,9 +484,10 @@ static SoftmaxPlan plan_softmax(int64_t sk, int E, int max_elems) {
   int vpl = need <= 1 ? 1 : need <= 2 ? 2 : need <= 4 ? 4 : 8;
   int rpw = 1;
   if (wpr == 1) {
-    // aim at 32 resident elements per lane per operand
+    // rows a wave handles at once; measured best on MI355X: one, or two
+    // for the forward with a mask tensor (its loads wait for the mask bytes)
     int want = g_tune.softmax_rows_per_wave > 0 ? g_tune.softmax_rows_per_wave
-                                                : 32 / (vpl * E);
+                                                : default_rpw;
     rpw = want >= 4 ? 4 : (want >= 2 ? 2 : 1);
     while (rpw > 1 && (rpw * vpl * E > max_elems || rpw * vpl > 8)) rpw >>= 1;
   }
@@ -476,7 +528,8 @@ template <typename T, int MODE>
 static int launch_softmax_fwd(const void *x, const uint8_t *mask, void *y,
                               SoftmaxGeom g, float scale, hipStream_t st) {
   constexpr int E = io<T>::EPV;
-  SoftmaxPlan pl = plan_softmax(g.sk, E, kFwdMaxElems);
+  SoftmaxPlan pl =
+      plan_softmax(g.sk, E, kFwdMaxElems, MODE == kModeMasked ? 2 : 1);
   const bool vec_ok = pl.ok && aligned16(x) && aligned16(y) &&
                       (MODE != kModeMasked ||
                        (reinterpret_cast<uintptr_t>(mask) % E) == 0);
@@ -508,7 +561,7 @@ static int launch_softmax_bwd(const void *dy, const void *y,
                               const uint8_t *mask, void *dx, SoftmaxGeom g,
                               float scale, hipStream_t st) {
   constexpr int E = io<T>::EPV;
-  SoftmaxPlan pl = plan_softmax(g.sk, E, kBwdMaxElems);
+  SoftmaxPlan pl = plan_softmax(g.sk, E, kBwdMaxElems, 1);
   const bool vec_ok = pl.ok && aligned16(dy) && aligned16(y) &&
                       aligned16(dx) &&
                       (MODE != kModeMasked ||
@@ -649,7 +702,7 @@ int oslo_softmax_batch_per_block(int64_t sq, int64_t sk, int64_t b,
                 "softmax_batch_per_block: bad shape");
   // rows per workgroup of the 16-bit masked kernel (the reference's shim only
   // admits fp16 / bf16); rows that do not vectorise run one row per workgroup
-  SoftmaxPlan pl = plan_softmax(sk, 8, kFwdMaxElems);
+  SoftmaxPlan pl = plan_softmax(sk, 8, kFwdMaxElems, 2);
   if (!pl.ok) return 1;
   return pl.rpb * pl.rpw;
 }

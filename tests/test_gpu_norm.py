@@ -105,10 +105,12 @@ def test_rms_norm(device, n1, n2, tin, tout, affine):
         y, invvar = k.rms_norm_forward(xd, (n2,), eps)
     assert y.dtype == tout and invvar.dtype == F32
     # the oracle rounds twice (normalised value, then the product with gamma);
-    # compare in the storage type, allowing 1 ulp where fp32 vs fp64 arithmetic
-    # tips the first rounding
+    # compare in the storage type.  Where fp32 vs fp64 arithmetic tips the
+    # first rounding the intermediate moves by 1 ulp, and its product with a
+    # gamma > 1 can then land 2 ulp away after the second rounding
     oy, oinv = cf.rms_norm_fwd(f64(x), f64(gamma) if affine else None, eps, out=NAME[tout])
-    check(y, np.asarray(oy, dtype=np.float64), "rms fwd y", atol=2e-6, min_exact=0.995)
+    check(y, np.asarray(oy, dtype=np.float64), "rms fwd y", atol=2e-6, min_exact=0.995,
+          max_ulp=2 if (affine and tout != F32) else 1)
     check_f32(invvar, oinv, "rms invvar", atol=0)
 
     if affine:
