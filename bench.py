@@ -31,6 +31,11 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published
 METRIC = "achieved HBM GB/s (% of MI355X peak) per fused fwd+bwd kernel; speedup vs CPU path"
+# HBM traffic of one LayerNorm-backward call on bf16 [16384, 4096], measured with
+# rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE and calibrated against a 1 GiB copy:
+# main kernel 270.6 MB read + 140.4 MB written, finalize 8.4 MB read
+# (summary: profiles/bench_all_kernels_hbm_traffic.txt).  Algorithmic: 402.7 MB.
+LN_BWD_TRAFFIC_BYTES = 419.4e6
 
 F32, F16, BF16 = 0, 1, 2
 
@@ -435,7 +440,8 @@ def main():
             "peak": HBM_PEAK_GBPS,
             "unit": "GB/s",
             "frac": round(achieved / HBM_PEAK_GBPS, 4),
-            "traffic": None,
+            "traffic": LN_BWD_TRAFFIC_BYTES,
+            "traffic_unit": "HBM bytes per oslo_ln_bwd call, rocprofv3 FETCH_SIZE + WRITE_SIZE scaled by a 1 GiB copy",
             "algorithmic_MB_per_launch": round(3 * T / 1e6, 1),
             "avg_us": round(bwd_ms * 1e3, 2),
         },

@@ -399,20 +399,14 @@ __global__ __launch_bounds__(256) void philox_words_kernel(
   }
 }
 
+// One 128-bit vector per thread, workgroups in memory order: the fastest copy
+// measured on MI355X (short-lived waves sweeping one compact window).
 __global__ __launch_bounds__(256) void copy_probe_kernel(
     const u32x4 *__restrict__ src, u32x4 *__restrict__ dst, int64_t nvec) {
   const int64_t stride = (int64_t)gridDim.x * 256;
-  int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  for (; i + 3 * stride < nvec; i += 4 * stride) {
-    u32x4 a = ld16_stream(src + i), b = ld16_stream(src + i + stride);
-    u32x4 c = ld16_stream(src + i + 2 * stride),
-          e = ld16_stream(src + i + 3 * stride);
-    st16_stream(dst + i, a);
-    st16_stream(dst + i + stride, b);
-    st16_stream(dst + i + 2 * stride, c);
-    st16_stream(dst + i + 3 * stride, e);
-  }
-  for (; i < nvec; i += stride) st16_stream(dst + i, ld16_stream(src + i));
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < nvec;
+       i += stride)
+    st16_stream(dst + i, ld16_stream(src + i));
 }
 
 __global__ __launch_bounds__(64) void wave_reduce_selftest_kernel(float *out) {
@@ -801,9 +795,8 @@ int oslo_copy_probe(const void *src, void *dst, int64_t bytes, void *stream) {
                "16-byte aligned");
   if (bytes == 0) return OSLO_OK;
   const int64_t nvec = bytes / 16;
-  int64_t grid = ceil_div(nvec, 256 * 4);
-  const int64_t cap = (int64_t)device_cu_count() * 16;
-  if (grid > cap) grid = cap;
+  int64_t grid = ceil_div(nvec, 256);
+  if (grid > 0x7fffffff) grid = 0x7fffffff;
   copy_probe_kernel<<<dim3((unsigned)grid), 256, 0, (hipStream_t)stream>>>(
       (const u32x4 *)src, (u32x4 *)dst, nvec);
   return check_launch("copy_probe_kernel");
