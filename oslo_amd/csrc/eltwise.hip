@@ -4,12 +4,14 @@
 // Thread mapping (all vector kernels): a lane owns one chunk of 8 consecutive
 // columns.  A 256-thread workgroup is tx lanes wide (64, 128 or 256: up to
 // 2048 columns, one contiguous 4 KB piece of a row) and ty = 256 / tx rows
-// tall, and walks a band of consecutive rows, U row-steps at a time so that a
-// lane keeps U independent 128-bit loads in flight.  Workgroups are numbered
-// column tile first, then band, so the launch sweeps memory front to back.
-// Forward kernels use short bands (one step); backward kernels use longer
-// bands, keep the column sums of dx for their 8 columns in registers, fold the
-// ty rows through LDS and write one fp32 partial row per band, which
+// tall.  The rows are cut into steps of ty * U consecutive rows (a lane keeps
+// U independent 128-bit loads in flight); workgroups are numbered column tile
+// first, then slot, and slot s visits steps s, s + slots, s + 2 slots, ...
+// Forward kernels launch one workgroup per step, so the launch sweeps memory
+// front to back with short-lived waves.  Backward kernels launch about three
+// workgroups per CU; they advance through the rows in lockstep (one compact
+// moving window), keep the column sums of dx for their 8 columns in registers,
+// fold the ty rows through LDS and write one fp32 partial row per slot, which
 // colsum_finalize_kernel reduces deterministically.
 //
 // Formulas: oslo/torch/nn/modules/functional.py:23-50 (GeLU forward and

@@ -3,15 +3,16 @@
 // Register-resident path (rows of up to 64 * 16 * 8 chunks): a row is split
 // over `wpr` consecutive wavefronts, every lane holds VPL chunks of E
 // elements in registers, so x (and dy) are read from HBM exactly once.
-// Statistics are the exact two-pass form of Welford/Chan for resident data:
-// mean first, then the sum of squared deviations, both reduced with DPP
-// inside a wave and through LDS across the waves of a row.
+// LayerNorm statistics are Welford/Chan: each lane takes the exact mean and
+// sum of squared deviations of its own resident elements, the equal-sized
+// partials are merged pairwise by a DPP butterfly inside the wave and through
+// LDS across the waves of a row (one barrier).  RMSNorm needs one sum.
 //
-// Backward is a single pass over dy and x: persistent workgroups stride over
-// the rows, keep the per-column partial sums of dgamma / dbeta in registers
-// for the columns their lanes own, and write one fp32 partial row per
-// workgroup; a small finalize kernel reduces the partial rows in a fixed
-// order (deterministic, no atomics).
+// Backward is a single pass over dy and x: one persistent workgroup per CU
+// strides over the rows (the next row is prefetched in packed form), keeps
+// the per-column partial sums of dgamma / dbeta in registers for the columns
+// its lanes own, and writes one fp32 partial row; a small finalize kernel
+// reduces the partial rows in a fixed order (deterministic, no atomics).
 //
 // Formulas follow oslo/torch/_C/csrc/fused_layer_norm.cu:310-359 (forward)
 // and :594-741 (grad input), :458-591 (grad gamma/beta) of the reference.
@@ -238,17 +239,6 @@ __global__ __launch_bounds__(MAXT) void norm_fwd_reg_kernel(
 // streaming Welford per thread merged with Chan's formula; second pass
 // re-reads the row (L2-resident).
 // ---------------------------------------------------------------------------
-struct Wf {
-  float n, mu, m2;
-};
-__device__ __forceinline__ Wf wf_merge(Wf a, Wf b) {
-  const float n = a.n + b.n;
-  if (n == 0.f) return Wf{0.f, 0.f, 0.f};
-  const float d = b.mu - a.mu;
-  const float fb = b.n / n;
-  return Wf{n, a.mu + d * fb, a.m2 + b.m2 + d * d * a.n * fb};
-}
-
 template <typename T, typename V, bool RMS>
 __global__ __launch_bounds__(256) void norm_fwd_generic_kernel(
     const T *__restrict__ x, const V *__restrict__ gamma,
@@ -258,43 +248,39 @@ __global__ __launch_bounds__(256) void norm_fwd_generic_kernel(
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   for (int64_t row = blockIdx.x; row < n1; row += gridDim.x) {
     const T *xr = x + row * n2;
-    Wf w{0.f, 0.f, 0.f};
+    Welford w{0.f, 0.f, 0.f};
     for (int64_t i = tid; i < n2; i += 256) {
       const float v = io<T>::from_scalar(xr[i]);
       if constexpr (RMS) {
         w.m2 += v * v;
       } else {
+        // Welford's online update (fused_layer_norm.cu:12-19 of the reference)
         w.n += 1.f;
-        const float d = v - w.mu;
-        w.mu += d / w.n;
-        w.m2 += d * (v - w.mu);
+        const float d = v - w.mean;
+        w.mean += d / w.n;
+        w.m2 += d * (v - w.mean);
       }
     }
-#pragma unroll
-    for (int m = 1; m < 64; m <<= 1) {
-      Wf o{__shfl_xor(w.n, m, 64), __shfl_xor(w.mu, m, 64),
-           __shfl_xor(w.m2, m, 64)};
-      if constexpr (RMS)
-        w.m2 += o.m2;
-      else
-        w = wf_merge(w, o);
-    }
+    if constexpr (RMS)
+      w.m2 = wave_sum(w.m2);
+    else
+      w = wave_welford(w);
     if (lane == 0) {
       sh[0][wave] = w.n;
-      sh[1][wave] = w.mu;
+      sh[1][wave] = w.mean;
       sh[2][wave] = w.m2;
     }
     __syncthreads();
-    Wf t{sh[0][0], sh[1][0], sh[2][0]};
+    Welford t{sh[0][0], sh[1][0], sh[2][0]};
     for (int k = 1; k < 4; ++k) {
-      Wf o{sh[0][k], sh[1][k], sh[2][k]};
+      const Welford o{sh[0][k], sh[1][k], sh[2][k]};
       if constexpr (RMS)
         t.m2 += o.m2;
       else
-        t = wf_merge(t, o);
+        t = chan_merge(t, o);
     }
     __syncthreads();
-    const float mu = RMS ? 0.f : t.mu;
+    const float mu = RMS ? 0.f : t.mean;
     const float rs = 1.0f / sqrtf(t.m2 / (float)n2 + eps);
     V *yr = y + row * n2;
     for (int64_t i = tid; i < n2; i += 256) {
