@@ -222,7 +222,8 @@ int oslo_wave_reduce_selftest(float *out4, void *stream);
 /* Overrides a launch heuristic (for tuning sweeps): key is one of
  * "norm_fwd_vpl", "norm_bwd_vpl", "norm_bwd_blocks_per_cu",
  * "softmax_rows_per_wave", "eltwise_unroll", "eltwise_rowgroups",
- * "eltwise_fwd_steps", "norm_bwd_waves", "norm_fwd_waves";
+ * "eltwise_fwd_steps", "norm_bwd_waves", "norm_fwd_waves",
+ * "norm_bwd_prefetch", "norm_fwd_iters";
  * value 0 restores the default.  Process-wide, not thread-safe.            */
 int oslo_tune(const char *key, int value);
 

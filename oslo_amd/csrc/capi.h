@@ -31,6 +31,8 @@ struct Tuning {
   int eltwise_fwd_steps;
   int norm_bwd_waves;
   int norm_fwd_waves;
+  int norm_bwd_prefetch;
+  int norm_fwd_iters;
 };
 extern Tuning g_tune;
 

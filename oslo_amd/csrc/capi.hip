@@ -86,6 +86,8 @@ int oslo_tune(const char *key, int value) {
       {"eltwise_fwd_steps", &oslo::g_tune.eltwise_fwd_steps},
       {"norm_bwd_waves", &oslo::g_tune.norm_bwd_waves},
       {"norm_fwd_waves", &oslo::g_tune.norm_fwd_waves},
+      {"norm_bwd_prefetch", &oslo::g_tune.norm_bwd_prefetch},
+      {"norm_fwd_iters", &oslo::g_tune.norm_fwd_iters},
   };
   for (const Entry &e : table) {
     if (strcmp(e.name, key) == 0) {

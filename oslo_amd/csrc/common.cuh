@@ -307,6 +307,18 @@ __device__ __forceinline__ float rsqrt_refined(float a) {
   return fmaf(y, 0.5f - h * y, y);
 }
 
+// Reduction of the values held by lanes 0..15 (one DPP row), returned to every
+// lane through lane 0.  Used to combine the per-wave results of the up to 16
+// waves that share a row: lane l < wpr reads wave l's value from LDS, the
+// other lanes pass the identity.
+template <typename Op> __device__ __forceinline__ float row16_allreduce(float v) {
+  v = Op::apply(v, dpp_mov<kDppQuadSwap1>(v));
+  v = Op::apply(v, dpp_mov<kDppQuadSwap2>(v));
+  v = Op::apply(v, dpp_mov<kDppRowHalfMirror>(v));
+  v = Op::apply(v, dpp_mov<kDppRowMirror>(v));
+  return readlane(v, 0);
+}
+
 // Reduction over the WPR consecutive waves that share one row.  `red` is LDS
 // scratch of at least (waves in block) floats, `slot` selects one of two such
 // areas so that back-to-back reductions need only one barrier each.

@@ -25,6 +25,10 @@ namespace oslo {
 // ---------------------------------------------------------------------------
 // helpers
 // ---------------------------------------------------------------------------
+// Sums over the wpr (<= 16) consecutive waves that share a row: lane 0 of every
+// wave publishes its wave's sum in LDS, then lane l < wpr of every wave reads
+// the sum of wave first + l and one DPP row reduction combines them, which
+// costs a fixed dozen instructions instead of a loop over wpr.
 // Two simultaneous row sums sharing one barrier.  red is [2][16] floats.
 __device__ __forceinline__ void row_sum2(float &a, float &b, float *red,
                                          int wave, int first, int wpr,
@@ -37,13 +41,11 @@ __device__ __forceinline__ void row_sum2(float &a, float &b, float *red,
       red[16 + wave] = b;
     }
     __syncthreads();
-    float ra = red[first], rb = red[16 + first];
-    for (int w = 1; w < wpr; ++w) {
-      ra += red[first + w];
-      rb += red[16 + first + w];
-    }
-    a = ra;
-    b = rb;
+    const bool own = lane < wpr;
+    const int src = own ? first + lane : first;
+    const float ra = red[src], rb = red[16 + src];
+    a = row16_allreduce<OpSum>(own ? ra : 0.f);
+    b = row16_allreduce<OpSum>(own ? rb : 0.f);
   }
 }
 
@@ -53,17 +55,19 @@ __device__ __forceinline__ float row_sum1(float a, float *red, int wave,
   if (wpr > 1) {
     if (lane == 0) red[wave] = a;
     __syncthreads();
-    float ra = red[first];
-    for (int w = 1; w < wpr; ++w) ra += red[first + w];
-    a = ra;
+    const bool own = lane < wpr;
+    const float ra = red[own ? first + lane : first];
+    a = row16_allreduce<OpSum>(own ? ra : 0.f);
   }
   return a;
 }
 
 // Welford partials of equal size (every lane holds w.n values) merged over
-// the wave and then over the wpr waves of a row.  red holds two areas of 48
-// floats; `parity` alternates between them from one call to the next so that
-// a single barrier per call suffices.
+// the wave and then over the wpr waves of a row.  The waves hold equal
+// counts c, so the row's mean is the average of the wave means and its M2 is
+// sum_w (M2_w + c (mean_w - mean)^2).  red holds two areas of 48 floats;
+// `parity` alternates between them from one call to the next so that a
+// single barrier per call suffices.
 __device__ __forceinline__ Welford row_welford(Welford w, float *red, int wave,
                                                int first, int wpr, int lane,
                                                int parity) {
@@ -75,12 +79,16 @@ __device__ __forceinline__ Welford row_welford(Welford w, float *red, int wave,
       area[16 + wave] = w.m2;
     }
     __syncthreads();
-    Welford t{w.n, area[first], area[16 + first]};
-    for (int k = 1; k < wpr; ++k) {
-      const Welford o{w.n, area[first + k], area[16 + first + k]};
-      t = chan_merge(t, o);
-    }
-    w = t;
+    const bool own = lane < wpr;
+    const int src = own ? first + lane : first;
+    const float mw = area[src], qw = area[16 + src];
+    const float mean =
+        row16_allreduce<OpSum>(own ? mw : 0.f) * __builtin_amdgcn_rcpf((float)wpr);
+    const float d = mw - mean;
+    const float m2 = row16_allreduce<OpSum>(own ? fmaf(w.n * d, d, qw) : 0.f);
+    w.mean = mean;
+    w.m2 = m2;
+    w.n *= (float)wpr;
   }
   return w;
 }
@@ -95,7 +103,7 @@ __global__ __launch_bounds__(MAXT) void norm_fwd_reg_kernel(
     const T *__restrict__ x, const V *__restrict__ gamma,
     const V *__restrict__ beta, V *__restrict__ y, float *__restrict__ mean,
     float *__restrict__ invvar, int64_t n1, int n2, float eps, int wpr,
-    int rpb) {
+    int rpb, int iters) {
   constexpr int E = chunk_elems<T, V>::value;
   __shared__ float red[2][48];
   const int lane = threadIdx.x & 63;
@@ -109,35 +117,55 @@ __global__ __launch_bounds__(MAXT) void norm_fwd_reg_kernel(
   const float fn = (float)n2;
   int parity = 0;
 
-  for (int64_t base = (int64_t)blockIdx.x * rpb; base < n1;
-       base += (int64_t)gridDim.x * rpb) {
-    const int64_t row = base + rslot;
-    const bool rvalid = row < n1;
-    // a slot past the last row re-reads row n1 - 1 and stores nothing
-    const T *xr = x + (rvalid ? row : n1 - 1) * n2;
-    float v[VPL][E];
+  // the affine parameters of this lane's columns stay packed in registers
+  // for all rows of the workgroup
+  RawChunk<V, E> graw[VPL], braw[VPL];
+  if (gamma != nullptr) {
 #pragma unroll
     for (int k = 0; k < VPL; ++k) {
       const int c = c0 + k * cstride;
-      if (EVEN || c < nchunks) {
-        load_chunk<T, E>(xr + (int64_t)c * E, v[k]);
-      } else {
-#pragma unroll
-        for (int e = 0; e < E; ++e) v[k][e] = 0.f;
+      if (c < nchunks) {
+        graw[k].load_cached(gamma + (int64_t)c * E);
+        if constexpr (!RMS) braw[k].load_cached(beta + (int64_t)c * E);
       }
     }
+  }
 
-    // the affine parameters of this lane's columns: requested now, used last
-    RawChunk<V, E> graw[VPL], braw[VPL];
-    if (gamma != nullptr) {
+  // A workgroup takes `iters` consecutive groups of rpb rows, then strides
+  // by the grid.
+  const int64_t total_groups = (n1 + rpb - 1) / rpb;
+  // The next row of a workgroup is requested, in packed form, before the
+  // current one is reduced, so that every wave keeps loads in flight.
+  // (not in the 1024-thread build with 32 elements per lane, whose register
+  // budget of 128 has no room for the second row)
+  constexpr bool kPrefetch = !(MAXT > 256 && VPL * E >= 32);
+  RawChunk<T, E> nx[VPL];
+  auto fetch = [&](int64_t group) {
+    int64_t frow = group * rpb + rslot;
+    // a slot past the last row re-reads row n1 - 1 and stores nothing
+    frow = frow < n1 ? frow : n1 - 1;
+    const T *xr = x + frow * n2;
 #pragma unroll
-      for (int k = 0; k < VPL; ++k) {
-        const int c = c0 + k * cstride;
-        if (c < nchunks) {
-          graw[k].load_cached(gamma + (int64_t)c * E);
-          if constexpr (!RMS) braw[k].load_cached(beta + (int64_t)c * E);
-        }
-      }
+    for (int k = 0; k < VPL; ++k) {
+      const int c = c0 + k * cstride;
+      if (EVEN || c < nchunks)
+        nx[k].load(xr + (int64_t)c * E);
+      else
+        nx[k].zero();
+    }
+  };
+  for (int64_t g0 = (int64_t)blockIdx.x * iters; g0 < total_groups;
+       g0 += (int64_t)gridDim.x * iters) {
+  if constexpr (kPrefetch) fetch(g0);
+  for (int it = 0; it < iters && g0 + it < total_groups; ++it) {
+    const int64_t row = (g0 + it) * rpb + rslot;
+    const bool rvalid = row < n1;
+    float v[VPL][E];
+    if constexpr (!kPrefetch) fetch(g0 + it);
+#pragma unroll
+    for (int k = 0; k < VPL; ++k) nx[k].unpack(v[k]);
+    if constexpr (kPrefetch) {
+      if (it + 1 < iters && g0 + it + 1 < total_groups) fetch(g0 + it + 1);
     }
 
     float mu = 0.f, q = 0.f;
@@ -232,6 +260,7 @@ __global__ __launch_bounds__(MAXT) void norm_fwd_reg_kernel(
       }
     }
   }
+  }
 }
 
 // ---------------------------------------------------------------------------
@@ -307,7 +336,7 @@ __global__ __launch_bounds__(256) void norm_fwd_generic_kernel(
 // backward, register-resident, single pass
 // ---------------------------------------------------------------------------
 // EVEN: every lane holds exactly VPL chunks of its row (no column guards).
-template <typename T, typename V, int VPL, bool RMS, bool EVEN>
+template <typename T, typename V, int VPL, bool RMS, bool EVEN, int PF>
 __global__ __launch_bounds__(1024) void norm_bwd_reg_kernel(
     const V *__restrict__ dy, const T *__restrict__ x,
     const float *__restrict__ mean, const float *__restrict__ invvar,
@@ -344,42 +373,45 @@ __global__ __launch_bounds__(1024) void norm_bwd_reg_kernel(
     }
   }
 
-  // The loads of a row are issued one iteration ahead, in packed form, so
-  // that they are in flight while the previous row is reduced and stored.
-  RawChunk<V, E> nd[VPL];
-  RawChunk<T, E> nx[VPL];
-  float nmu = 0.f, nrs = 0.f;
+  // The loads of a row are issued PF iterations ahead, in packed form, so
+  // that they are in flight while the previous rows are reduced and stored.
+  struct RowFetch {
+    RawChunk<V, E> d[VPL];
+    RawChunk<T, E> x[VPL];
+    float mu, rs;
+  };
   const int64_t rstride = (int64_t)gridDim.x * rpb;
   // A slot past the last row re-reads row n1 - 1 (its results are discarded),
   // which keeps the loads unconditional.
-#define OSLO_FETCH_ROW(BASE)                                       \
-  do {                                                             \
-    int64_t frow = (BASE) + rslot;                                 \
-    frow = frow < n1 ? frow : n1 - 1;                              \
-    _Pragma("unroll") for (int k = 0; k < VPL; ++k) {              \
-      const int c = c0 + k * cstride;                              \
-      if (EVEN || c < nchunks) {                                   \
-        nd[k].load(dy + frow * n2 + (int64_t)c * E);               \
-        nx[k].load(x + frow * n2 + (int64_t)c * E);                \
-      } else {                                                     \
-        nd[k].zero();                                              \
-        nx[k].zero();                                              \
-      }                                                            \
-    }                                                              \
-    if constexpr (!RMS) nmu = mean[frow];                          \
-    nrs = invvar[frow];                                            \
-  } while (0)
+  auto fetch = [&](RowFetch &f, int64_t base) {
+    int64_t frow = base + rslot;
+    frow = frow < n1 ? frow : n1 - 1;
+#pragma unroll
+    for (int k = 0; k < VPL; ++k) {
+      const int c = c0 + k * cstride;
+      if (EVEN || c < nchunks) {
+        f.d[k].load(dy + frow * n2 + (int64_t)c * E);
+        f.x[k].load(x + frow * n2 + (int64_t)c * E);
+      } else {
+        f.d[k].zero();
+        f.x[k].zero();
+      }
+    }
+    f.mu = RMS ? 0.f : mean[frow];
+    f.rs = invvar[frow];
+  };
 
-  OSLO_FETCH_ROW((int64_t)blockIdx.x * rpb);
   int parity = 0;
-  for (int64_t base = (int64_t)blockIdx.x * rpb; base < n1; base += rstride) {
+  // One row per slot: consume the fetched row, refill the buffer with the row
+  // PF iterations later, reduce, store dx.
+  auto process = [&](RowFetch &f, int64_t base) {
     const int64_t row = base + rslot;
     const bool rvalid = row < n1;
     float d[VPL][E], xh[VPL][E];
 #pragma unroll
     for (int k = 0; k < VPL; ++k) {
-      nd[k].unpack(d[k]);
-      nx[k].unpack(xh[k]);
+      f.d[k].unpack(d[k]);
+      f.x[k].unpack(xh[k]);
     }
     if (!rvalid) {  // wave-uniform: a slot past the end contributes nothing
 #pragma unroll
@@ -387,8 +419,8 @@ __global__ __launch_bounds__(1024) void norm_bwd_reg_kernel(
 #pragma unroll
         for (int e = 0; e < E; ++e) d[k][e] = 0.f;
     }
-    const float mu = nmu, rs = nrs;
-    OSLO_FETCH_ROW(base + rstride);
+    const float mu = f.mu, rs = f.rs;
+    fetch(f, base + PF * rstride);
     float s1 = 0.f, s2 = 0.f;
 #pragma unroll
     for (int k = 0; k < VPL; ++k) {
@@ -431,6 +463,22 @@ __global__ __launch_bounds__(1024) void norm_bwd_reg_kernel(
           store_chunk<T, E>(dxr + (int64_t)c * E, o);
         }
       }
+    }
+  };
+
+  const int64_t base0 = (int64_t)blockIdx.x * rpb;
+  if constexpr (PF == 1) {
+    RowFetch f0;
+    fetch(f0, base0);
+    for (int64_t base = base0; base < n1; base += rstride) process(f0, base);
+  } else {
+    RowFetch f0, f1;
+    fetch(f0, base0);
+    fetch(f1, base0 + rstride);
+    for (int64_t base = base0; base < n1; base += 2 * rstride) {
+      process(f0, base);
+      if (base + rstride >= n1) break;  // uniform over the workgroup
+      process(f1, base + rstride);
     }
   }
 
@@ -608,8 +656,11 @@ static int launch_norm_fwd(const void *x, const void *gamma, const void *beta,
   static const int kVpl[] = {1, 2, 4, 8};
   RowSplit sp{0, 1, 1, false};
   if (vec_ok) {
-    // up to four chunks per lane measured fastest on MI355X
-    const int cap = g_tune.norm_fwd_vpl > 0 ? g_tune.norm_fwd_vpl : 4;
+    // measured fastest on MI355X: up to four chunks per lane; LayerNorm,
+    // whose kernel holds more live registers, takes two while the row then
+    // still fits four waves
+    int cap = (!RMS && n2 / E <= kWave * 2 * 4) ? 2 : 4;
+    if (g_tune.norm_fwd_vpl > 0) cap = g_tune.norm_fwd_vpl;
     const int waves = g_tune.norm_fwd_waves > 0 ? g_tune.norm_fwd_waves : 4;
     sp = split_row(n2 / E, cap > 8 ? 8 : cap, kVpl, 4, waves);
     // more than 32 resident elements per lane only fit the register budget
@@ -627,7 +678,12 @@ static int launch_norm_fwd(const void *x, const void *gamma, const void *beta,
   const int threads = kWave * sp.wpr * sp.rpb;
   // every lane holds exactly vpl chunks: LayerNorm takes the Welford path
   const bool even = (n2 / E) == (int64_t)sp.vpl * kWave * sp.wpr;
-  int64_t grid = ceil_div(n1, sp.rpb);
+  // rows per workgroup = rpb * iters: the workgroup's loads of gamma and beta
+  // are spread over that many rows
+  // (LayerNorm: two groups, the second one prefetched; RMSNorm is fastest
+  // with short-lived workgroups)
+  int iters = g_tune.norm_fwd_iters > 0 ? g_tune.norm_fwd_iters : (RMS ? 1 : 2);
+  int64_t grid = ceil_div(ceil_div(n1, sp.rpb), iters);
   const int64_t maxgrid = (int64_t)device_cu_count() * 64;
   if (grid > maxgrid) grid = maxgrid;
 #define OSLO_FWD_CASE(VPL)                                                  \
@@ -636,23 +692,23 @@ static int launch_norm_fwd(const void *x, const void *gamma, const void *beta,
       norm_fwd_reg_kernel<T, V, VPL, RMS, true, 256>                        \
           <<<dim3((unsigned)grid), threads, 0, st>>>(                       \
               (const T *)x, (const V *)gamma, (const V *)beta, (V *)y,      \
-              mean, invvar, n1, (int)n2, eps, sp.wpr, sp.rpb);              \
+              mean, invvar, n1, (int)n2, eps, sp.wpr, sp.rpb, iters);             \
     else if (threads <= 256)                                                \
       norm_fwd_reg_kernel<T, V, VPL, RMS, false, 256>                       \
           <<<dim3((unsigned)grid), threads, 0, st>>>(                       \
               (const T *)x, (const V *)gamma, (const V *)beta, (V *)y,      \
-              mean, invvar, n1, (int)n2, eps, sp.wpr, sp.rpb);              \
+              mean, invvar, n1, (int)n2, eps, sp.wpr, sp.rpb, iters);             \
     else if constexpr (VPL * E <= 32) {                                     \
       if (even)                                                             \
         norm_fwd_reg_kernel<T, V, VPL, RMS, true, 1024>                     \
             <<<dim3((unsigned)grid), threads, 0, st>>>(                     \
                 (const T *)x, (const V *)gamma, (const V *)beta, (V *)y,    \
-                mean, invvar, n1, (int)n2, eps, sp.wpr, sp.rpb);            \
+                mean, invvar, n1, (int)n2, eps, sp.wpr, sp.rpb, iters);           \
       else                                                                  \
         norm_fwd_reg_kernel<T, V, VPL, RMS, false, 1024>                    \
             <<<dim3((unsigned)grid), threads, 0, st>>>(                     \
                 (const T *)x, (const V *)gamma, (const V *)beta, (V *)y,    \
-                mean, invvar, n1, (int)n2, eps, sp.wpr, sp.rpb);            \
+                mean, invvar, n1, (int)n2, eps, sp.wpr, sp.rpb, iters);           \
     }                                                                       \
     else                                                                    \
       return fail(OSLO_ERR_UNSUPPORTED,                                     \
@@ -697,10 +753,10 @@ static int launch_norm_bwd(const void *dy, const void *x, const float *mean,
       if (cap > 16 / E) cap = 16 / E;
       sp = split_row(n2 / E, cap, allowed, nallowed, waves);
     } else {
-      // measured best on MI355X: 8 elements per lane as long as a workgroup
-      // still holds two rows, else 16 elements per lane
+      // measured best on MI355X: 8 elements per lane wherever a row then
+      // fits one workgroup, else 16 elements per lane
       sp = split_row(n2 / E, 8 / E, allowed, nallowed, waves);
-      if (!sp.ok || sp.rpb < 2) {
+      if (!sp.ok) {
         const RowSplit wide = split_row(n2 / E, 16 / E, allowed, nallowed, waves);
         if (wide.ok) sp = wide;
       }
@@ -733,20 +789,27 @@ static int launch_norm_bwd(const void *dy, const void *x, const float *mean,
   const int threads = kWave * sp.wpr * sp.rpb;
   const size_t lds = sp.rpb > 1 ? (size_t)n2 * sizeof(float) : 0;
   const bool even = (n2 / E) == (int64_t)sp.vpl * kWave * sp.wpr;
-#define OSLO_BWD_CASE(VPL)                                                  \
-  case VPL:                                                                  \
-    if constexpr (VPL * E <= 16) {                                           \
-      if (even)                                                              \
-        norm_bwd_reg_kernel<T, V, VPL, RMS, true>                            \
-            <<<dim3((unsigned)P), threads, lds, st>>>(                       \
-                (const V *)dy, (const T *)x, mean, invvar, (const V *)gamma, \
-                (T *)dx, part, n1, (int)n2, sp.wpr, sp.rpb);                 \
-      else                                                                   \
-        norm_bwd_reg_kernel<T, V, VPL, RMS, false>                           \
-            <<<dim3((unsigned)P), threads, lds, st>>>(                       \
-                (const V *)dy, (const T *)x, mean, invvar, (const V *)gamma, \
-                (T *)dx, part, n1, (int)n2, sp.wpr, sp.rpb);                 \
-    }                                                                        \
+  // rows in flight ahead of the one being reduced: two while the packed row
+  // buffers are small (8 elements per lane), else one
+  int pf = sp.vpl * E <= 8 ? 2 : 1;
+  if (g_tune.norm_bwd_prefetch > 0) pf = g_tune.norm_bwd_prefetch >= 2 ? 2 : 1;
+#define OSLO_BWD_LAUNCH(VPL, EVEN_, PF_)                                   \
+  norm_bwd_reg_kernel<T, V, VPL, RMS, EVEN_, PF_>                          \
+      <<<dim3((unsigned)P), threads, lds, st>>>(                           \
+          (const V *)dy, (const T *)x, mean, invvar, (const V *)gamma,     \
+          (T *)dx, part, n1, (int)n2, sp.wpr, sp.rpb)
+#define OSLO_BWD_CASE(VPL)                                                 \
+  case VPL:                                                                \
+    if constexpr (VPL * E <= 16) {                                         \
+      if (even && pf == 2)                                                 \
+        OSLO_BWD_LAUNCH(VPL, true, 2);                                     \
+      else if (even)                                                       \
+        OSLO_BWD_LAUNCH(VPL, true, 1);                                     \
+      else if (pf == 2)                                                    \
+        OSLO_BWD_LAUNCH(VPL, false, 2);                                    \
+      else                                                                 \
+        OSLO_BWD_LAUNCH(VPL, false, 1);                                    \
+    }                                                                      \
     break;
   switch (sp.vpl) {
     OSLO_BWD_CASE(1)
@@ -755,6 +818,7 @@ static int launch_norm_bwd(const void *dy, const void *x, const float *mean,
     default:
       return fail(OSLO_ERR_UNSUPPORTED, "norm bwd: no kernel for vpl=%d", sp.vpl);
   }
+#undef OSLO_BWD_LAUNCH
 #undef OSLO_BWD_CASE
   int rc = check_launch("norm_bwd_reg_kernel");
   if (rc != OSLO_OK || !want_params) return rc;

@@ -33,15 +33,18 @@ struct SoftmaxGeom {
   int wpr, rpb;     // waves per row, rows per workgroup pass (without RPW)
 };
 
+// Reductions over the wpr (<= 16) consecutive waves of a row: lane 0 of each
+// wave publishes its wave's value in LDS, lane l < wpr then reads the value of
+// wave first + l and one DPP row reduction combines them.
 __device__ __forceinline__ float row_reduce_sum(float a, float *red, int wave,
                                                 int first, int wpr, int lane) {
   a = wave_sum(a);
   if (wpr > 1) {
     if (lane == 0) red[wave] = a;
     __syncthreads();
-    float r = red[first];
-    for (int w = 1; w < wpr; ++w) r += red[first + w];
-    a = r;
+    const bool own = lane < wpr;
+    const float r = red[own ? first + lane : first];
+    a = row16_allreduce<OpSum>(own ? r : 0.f);
   }
   return a;
 }
@@ -51,9 +54,8 @@ __device__ __forceinline__ float row_reduce_max(float a, float *red, int wave,
   if (wpr > 1) {
     if (lane == 0) red[wave] = a;
     __syncthreads();
-    float r = red[first];
-    for (int w = 1; w < wpr; ++w) r = fmaxf(r, red[first + w]);
-    a = r;
+    // lanes >= wpr repeat the first wave's value, which leaves the maximum unchanged
+    a = row16_allreduce<OpMax>(red[lane < wpr ? first + lane : first]);
   }
   return a;
 }
