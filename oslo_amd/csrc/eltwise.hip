@@ -144,17 +144,29 @@ __global__ __launch_bounds__(256) void bias_gelu_bwd_kernel(
   if (ps.cc < g.nchunks) {
     if constexpr (HAS_BIAS) load_chunk<T, kE, false>(bias + (int64_t)ps.cc * kE, b);
     const int64_t coff = (int64_t)ps.cc * kE;
-    for (int64_t r0 = ps.slot * g.ty * U + ps.ry; r0 < g.rows;
-       r0 += g.slots * g.ty * U) {
+    // The loads of the next step are requested, in packed form, before the
+    // current step is evaluated; a row past the end re-reads the last row.
+    RawChunk<T, kE> nx[U], ng[U];
+    auto fetch = [&](int64_t r0) {
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        int64_t r = r0 + u * g.ty;
+        r = r < g.rows ? r : g.rows - 1;
+        nx[u].load(x + r * g.cols + coff);
+        ng[u].load(gr + r * g.cols + coff);
+      }
+    };
+    const int64_t step = g.slots * g.ty * U;
+    int64_t r0 = ps.slot * g.ty * U + ps.ry;
+    if (r0 < g.rows) fetch(r0);
+    for (; r0 < g.rows; r0 += step) {
       float v[U][kE], gv[U][kE];
 #pragma unroll
       for (int u = 0; u < U; ++u) {
-        const int64_t r = r0 + u * g.ty;
-        if (r < g.rows) {
-          load_chunk<T, kE>(x + r * g.cols + coff, v[u]);
-          load_chunk<T, kE>(gr + r * g.cols + coff, gv[u]);
-        }
+        nx[u].unpack(v[u]);
+        ng[u].unpack(gv[u]);
       }
+      if (r0 + step < g.rows) fetch(r0 + step);
 #pragma unroll
       for (int u = 0; u < U; ++u) {
         const int64_t r = r0 + u * g.ty;
@@ -245,14 +257,24 @@ __global__ __launch_bounds__(256) void bias_dropout_add_bwd_kernel(
   for (int e = 0; e < kE; ++e) acc[e] = 0.f;
   if (ps.cc < g.nchunks) {
     const int64_t coff = (int64_t)ps.cc * kE;
-    for (int64_t r0 = ps.slot * g.ty * U + ps.ry; r0 < g.rows;
-       r0 += g.slots * g.ty * U) {
-      float gv[U][kE];
+    // next step requested before the current one is evaluated, as above
+    RawChunk<T, kE> ng[U];
+    auto fetch = [&](int64_t r0) {
 #pragma unroll
       for (int u = 0; u < U; ++u) {
-        const int64_t r = r0 + u * g.ty;
-        if (r < g.rows) load_chunk<T, kE>(gr + r * g.cols + coff, gv[u]);
+        int64_t r = r0 + u * g.ty;
+        r = r < g.rows ? r : g.rows - 1;
+        ng[u].load(gr + r * g.cols + coff);
       }
+    };
+    const int64_t step = g.slots * g.ty * U;
+    int64_t r0 = ps.slot * g.ty * U + ps.ry;
+    if (r0 < g.rows) fetch(r0);
+    for (; r0 < g.rows; r0 += step) {
+      float gv[U][kE];
+#pragma unroll
+      for (int u = 0; u < U; ++u) ng[u].unpack(gv[u]);
+      if (r0 + step < g.rows) fetch(r0 + step);
 #pragma unroll
       for (int u = 0; u < U; ++u) {
         const int64_t r = r0 + u * g.ty;
@@ -444,16 +466,17 @@ static inline void eltwise_tile(int64_t cols, int *tx, int *ty, int *tiles) {
   *tiles = (int)ceil_div(nchunks, t);
 }
 
-// Backward: workgroups per column tile = fp32 partial rows.  Enough workgroups
-// for about three per CU (measured best on MI355X: the workgroups advance
-// through the rows in step and each lane keeps several loads in flight), so
-// the partial rows stay around one percent of the tensor traffic.
+// Backward: workgroups per column tile = fp32 partial rows.  Two workgroups
+// per CU measured best on MI355X (three or more lose 5-10 %): the workgroups
+// advance through the rows in step, every lane keeps four chunks per operand
+// in flight plus the prefetch of the next step, and the partial rows stay
+// below one percent of the tensor traffic.
 int64_t colsum_parts_eltwise(int64_t rows, int64_t cols) {
   int tx, ty, tiles;
   eltwise_tile(cols, &tx, &ty, &tiles);
   int64_t parts = g_tune.eltwise_rowgroups > 0
                       ? g_tune.eltwise_rowgroups
-                      : ceil_div((int64_t)device_cu_count() * 3, tiles);
+                      : ((int64_t)device_cu_count() * 2) / tiles;  // never more than two per CU
   const int64_t min_band =
       g_tune.eltwise_rowgroups > 0 ? ty : (16 > ty ? 16 : ty);
   const int64_t maxp = ceil_div(rows, min_band);
@@ -554,7 +577,7 @@ static int run_bias_gelu_bwd(const void *gr, const void *x, const void *bias,
         (const T *)dx, (T *)dbias, rows, cols);
     return check_launch("colsum_generic_kernel");
   }
-  const int unroll = eltwise_unroll(2) > 2 ? 2 : eltwise_unroll(2);
+  const int unroll = eltwise_unroll(4);
   const EltGeom g = eltwise_geom_bwd(rows, cols, unroll);
   const int64_t parts = g.slots;
   const int64_t nblocks = parts * g.tiles;
