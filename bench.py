@@ -35,7 +35,7 @@ METRIC = "achieved HBM GB/s (% of MI355X peak) per fused fwd+bwd kernel; speedup
 # rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE and calibrated against a 1 GiB copy:
 # main kernel 270.6 MB read + 140.4 MB written, finalize 8.4 MB read
 # (summary: profiles/bench_all_kernels_hbm_traffic.txt).  Algorithmic: 402.7 MB.
-LN_BWD_TRAFFIC_BYTES = 419.4e6
+LN_BWD_TRAFFIC_BYTES = 421.9e6
 
 F32, F16, BF16 = 0, 1, 2
 
@@ -205,7 +205,25 @@ def kernel_table(L, dev, iters):
 
         rows.append(table_row("softmax_causal_fwd", cfg, [ab, s, s], str(tdt).split(".")[-1], (1 + f) * T, timed(fwd, ns)))
         rows.append(table_row("softmax_causal_bwd", cfg, [ab, s, s], str(tdt).split(".")[-1], (1 + 2 * f) * T, timed(bwd, ns)))
-        del bufs
+
+        # softmax with the attention dropout (p = 0.1) fused in: the same
+        # compulsory bytes (backward reads the logits instead of the
+        # probabilities; the row statistics are 8 bytes a row)
+        stats = torch.empty(ab * s, 2, device=dev, dtype=torch.float32)
+
+        def dfwd(i):
+            x, y, dy, dx = bufs[i]
+            L.ok(lib.oslo_softmax_causal_dropout_fwd(p(x), p(y), p(stats), ab, s, s, scale, 0.1, 1234, 0, code, L.stream()))
+
+        def dbwd(i):
+            x, y, dy, dx = bufs[i]
+            L.ok(lib.oslo_softmax_causal_dropout_bwd(p(dy), p(x), p(stats), p(dx), ab, s, s, scale, 0.1, 1234, 0, code, L.stream()))
+
+        for name, fn, nbytes in (("softmax_causal_dropout_fwd", dfwd, (1 + f) * T), ("softmax_causal_dropout_bwd", dbwd, (1 + 2 * f) * T)):
+            row = table_row(name, cfg, [ab, s, s], str(tdt).split(".")[-1], nbytes, timed(fn, ns))
+            row["p"] = 0.1
+            rows.append(row)
+        del bufs, stats
         torch.cuda.empty_cache()
 
     # ---- padding-masked softmax: cfg3 ----

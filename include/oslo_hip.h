@@ -153,6 +153,47 @@ int oslo_softmax_masked_bwd(const void *dy, const void *y, const uint8_t *mask,
 int oslo_softmax_batch_per_block(int64_t sq, int64_t sk, int64_t b,
                                  int64_t np);
 
+/* ---- softmax with the attention-probability dropout fused in ------------ *
+ * Replaces the pair softmax -> attn_dropout that follows the scores in
+ * oslo/transformers/models/gpt2/modeling_gpt2.py:138-142 (causal) and
+ * oslo/transformers/models/bert/modeling_bert.py:306-310 (padding mask):
+ *   out = keep * softmax(mask(scale * x)) / (1 - p).
+ * The keep decisions are the Philox stream of oslo_philox_mask over the
+ * flattened output (element i = row * sk + key: group i >> 3, bit i & 7), so
+ * nothing but the row statistics is stored for the backward pass:
+ * stats is float [rows][2] = {max_j of scale * log2(e) * x_j over the visible
+ * keys, 1 / sum_j exp2(scale * log2(e) * x_j - max)}, or {0, -1/sk} for a row
+ * without a visible key.  The backward pass takes the saved *input* x (not
+ * the output), recomputes the probabilities y from x and stats, regenerates
+ * the keep bits from the same (p, seed, offset) and returns
+ *   dx = scale * y * (dp - sum_k dp_k y_k),  dp = keep * dout / (1 - p).
+ * With p == 0 the forward output equals oslo_softmax_*_fwd bit for bit.
+ * dx may alias dout or x.  Shapes and mask rules as for the entry points
+ * above; advance the generator offset by 4 per call.                        */
+int oslo_softmax_causal_dropout_fwd(const void *x, void *out, float *stats,
+                                    int64_t attn_batches, int64_t sq,
+                                    int64_t sk, float scale, float p,
+                                    uint64_t seed, uint64_t offset, int dtype,
+                                    void *stream);
+int oslo_softmax_causal_dropout_bwd(const void *dout, const void *x,
+                                    const float *stats, void *dx,
+                                    int64_t attn_batches, int64_t sq,
+                                    int64_t sk, float scale, float p,
+                                    uint64_t seed, uint64_t offset, int dtype,
+                                    void *stream);
+int oslo_softmax_masked_dropout_fwd(const void *x, const uint8_t *mask,
+                                    void *out, float *stats, int64_t b,
+                                    int64_t np, int64_t sq, int64_t sk,
+                                    int64_t mask_b, int64_t mask_sq,
+                                    float scale, float p, uint64_t seed,
+                                    uint64_t offset, int dtype, void *stream);
+int oslo_softmax_masked_dropout_bwd(const void *dout, const void *x,
+                                    const uint8_t *mask, const float *stats,
+                                    void *dx, int64_t b, int64_t np, int64_t sq,
+                                    int64_t sk, int64_t mask_b, int64_t mask_sq,
+                                    float scale, float p, uint64_t seed,
+                                    uint64_t offset, int dtype, void *stream);
+
 /* ---- bias-GeLU (tanh approximation) ------------------------------------ *
  * x, y, g, dx are [rows, cols]; bias, dbias are [cols]; one dtype for all. */
 

@@ -110,6 +110,37 @@ def softmax_bwd(dy, y, scale, out="f64", acc=np.float64):
     return round_to(acc(scale) * (y * (dy - s)), out)
 
 
+def _dropout_scale(p, acc):
+    return acc(np.float32(1.0) / (np.float32(1.0) - np.float32(p))) if p < 1.0 else acc(0.0)
+
+
+def softmax_dropout_fwd(x, hidden, scale, keep, p, out="f64", acc=np.float64):
+    """out = keep * softmax(mask(scale * x)) / (1 - p), rounded once.
+
+    The softmax of modeling_gpt2.py:138 / modeling_bert.py:306 followed by
+    attn_dropout (modeling_gpt2.py:142, modeling_bert.py:310), i.e.
+    torch.nn.functional.dropout of the probabilities.  `keep` is the 0/1 mask
+    over the output (None = keep everything).
+    """
+    y = softmax_masked_fwd(x, hidden, scale, "f64", acc)
+    if keep is not None:
+        y = np.where(np.asarray(keep, dtype=bool), y * _dropout_scale(p, acc), 0.0)
+    return round_to(y, out)
+
+
+def softmax_dropout_bwd(dout, x, hidden, scale, keep, p, out="f64", acc=np.float64):
+    """dx of out = dropout(softmax(mask(scale * x))) given d(out):
+    dp = keep * dout / (1 - p) is the gradient of the probabilities y, then the
+    softmax backward dx = scale * y * (dp - sum_k dp_k y_k), with y recomputed
+    from x in `acc` precision (the fused backward keeps x, not y)."""
+    y = softmax_masked_fwd(x, hidden, scale, "f64", acc)
+    dp = np.asarray(dout, dtype=acc)
+    if keep is not None:
+        dp = np.where(np.asarray(keep, dtype=bool), dp * _dropout_scale(p, acc), 0.0)
+    s = (dp * y).sum(axis=-1, keepdims=True)
+    return round_to(acc(scale) * (y * (dp - s)), out)
+
+
 # ---------------------------------------------------------------------------
 # LayerNorm / RMSNorm
 # ---------------------------------------------------------------------------

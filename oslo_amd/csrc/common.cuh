@@ -391,4 +391,28 @@ dropout_keep_bits(uint64_t group, uint64_t seed, uint64_t offset,
   return bits;
 }
 
+// Dropout parameters of one call.  Element i of the flattened tensor belongs
+// to group i >> 3 and is kept when bit i & 7 of that group's keep bits is set.
+struct DropArgs {
+  uint64_t seed, offset;
+  uint32_t threshold;  // keep when the 16-bit draw >= threshold
+  float scale;         // 1 / (1 - p), 0 when p >= 1
+};
+
+__device__ __host__ __forceinline__ bool keep_element(int64_t i, const DropArgs &d) {
+  const uint32_t bits =
+      dropout_keep_bits((uint64_t)i >> 3, d.seed, d.offset, d.threshold);
+  return (bits >> (i & 7)) & 1u;
+}
+
+static inline DropArgs make_drop(float p, uint64_t seed, uint64_t offset) {
+  DropArgs d;
+  d.seed = seed;
+  d.offset = offset;
+  double t = (double)p * 65536.0 + 0.5;
+  d.threshold = t >= 65536.0 ? 65536u : (uint32_t)t;
+  d.scale = p < 1.0f ? 1.0f / (1.0f - p) : 0.f;
+  return d;
+}
+
 }  // namespace oslo

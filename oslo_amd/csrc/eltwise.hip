@@ -188,11 +188,6 @@ __global__ __launch_bounds__(256) void bias_gelu_bwd_kernel(
 // ---------------------------------------------------------------------------
 // bias-dropout-add
 // ---------------------------------------------------------------------------
-struct DropArgs {
-  uint64_t seed, offset;
-  uint32_t threshold;  // keep when the 16-bit draw >= threshold
-  float scale;         // 1 / (1 - p), 0 when p >= 1
-};
 
 template <typename T, int U, bool HAS_BIAS, bool HAS_RES, bool DROP>
 __global__ __launch_bounds__(256) void bias_dropout_add_fwd_kernel(
@@ -303,11 +298,6 @@ __global__ __launch_bounds__(256) void bias_dropout_add_bwd_kernel(
 // generic (cols not a multiple of 8, or unaligned pointers): one thread per
 // element, grid-stride; the mask is the same function of the element index.
 // ---------------------------------------------------------------------------
-__device__ __forceinline__ bool keep_element(int64_t i, const DropArgs &d) {
-  const uint32_t bits =
-      dropout_keep_bits((uint64_t)i >> 3, d.seed, d.offset, d.threshold);
-  return (bits >> (i & 7)) & 1u;
-}
 
 template <typename T>
 __global__ __launch_bounds__(256) void bias_gelu_fwd_generic_kernel(
@@ -514,15 +504,6 @@ static inline int64_t flat_grid(int64_t n) {
   return grid < cap ? (grid < 1 ? 1 : grid) : cap;
 }
 
-static DropArgs make_drop(float p, uint64_t seed, uint64_t offset) {
-  DropArgs d;
-  d.seed = seed;
-  d.offset = offset;
-  double t = (double)p * 65536.0 + 0.5;
-  d.threshold = t >= 65536.0 ? 65536u : (uint32_t)t;
-  d.scale = p < 1.0f ? 1.0f / (1.0f - p) : 0.f;
-  return d;
-}
 
 #define OSLO_ELT_U(U_, ...)  \
   do {                       \

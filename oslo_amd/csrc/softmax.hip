@@ -108,10 +108,29 @@ __device__ __forceinline__ void row_setup(const SoftmaxGeom &g, int64_t r,
   }
 }
 
-template <typename T, int VPL, int RPW, int MODE>
+// Keep bits of the E elements of chunk c of `row` (dropout on the flattened
+// [rows, sk] tensor: element i belongs to group i >> 3).  A 4-element chunk
+// takes the low or the high half of its group's eight bits.
+template <int E>
+__device__ __forceinline__ uint32_t chunk_keep_bits(int64_t row, int sk, int c,
+                                                    const DropArgs &d) {
+  const uint64_t flat = (uint64_t)row * (uint64_t)sk + (uint64_t)c * E;
+  uint32_t keep = dropout_keep_bits(flat >> 3, d.seed, d.offset, d.threshold);
+  if constexpr (E == 4) keep >>= (uint32_t)(flat & 4u);
+  return keep;
+}
+
+// DROP: dropout is applied to the probabilities before they are written
+// (oslo/transformers/models/gpt2/modeling_gpt2.py:138-142,
+// oslo/transformers/models/bert/modeling_bert.py:306-310) and the row
+// statistics {max of the log2-domain logits, 1 / sum} go to stats[row], from
+// which the backward pass recomputes the probabilities.  A row without a
+// visible key stores {0, -1 / sk}.
+template <typename T, int VPL, int RPW, int MODE, bool DROP>
 __global__ __launch_bounds__(1024) void softmax_fwd_kernel(
     const T *__restrict__ x, const uint8_t *__restrict__ mask,
-    T *__restrict__ y, SoftmaxGeom g, float scale) {
+    T *__restrict__ y, float *__restrict__ stats, SoftmaxGeom g, float scale,
+    DropArgs d) {
   constexpr int E = io<T>::EPV;
   constexpr uint32_t kAll = (1u << E) - 1u;
   __shared__ float red[2][16];
@@ -246,6 +265,12 @@ __global__ __launch_bounds__(1024) void softmax_fwd_kernel(
     const float inv = empty ? 0.f : 1.0f / sm[j];
     const float fill = empty ? 1.0f / (float)g.sk : 0.f;
     T *yr = y + row[j] * g.sk;
+    if constexpr (DROP) {
+      if (c0 == 0) {
+        stats[2 * row[j]] = empty ? 0.f : mx[j];
+        stats[2 * row[j] + 1] = empty ? -fill : inv;
+      }
+    }
 #pragma unroll
     for (int k = 0; k < VPL; ++k) {
       const int c = c0 + k * cstride;
@@ -258,7 +283,153 @@ __global__ __launch_bounds__(1024) void softmax_fwd_kernel(
 #pragma unroll
           for (int e = 0; e < E; ++e) o[e] = v[j][k][e] * inv + fill;
         }
+        if constexpr (DROP) {
+          // exact zeros need no draw (wave-uniform test)
+          if (!none_visible[j][k] || empty) {
+            const uint32_t keep = chunk_keep_bits<E>(row[j], g.sk, c, d);
+#pragma unroll
+            for (int e = 0; e < E; ++e)
+              o[e] = (keep >> e) & 1u ? o[e] * d.scale : 0.f;
+          }
+        }
         store_chunk<T, E>(yr + (int64_t)c * E, o);
+      }
+    }
+  }
+}
+
+// Backward of softmax + dropout from the saved logits: the probabilities are
+// recomputed as exp2(x * scale * log2 e - stats[row][0]) * stats[row][1], the
+// keep bits are regenerated from (seed, offset), and
+// dx = scale * y * (dp - sum_k dp_k y_k) with dp = keep * dy / (1 - p).
+template <typename T, int VPL, int RPW, int MODE>
+__global__ __launch_bounds__(1024) void softmax_dropout_bwd_kernel(
+    const T *__restrict__ dy, const T *__restrict__ x,
+    const float *__restrict__ stats, const uint8_t *__restrict__ mask,
+    T *__restrict__ dx, SoftmaxGeom g, float scale, DropArgs d) {
+  constexpr int E = io<T>::EPV;
+  constexpr uint32_t kAll = (1u << E) - 1u;
+  __shared__ float red[16];
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int rslot = wave / g.wpr;
+  const int first = rslot * g.wpr;
+  const int nchunks = g.sk / E;
+  const int cstride = kWave * g.wpr;
+  const int c0 = (wave - first) * kWave + lane;
+  const int64_t rbase = ((int64_t)blockIdx.x * g.rpb + rslot) * RPW;
+  const float c2 = scale * kLog2e;
+
+  float yv[RPW][VPL][E], gv[RPW][VPL][E];
+  uint32_t mbits[RPW][VPL];  // bit e set: key masked out
+  int64_t row[RPW];
+  bool rvalid[RPW];
+  float rmax[RPW], rinv[RPW];
+
+#pragma unroll
+  for (int j = 0; j < RPW; ++j) {
+    const int64_t r = rbase + j;
+    rvalid[j] = r < g.rows;
+    int visible = 0;
+    const uint8_t *mrow = nullptr;
+    row[j] = 0;
+    rmax[j] = 0.f;
+    rinv[j] = 0.f;
+    if (rvalid[j]) {
+      row_setup<MODE>(g, r, mask, row[j], visible, mrow);
+      rmax[j] = stats[2 * row[j]];
+      rinv[j] = stats[2 * row[j] + 1];
+    }
+    const bool empty = rinv[j] < 0.f;  // uniform row: every key counts
+#pragma unroll
+    for (int k = 0; k < VPL; ++k) {
+      const int c = c0 + k * cstride;
+      uint32_t mb = kAll;
+      if (rvalid[j] && c < nchunks) {
+        if (empty) {
+          mb = 0u;
+        } else if constexpr (MODE == kModeCausal) {
+          const int left = visible - c * E;
+          mb = left >= E ? 0u : (left <= 0 ? mb : (mb & ~((1u << left) - 1u)));
+        } else {
+          mb = load_mask_bits<E>(mrow + (int64_t)c * E);
+        }
+      }
+      mbits[j][k] = mb;
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < RPW; ++j) {
+    const T *xr = x + row[j] * g.sk;
+    const T *gr = dy + row[j] * g.sk;
+#pragma unroll
+    for (int k = 0; k < VPL; ++k) {
+      const int c = c0 + k * cstride;
+      if (mbits[j][k] != kAll) {
+        load_chunk<T, E>(xr + (int64_t)c * E, yv[j][k]);
+        load_chunk<T, E>(gr + (int64_t)c * E, gv[j][k]);
+      } else {
+#pragma unroll
+        for (int e = 0; e < E; ++e) {
+          yv[j][k][e] = 0.f;
+          gv[j][k][e] = 0.f;
+        }
+      }
+    }
+  }
+  bool none_loaded[RPW][VPL];
+#pragma unroll
+  for (int j = 0; j < RPW; ++j)
+#pragma unroll
+    for (int k = 0; k < VPL; ++k)
+      none_loaded[j][k] = __builtin_amdgcn_ballot_w64(mbits[j][k] != kAll) == 0;
+
+  float s[RPW];
+#pragma unroll
+  for (int j = 0; j < RPW; ++j) {
+    float a = 0.f;
+    const bool empty = rinv[j] < 0.f;
+#pragma unroll
+    for (int k = 0; k < VPL; ++k) {
+      if (none_loaded[j][k]) continue;
+      const int c = c0 + k * cstride;
+      const uint32_t keep =
+          mbits[j][k] != kAll ? chunk_keep_bits<E>(row[j], g.sk, c, d) : 0u;
+#pragma unroll
+      for (int e = 0; e < E; ++e) {
+        float p = __builtin_amdgcn_exp2f(fmaf(yv[j][k][e], c2, -rmax[j])) * rinv[j];
+        if (empty) p = -rinv[j];
+        if ((mbits[j][k] >> e) & 1u) p = 0.f;
+        const float dp = (keep >> e) & 1u ? gv[j][k][e] * d.scale : 0.f;
+        yv[j][k][e] = p;
+        gv[j][k][e] = dp;
+        a += p * dp;
+      }
+    }
+    s[j] = a;
+  }
+#pragma unroll
+  for (int j = 0; j < RPW; ++j)
+    s[j] = row_reduce_sum(s[j], red, wave, first, g.wpr, lane);
+
+#pragma unroll
+  for (int j = 0; j < RPW; ++j) {
+    if (!rvalid[j]) continue;
+    T *dxr = dx + row[j] * g.sk;
+#pragma unroll
+    for (int k = 0; k < VPL; ++k) {
+      const int c = c0 + k * cstride;
+      if (c < nchunks) {
+        float o[E];
+        if (none_loaded[j][k]) {
+#pragma unroll
+          for (int e = 0; e < E; ++e) o[e] = 0.f;
+        } else {
+#pragma unroll
+          for (int e = 0; e < E; ++e)
+            o[e] = scale * (yv[j][k][e] * (gv[j][k][e] - s[j]));
+        }
+        store_chunk<T, E>(dxr + (int64_t)c * E, o);
       }
     }
   }
@@ -404,10 +575,11 @@ __device__ __forceinline__ float block_reduce_256(float v, float *sh, bool is_ma
                 : (sh[0] + sh[1]) + (sh[2] + sh[3]);
 }
 
-template <typename T, int MODE>
+template <typename T, int MODE, bool DROP>
 __global__ __launch_bounds__(256) void softmax_fwd_generic_kernel(
     const T *__restrict__ x, const uint8_t *__restrict__ mask,
-    T *__restrict__ y, SoftmaxGeom g, float scale) {
+    T *__restrict__ y, float *__restrict__ stats, SoftmaxGeom g, float scale,
+    DropArgs d) {
   __shared__ float sh[4];
   const float ninf = -__builtin_inff();
   for (int64_t r = blockIdx.x; r < g.rows; r += gridDim.x) {
@@ -440,8 +612,53 @@ __global__ __launch_bounds__(256) void softmax_fwd_generic_kernel(
       if (!hidden)
         p = __builtin_amdgcn_exp2f((io<T>::from_scalar(xr[i]) * scale - m) *
                                    kLog2e);
-      yr[i] = io<T>::to_scalar(p * inv + fill);
+      float o = p * inv + fill;
+      if constexpr (DROP)
+        o = keep_element(row * g.sk + i, d) ? o * d.scale : 0.f;
+      yr[i] = io<T>::to_scalar(o);
     }
+    if constexpr (DROP) {
+      if (threadIdx.x == 0) {
+        // statistics in the log2 domain, as the register kernel stores them
+        stats[2 * row] = empty ? 0.f : m * kLog2e;
+        stats[2 * row + 1] = empty ? -fill : inv;
+      }
+    }
+  }
+}
+
+template <typename T, int MODE>
+__global__ __launch_bounds__(256) void softmax_dropout_bwd_generic_kernel(
+    const T *__restrict__ dy, const T *__restrict__ x,
+    const float *__restrict__ stats, const uint8_t *__restrict__ mask,
+    T *__restrict__ dx, SoftmaxGeom g, float scale, DropArgs d) {
+  __shared__ float sh[4];
+  const float c2 = scale * kLog2e;
+  for (int64_t r = blockIdx.x; r < g.rows; r += gridDim.x) {
+    int64_t row;
+    int visible;
+    const uint8_t *mrow;
+    row_setup<MODE>(g, r, mask, row, visible, mrow);
+    const T *xr = x + row * g.sk;
+    const T *gr = dy + row * g.sk;
+    T *dxr = dx + row * g.sk;
+    const float m = stats[2 * row], inv = stats[2 * row + 1];
+    const bool empty = inv < 0.f;
+    auto prob = [&](int i) {
+      if (empty) return -inv;
+      const bool hidden = MODE == kModeCausal ? i >= visible : mrow[i] != 0;
+      if (hidden) return 0.f;
+      return __builtin_amdgcn_exp2f(fmaf(io<T>::from_scalar(xr[i]), c2, -m)) * inv;
+    };
+    auto dprob = [&](int i) {
+      return keep_element(row * g.sk + i, d) ? io<T>::from_scalar(gr[i]) * d.scale
+                                             : 0.f;
+    };
+    float s = 0.f;
+    for (int i = threadIdx.x; i < g.sk; i += 256) s += prob(i) * dprob(i);
+    s = block_reduce_256(s, sh, false);
+    for (int i = threadIdx.x; i < g.sk; i += 256)
+      dxr[i] = io<T>::to_scalar(scale * (prob(i) * (dprob(i) - s)));
   }
 }
 
@@ -526,10 +743,13 @@ constexpr int kBwdMaxElems = 32;  // two operands resident
     LAUNCH(8, 1);                    \
   }
 
+// stats != nullptr selects the dropout variant (d is ignored otherwise).
 template <typename T, int MODE>
 static int launch_softmax_fwd(const void *x, const uint8_t *mask, void *y,
-                              SoftmaxGeom g, float scale, hipStream_t st) {
+                              float *stats, DropArgs d, SoftmaxGeom g,
+                              float scale, hipStream_t st) {
   constexpr int E = io<T>::EPV;
+  const bool drop = stats != nullptr;
   SoftmaxPlan pl =
       plan_softmax(g.sk, E, kFwdMaxElems, MODE == kModeMasked ? 2 : 1);
   const bool vec_ok = pl.ok && aligned16(x) && aligned16(y) &&
@@ -539,8 +759,14 @@ static int launch_softmax_fwd(const void *x, const uint8_t *mask, void *y,
     const int64_t grid = g.rows < (int64_t)device_cu_count() * 32
                              ? g.rows
                              : (int64_t)device_cu_count() * 32;
-    softmax_fwd_generic_kernel<T, MODE><<<dim3((unsigned)grid), 256, 0, st>>>(
-        (const T *)x, mask, (T *)y, g, scale);
+    if (drop)
+      softmax_fwd_generic_kernel<T, MODE, true>
+          <<<dim3((unsigned)grid), 256, 0, st>>>((const T *)x, mask, (T *)y,
+                                                 stats, g, scale, d);
+    else
+      softmax_fwd_generic_kernel<T, MODE, false>
+          <<<dim3((unsigned)grid), 256, 0, st>>>((const T *)x, mask, (T *)y,
+                                                 nullptr, g, scale, d);
     return check_launch("softmax_fwd_generic_kernel");
   }
   g.wpr = pl.wpr;
@@ -548,11 +774,17 @@ static int launch_softmax_fwd(const void *x, const uint8_t *mask, void *y,
   const int threads = kWave * pl.wpr * pl.rpb;
   const int64_t grid = ceil_div(g.rows, (int64_t)pl.rpb * pl.rpw);
   OSLO_REQUIRE(grid <= 0x7fffffff, "softmax fwd: too many rows");
-#define OSLO_SM_FWD(VPL, RPW)                              \
-  if constexpr (VPL * RPW * E <= kFwdMaxElems)             \
-    softmax_fwd_kernel<T, VPL, RPW, MODE>                  \
-        <<<dim3((unsigned)grid), threads, 0, st>>>(        \
-            (const T *)x, mask, (T *)y, g, scale)
+#define OSLO_SM_FWD(VPL, RPW)                                        \
+  if constexpr (VPL * RPW * E <= kFwdMaxElems) {                     \
+    if (drop)                                                        \
+      softmax_fwd_kernel<T, VPL, RPW, MODE, true>                    \
+          <<<dim3((unsigned)grid), threads, 0, st>>>(                \
+              (const T *)x, mask, (T *)y, stats, g, scale, d);       \
+    else                                                             \
+      softmax_fwd_kernel<T, VPL, RPW, MODE, false>                   \
+          <<<dim3((unsigned)grid), threads, 0, st>>>(                \
+              (const T *)x, mask, (T *)y, nullptr, g, scale, d);     \
+  }
   OSLO_SM_CASES(OSLO_SM_FWD)
 #undef OSLO_SM_FWD
   return check_launch("softmax_fwd_kernel");
@@ -591,6 +823,42 @@ static int launch_softmax_bwd(const void *dy, const void *y,
   return check_launch("softmax_bwd_kernel");
 }
 
+template <typename T, int MODE>
+static int launch_softmax_dropout_bwd(const void *dy, const void *x,
+                                      const float *stats, const uint8_t *mask,
+                                      void *dx, DropArgs d, SoftmaxGeom g,
+                                      float scale, hipStream_t st) {
+  constexpr int E = io<T>::EPV;
+  SoftmaxPlan pl = plan_softmax(g.sk, E, kBwdMaxElems, 1);
+  const bool vec_ok = pl.ok && aligned16(dy) && aligned16(x) && aligned16(dx) &&
+                      (MODE != kModeMasked ||
+                       (reinterpret_cast<uintptr_t>(mask) % E) == 0);
+  if (!vec_ok) {
+    const int64_t grid = g.rows < (int64_t)device_cu_count() * 32
+                             ? g.rows
+                             : (int64_t)device_cu_count() * 32;
+    softmax_dropout_bwd_generic_kernel<T, MODE>
+        <<<dim3((unsigned)grid), 256, 0, st>>>((const T *)dy, (const T *)x,
+                                               stats, mask, (T *)dx, g, scale,
+                                               d);
+    return check_launch("softmax_dropout_bwd_generic_kernel");
+  }
+  g.wpr = pl.wpr;
+  g.rpb = pl.rpb;
+  const int threads = kWave * pl.wpr * pl.rpb;
+  const int64_t grid = ceil_div(g.rows, (int64_t)pl.rpb * pl.rpw);
+  OSLO_REQUIRE(grid <= 0x7fffffff, "softmax dropout bwd: too many rows");
+#define OSLO_SM_DBWD(VPL, RPW)                                      \
+  if constexpr (VPL * RPW * E <= kBwdMaxElems)                      \
+    softmax_dropout_bwd_kernel<T, VPL, RPW, MODE>                   \
+        <<<dim3((unsigned)grid), threads, 0, st>>>(                 \
+            (const T *)dy, (const T *)x, stats, mask, (T *)dx, g,   \
+            scale, d)
+  OSLO_SM_CASES(OSLO_SM_DBWD)
+#undef OSLO_SM_DBWD
+  return check_launch("softmax_dropout_bwd_kernel");
+}
+
 #define OSLO_SM_DISPATCH(dtype, MODE, FN, ...)                       \
   do {                                                               \
     if (dtype == OSLO_DTYPE_F32) return FN<float, MODE>(__VA_ARGS__); \
@@ -622,8 +890,8 @@ int oslo_softmax_causal_fwd(const void *x, void *y, int64_t attn_batches,
   if (attn_batches * sq == 0) return OSLO_OK;
   OSLO_REQUIRE(x && y, "softmax causal fwd: null tensor pointer");
   SoftmaxGeom g{attn_batches * sq, (int)sq, (int)sk, 1, 0, 0, 1, 1};
-  OSLO_SM_DISPATCH(dtype, kModeCausal, launch_softmax_fwd, x, nullptr, y, g,
-                   scale, (hipStream_t)stream);
+  OSLO_SM_DISPATCH(dtype, kModeCausal, launch_softmax_fwd, x, nullptr, y,
+                   nullptr, DropArgs{}, g, scale, (hipStream_t)stream);
 }
 
 int oslo_softmax_causal_bwd(const void *dy, const void *y, void *dx,
@@ -671,8 +939,8 @@ int oslo_softmax_masked_fwd(const void *x, const uint8_t *mask, void *y,
   if (rc != OSLO_OK) return rc;
   if (g.rows == 0) return OSLO_OK;
   OSLO_REQUIRE(x && y && mask, "softmax masked fwd: null tensor pointer");
-  OSLO_SM_DISPATCH(dtype, kModeMasked, launch_softmax_fwd, x, mask, y, g, scale,
-                   (hipStream_t)stream);
+  OSLO_SM_DISPATCH(dtype, kModeMasked, launch_softmax_fwd, x, mask, y, nullptr,
+                   DropArgs{}, g, scale, (hipStream_t)stream);
 }
 
 int oslo_softmax_masked_bwd(const void *dy, const void *y, const uint8_t *mask,
@@ -709,4 +977,89 @@ int oslo_softmax_batch_per_block(int64_t sq, int64_t sk, int64_t b,
   return pl.rpb * pl.rpw;
 }
 
-}  // extern "C"
+
+static int check_dropout_p(const char *what, float p) {
+  if (!(p >= 0.f && p <= 1.f))
+    return fail(OSLO_ERR_INVALID_ARGUMENT, "%s: p = %g outside [0, 1]", what,
+                (double)p);
+  return OSLO_OK;
+}
+
+int oslo_softmax_causal_dropout_fwd(const void *x, void *out, float *stats,
+                                    int64_t attn_batches, int64_t sq,
+                                    int64_t sk, float scale, float p,
+                                    uint64_t seed, uint64_t offset, int dtype,
+                                    void *stream) {
+  const char *what = "softmax causal dropout fwd";
+  int rc = check_softmax_shape(what, attn_batches, sq, sk, dtype);
+  if (rc == OSLO_OK) rc = check_dropout_p(what, p);
+  if (rc != OSLO_OK) return rc;
+  if (attn_batches * sq == 0) return OSLO_OK;
+  OSLO_REQUIRE(x && out && stats, "softmax causal dropout fwd: null pointer");
+  SoftmaxGeom g{attn_batches * sq, (int)sq, (int)sk, 1, 0, 0, 1, 1};
+  OSLO_SM_DISPATCH(dtype, kModeCausal, launch_softmax_fwd, x, nullptr, out,
+                   stats, make_drop(p, seed, offset), g, scale,
+                   (hipStream_t)stream);
+}
+
+int oslo_softmax_causal_dropout_bwd(const void *dout, const void *x,
+                                    const float *stats, void *dx,
+                                    int64_t attn_batches, int64_t sq,
+                                    int64_t sk, float scale, float p,
+                                    uint64_t seed, uint64_t offset, int dtype,
+                                    void *stream) {
+  const char *what = "softmax causal dropout bwd";
+  int rc = check_softmax_shape(what, attn_batches, sq, sk, dtype);
+  if (rc == OSLO_OK) rc = check_dropout_p(what, p);
+  if (rc != OSLO_OK) return rc;
+  if (attn_batches * sq == 0) return OSLO_OK;
+  OSLO_REQUIRE(dout && x && stats && dx,
+               "softmax causal dropout bwd: null pointer");
+  SoftmaxGeom g{attn_batches * sq, (int)sq, (int)sk, 1, 0, 0, 1, 1};
+  OSLO_SM_DISPATCH(dtype, kModeCausal, launch_softmax_dropout_bwd, dout, x,
+                   stats, nullptr, dx, make_drop(p, seed, offset), g, scale,
+                   (hipStream_t)stream);
+}
+
+int oslo_softmax_masked_dropout_fwd(const void *x, const uint8_t *mask,
+                                    void *out, float *stats, int64_t b,
+                                    int64_t np, int64_t sq, int64_t sk,
+                                    int64_t mask_b, int64_t mask_sq,
+                                    float scale, float p, uint64_t seed,
+                                    uint64_t offset, int dtype, void *stream) {
+  const char *what = "softmax masked dropout fwd";
+  int rc = check_softmax_shape(what, b, sq, sk, dtype);
+  if (rc == OSLO_OK) rc = check_dropout_p(what, p);
+  if (rc != OSLO_OK) return rc;
+  SoftmaxGeom g;
+  rc = masked_geom(what, b, np, sq, sk, mask_b, mask_sq, &g);
+  if (rc != OSLO_OK) return rc;
+  if (g.rows == 0) return OSLO_OK;
+  OSLO_REQUIRE(x && out && mask && stats,
+               "softmax masked dropout fwd: null pointer");
+  OSLO_SM_DISPATCH(dtype, kModeMasked, launch_softmax_fwd, x, mask, out, stats,
+                   make_drop(p, seed, offset), g, scale, (hipStream_t)stream);
+}
+
+int oslo_softmax_masked_dropout_bwd(const void *dout, const void *x,
+                                    const uint8_t *mask, const float *stats,
+                                    void *dx, int64_t b, int64_t np, int64_t sq,
+                                    int64_t sk, int64_t mask_b, int64_t mask_sq,
+                                    float scale, float p, uint64_t seed,
+                                    uint64_t offset, int dtype, void *stream) {
+  const char *what = "softmax masked dropout bwd";
+  int rc = check_softmax_shape(what, b, sq, sk, dtype);
+  if (rc == OSLO_OK) rc = check_dropout_p(what, p);
+  if (rc != OSLO_OK) return rc;
+  SoftmaxGeom g;
+  rc = masked_geom(what, b, np, sq, sk, mask_b, mask_sq, &g);
+  if (rc != OSLO_OK) return rc;
+  if (g.rows == 0) return OSLO_OK;
+  OSLO_REQUIRE(dout && x && mask && stats && dx,
+               "softmax masked dropout bwd: null pointer");
+  OSLO_SM_DISPATCH(dtype, kModeMasked, launch_softmax_dropout_bwd, dout, x,
+                   stats, mask, dx, make_drop(p, seed, offset), g, scale,
+                   (hipStream_t)stream);
+}
+
+}

@@ -71,6 +71,24 @@ _SIGNATURES = {
         [_p, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _i64, _f32, _int, _p],
     ),
     "oslo_softmax_batch_per_block": (_int, [_i64, _i64, _i64, _i64]),
+    "oslo_softmax_causal_dropout_fwd": (
+        _int,
+        [_p, _p, _p, _i64, _i64, _i64, _f32, _f32, _u64, _u64, _int, _p],
+    ),
+    "oslo_softmax_causal_dropout_bwd": (
+        _int,
+        [_p, _p, _p, _p, _i64, _i64, _i64, _f32, _f32, _u64, _u64, _int, _p],
+    ),
+    "oslo_softmax_masked_dropout_fwd": (
+        _int,
+        [_p, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _i64, _f32, _f32, _u64, _u64,
+         _int, _p],
+    ),
+    "oslo_softmax_masked_dropout_bwd": (
+        _int,
+        [_p, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _i64, _f32, _f32, _u64,
+         _u64, _int, _p],
+    ),
     "oslo_bias_gelu_fwd": (_int, [_p, _p, _p, _i64, _i64, _int, _p]),
     "oslo_bias_gelu_bwd": (_int, [_p, _p, _p, _p, _p, _p, _i64, _i64, _i64, _int, _p]),
     "oslo_bias_dropout_add_fwd": (
@@ -462,6 +480,91 @@ class _SoftmaxKernel:
                 float(scale_factor), _dtype_code(output_grads, "output_grads"),
                 _stream(output_grads),
             )
+            _check(rc, lib)
+        return grad_input
+
+    # -- softmax with the attention dropout fused in (no counterpart in the
+    #    reference's shim: the models apply nn.Dropout to the probabilities,
+    #    oslo/transformers/models/gpt2/modeling_gpt2.py:138-142) -------------
+    def _masked_dims(self, input, mask):
+        if input.dim() != 4 or mask.dim() != 4:
+            raise RuntimeError("expected 4D tensor")
+        b, np_, sq, sk = input.shape
+        mb, mh, msq, msk = mask.shape
+        if mh != 1 or msk != sk or mb not in (1, b) or msq not in (1, sq):
+            raise RuntimeError(
+                "mask of size %s does not broadcast to [%d, 1, %d, %d]"
+                % (list(mask.shape), b, sq, sk)
+            )
+        return b, np_, sq, sk, mb, msq
+
+    def softmax_dropout_forward(self, input, mask, scale_factor, p, seed, offset):
+        """``dropout(softmax(mask(scale * input)), p)`` -> ``[out, stats]``.
+
+        ``mask=None`` selects the causal form on a 3-D ``[attn_batches, sq, sk]``
+        input, otherwise ``input`` is ``[b, np, sq, sk]`` and ``mask`` a 4-D
+        padding mask.  ``stats`` (float32 ``[rows, 2]``) and ``input`` are what
+        the backward pass needs.
+        """
+        lib = self._lib
+        _check_input(input, "input")
+        out = torch.empty_like(input)
+        rows = input.numel() // input.shape[-1] if input.numel() else 0
+        stats = torch.empty((rows, 2), dtype=torch.float32, device=input.device)
+        with torch.cuda.device_of(input):
+            if mask is None:
+                if input.dim() != 3:
+                    raise RuntimeError("expected 3D tensor")
+                ab, sq, sk = input.shape
+                rc = lib.oslo_softmax_causal_dropout_fwd(
+                    _ptr(input), _ptr(out), _ptr(stats), ab, sq, sk,
+                    float(scale_factor), float(p), int(seed), int(offset),
+                    _dtype_code(input, "input"), _stream(input),
+                )
+            else:
+                b, np_, sq, sk, mb, msq = self._masked_dims(input, mask)
+                m8 = self._mask_u8(mask)
+                rc = lib.oslo_softmax_masked_dropout_fwd(
+                    _ptr(input), _ptr(m8), _ptr(out), _ptr(stats), b, np_, sq, sk,
+                    mb, msq, float(scale_factor), float(p), int(seed), int(offset),
+                    _dtype_code(input, "input"), _stream(input),
+                )
+            _check(rc, lib)
+        return [out, stats]
+
+    def softmax_dropout_backward(
+        self, output_grads, input, stats, mask, scale_factor, p, seed, offset,
+        inplace=False,
+    ):
+        lib = self._lib
+        _check_input(output_grads, "output_grads")
+        _check_input(input, "input")
+        _check_input(stats, "stats")
+        if output_grads.dtype != input.dtype or output_grads.shape != input.shape:
+            raise RuntimeError("output_grads and input differ in dtype or shape")
+        rows = input.numel() // input.shape[-1] if input.numel() else 0
+        if stats.dtype != torch.float32 or stats.numel() != 2 * rows:
+            raise RuntimeError("stats must be float32 [rows, 2]")
+        grad_input = output_grads if inplace else torch.empty_like(output_grads)
+        with torch.cuda.device_of(input):
+            if mask is None:
+                if input.dim() != 3:
+                    raise RuntimeError("expected 3D tensor")
+                ab, sq, sk = input.shape
+                rc = lib.oslo_softmax_causal_dropout_bwd(
+                    _ptr(output_grads), _ptr(input), _ptr(stats), _ptr(grad_input),
+                    ab, sq, sk, float(scale_factor), float(p), int(seed), int(offset),
+                    _dtype_code(input, "input"), _stream(input),
+                )
+            else:
+                b, np_, sq, sk, mb, msq = self._masked_dims(input, mask)
+                m8 = self._mask_u8(mask)
+                rc = lib.oslo_softmax_masked_dropout_bwd(
+                    _ptr(output_grads), _ptr(input), _ptr(m8), _ptr(stats),
+                    _ptr(grad_input), b, np_, sq, sk, mb, msq, float(scale_factor),
+                    float(p), int(seed), int(offset), _dtype_code(input, "input"),
+                    _stream(input),
+                )
             _check(rc, lib)
         return grad_input
 

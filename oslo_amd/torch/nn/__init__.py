@@ -15,7 +15,9 @@ from oslo_amd.torch.nn.modules.functional import (
     mixed_dtype_fused_layer_norm_affine,
     mixed_dtype_fused_rms_norm_affine,
     scaled_masked_softmax,
+    scaled_masked_softmax_dropout,
     scaled_upper_triang_masked_softmax,
+    scaled_upper_triang_masked_softmax_dropout,
 )
 from oslo_amd.torch.nn.modules.layer_norm import (
     FusedLayerNorm,
@@ -52,5 +54,7 @@ __all__ = [
     "mixed_dtype_fused_layer_norm_affine",
     "mixed_dtype_fused_rms_norm_affine",
     "scaled_masked_softmax",
+    "scaled_masked_softmax_dropout",
     "scaled_upper_triang_masked_softmax",
+    "scaled_upper_triang_masked_softmax_dropout",
 ]

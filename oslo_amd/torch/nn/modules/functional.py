@@ -323,6 +323,47 @@ class _ScaledMaskedSoftmax(torch.autograd.Function):
         return input_grads, None, None
 
 
+class _ScaledMaskedSoftmaxDropout(torch.autograd.Function):
+    """
+    Fused: scale -> causal or padding mask -> softmax -> dropout, the pair
+    ``nn.functional.softmax`` + ``attn_dropout`` of
+    oslo/transformers/models/gpt2/modeling_gpt2.py:138-142 and
+    oslo/transformers/models/bert/modeling_bert.py:306-310 in one pass.
+
+    ``mask=None``: causal, inputs [attn_batches, sq, sk]; otherwise inputs
+    [b, np, sq, sk] with a padding mask.  Saves the *input* and two floats per
+    row; backward recomputes the probabilities and regenerates the keep bits
+    from (seed, offset), so neither the probabilities nor a mask are stored.
+    """
+
+    @staticmethod
+    def forward(ctx, inputs, mask, scale, p, seed, offset):
+        scale = float(scale)
+        inputs = inputs.contiguous()
+        out, stats = get_softmax_kernel().softmax_dropout_forward(
+            inputs, mask, scale, p, seed, offset
+        )
+        ctx.scale, ctx.p, ctx.seed, ctx.offset = scale, p, seed, offset
+        ctx.has_mask = mask is not None
+        if mask is not None:
+            ctx.save_for_backward(inputs, stats, mask)
+        else:
+            ctx.save_for_backward(inputs, stats)
+        return out
+
+    @staticmethod
+    def backward(ctx, output_grads):
+        if ctx.has_mask:
+            inputs, stats, mask = ctx.saved_tensors
+        else:
+            (inputs, stats), mask = ctx.saved_tensors, None
+        input_grads = get_softmax_kernel().softmax_dropout_backward(
+            output_grads.contiguous(), inputs, stats, mask, ctx.scale, ctx.p,
+            ctx.seed, ctx.offset,
+        )
+        return input_grads, None, None, None, None, None
+
+
 """
 User Functions
 """
@@ -412,3 +453,30 @@ def scaled_upper_triang_masked_softmax(input, scale=1.0):
 def scaled_masked_softmax(input, mask, scale=1.0):
     """softmax(scale * input) with `mask` (True = masked out); input is [b, np, sq, sk]."""
     return _ScaledMaskedSoftmax.apply(input, mask, scale)
+
+
+def _check_dropout_p(p):
+    if p < 0.0 or p > 1.0:
+        raise ValueError(
+            "dropout probability has to be between 0 and 1, but got {}".format(p)
+        )
+
+
+def scaled_upper_triang_masked_softmax_dropout(input, scale=1.0, p=0.0, training=True):
+    """dropout(softmax(scale * input) under a causal mask, p); [attn_batches, sq, sk]."""
+    _check_dropout_p(p)
+    p_eff = float(p) if training else 0.0
+    if p_eff == 0.0:
+        return _ScaledUpperTriangMaskedSoftmax.apply(input, scale)
+    seed, offset = _next_philox_state(input.device)
+    return _ScaledMaskedSoftmaxDropout.apply(input, None, scale, p_eff, seed, offset)
+
+
+def scaled_masked_softmax_dropout(input, mask, scale=1.0, p=0.0, training=True):
+    """dropout(softmax(scale * input) with `mask`, p); input is [b, np, sq, sk]."""
+    _check_dropout_p(p)
+    p_eff = float(p) if training else 0.0
+    if p_eff == 0.0:
+        return _ScaledMaskedSoftmax.apply(input, mask, scale)
+    seed, offset = _next_philox_state(input.device)
+    return _ScaledMaskedSoftmaxDropout.apply(input, mask, scale, p_eff, seed, offset)

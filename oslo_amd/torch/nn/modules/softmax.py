@@ -39,6 +39,11 @@ class FusedScaleMaskSoftmax(nn.Module):
         softmax_in_fp32: unfused branch computes the softmax in fp32 (the fused
             kernels always accumulate in fp32).
         scale: factor applied to the scores before masking (None = 1).
+        attn_dropout: probability of the dropout the models apply to the
+            probabilities right after the softmax
+            (``modeling_gpt2.py:142``, ``modeling_bert.py:310``); fused into the
+            same kernel while the module is in training mode.  0 (default)
+            leaves the module a plain softmax.
 
     ``forward(input, mask)``: ``input`` is ``[b, np, sq, sk]``; ``mask`` is a
     boolean ``[b or 1, 1, sq or 1, sk]`` tensor with True = masked out, or None.
@@ -55,8 +60,16 @@ class FusedScaleMaskSoftmax(nn.Module):
         mask_func=attention_mask_func,
         softmax_in_fp32=True,
         scale=None,
+        attn_dropout=0.0,
     ):
         super().__init__()
+        if attn_dropout < 0.0 or attn_dropout > 1.0:
+            raise ValueError(
+                "dropout probability has to be between 0 and 1, but got {}".format(
+                    attn_dropout
+                )
+            )
+        self.attn_dropout = float(attn_dropout)
         self.input_in_fp16 = input_in_fp16
         self.input_in_bf16 = input_in_bf16
         if self.input_in_fp16 and self.input_in_bf16:
@@ -95,14 +108,15 @@ class FusedScaleMaskSoftmax(nn.Module):
     def forward_fused_softmax(self, input, mask):
         b, np, sq, sk = input.size()
         scale = self.scale if self.scale is not None else 1.0
+        p, training = self.attn_dropout, self.training
         if self.attn_mask_type == AttnMaskType.causal and mask is None:
-            probs = onn_f.scaled_upper_triang_masked_softmax(
-                input.reshape(-1, sq, sk), scale
+            probs = onn_f.scaled_upper_triang_masked_softmax_dropout(
+                input.reshape(-1, sq, sk), scale, p, training
             )
             return probs.view(b, np, sq, sk)
         if mask is None:
             mask = torch.zeros(1, 1, 1, sk, dtype=torch.bool, device=input.device)
-        return onn_f.scaled_masked_softmax(input, mask, scale)
+        return onn_f.scaled_masked_softmax_dropout(input, mask, scale, p, training)
 
     def forward_torch_softmax(self, input, mask):
         orig_dtype = input.dtype
@@ -120,6 +134,10 @@ class FusedScaleMaskSoftmax(nn.Module):
         probs = torch.nn.Softmax(dim=-1)(mask_output)
         if self.input_in_float16 and self.softmax_in_fp32:
             probs = probs.to(orig_dtype)
+        if self.attn_dropout > 0.0:
+            probs = torch.nn.functional.dropout(
+                probs, p=self.attn_dropout, training=self.training
+            )
         return probs
 
     @staticmethod

@@ -78,6 +78,51 @@ def test_causal_softmax_full_size(device, name, ab, s, dtype, scale):
     check(dxb, cf.softmax_bwd(f64(gb), f64(yb), scale), name + " bwd rows", atol=1e-7)
 
 
+@pytest.mark.parametrize(
+    "name,ab,s,dtype,scale",
+    [("cfg1", 48, 512, F32, 0.125), ("cfg5", 256, 2048, BF16, 1.0 / math.sqrt(96.0))],
+)
+def test_causal_softmax_dropout_full_size(device, name, ab, s, dtype, scale):
+    """Softmax with fused dropout at full size: the keep decisions equal the
+    Philox mask of the flattened output, kept values are the plain
+    probabilities over 1 - p, gradient rows sum to 0, sampled rows match the
+    oracle."""
+    p, seed, offset = 0.1, 4242, 16
+    x = gpu_randn((ab, s, s), dtype, 1, device)
+    g = gpu_randn((ab, s, s), dtype, 2, device)
+    k = _C.get_softmax_kernel()
+    ek = _C.get_fused_elementwise_kernel()
+    out, stats = k.softmax_dropout_forward(x, None, scale, p, seed, offset)
+    y = k.fused_scaled_upper_triang_masked_softmax_forward(x, scale)
+    keep = ek.philox_mask(x.numel(), p, seed, offset, device).view(ab, s, s)
+    tol = 1e-5 if dtype == F32 else 2.0 ** -7
+    for b0 in range(0, ab, 32):
+        ob, yb, kb = out[b0:b0 + 32].float(), y[b0:b0 + 32].float(), keep[b0:b0 + 32].bool()
+        assert ob[~kb].count_nonzero().item() == 0
+        assert torch.triu(ob, diagonal=1).count_nonzero().item() == 0
+        want = yb / (1.0 - p)
+        assert ((ob - want)[kb].abs() <= tol * want[kb] + 1e-30).all()
+    del y, keep
+    dx = k.softmax_dropout_backward(g, x, stats, None, scale, p, seed, offset)
+    for b0 in range(0, ab, 32):
+        dxb = dx[b0:b0 + 32].float()
+        assert torch.triu(dxb, diagonal=1).count_nonzero().item() == 0
+        gscale = g[b0:b0 + 32].float().abs().amax(-1) * abs(scale) / (1.0 - p)
+        rtol = 1e-5 if dtype == F32 else 2e-3
+        assert (dxb.sum(-1).abs() <= (4 * rtol) * gscale + 1e-6).all()
+    rows = sample_rows(ab * s)
+    sel = rows.to(device)
+    xb, ob = x.view(ab * s, s)[sel].cpu(), out.view(ab * s, s)[sel].cpu()
+    gb, dxb = g.view(ab * s, s)[sel].cpu(), dx.view(ab * s, s)[sel].cpu()
+    qi = (rows % s).numpy()
+    hidden = np.arange(s)[None, :] > qi[:, None]
+    keep_rows = np.stack(
+        [philox.keep_mask(s, p, seed, offset, first_element=int(r) * s) for r in rows]
+    ).astype(bool)
+    check(ob, cf.softmax_dropout_fwd(f64(xb), hidden, scale, keep_rows, p), name + " dropout fwd rows", atol=1e-9)
+    check(dxb, cf.softmax_dropout_bwd(f64(gb), f64(xb), hidden, scale, keep_rows, p), name + " dropout bwd rows", atol=2e-7)
+
+
 # --------------------------------------------------------------------------- cfg3
 def test_padding_softmax_full_size(device):
     b, h, s = 16, 16, 1024

@@ -286,3 +286,38 @@ def test_autograd_sums_full_size_bias_grad():
     g = torch.randn(5, 3, dtype=torch.float64)
     Fn.apply(x, b).backward(g)
     assert torch.allclose(b.grad, g.sum(0))
+
+
+# ------------------------------------------------------- softmax + dropout
+def test_softmax_dropout_vs_autograd_of_the_unfused_chain():
+    """softmax -> dropout as the models chain them (modeling_gpt2.py:138-142):
+    forward and backward of the oracle against torch autograd through
+    softmax(where(hidden, -1e4, scale * x)) * keep / (1 - p) in float64, with an
+    explicit keep mask; a wrong scale placement or a missing keep factor in the
+    backward fails here."""
+    r = np.random.default_rng(11)
+    b, sq, sk, scale, p = 3, 5, 24, 0.37, 0.25
+    x = torch.from_numpy(r.standard_normal((b, sq, sk))).requires_grad_(True)
+    g = torch.from_numpy(r.standard_normal((b, sq, sk)))
+    keep = r.random((b, sq, sk)) >= p
+    hidden = cf.causal_hidden(sq, sk)
+    t = torch.where(torch.from_numpy(hidden), torch.tensor(-1e4, dtype=torch.float64), x * scale)
+    out = torch.softmax(t, -1) * torch.from_numpy(keep) / (1.0 - p)
+    out.backward(g)
+    o = cf.softmax_dropout_fwd(x.detach().numpy(), hidden, scale, keep, p)
+    # the oracle's dropout scale is the float32 quotient 1 / (1 - p), as in the kernel
+    assert np.allclose(o, out.detach().numpy(), rtol=1e-7, atol=1e-300)
+    dx = cf.softmax_dropout_bwd(g.numpy(), x.detach().numpy(), hidden, scale, keep, p)
+    assert np.allclose(dx, x.grad.numpy(), rtol=1e-6, atol=1e-12)
+    # p = 0 / no mask: the plain softmax pair
+    assert np.array_equal(
+        cf.softmax_dropout_fwd(x.detach().numpy(), hidden, scale, None, 0.0),
+        cf.softmax_causal_fwd(x.detach().numpy(), scale),
+    )
+    y = cf.softmax_causal_fwd(x.detach().numpy(), scale)
+    assert np.allclose(
+        cf.softmax_dropout_bwd(g.numpy(), x.detach().numpy(), hidden, scale, None, 0.0),
+        cf.softmax_bwd(g.numpy(), y, scale), rtol=1e-13, atol=1e-300,
+    )
+    # dropped positions still receive a gradient through the normaliser
+    assert (dx[~keep & ~np.broadcast_to(hidden, keep.shape)] != 0).any()
