@@ -316,6 +316,39 @@ def kernel_table(L, dev, iters):
         r2 = table_row("bias_dropout_add_bwd", cfg, [n1, n2], "bf16", 2 * T, timed(dbwd, ns))
         r1["p"] = r2["p"] = pdrop
         rows += [r1, r2]
+
+        # the same op fused into the LayerNorm that follows it (post-LN block):
+        # forward reads x, residual and writes h, y (4T instead of 3T + 2T);
+        # backward reads dy, h and writes the residual and x gradients (4T
+        # instead of 3T + 2T)
+        if pdrop > 0:
+            gamma = (1 + 0.02 * torch.randn(n2, generator=g, device=dev)).to(torch.bfloat16)
+            beta = (0.02 * torch.randn(n2, generator=g, device=dev)).to(torch.bfloat16)
+            dgamma, dbeta = torch.empty_like(gamma), torch.empty_like(beta)
+            mean = torch.empty(n1, device=dev, dtype=torch.float32)
+            invvar = torch.empty(n1, device=dev, dtype=torch.float32)
+            ws2, wsb2 = L.ws(L._C.OSLO_OP_BIAS_DROPOUT_ADD_NORM_BWD, n1, n2, dev)
+            extra = [(torch.empty_like(b[0]), torch.empty_like(b[0])) for b in bufs]  # h, dres
+
+            def ffwd(i):
+                x, res, out, gg, dx = bufs[i]
+                L.ok(lib.oslo_bias_dropout_add_norm_fwd(p(x), p(bias), p(res), p(gamma), p(beta), p(extra[i][0]),
+                                                        p(out), p(mean), p(invvar), n1, n2, 1e-5, pdrop, 1234, 0, 0,
+                                                        BF16, L.stream()))
+
+            def fbwd(i):
+                x, res, out, gg, dx = bufs[i]
+                L.ok(lib.oslo_bias_dropout_add_norm_bwd(p(gg), None, p(extra[i][0]), p(mean), p(invvar), p(gamma),
+                                                        p(extra[i][1]), p(dx), p(dgamma), p(dbeta), p(dbias), p(ws2),
+                                                        wsb2, n1, n2, pdrop, 1234, 0, 0, BF16, L.stream()))
+
+            r3 = table_row("bias_dropout_add_ln_fwd", cfg, [n1, n2], "bf16", 4 * T, timed(ffwd, ns))
+            for i in range(ns):
+                ffwd(i)
+            r4 = table_row("bias_dropout_add_ln_bwd", cfg, [n1, n2], "bf16", 4 * T, timed(fbwd, ns))
+            r3["p"] = r4["p"] = pdrop
+            rows += [r3, r4]
+            del extra
         del bufs
         torch.cuda.empty_cache()
 

@@ -43,6 +43,7 @@ extern "C" {
 #define OSLO_OP_RMS_BWD 2
 #define OSLO_OP_BIAS_GELU_BWD 3
 #define OSLO_OP_BIAS_DROPOUT_ADD_BWD 4
+#define OSLO_OP_BIAS_DROPOUT_ADD_NORM_BWD 5
 
 /* ---- library state ----------------------------------------------------- */
 
@@ -239,6 +240,50 @@ int oslo_bias_dropout_add_bwd(const void *g, void *dx, void *dbias,
                               int64_t rows, int64_t cols, float p,
                               uint64_t seed, uint64_t offset, int dtype,
                               void *stream);
+
+/* ---- bias-dropout-add fused into the following LayerNorm / RMSNorm ------ *
+ * Replaces the chain FusedBiasDropout -> residual add -> LayerNorm of the
+ * post-LN blocks (oslo/transformers/models/bert/modeling_bert.py:343-346,
+ * 446-449: LayerNorm(dropout(dense(x) + bias) + input_tensor)) and the
+ * residual add -> ln_2 of the pre-LN blocks (modeling_gpt2.py:369-393):
+ *   h = keep * (x + bias) / (1 - p) + residual   (rounded once, as
+ *                                                 oslo_bias_dropout_add_fwd)
+ *   y = norm(h)                                  (as oslo_ln_fwd / oslo_rms_fwd
+ *                                                 of the stored h)
+ * One dtype for x, bias, residual, h_out, y, gamma, beta.  bias, residual,
+ * gamma/beta and h_out may be NULL; h_out receives h, which the backward
+ * pass (and a pre-LN block's next residual) needs.  rms != 0 selects RMSNorm
+ * (beta and mean are then ignored).  Keep mask: that of
+ * oslo_bias_dropout_add_fwd for the same (p, seed, offset).                 */
+int oslo_bias_dropout_add_norm_fwd(const void *x, const void *bias,
+                                   const void *residual, const void *gamma,
+                                   const void *beta, void *h_out, void *y,
+                                   float *mean, float *invvar, int64_t n1,
+                                   int64_t n2, double eps, float p,
+                                   uint64_t seed, uint64_t offset, int rms,
+                                   int dtype, void *stream);
+
+/* Backward of the above in one pass over dy and h (plus a finalize launch):
+ *   dh    = norm_backward(dy; h, mean, invvar, gamma) + dh_extra
+ *   dres  = dh                      gradient of the residual (and of h)
+ *   dx    = keep * dh / (1 - p)     gradient of x; NULL allowed when p == 0,
+ *                                   where it equals dres
+ *   dbias = column sums of dx as stored; dgamma, dbeta as oslo_ln_bwd.
+ * dh_extra (may be NULL) is the gradient that reaches h from its other
+ * consumers -- in a pre-LN block h is also the next residual -- the fused
+ * residual-gradient add of the reference's
+ * oslo/lightseq2/csrc/kernels/cuda/normalize_kernels.cu:608-616.
+ * Workspace: oslo_workspace_bytes(OSLO_OP_BIAS_DROPOUT_ADD_NORM_BWD, n1, n2).
+ * Outputs must not alias inputs.                                            */
+int oslo_bias_dropout_add_norm_bwd(const void *dy, const void *dh_extra,
+                                   const void *h, const float *mean,
+                                   const float *invvar, const void *gamma,
+                                   void *dres, void *dx, void *dgamma,
+                                   void *dbeta, void *dbias, void *workspace,
+                                   int64_t workspace_bytes, int64_t n1,
+                                   int64_t n2, float p, uint64_t seed,
+                                   uint64_t offset, int rms, int dtype,
+                                   void *stream);
 
 /* ---- test and measurement hooks (no counterpart in the reference) ------ */
 

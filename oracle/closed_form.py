@@ -277,3 +277,52 @@ def bias_dropout_add_bwd(g, keep, p, out="f64", acc=np.float64):
     cols = dx.shape[-1]
     dbias = np.asarray(dx, dtype=acc).reshape(-1, cols).sum(axis=0)
     return dx, round_to(dbias, out)
+
+
+# ---------------------------------------------------------------------------
+# bias-dropout-add fused into the following norm
+# ---------------------------------------------------------------------------
+def bias_dropout_add_norm_fwd(x, bias, residual, keep, p, gamma, beta, eps, rms=False,
+                              out="f64", acc=np.float64):
+    """Returns (y, h, mean, invvar): h = dropout(x + bias) + residual rounded once
+    to the storage type, y = LayerNorm / RMSNorm of that stored h.
+
+    The chain FusedBiasDropout -> residual add -> LayerNorm of
+    oslo/transformers/models/bert/modeling_bert.py:343-346; composed from
+    bias_dropout_add_fwd and layer_norm_fwd / rms_norm_fwd above.  mean is None
+    for RMSNorm.
+    """
+    h = bias_dropout_add_fwd(x, bias, residual, keep, p, out, acc)
+    h = np.asarray(h, dtype=acc)
+    if rms:
+        y, invvar = rms_norm_fwd(h, gamma, eps, out, acc)
+        return y, h, None, invvar
+    y, mean, invvar = layer_norm_fwd(h, gamma, beta, eps, out, acc)
+    return y, h, mean, invvar
+
+
+def bias_dropout_add_norm_bwd(dy, dh_extra, h, mean, invvar, gamma, keep, p, rms=False,
+                              out="f64", acc=np.float64):
+    """Returns (dres, dx, dgamma, dbeta, dbias) of the fused chain.
+
+    dh = norm_backward(dy) + dh_extra is formed in `acc`; dres = dh and
+    dx = keep * dh / (1 - p) are each rounded once from it; dbias is the column
+    sum of dx as stored; dgamma / dbeta as the plain norm backward (dbeta None
+    for RMSNorm).
+    """
+    if rms:
+        dh, dgamma = rms_norm_bwd(dy, h, invvar, gamma, "f64", out, acc)
+        dbeta = None
+    else:
+        dh, dgamma, dbeta = layer_norm_bwd(dy, h, mean, invvar, gamma, "f64", out, acc)
+    dh = np.asarray(dh, dtype=acc)
+    if dh_extra is not None:
+        dh = dh + np.asarray(dh_extra, dtype=acc)
+    dres = round_to(dh, out)
+    t = dh
+    if keep is not None:
+        t = np.where(np.asarray(keep, dtype=bool), dh * _dropout_scale(p, acc), 0.0)
+    dx = round_to(t, out)
+    n2 = dx.shape[-1]
+    dbias = round_to(np.asarray(dx, dtype=acc).reshape(-1, n2).sum(axis=0), out)
+    return dres, dx, dgamma, dbeta, dbias

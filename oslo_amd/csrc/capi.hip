@@ -58,6 +58,8 @@ int64_t oslo_workspace_bytes(int op, int64_t n1, int64_t n2) {
   switch (op) {
     case OSLO_OP_LN_BWD:
       return 2 * oslo::colsum_parts_norm(n1, n2) * n2 * (int64_t)sizeof(float);
+    case OSLO_OP_BIAS_DROPOUT_ADD_NORM_BWD:
+      return 3 * oslo::colsum_parts_norm(n1, n2) * n2 * (int64_t)sizeof(float);
     case OSLO_OP_RMS_BWD:
       return oslo::colsum_parts_norm(n1, n2) * n2 * (int64_t)sizeof(float);
     case OSLO_OP_BIAS_GELU_BWD:

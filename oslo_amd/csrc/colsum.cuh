@@ -8,14 +8,15 @@
 namespace oslo {
 
 // Reduces fp32 partial rows part[a][0..P)[cols] to out_a[cols] in dtype V;
-// blockIdx.y selects the array a.  A workgroup owns 32 columns: 8 column quads
+// blockIdx.y selects the array a (up to three; a null output is skipped).
+// A workgroup owns 32 columns: 8 column quads
 // times 128 slices of the partial rows, so that for the usual P of a few
 // hundred every thread issues all its loads at once; the slices are then
 // folded through LDS in a fixed order.  cols % 4 == 0.
 template <typename V>
 __global__ __launch_bounds__(1024) void colsum_finalize_kernel(
     const float *__restrict__ part, int64_t P, int64_t cols,
-    V *__restrict__ out0, V *__restrict__ out1) {
+    V *__restrict__ out0, V *__restrict__ out1, V *__restrict__ out2) {
   __shared__ float sh[128][33];
   __shared__ float sh2[8][33];
   const int tid = threadIdx.x;
@@ -49,21 +50,23 @@ __global__ __launch_bounds__(1024) void colsum_finalize_kernel(
 #pragma unroll
     for (int g = 0; g < 8; ++g) s += sh2[g][tid];
     const int64_t oc = (int64_t)blockIdx.x * 32 + tid;
-    if (oc < cols) {
-      V *o = a == 0 ? out0 : out1;
-      o[oc] = io<V>::to_scalar(s);
-    }
+    V *o = a == 0 ? out0 : (a == 1 ? out1 : out2);
+    if (oc < cols && o != nullptr) o[oc] = io<V>::to_scalar(s);
   }
 }
 
 template <typename V>
 static inline int launch_colsum_finalize(const float *part, int64_t P,
                                          int64_t cols, void *out0, void *out1,
-                                         hipStream_t st) {
+                                         hipStream_t st, void *out2 = nullptr,
+                                         int narrays = 0) {
   const int64_t grid = ceil_div(cols, 32);
+  // narrays = number of arrays of partial rows (outputs that are null are
+  // skipped); by default one per non-null output
+  if (narrays <= 0) narrays = out1 != nullptr ? 2 : 1;
   colsum_finalize_kernel<V>
-      <<<dim3((unsigned)grid, out1 != nullptr ? 2 : 1), 1024, 0, st>>>(
-          part, P, cols, (V *)out0, (V *)out1);
+      <<<dim3((unsigned)grid, (unsigned)narrays), 1024, 0, st>>>(
+          part, P, cols, (V *)out0, (V *)out1, (V *)out2);
   return check_launch("colsum_finalize_kernel");
 }
 

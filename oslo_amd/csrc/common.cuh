@@ -415,4 +415,16 @@ static inline DropArgs make_drop(float p, uint64_t seed, uint64_t offset) {
   return d;
 }
 
+// Keep bits of the E elements of chunk c of `row` (dropout on the flattened
+// [rows, row_length] tensor: element i belongs to group i >> 3).  A 4-element chunk
+// takes the low or the high half of its group's eight bits.
+template <int E>
+__device__ __forceinline__ uint32_t chunk_keep_bits(int64_t row, int row_length, int c,
+                                                    const DropArgs &d) {
+  const uint64_t flat = (uint64_t)row * (uint64_t)row_length + (uint64_t)c * E;
+  uint32_t keep = dropout_keep_bits(flat >> 3, d.seed, d.offset, d.threshold);
+  if constexpr (E == 4) keep >>= (uint32_t)(flat & 4u);
+  return keep;
+}
+
 }  // namespace oslo

@@ -96,15 +96,30 @@ __device__ __forceinline__ Welford row_welford(Welford w, float *red, int wave,
 // ---------------------------------------------------------------------------
 // forward, register-resident
 // ---------------------------------------------------------------------------
+// Operands of the fused prologue h = dropout(x + bias) + residual, which the
+// FUSE build of the forward kernel evaluates, rounds to the storage type and
+// (optionally) stores before it normalises h: the chain FusedBiasDropout ->
+// residual add -> LayerNorm of oslo/transformers/models/bert/modeling_bert.py:
+// 343-346, 446-449 in one pass.  One dtype for all tensors.
+struct FusePrologue {
+  const void *bias;      // [n2] or null
+  const void *residual;  // [n1, n2] or null
+  void *h_out;           // [n1, n2] or null
+  DropArgs d;
+  int drop;              // 1: dropout with d, 0: none
+};
+
 // EVEN: every lane holds exactly VPL chunks of its row (no column guards;
 // LayerNorm then merges equal-sized Welford partials).
-template <typename T, typename V, int VPL, bool RMS, bool EVEN, int MAXT>
+template <typename T, typename V, int VPL, bool RMS, bool EVEN, int MAXT,
+          bool FUSE = false>
 __global__ __launch_bounds__(MAXT) void norm_fwd_reg_kernel(
     const T *__restrict__ x, const V *__restrict__ gamma,
     const V *__restrict__ beta, V *__restrict__ y, float *__restrict__ mean,
     float *__restrict__ invvar, int64_t n1, int n2, float eps, int wpr,
-    int rpb, int iters) {
+    int rpb, int iters, FusePrologue fp) {
   constexpr int E = chunk_elems<T, V>::value;
+  static_assert(!FUSE || sizeof(T) == sizeof(V), "fused prologue: one dtype");
   __shared__ float red[2][48];
   const int lane = threadIdx.x & 63;
   // the wave index is uniform: keep it (and the row arithmetic) in scalar registers
@@ -131,6 +146,21 @@ __global__ __launch_bounds__(MAXT) void norm_fwd_reg_kernel(
     }
   }
 
+  const T *fbias = static_cast<const T *>(fp.bias);
+  const T *fres = static_cast<const T *>(fp.residual);
+  T *fh = static_cast<T *>(fp.h_out);
+  RawChunk<T, E> biasraw[FUSE ? VPL : 1];
+  if constexpr (FUSE) {
+#pragma unroll
+    for (int k = 0; k < VPL; ++k) {
+      const int c = c0 + k * cstride;
+      if (fbias != nullptr && c < nchunks)
+        biasraw[k].load_cached(fbias + (int64_t)c * E);
+      else
+        biasraw[k].zero();
+    }
+  }
+
   // A workgroup takes `iters` consecutive groups of rpb rows, then strides
   // by the grid.
   const int64_t total_groups = (n1 + rpb - 1) / rpb;
@@ -140,6 +170,7 @@ __global__ __launch_bounds__(MAXT) void norm_fwd_reg_kernel(
   // budget of 128 has no room for the second row)
   constexpr bool kPrefetch = !(MAXT > 256 && VPL * E >= 32);
   RawChunk<T, E> nx[VPL];
+  RawChunk<T, E> nr[FUSE ? VPL : 1];  // residual of the fused prologue
   auto fetch = [&](int64_t group) {
     int64_t frow = group * rpb + rslot;
     // a slot past the last row re-reads row n1 - 1 and stores nothing
@@ -152,6 +183,12 @@ __global__ __launch_bounds__(MAXT) void norm_fwd_reg_kernel(
         nx[k].load(xr + (int64_t)c * E);
       else
         nx[k].zero();
+      if constexpr (FUSE) {
+        if (fres != nullptr && (EVEN || c < nchunks))
+          nr[k].load(fres + frow * n2 + (int64_t)c * E);
+        else
+          nr[k].zero();
+      }
     }
   };
   for (int64_t g0 = (int64_t)blockIdx.x * iters; g0 < total_groups;
@@ -164,6 +201,30 @@ __global__ __launch_bounds__(MAXT) void norm_fwd_reg_kernel(
     if constexpr (!kPrefetch) fetch(g0 + it);
 #pragma unroll
     for (int k = 0; k < VPL; ++k) nx[k].unpack(v[k]);
+    if constexpr (FUSE) {
+      // h = dropout(x + bias) + residual, rounded once to the storage type;
+      // the statistics below are those of the stored h.  Done before the
+      // next row is requested, so the packed residual is dead by then.
+#pragma unroll
+      for (int k = 0; k < VPL; ++k) {
+        const int c = c0 + k * cstride;
+        if (EVEN || c < nchunks) {
+          float b[E], res[E];
+          biasraw[k].unpack(b);
+          nr[k].unpack(res);
+          uint32_t keep = (1u << E) - 1u;
+          if (fp.drop) keep = chunk_keep_bits<E>(rvalid ? row : n1 - 1, n2, c, fp.d);
+#pragma unroll
+          for (int e = 0; e < E; ++e) {
+            float t = v[k][e] + b[e];
+            if (fp.drop) t = (keep >> e) & 1u ? t * fp.d.scale : 0.f;
+            v[k][e] = io<T>::round(t + res[e]);
+          }
+          if (fh != nullptr && rvalid)
+            store_chunk<T, E>(fh + row * n2 + (int64_t)c * E, v[k]);
+        }
+      }
+    }
     if constexpr (kPrefetch) {
       if (it + 1 < iters && g0 + it + 1 < total_groups) fetch(g0 + it + 1);
     }
@@ -336,13 +397,29 @@ __global__ __launch_bounds__(256) void norm_fwd_generic_kernel(
 // backward, register-resident, single pass
 // ---------------------------------------------------------------------------
 // EVEN: every lane holds exactly VPL chunks of its row (no column guards).
-template <typename T, typename V, int VPL, bool RMS, bool EVEN, int PF>
+// Operands of the fused epilogue, the backward of the forward kernel's
+// prologue h = dropout(x + bias) + residual: the gradient of h is the norm's
+// input gradient plus dh_extra (what reaches h from its other consumers); it
+// is stored through the kernel's dx pointer (= gradient of the residual) and,
+// masked and scaled, through dx_drop (= gradient of x); the column sums of
+// dx_drop as stored are the bias gradient (an extra array of partial rows).
+struct FuseEpilogue {
+  const void *dh_extra;  // [n1, n2] or null
+  void *dx_drop;         // [n1, n2] or null
+  DropArgs d;
+  int drop;              // 1: dropout with d, 0: none
+  int want_dbias;        // 1: partial rows of the bias gradient are written
+};
+
+template <typename T, typename V, int VPL, bool RMS, bool EVEN, int PF,
+          bool FUSE = false>
 __global__ __launch_bounds__(1024) void norm_bwd_reg_kernel(
     const V *__restrict__ dy, const T *__restrict__ x,
     const float *__restrict__ mean, const float *__restrict__ invvar,
     const V *__restrict__ gamma, T *__restrict__ dx, float *__restrict__ part,
-    int64_t n1, int n2, int wpr, int rpb) {
+    int64_t n1, int n2, int wpr, int rpb, FuseEpilogue fe) {
   constexpr int E = chunk_elems<T, V>::value;
+  static_assert(!FUSE || sizeof(T) == sizeof(V), "fused epilogue: one dtype");
   extern __shared__ float xslot[];  // [n2] when rpb > 1
   __shared__ float red[2][32];
   const int lane = threadIdx.x & 63;
@@ -359,6 +436,7 @@ __global__ __launch_bounds__(1024) void norm_bwd_reg_kernel(
   // gamma stays packed (half the registers) and is unpacked once per row
   RawChunk<V, E> gmraw[VPL];
   float acc_g[VPL][E], acc_b[VPL][E];
+  float acc_d[FUSE ? VPL : 1][E];  // bias gradient of the fused epilogue
 #pragma unroll
   for (int k = 0; k < VPL; ++k) {
     const int c = c0 + k * cstride;
@@ -370,14 +448,18 @@ __global__ __launch_bounds__(1024) void norm_bwd_reg_kernel(
     for (int e = 0; e < E; ++e) {
       acc_g[k][e] = 0.f;
       acc_b[k][e] = 0.f;
+      if constexpr (FUSE) acc_d[k][e] = 0.f;
     }
   }
+  const T *fextra = static_cast<const T *>(fe.dh_extra);
+  T *fdrop = static_cast<T *>(fe.dx_drop);
 
   // The loads of a row are issued PF iterations ahead, in packed form, so
   // that they are in flight while the previous rows are reduced and stored.
   struct RowFetch {
     RawChunk<V, E> d[VPL];
     RawChunk<T, E> x[VPL];
+    RawChunk<T, E> extra[FUSE ? VPL : 1];
     float mu, rs;
   };
   const int64_t rstride = (int64_t)gridDim.x * rpb;
@@ -395,6 +477,12 @@ __global__ __launch_bounds__(1024) void norm_bwd_reg_kernel(
       } else {
         f.d[k].zero();
         f.x[k].zero();
+      }
+      if constexpr (FUSE) {
+        if (fextra != nullptr && (EVEN || c < nchunks))
+          f.extra[k].load(fextra + frow * n2 + (int64_t)c * E);
+        else
+          f.extra[k].zero();
       }
     }
     f.mu = RMS ? 0.f : mean[frow];
@@ -420,6 +508,11 @@ __global__ __launch_bounds__(1024) void norm_bwd_reg_kernel(
         for (int e = 0; e < E; ++e) d[k][e] = 0.f;
     }
     const float mu = f.mu, rs = f.rs;
+    float extra[FUSE ? VPL : 1][E];
+    if constexpr (FUSE) {
+#pragma unroll
+      for (int k = 0; k < VPL; ++k) f.extra[k].unpack(extra[k]);
+    }
     fetch(f, base + PF * rstride);
     float s1 = 0.f, s2 = 0.f;
 #pragma unroll
@@ -460,7 +553,24 @@ __global__ __launch_bounds__(1024) void norm_bwd_reg_kernel(
 #pragma unroll
           for (int e = 0; e < E; ++e)
             o[e] = fmaf(-c2, xh[k][e], fmaf(rs, d[k][e], -b1));
+          if constexpr (FUSE) {
+#pragma unroll
+            for (int e = 0; e < E; ++e) o[e] += extra[k][e];
+          }
           store_chunk<T, E>(dxr + (int64_t)c * E, o);
+          if constexpr (FUSE) {
+            // gradient of x of the prologue, from the unrounded gradient of h
+            if (fe.drop) {
+              const uint32_t keep = chunk_keep_bits<E>(row, n2, c, fe.d);
+#pragma unroll
+              for (int e = 0; e < E; ++e)
+                o[e] = (keep >> e) & 1u ? o[e] * fe.d.scale : 0.f;
+            }
+            if (fdrop != nullptr)
+              store_chunk<T, E>(fdrop + row * n2 + (int64_t)c * E, o);
+#pragma unroll
+            for (int e = 0; e < E; ++e) acc_d[k][e] += io<T>::round(o[e]);
+          }
         }
       }
     }
@@ -485,9 +595,13 @@ __global__ __launch_bounds__(1024) void norm_bwd_reg_kernel(
   if (part == nullptr) return;  // uniform: no parameter gradients wanted
 
   // Fold the row slots of this workgroup into slot 0, one slot at a time.
+  // Arrays: 0 = dgamma, then dbeta (LayerNorm only), then the bias gradient of
+  // the fused epilogue (last, when wanted).
   constexpr int NARR = RMS ? 1 : 2;
-#pragma unroll
-  for (int a = 0; a < NARR; ++a) {
+  const int64_t P = gridDim.x;
+  // (a lambda over one accumulator array at a time keeps the arrays in
+  // registers: none of them is indexed by a run-time value)
+  auto fold_and_store = [&](auto &acc, int a) {
     for (int s = 1; s < rpb; ++s) {
       __syncthreads();
       if (rslot == s) {
@@ -496,8 +610,7 @@ __global__ __launch_bounds__(1024) void norm_bwd_reg_kernel(
           const int c = c0 + k * cstride;
           if (c < nchunks) {
 #pragma unroll
-            for (int e = 0; e < E; ++e)
-              xslot[c * E + e] = a == 0 ? acc_g[k][e] : acc_b[k][e];
+            for (int e = 0; e < E; ++e) xslot[c * E + e] = acc[k][e];
           }
         }
       }
@@ -508,30 +621,24 @@ __global__ __launch_bounds__(1024) void norm_bwd_reg_kernel(
           const int c = c0 + k * cstride;
           if (c < nchunks) {
 #pragma unroll
-            for (int e = 0; e < E; ++e) {
-              if (a == 0)
-                acc_g[k][e] += xslot[c * E + e];
-              else
-                acc_b[k][e] += xslot[c * E + e];
-            }
+            for (int e = 0; e < E; ++e) acc[k][e] += xslot[c * E + e];
           }
         }
       }
     }
-  }
-  if (rslot == 0) {
-    const int64_t P = gridDim.x;
-#pragma unroll
-    for (int a = 0; a < NARR; ++a) {
+    if (rslot == 0) {
       float *prow = part + ((int64_t)a * P + blockIdx.x) * n2;
 #pragma unroll
       for (int k = 0; k < VPL; ++k) {
         const int c = c0 + k * cstride;
-        if (c < nchunks)
-          store_chunk<float, E>(prow + (int64_t)c * E,
-                                a == 0 ? acc_g[k] : acc_b[k]);
+        if (c < nchunks) store_chunk<float, E>(prow + (int64_t)c * E, acc[k]);
       }
     }
+  };
+  fold_and_store(acc_g, 0);
+  if constexpr (!RMS) fold_and_store(acc_b, 1);
+  if constexpr (FUSE) {
+    if (fe.want_dbias) fold_and_store(acc_d, NARR);
   }
 }
 
@@ -543,7 +650,12 @@ template <typename T, typename V, bool RMS>
 __global__ __launch_bounds__(256) void norm_bwd_dx_generic_kernel(
     const V *__restrict__ dy, const T *__restrict__ x,
     const float *__restrict__ mean, const float *__restrict__ invvar,
-    const V *__restrict__ gamma, T *__restrict__ dx, int64_t n1, int64_t n2) {
+    const V *__restrict__ gamma, T *__restrict__ dx, int64_t n1, int64_t n2,
+    FuseEpilogue fe) {
+  // fe: the fused epilogue (all-null for the plain backward): dh_extra is added
+  // before the single rounding, dx_drop receives the masked, scaled gradient
+  const T *extra = static_cast<const T *>(fe.dh_extra);
+  T *dx_drop = static_cast<T *>(fe.dx_drop);
   __shared__ float sh[2][4];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   for (int64_t row = blockIdx.x; row < n1; row += gridDim.x) {
@@ -579,7 +691,13 @@ __global__ __launch_bounds__(256) void norm_bwd_dx_generic_kernel(
       float f = fn * io<V>::from_scalar(dyr[i]) * g;
       f -= s1;
       f -= h * s2;
-      dxr[i] = io<T>::to_scalar(f * term);
+      float o = f * term;
+      if (extra != nullptr) o += io<T>::from_scalar(extra[row * n2 + i]);
+      dxr[i] = io<T>::to_scalar(o);
+      if (dx_drop != nullptr) {
+        if (fe.drop) o = keep_element(row * n2 + i, fe.d) ? o * fe.d.scale : 0.f;
+        dx_drop[row * n2 + i] = io<T>::to_scalar(o);
+      }
     }
   }
 }
@@ -645,13 +763,22 @@ int64_t colsum_parts_norm(int64_t n1, int64_t n2) {
   return p;
 }
 
+constexpr int kNotFused = 1;  // launch_norm_fwd: shape needs the composed path
+
+// fp != nullptr selects the fused prologue (T == V); shapes outside the
+// register path then return kNotFused without launching anything.
 template <typename T, typename V, bool RMS>
 static int launch_norm_fwd(const void *x, const void *gamma, const void *beta,
                            void *y, float *mean, float *invvar, int64_t n1,
-                           int64_t n2, float eps, hipStream_t st) {
+                           int64_t n2, float eps, hipStream_t st,
+                           const FusePrologue *fp = nullptr) {
   constexpr int E = chunk_elems<T, V>::value;
+  constexpr bool kCanFuse = sizeof(T) == sizeof(V);
+  const bool fused = fp != nullptr;
   const bool vec_ok = n2 % E == 0 && aligned16(x) && aligned16(y) &&
                       aligned16(gamma) && aligned16(beta) &&
+                      (!fused || (aligned16(fp->bias) && aligned16(fp->residual) &&
+                                  aligned16(fp->h_out))) &&
                       n2 <= (int64_t)kWave * 16 * 8 * E;
   static const int kVpl[] = {1, 2, 4, 8};
   RowSplit sp{0, 1, 1, false};
@@ -668,6 +795,26 @@ static int launch_norm_fwd(const void *x, const void *gamma, const void *beta,
     if (sp.ok && sp.wpr * sp.rpb > 4 && sp.vpl * E > 32)
       sp = split_row(n2 / E, 32 / E, kVpl, 4, waves);
   }
+  // The fused build holds two more packed operands per chunk: at most 16
+  // elements per lane.  Measured on MI355X: 16 per lane while a row then fits
+  // four waves, else 8 per lane over up to sixteen waves, else 16 per lane.
+  bool fused_big = false;
+  if (fused && vec_ok) {
+    const int waves = g_tune.norm_fwd_waves > 0 ? g_tune.norm_fwd_waves : 4;
+    if (g_tune.norm_fwd_vpl > 0) {
+      const int cap = g_tune.norm_fwd_vpl < 16 / E ? g_tune.norm_fwd_vpl : 16 / E;
+      sp = split_row(n2 / E, cap, kVpl, 4, waves);
+    } else {
+      sp = split_row(n2 / E, 16 / E, kVpl, 4, waves);
+      if (!sp.ok || sp.wpr > 4) {
+        const RowSplit narrow = split_row(n2 / E, 8 / E, kVpl, 4, waves);
+        if (narrow.ok) sp = narrow;
+      }
+    }
+    if (sp.ok && sp.vpl * E > 16) sp.ok = false;
+    fused_big = sp.ok && sp.wpr * sp.rpb > 4;
+  }
+  if (fused && !sp.ok) return kNotFused;
   if (!sp.ok) {
     int64_t grid = n1 < 65535 * 16 ? n1 : 65535 * 16;
     norm_fwd_generic_kernel<T, V, RMS><<<dim3((unsigned)grid), 256, 0, st>>>(
@@ -686,29 +833,61 @@ static int launch_norm_fwd(const void *x, const void *gamma, const void *beta,
   int64_t grid = ceil_div(ceil_div(n1, sp.rpb), iters);
   const int64_t maxgrid = (int64_t)device_cu_count() * 64;
   if (grid > maxgrid) grid = maxgrid;
+  if constexpr (kCanFuse) {
+    if (fused) {
+#define OSLO_FWD_FUSED_L(VPL, EVEN_, MAXT_)                                 \
+  norm_fwd_reg_kernel<T, V, VPL, RMS, EVEN_, MAXT_, true>                   \
+      <<<dim3((unsigned)grid), threads, 0, st>>>(                           \
+          (const T *)x, (const V *)gamma, (const V *)beta, (V *)y, mean,    \
+          invvar, n1, (int)n2, eps, sp.wpr, sp.rpb, iters, *fp)
+#define OSLO_FWD_FUSED(VPL)                                                 \
+  case VPL:                                                                 \
+    if constexpr (VPL * E <= 16) {                                          \
+      if (!fused_big) {                                                     \
+        if (even) OSLO_FWD_FUSED_L(VPL, true, 256);                         \
+        else OSLO_FWD_FUSED_L(VPL, false, 256);                             \
+      } else {                                                              \
+        if (even) OSLO_FWD_FUSED_L(VPL, true, 1024);                        \
+        else OSLO_FWD_FUSED_L(VPL, false, 1024);                            \
+      }                                                                     \
+      break;                                                                \
+    }                                                                       \
+    return fail(OSLO_ERR_UNSUPPORTED, "fused norm fwd: no kernel for vpl=%d", VPL);
+      switch (sp.vpl) {
+        OSLO_FWD_FUSED(1)
+        OSLO_FWD_FUSED(2)
+        OSLO_FWD_FUSED(4)
+        default:
+          return fail(OSLO_ERR_UNSUPPORTED, "fused norm fwd: no kernel for vpl=%d", sp.vpl);
+      }
+#undef OSLO_FWD_FUSED
+#undef OSLO_FWD_FUSED_L
+      return check_launch("norm_fwd_reg_kernel (fused)");
+    }
+  }
 #define OSLO_FWD_CASE(VPL)                                                  \
   case VPL:                                                                 \
     if (threads <= 256 && even)                                             \
       norm_fwd_reg_kernel<T, V, VPL, RMS, true, 256>                        \
           <<<dim3((unsigned)grid), threads, 0, st>>>(                       \
               (const T *)x, (const V *)gamma, (const V *)beta, (V *)y,      \
-              mean, invvar, n1, (int)n2, eps, sp.wpr, sp.rpb, iters);             \
+              mean, invvar, n1, (int)n2, eps, sp.wpr, sp.rpb, iters, FusePrologue{});             \
     else if (threads <= 256)                                                \
       norm_fwd_reg_kernel<T, V, VPL, RMS, false, 256>                       \
           <<<dim3((unsigned)grid), threads, 0, st>>>(                       \
               (const T *)x, (const V *)gamma, (const V *)beta, (V *)y,      \
-              mean, invvar, n1, (int)n2, eps, sp.wpr, sp.rpb, iters);             \
+              mean, invvar, n1, (int)n2, eps, sp.wpr, sp.rpb, iters, FusePrologue{});             \
     else if constexpr (VPL * E <= 32) {                                     \
       if (even)                                                             \
         norm_fwd_reg_kernel<T, V, VPL, RMS, true, 1024>                     \
             <<<dim3((unsigned)grid), threads, 0, st>>>(                     \
                 (const T *)x, (const V *)gamma, (const V *)beta, (V *)y,    \
-                mean, invvar, n1, (int)n2, eps, sp.wpr, sp.rpb, iters);           \
+                mean, invvar, n1, (int)n2, eps, sp.wpr, sp.rpb, iters, FusePrologue{});           \
       else                                                                  \
         norm_fwd_reg_kernel<T, V, VPL, RMS, false, 1024>                    \
             <<<dim3((unsigned)grid), threads, 0, st>>>(                     \
                 (const T *)x, (const V *)gamma, (const V *)beta, (V *)y,    \
-                mean, invvar, n1, (int)n2, eps, sp.wpr, sp.rpb, iters);           \
+                mean, invvar, n1, (int)n2, eps, sp.wpr, sp.rpb, iters, FusePrologue{});           \
     }                                                                       \
     else                                                                    \
       return fail(OSLO_ERR_UNSUPPORTED,                                     \
@@ -727,17 +906,34 @@ static int launch_norm_fwd(const void *x, const void *gamma, const void *beta,
   return check_launch("norm_fwd_reg_kernel");
 }
 
+// Column sums of a stored [rows, cols] tensor, one thread per column.
+template <typename T>
+__global__ __launch_bounds__(256) void norm_colsum_generic_kernel(
+    const T *__restrict__ a, T *__restrict__ out, int64_t rows, int64_t cols) {
+  const int64_t col = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (col >= cols) return;
+  float s = 0.f;
+  for (int64_t r = 0; r < rows; ++r) s += io<T>::from_scalar(a[r * cols + col]);
+  out[col] = io<T>::to_scalar(s);
+}
+
+// fe != nullptr selects the fused epilogue (T == V); dbias is then the bias
+// gradient (may be null).
 template <typename T, typename V, bool RMS>
 static int launch_norm_bwd(const void *dy, const void *x, const float *mean,
                            const float *invvar, const void *gamma, void *dx,
                            void *dgamma, void *dbeta, void *ws,
                            int64_t ws_bytes, int64_t n1, int64_t n2,
-                           hipStream_t st) {
+                           hipStream_t st, const FuseEpilogue *fe = nullptr,
+                           void *dbias = nullptr) {
   constexpr int E = chunk_elems<T, V>::value;
   constexpr int NARR = RMS ? 1 : 2;
-  const bool want_params = dgamma != nullptr;
+  constexpr bool kCanFuse = sizeof(T) == sizeof(V);
+  const bool fused = fe != nullptr;
+  const bool want_params = dgamma != nullptr || (fused && dbias != nullptr);
   const bool vec_ok = n2 % E == 0 && aligned16(dy) && aligned16(x) &&
                       aligned16(dx) && aligned16(gamma) && aligned16(ws) &&
+                      (!fused || (aligned16(fe->dh_extra) && aligned16(fe->dx_drop))) &&
                       n2 <= (int64_t)kWave * 16 * (16 / E) * E;
   // at most 16 elements per lane: 5 register arrays of that size stay
   // below the 128-VGPR budget of a 1024-thread workgroup
@@ -766,9 +962,25 @@ static int launch_norm_bwd(const void *dy, const void *x, const float *mean,
     int64_t grid = n1 < 65535 * 16 ? n1 : 65535 * 16;
     norm_bwd_dx_generic_kernel<T, V, RMS><<<dim3((unsigned)grid), 256, 0, st>>>(
         (const V *)dy, (const T *)x, mean, invvar, (const V *)gamma, (T *)dx,
-        n1, n2);
+        n1, n2, fused ? *fe : FuseEpilogue{});
     int rc = check_launch("norm_bwd_dx_generic_kernel");
-    if (rc != OSLO_OK || !want_params) return rc;
+    if (rc != OSLO_OK) return rc;
+    if constexpr (kCanFuse) {
+      if (fused) {
+        if (dbias != nullptr) {
+          const void *src = fe->dx_drop != nullptr ? fe->dx_drop : dx;
+          if (fe->drop && fe->dx_drop == nullptr)
+            return fail(OSLO_ERR_INVALID_ARGUMENT,
+                        "fused norm bwd: dbias with dropout needs dx_drop");
+          norm_colsum_generic_kernel<T>
+              <<<dim3((unsigned)ceil_div(n2, 256)), 256, 0, st>>>(
+                  (const T *)src, (T *)dbias, n1, n2);
+          rc = check_launch("norm_colsum_generic_kernel");
+          if (rc != OSLO_OK) return rc;
+        }
+      }
+    }
+    if (dgamma == nullptr) return rc;
     norm_bwd_param_generic_kernel<T, V, RMS>
         <<<dim3((unsigned)ceil_div(n2, 256)), 256, 0, st>>>(
             (const V *)dy, (const T *)x, mean, invvar, (V *)dgamma,
@@ -778,8 +990,14 @@ static int launch_norm_bwd(const void *dy, const void *x, const float *mean,
   int64_t P = colsum_parts_norm(n1, n2);
   if (P > ceil_div(n1, sp.rpb)) P = ceil_div(n1, sp.rpb);
   float *part = nullptr;
+  FuseEpilogue fev{};
+  if (fused) {
+    fev = *fe;
+    fev.want_dbias = dbias != nullptr ? 1 : 0;
+  }
+  const int narr = NARR + (fev.want_dbias ? 1 : 0);
   if (want_params) {
-    const int64_t need = (int64_t)NARR * P * n2 * (int64_t)sizeof(float);
+    const int64_t need = (int64_t)narr * P * n2 * (int64_t)sizeof(float);
     if (ws == nullptr || ws_bytes < need)
       return fail(OSLO_ERR_WORKSPACE,
                   "norm bwd: workspace of %lld bytes needed, %lld given",
@@ -794,10 +1012,22 @@ static int launch_norm_bwd(const void *dy, const void *x, const float *mean,
   int pf = sp.vpl * E <= 8 ? 2 : 1;
   if (g_tune.norm_bwd_prefetch > 0) pf = g_tune.norm_bwd_prefetch >= 2 ? 2 : 1;
 #define OSLO_BWD_LAUNCH(VPL, EVEN_, PF_)                                   \
-  norm_bwd_reg_kernel<T, V, VPL, RMS, EVEN_, PF_>                          \
-      <<<dim3((unsigned)P), threads, lds, st>>>(                           \
-          (const V *)dy, (const T *)x, mean, invvar, (const V *)gamma,     \
-          (T *)dx, part, n1, (int)n2, sp.wpr, sp.rpb)
+  do {                                                                     \
+    if constexpr (kCanFuse) {                                              \
+      if (fused) {                                                         \
+        norm_bwd_reg_kernel<T, V, VPL, RMS, EVEN_, PF_, true>              \
+            <<<dim3((unsigned)P), threads, lds, st>>>(                     \
+                (const V *)dy, (const T *)x, mean, invvar,                 \
+                (const V *)gamma, (T *)dx, part, n1, (int)n2, sp.wpr,      \
+                sp.rpb, fev);                                              \
+        break;                                                             \
+      }                                                                    \
+    }                                                                      \
+    norm_bwd_reg_kernel<T, V, VPL, RMS, EVEN_, PF_, false>                 \
+        <<<dim3((unsigned)P), threads, lds, st>>>(                         \
+            (const V *)dy, (const T *)x, mean, invvar, (const V *)gamma,   \
+            (T *)dx, part, n1, (int)n2, sp.wpr, sp.rpb, fev);              \
+  } while (0)
 #define OSLO_BWD_CASE(VPL)                                                 \
   case VPL:                                                                \
     if constexpr (VPL * E <= 16) {                                         \
@@ -822,8 +1052,12 @@ static int launch_norm_bwd(const void *dy, const void *x, const float *mean,
 #undef OSLO_BWD_CASE
   int rc = check_launch("norm_bwd_reg_kernel");
   if (rc != OSLO_OK || !want_params) return rc;
-  return launch_colsum_finalize<V>(part, P, n2, dgamma, RMS ? nullptr : dbeta,
-                                   st);
+  // arrays of partial rows: dgamma, dbeta (LayerNorm), bias gradient (fused)
+  void *outs[3] = {dgamma, nullptr, nullptr};
+  int na = 1;
+  if (!RMS) outs[na++] = dbeta;
+  if (fev.want_dbias) outs[na++] = dbias;
+  return launch_colsum_finalize<V>(part, P, n2, outs[0], outs[1], st, outs[2], na);
 }
 
 static int check_norm_dtypes(int din, int dout) {
@@ -942,6 +1176,102 @@ int oslo_rms_bwd(const void *dy, const void *x, const float *invvar,
   return oslo::norm_bwd_entry(true, dy, x, nullptr, invvar, gamma, dx, dgamma,
                               nullptr, workspace, workspace_bytes, n1, n2,
                               dtype_in, dtype_out, stream);
+}
+
+int oslo_bias_dropout_add_norm_fwd(const void *x, const void *bias,
+                                   const void *residual, const void *gamma,
+                                   const void *beta, void *h_out, void *y,
+                                   float *mean, float *invvar, int64_t n1,
+                                   int64_t n2, double eps, float p,
+                                   uint64_t seed, uint64_t offset, int rms,
+                                   int dtype, void *stream) {
+  using namespace oslo;
+  int rc = check_norm_dtypes(dtype, dtype);
+  if (rc != OSLO_OK) return rc;
+  OSLO_REQUIRE(n1 >= 0 && n2 >= 1 && n2 <= 0x7fffffff,
+               "fused norm fwd: bad shape [%lld, %lld]", (long long)n1,
+               (long long)n2);
+  OSLO_REQUIRE(p >= 0.f && p <= 1.f, "fused norm fwd: p = %g outside [0, 1]",
+               (double)p);
+  if (n1 == 0) return OSLO_OK;
+  OSLO_REQUIRE(x && y && invvar, "fused norm fwd: null tensor pointer");
+  OSLO_REQUIRE(rms || mean, "fused layer norm fwd: null mean pointer");
+  OSLO_REQUIRE(rms || (gamma == nullptr) == (beta == nullptr),
+               "fused layer norm fwd: gamma and beta must both be given or "
+               "both be NULL");
+  hipStream_t st = (hipStream_t)stream;
+  FusePrologue fp{bias, residual, h_out, make_drop(p, seed, offset),
+                  p > 0.f ? 1 : 0};
+  if (rms) beta = nullptr;
+#define OSLO_FUSED_FWD(T_)                                                    \
+  (rms ? launch_norm_fwd<T_, T_, true>(x, gamma, nullptr, y, nullptr, invvar, \
+                                       n1, n2, (float)eps, st, &fp)           \
+       : launch_norm_fwd<T_, T_, false>(x, gamma, beta, y, mean, invvar, n1,  \
+                                        n2, (float)eps, st, &fp))
+  rc = dtype == OSLO_DTYPE_F32   ? OSLO_FUSED_FWD(float)
+       : dtype == OSLO_DTYPE_F16 ? OSLO_FUSED_FWD(_Float16)
+                                 : OSLO_FUSED_FWD(__bf16);
+#undef OSLO_FUSED_FWD
+  if (rc != kNotFused) return rc;
+  // Rows outside the register path: the same arithmetic as two launches, h
+  // staged in h_out (or in y, which the norm then overwrites in place).
+  void *buf = h_out != nullptr ? h_out : y;
+  rc = oslo_bias_dropout_add_fwd(x, bias, residual, buf, nullptr, n1, n2, p,
+                                 seed, offset, dtype, stream);
+  if (rc != OSLO_OK) return rc;
+  return norm_fwd_entry(rms != 0, buf, gamma, beta, y, mean, invvar, n1, n2,
+                        eps, dtype, dtype, stream);
+}
+
+int oslo_bias_dropout_add_norm_bwd(const void *dy, const void *dh_extra,
+                                   const void *h, const float *mean,
+                                   const float *invvar, const void *gamma,
+                                   void *dres, void *dx, void *dgamma,
+                                   void *dbeta, void *dbias, void *workspace,
+                                   int64_t workspace_bytes, int64_t n1,
+                                   int64_t n2, float p, uint64_t seed,
+                                   uint64_t offset, int rms, int dtype,
+                                   void *stream) {
+  using namespace oslo;
+  int rc = check_norm_dtypes(dtype, dtype);
+  if (rc != OSLO_OK) return rc;
+  OSLO_REQUIRE(n1 >= 0 && n2 >= 1 && n2 <= 0x7fffffff,
+               "fused norm bwd: bad shape [%lld, %lld]", (long long)n1,
+               (long long)n2);
+  OSLO_REQUIRE(p >= 0.f && p <= 1.f, "fused norm bwd: p = %g outside [0, 1]",
+               (double)p);
+  OSLO_REQUIRE(gamma != nullptr || dgamma == nullptr,
+               "fused norm bwd: dgamma requested without gamma");
+  OSLO_REQUIRE(rms || (dgamma == nullptr) == (dbeta == nullptr),
+               "fused layer norm bwd: dgamma and dbeta must both be given or "
+               "both be NULL");
+  OSLO_REQUIRE(p == 0.f || dx != nullptr,
+               "fused norm bwd: with dropout the gradient of x needs its own "
+               "tensor (dx)");
+  hipStream_t st = (hipStream_t)stream;
+  if (n1 == 0) {
+    const size_t nb = (size_t)n2 * dtype_size(dtype);
+    if (dgamma) (void)hipMemsetAsync(dgamma, 0, nb, st);
+    if (dbeta && !rms) (void)hipMemsetAsync(dbeta, 0, nb, st);
+    if (dbias) (void)hipMemsetAsync(dbias, 0, nb, st);
+    return OSLO_OK;
+  }
+  OSLO_REQUIRE(dy && h && invvar && dres, "fused norm bwd: null tensor pointer");
+  OSLO_REQUIRE(rms || mean, "fused layer norm bwd: null mean pointer");
+  FuseEpilogue fe{dh_extra, dx, make_drop(p, seed, offset), p > 0.f ? 1 : 0, 0};
+#define OSLO_FUSED_BWD(T_)                                                     \
+  (rms ? launch_norm_bwd<T_, T_, true>(dy, h, nullptr, invvar, gamma, dres,    \
+                                       dgamma, nullptr, workspace,             \
+                                       workspace_bytes, n1, n2, st, &fe,       \
+                                       dbias)                                  \
+       : launch_norm_bwd<T_, T_, false>(dy, h, mean, invvar, gamma, dres,      \
+                                        dgamma, dbeta, workspace,              \
+                                        workspace_bytes, n1, n2, st, &fe,      \
+                                        dbias))
+  return dtype == OSLO_DTYPE_F32   ? OSLO_FUSED_BWD(float)
+         : dtype == OSLO_DTYPE_F16 ? OSLO_FUSED_BWD(_Float16)
+                                   : OSLO_FUSED_BWD(__bf16);
+#undef OSLO_FUSED_BWD
 }
 
 }  // extern "C"

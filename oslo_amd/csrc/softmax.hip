@@ -108,18 +108,6 @@ __device__ __forceinline__ void row_setup(const SoftmaxGeom &g, int64_t r,
   }
 }
 
-// Keep bits of the E elements of chunk c of `row` (dropout on the flattened
-// [rows, sk] tensor: element i belongs to group i >> 3).  A 4-element chunk
-// takes the low or the high half of its group's eight bits.
-template <int E>
-__device__ __forceinline__ uint32_t chunk_keep_bits(int64_t row, int sk, int c,
-                                                    const DropArgs &d) {
-  const uint64_t flat = (uint64_t)row * (uint64_t)sk + (uint64_t)c * E;
-  uint32_t keep = dropout_keep_bits(flat >> 3, d.seed, d.offset, d.threshold);
-  if constexpr (E == 4) keep >>= (uint32_t)(flat & 4u);
-  return keep;
-}
-
 // DROP: dropout is applied to the probabilities before they are written
 // (oslo/transformers/models/gpt2/modeling_gpt2.py:138-142,
 // oslo/transformers/models/bert/modeling_bert.py:306-310) and the row

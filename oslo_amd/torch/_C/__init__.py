@@ -29,6 +29,7 @@ OSLO_OP_LN_BWD = 1
 OSLO_OP_RMS_BWD = 2
 OSLO_OP_BIAS_GELU_BWD = 3
 OSLO_OP_BIAS_DROPOUT_ADD_BWD = 4
+OSLO_OP_BIAS_DROPOUT_ADD_NORM_BWD = 5
 
 ABI_VERSION = 1
 
@@ -98,6 +99,16 @@ _SIGNATURES = {
     "oslo_bias_dropout_add_bwd": (
         _int,
         [_p, _p, _p, _p, _i64, _i64, _i64, _f32, _u64, _u64, _int, _p],
+    ),
+    "oslo_bias_dropout_add_norm_fwd": (
+        _int,
+        [_p, _p, _p, _p, _p, _p, _p, _p, _p, _i64, _i64, _f64, _f32, _u64, _u64, _int,
+         _int, _p],
+    ),
+    "oslo_bias_dropout_add_norm_bwd": (
+        _int,
+        [_p, _p, _p, _p, _p, _p, _p, _p, _p, _p, _p, _p, _i64, _i64, _i64, _f32, _u64,
+         _u64, _int, _int, _p],
     ),
     "oslo_philox_mask": (_int, [_p, _i64, _f32, _u64, _u64, _p]),
     "oslo_philox_words": (_int, [_p, _i64, _i64, _u64, _u64, _p]),
@@ -361,6 +372,93 @@ class _LayerNormKernel:
             True, dout, None, invvar, input, normalized_shape, gamma, None
         )
         return [gi, gg]
+
+    # -- bias-dropout-add fused into the norm (no counterpart in the
+    #    reference's module: its models chain FusedBiasDropout, the residual
+    #    add and LayerNorm, oslo/transformers/models/bert/modeling_bert.py:
+    #    343-346) ----------------------------------------------------------
+    def bias_dropout_add_norm_forward(
+        self, rms, input, bias, residual, normalized_shape, gamma, beta, eps,
+        p, seed, offset, want_h=True,
+    ):
+        """``h = dropout(input + bias, p) + residual; y = norm(h)``.
+
+        Returns ``[y, h, mean, invvar]`` (``h`` None when ``want_h`` is false,
+        ``mean`` None for RMSNorm).  One dtype throughout.
+        """
+        lib = self._lib
+        _check_input(input, "input")
+        n1, n2 = _compute_n1_n2(input, normalized_shape)
+        for name, t in (("gamma", gamma), ("beta", beta), ("bias", bias)):
+            if t is not None:
+                _check_input(t, name)
+                _check_param(t, normalized_shape, name)
+        if residual is not None:
+            _check_input(residual, "residual")
+            if residual.shape != input.shape:
+                raise RuntimeError("residual and input differ in shape")
+        for name, t in (("gamma", gamma), ("beta", beta), ("bias", bias), ("residual", residual)):
+            if t is not None and t.dtype != input.dtype:
+                raise RuntimeError(
+                    "%s has dtype %s but input has dtype %s" % (name, t.dtype, input.dtype)
+                )
+        code = _dtype_code(input, "input")
+        y = torch.empty_like(input)
+        h = torch.empty_like(input) if want_h else None
+        invvar = torch.empty(n1, dtype=torch.float32, device=input.device)
+        mean = None if rms else torch.empty(n1, dtype=torch.float32, device=input.device)
+        with torch.cuda.device_of(input):
+            rc = lib.oslo_bias_dropout_add_norm_fwd(
+                _ptr(input), _ptr(bias), _ptr(residual), _ptr(gamma), _ptr(beta), _ptr(h),
+                _ptr(y), _ptr(mean), _ptr(invvar), n1, n2, float(eps), float(p),
+                int(seed), int(offset), 1 if rms else 0, code, _stream(input),
+            )
+            _check(rc, lib)
+        return [y, h, mean, invvar]
+
+    def bias_dropout_add_norm_backward(
+        self, rms, dout, dh_extra, h, mean, invvar, normalized_shape, gamma,
+        p, seed, offset, need_bias_grad=True,
+    ):
+        """Returns ``(grad_residual, grad_input, grad_gamma, grad_beta, grad_bias)``;
+        ``grad_input`` is ``grad_residual`` itself when ``p == 0``."""
+        lib = self._lib
+        for name, t in (("dout", dout), ("h", h), ("invvar", invvar)):
+            _check_input(t, name)
+        n1, n2 = _compute_n1_n2(h, normalized_shape)
+        if dout.shape != h.shape or dout.dtype != h.dtype:
+            raise RuntimeError("dout and h differ in shape or dtype")
+        if dh_extra is not None:
+            _check_input(dh_extra, "dh_extra")
+            if dh_extra.shape != h.shape or dh_extra.dtype != h.dtype:
+                raise RuntimeError("dh_extra and h differ in shape or dtype")
+        code = _dtype_code(h, "h")
+        grad_res = torch.empty_like(h)
+        grad_in = torch.empty_like(h) if p > 0.0 else None
+        grad_gamma = grad_beta = grad_bias = None
+        if gamma is not None:
+            _check_input(gamma, "gamma")
+            grad_gamma = torch.empty_like(gamma)
+            if not rms:
+                grad_beta = torch.empty_like(gamma)
+        if need_bias_grad:
+            grad_bias = torch.empty(n2, dtype=h.dtype, device=h.device)
+        ws, ws_bytes = None, 0
+        if gamma is not None or need_bias_grad:
+            ws, ws_bytes = _workspace(lib, OSLO_OP_BIAS_DROPOUT_ADD_NORM_BWD, n1, n2, h.device)
+        with torch.cuda.device_of(h):
+            rc = lib.oslo_bias_dropout_add_norm_bwd(
+                _ptr(dout), _ptr(dh_extra), _ptr(h), _ptr(mean), _ptr(invvar), _ptr(gamma),
+                _ptr(grad_res), _ptr(grad_in), _ptr(grad_gamma), _ptr(grad_beta),
+                _ptr(grad_bias), _ptr(ws), ws_bytes, n1, n2, float(p), int(seed),
+                int(offset), 1 if rms else 0, code, _stream(h),
+            )
+            _check(rc, lib)
+        if grad_in is None:
+            grad_in = grad_res
+        if grad_bias is not None:
+            grad_bias = grad_bias.view(tuple(int(s) for s in normalized_shape))
+        return grad_res, grad_in, grad_gamma, grad_beta, grad_bias
 
 
 # ---------------------------------------------------------------------------

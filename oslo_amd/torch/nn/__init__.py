@@ -6,6 +6,8 @@ from oslo_amd.torch.nn.modules.dropout import FusedBiasDropout
 from oslo_amd.torch.nn.modules.functional import (
     fused_bias_dropout,
     fused_bias_dropout_add,
+    fused_bias_dropout_add_layer_norm,
+    fused_bias_dropout_add_rms_norm,
     fused_bias_gelu,
     fused_gelu,
     fused_layer_norm,
@@ -26,6 +28,10 @@ from oslo_amd.torch.nn.modules.layer_norm import (
     MixedFusedRMSNorm,
 )
 from oslo_amd.torch.nn.modules.linear import Linear
+from oslo_amd.torch.nn.modules.residual_norm import (
+    FusedBiasDropoutAddLayerNorm,
+    FusedBiasDropoutAddRMSNorm,
+)
 from oslo_amd.torch.nn.modules.softmax import (
     AttnMaskType,
     FusedScaleMaskSoftmax,
@@ -36,6 +42,8 @@ __all__ = [
     "AttnMaskType",
     "Conv1D",
     "FusedBiasDropout",
+    "FusedBiasDropoutAddLayerNorm",
+    "FusedBiasDropoutAddRMSNorm",
     "FusedLayerNorm",
     "FusedRMSNorm",
     "FusedScaleMaskSoftmax",
@@ -45,6 +53,8 @@ __all__ = [
     "attention_mask_func",
     "fused_bias_dropout",
     "fused_bias_dropout_add",
+    "fused_bias_dropout_add_layer_norm",
+    "fused_bias_dropout_add_rms_norm",
     "fused_bias_gelu",
     "fused_gelu",
     "fused_layer_norm",

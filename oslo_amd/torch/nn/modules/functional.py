@@ -267,6 +267,69 @@ class _FusedRMSNormFunction(torch.autograd.Function):
         return _norm_backward(ctx, grad_output)[0], None, None
 
 
+class _FusedBiasDropoutAddNormFunction(torch.autograd.Function):
+    """
+    Kernel fusion function: Bias + Dropout + residual add + LayerNorm / RMSNorm
+
+    ``h = dropout(input + bias) + residual; y = norm(h) * weight + norm_bias`` --
+    the chain of oslo/transformers/models/bert/modeling_bert.py:343-346 in one
+    pass.  Returns ``(y, h)``; a gradient arriving at ``h`` (a pre-LN block
+    keeps it as the next residual) is added to the norm's input gradient inside
+    the backward kernel.
+    """
+
+    @staticmethod
+    def forward(ctx, input, bias, residual, weight, norm_bias, normalized_shape, eps,
+                p, seed, offset, rms):
+        kernel = get_layernorm_kernel()
+        y, h, mean, invvar = kernel.bias_dropout_add_norm_forward(
+            rms,
+            input.contiguous(),
+            None if bias is None else bias.contiguous(),
+            None if residual is None else residual.contiguous(),
+            normalized_shape,
+            None if weight is None else weight.contiguous(),
+            None if norm_bias is None else norm_bias.contiguous(),
+            eps, p, seed, offset,
+        )
+        ctx.rms, ctx.p, ctx.seed, ctx.offset = rms, p, seed, offset
+        ctx.normalized_shape = normalized_shape
+        ctx.has = (bias is not None, residual is not None, weight is not None,
+                   norm_bias is not None)
+        saved = [h, invvar]
+        if not rms:
+            saved.append(mean)
+        if weight is not None:
+            saved.append(weight)
+        ctx.save_for_backward(*saved)
+        return y, h
+
+    @staticmethod
+    def backward(ctx, grad_y, grad_h):
+        saved = list(ctx.saved_tensors)
+        h, invvar = saved[0], saved[1]
+        mean = None if ctx.rms else saved[2]
+        has_bias, has_res, has_weight, has_nbias = ctx.has
+        weight = saved[-1] if has_weight else None
+        need_b = has_bias and ctx.needs_input_grad[1]
+        g_res, g_in, g_gamma, g_beta, g_bias = (
+            get_layernorm_kernel().bias_dropout_add_norm_backward(
+                ctx.rms, grad_y.contiguous(),
+                None if grad_h is None else grad_h.contiguous(),
+                h, mean, invvar, ctx.normalized_shape, weight,
+                ctx.p, ctx.seed, ctx.offset, need_bias_grad=need_b,
+            )
+        )
+        return (
+            g_in,
+            g_bias if need_b else None,
+            g_res if has_res else None,
+            g_gamma if has_weight else None,
+            g_beta if has_nbias else None,
+            None, None, None, None, None, None,
+        )
+
+
 class _ScaledUpperTriangMaskedSoftmax(torch.autograd.Function):
     """
     Fused: scale -> causal (upper-triangular) mask -> softmax, on
@@ -443,6 +506,58 @@ def fused_bias_dropout_add(x, bias, residual, p, training, inplace=False):
     return _FusedBiasDropoutAddFunction.apply(
         x, bias, residual, p_eff, seed, offset, bool(inplace)
     )
+
+
+def _bias_dropout_add_norm(rms, x, bias, residual, weight, norm_bias, normalized_shape,
+                           eps, p, training, return_sum):
+    _check_dropout_p(p)
+    normalized_shape = (
+        (int(normalized_shape),) if isinstance(normalized_shape, int)
+        else tuple(int(s) for s in normalized_shape)
+    )
+    if not x.is_cuda:
+        # the reference's CPU path: the unfused chain of torch ops
+        h = x if bias is None else x + bias
+        h = F.dropout(h, p=p, training=training)
+        if residual is not None:
+            h = h + residual
+        if rms:
+            from oslo_amd.torch.nn.modules.layer_norm import manual_rms_norm
+
+            y = manual_rms_norm(h, normalized_shape, weight, eps)
+        else:
+            y = F.layer_norm(h, normalized_shape, weight, norm_bias, eps)
+        return (y, h) if return_sum else y
+    p_eff = float(p) if training else 0.0
+    seed, offset = _next_philox_state(x.device) if p_eff > 0.0 else (0, 0)
+    args = _cast_if_autocast_enabled(x, bias, residual, weight, norm_bias)
+    with torch.amp.autocast("cuda", enabled=False):
+        y, h = _FusedBiasDropoutAddNormFunction.apply(
+            *args, normalized_shape, eps, p_eff, seed, offset, bool(rms)
+        )
+    return (y, h) if return_sum else y
+
+
+def fused_bias_dropout_add_layer_norm(x, bias, residual, weight, norm_bias,
+                                      normalized_shape, eps=1e-5, p=0.0, training=True,
+                                      return_sum=False):
+    """``LayerNorm(dropout(x + bias, p) + residual)`` in one kernel.
+
+    The post-LN chain of oslo/transformers/models/bert/modeling_bert.py:343-346
+    (FusedBiasDropout, residual add, nn.LayerNorm).  ``bias``, ``residual``,
+    ``weight`` / ``norm_bias`` may be None.  With ``return_sum`` the normalised
+    tensor comes with ``h = dropout(x + bias) + residual`` -- what a pre-LN block
+    (modeling_gpt2.py:369-393) carries on as its residual.
+    """
+    return _bias_dropout_add_norm(False, x, bias, residual, weight, norm_bias,
+                                  normalized_shape, eps, p, training, return_sum)
+
+
+def fused_bias_dropout_add_rms_norm(x, bias, residual, weight, normalized_shape,
+                                    eps=1e-5, p=0.0, training=True, return_sum=False):
+    """``RMSNorm(dropout(x + bias, p) + residual)`` in one kernel (see above)."""
+    return _bias_dropout_add_norm(True, x, bias, residual, weight, None,
+                                  normalized_shape, eps, p, training, return_sum)
 
 
 def scaled_upper_triang_masked_softmax(input, scale=1.0):

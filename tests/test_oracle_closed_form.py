@@ -321,3 +321,49 @@ def test_softmax_dropout_vs_autograd_of_the_unfused_chain():
     )
     # dropped positions still receive a gradient through the normaliser
     assert (dx[~keep & ~np.broadcast_to(hidden, keep.shape)] != 0).any()
+
+
+# ------------------------------------------- bias-dropout-add fused into a norm
+@pytest.mark.parametrize("rms", [False, True])
+def test_bias_dropout_add_norm_vs_autograd_of_the_unfused_chain(rms):
+    """norm(keep * (x + b) / (1 - p) + residual) with an explicit keep mask and a
+    second consumer of h (its gradient is dh_extra): forward and every gradient
+    of the oracle against torch autograd in float64."""
+    r = np.random.default_rng(5)
+    n1, n2, p, eps = 7, 24, 0.2, 1e-5
+    # the reference's RMS formula takes the variance in float32 even for float64 input
+    rt = 2e-6 if rms else 1e-9
+    x = torch.from_numpy(r.standard_normal((n1, n2))).requires_grad_(True)
+    b = torch.from_numpy(r.standard_normal(n2)).requires_grad_(True)
+    res = torch.from_numpy(r.standard_normal((n1, n2))).requires_grad_(True)
+    gam = torch.from_numpy(1 + 0.1 * r.standard_normal(n2)).requires_grad_(True)
+    bet = torch.from_numpy(0.1 * r.standard_normal(n2)).requires_grad_(True)
+    keep = r.random((n1, n2)) >= p
+    gy = torch.from_numpy(r.standard_normal((n1, n2)))
+    gh = torch.from_numpy(r.standard_normal((n1, n2)))
+    scale = float(np.float32(1.0) / (np.float32(1.0) - np.float32(p)))
+    h = (x + b) * torch.from_numpy(keep) * scale + res
+    if rms:
+        y = tp.rms_norm(h, gam, eps)
+    else:
+        y = torch.nn.functional.layer_norm(h, (n2,), gam, bet, eps)
+    (y * gy).sum().backward(retain_graph=True)
+    (h * gh).sum().backward()
+    oy, oh, om, oi = cf.bias_dropout_add_norm_fwd(
+        x.detach().numpy(), b.detach().numpy(), res.detach().numpy(), keep, p,
+        gam.detach().numpy(), bet.detach().numpy(), eps, rms)
+    assert np.allclose(oh, h.detach().numpy(), rtol=1e-13, atol=1e-300)
+    assert np.allclose(oy, y.detach().numpy(), rtol=rt * 1e-2 if not rms else rt, atol=1e-13)
+    dres, dx, dg, dbt, dbias = cf.bias_dropout_add_norm_bwd(
+        gy.numpy(), gh.numpy(), oh, om, oi, gam.detach().numpy(), keep, p, rms)
+    assert np.allclose(dres, res.grad.numpy(), rtol=rt, atol=1e-12 if not rms else 1e-6)
+    assert np.allclose(dx, x.grad.numpy(), rtol=rt, atol=1e-12 if not rms else 1e-6)
+    assert np.allclose(dbias, b.grad.numpy(), rtol=rt, atol=1e-12 if not rms else 1e-6)
+    assert np.allclose(dg, gam.grad.numpy(), rtol=rt, atol=1e-12 if not rms else 1e-6)
+    if not rms:
+        assert np.allclose(dbt, bet.grad.numpy(), rtol=rt, atol=1e-12 if not rms else 1e-6)
+    # without the second consumer the residual gradient is the plain norm backward
+    d0 = cf.bias_dropout_add_norm_bwd(gy.numpy(), None, oh, om, oi, gam.detach().numpy(), None, 0.0, rms)
+    plain = (cf.rms_norm_bwd(gy.numpy(), oh, oi, gam.detach().numpy())[0] if rms
+             else cf.layer_norm_bwd(gy.numpy(), oh, om, oi, gam.detach().numpy())[0])
+    assert np.array_equal(d0[0], plain) and np.array_equal(d0[1], plain)
