@@ -1,0 +1,17 @@
+"""Model-level helpers that put the fused ops into existing models, mirroring
+``oslo/transformers/kernel_fusion_utils.py`` of the reference."""
+from oslo_amd.transformers.kernel_fusion_utils import (
+    fused_attention_forward,
+    fused_layer_norm,
+    fused_rms_norm,
+    fused_scale_mask_softmax,
+    register_fused_attention,
+)
+
+__all__ = [
+    "fused_attention_forward",
+    "fused_layer_norm",
+    "fused_rms_norm",
+    "fused_scale_mask_softmax",
+    "register_fused_attention",
+]

@@ -1,0 +1,149 @@
+"""Module swaps that route a model through the fused kernels.
+
+The reference swaps ``T5LayerNorm`` for ``FusedRMSNorm`` by rewriting the
+module's class in place (``oslo/transformers/kernel_fusion_utils.py:71-87``);
+``fused_rms_norm`` / ``fused_layer_norm`` do the same here.  The reference's
+attention blocks run scale -> mask -> softmax -> dropout unfused
+(``oslo/transformers/models/gpt2/modeling_gpt2.py:113-142``);
+``fused_scale_mask_softmax`` routes a Hugging Face model's attention through
+``FusedScaleMaskSoftmax`` (softmax and attention dropout in one kernel) by
+registering an attention function with the library's attention interface.
+"""
+import torch
+import torch.nn as nn
+
+from oslo_amd.torch.nn.modules import functional as onn_f
+from oslo_amd.torch.nn.modules.layer_norm import FusedLayerNorm, FusedRMSNorm
+
+ATTENTION_NAME = "oslo_fused_softmax"
+
+
+def _is_rms_norm(module):
+    """T5LayerNorm and its descendants (LlamaRMSNorm, ...): a ``weight`` vector,
+    a ``variance_epsilon`` and no bias."""
+    return (
+        hasattr(module, "variance_epsilon")
+        and isinstance(getattr(module, "weight", None), nn.Parameter)
+        and module.weight.dim() == 1
+        and getattr(module, "bias", None) is None
+        and not isinstance(module, (FusedRMSNorm, FusedLayerNorm))
+    )
+
+
+def fused_rms_norm(model):
+    """Turns every RMS-norm module of ``model`` into a ``FusedRMSNorm`` in place
+    (kernel_fusion_utils.py:71-87 of the reference, there for T5 only).
+    Returns the number of modules swapped."""
+    n = 0
+    for module in model.modules():
+        if _is_rms_norm(module):
+            module.elementwise_affine = True
+            module.normalized_shape = module.weight.size()
+            module.eps = module.variance_epsilon
+            module.__class__ = FusedRMSNorm
+            n += 1
+    return n
+
+
+def fused_layer_norm(model):
+    """Turns every ``nn.LayerNorm`` of ``model`` into a ``FusedLayerNorm`` in place."""
+    n = 0
+    for module in model.modules():
+        if type(module) is nn.LayerNorm:
+            if module.elementwise_affine and module.bias is None:
+                continue  # weight without bias: no fused counterpart
+            module.__class__ = FusedLayerNorm
+            n += 1
+    return n
+
+
+def _repeat_kv(hidden_states, n_rep):
+    if n_rep == 1:
+        return hidden_states
+    b, kv_heads, s, d = hidden_states.shape
+    hidden_states = hidden_states[:, :, None, :, :].expand(b, kv_heads, n_rep, s, d)
+    return hidden_states.reshape(b, kv_heads * n_rep, s, d)
+
+
+def fused_attention_forward(module, query, key, value, attention_mask, scaling=None,
+                            dropout=0.0, **kwargs):
+    """Attention with the scale -> mask -> softmax -> dropout chain in one kernel.
+
+    Signature and return value of the attention functions of Hugging Face
+    transformers (``(module, query, key, value, attention_mask, scaling,
+    dropout, **kwargs) -> (attn_output [b, sq, heads, d], attn_weights)``).
+    ``attention_mask`` is None (causal when the module is), a boolean
+    ``[b or 1, 1, sq or 1, sk]`` tensor with True = attend, or an additive float
+    mask of that shape.
+    """
+    if scaling is None:
+        scaling = query.size(-1) ** -0.5
+    n_rep = query.size(1) // key.size(1)
+    key = _repeat_kv(key, n_rep)
+    value = _repeat_kv(value, n_rep)
+    scores = torch.matmul(query, key.transpose(-1, -2))
+    b, heads, sq, sk = scores.shape
+    p = float(dropout) if module.training else 0.0
+    if attention_mask is None:
+        causal = kwargs.get("is_causal")
+        if causal is None:
+            causal = getattr(module, "is_causal", True)
+    else:
+        causal = False
+    if not scores.is_cuda:
+        # CPU tensors: the unfused chain
+        t = scores * scaling
+        if attention_mask is not None:
+            if attention_mask.dtype == torch.bool:
+                t = t.masked_fill(~attention_mask, -10000.0)
+            else:
+                t = t + attention_mask
+        elif causal:
+            hidden = torch.ones(sq, sk, dtype=torch.bool, device=t.device).triu(1 + sk - sq)
+            t = t.masked_fill(hidden, -10000.0)
+        probs = torch.softmax(t, dim=-1).to(value.dtype)
+        probs = torch.nn.functional.dropout(probs, p=p, training=module.training)
+    elif attention_mask is None and causal:
+        probs = onn_f.scaled_upper_triang_masked_softmax_dropout(
+            scores.reshape(b * heads, sq, sk), scaling, p, module.training
+        ).view(b, heads, sq, sk)
+    else:
+        if attention_mask is None:
+            hidden = torch.zeros(1, 1, 1, sk, dtype=torch.bool, device=scores.device)
+        elif attention_mask.dtype == torch.bool:
+            hidden = ~attention_mask
+        else:
+            hidden = attention_mask < -1.0
+        hidden = hidden[..., :sk]
+        probs = onn_f.scaled_masked_softmax_dropout(
+            scores, hidden, scaling, p, module.training
+        )
+    attn_output = torch.matmul(probs.to(value.dtype), value).transpose(1, 2).contiguous()
+    return attn_output, probs
+
+
+def register_fused_attention(name=ATTENTION_NAME):
+    """Registers ``fused_attention_forward`` (and a boolean mask builder) with
+    transformers' attention interface under ``name``."""
+    try:
+        from transformers import AttentionInterface
+        from transformers.masking_utils import AttentionMaskInterface, sdpa_mask
+    except ImportError as e:  # older transformers: no pluggable attention
+        raise ImportError(
+            "fused_scale_mask_softmax needs a transformers version with "
+            "AttentionInterface (%s)" % e
+        ) from None
+    AttentionInterface.register(name, fused_attention_forward)
+    AttentionMaskInterface.register(name, sdpa_mask)
+    return name
+
+
+def fused_scale_mask_softmax(model, name=ATTENTION_NAME):
+    """Routes the attention of a Hugging Face ``model`` through the fused
+    scale-mask-softmax(-dropout) kernels."""
+    register_fused_attention(name)
+    if hasattr(model, "set_attn_implementation"):
+        model.set_attn_implementation(name)
+    else:
+        model.config._attn_implementation = name
+    return model
