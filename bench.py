@@ -352,6 +352,37 @@ def kernel_table(L, dev, iters):
         del bufs
         torch.cuda.empty_cache()
 
+    # ---- multi-tensor Adam (AdamW mode): the parameters of 16 transformer
+    # layers of hidden size 2048 (12 tensors a layer, 0.8e9 bytes a state array
+    # in fp32); reads g, p, m, v and writes p, m, v: 7 values per element ----
+    import ctypes
+
+    shapes = []
+    for _ in range(16):
+        shapes += [(2048, 6144), (6144,), (2048, 2048), (2048,), (2048, 8192), (8192,), (8192, 2048), (2048,),
+                   (2048,), (2048,), (2048,), (2048,)]
+    for tdt, code, esz in ((torch.float32, F32, 4), (torch.bfloat16, BF16, 2)):
+        lists = [[torch.zeros(s, device=dev, dtype=tdt) for s in shapes] for _ in range(4)]
+        for t in lists[0]:
+            t.normal_()
+        nel = sum(t.numel() for t in lists[0])
+        n = len(shapes)
+        arr = ctypes.c_void_p * n
+        tables = [arr(*[t.data_ptr() for t in lst]) for lst in lists]
+        sizes = (ctypes.c_int64 * n)(*[t.numel() for t in lists[0]])
+        step_no = [0]
+
+        def adam(i):
+            step_no[0] += 1
+            L.ok(lib.oslo_multi_tensor_adam(tables[0], tables[1], tables[2], tables[3], sizes, n, 1e-3, 0.9, 0.999,
+                                            1e-8, step_no[0], 1, 1, 0.01, code, L.stream()))
+
+        row = table_row("multi_tensor_adam", "-", [n, nel], str(tdt).split(".")[-1], 7 * nel * esz, timed(adam, 1))
+        row["tensors"] = n
+        rows.append(row)
+        del lists, tables
+        torch.cuda.empty_cache()
+
     # ---- plain copy with the same load/store path: the practical ceiling ----
     nbytes = 1 << 30
     src = [torch.empty(nbytes, dtype=torch.uint8, device=dev) for _ in range(2)]

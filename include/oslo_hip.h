@@ -285,6 +285,30 @@ int oslo_bias_dropout_add_norm_bwd(const void *dy, const void *dh_extra,
                                    uint64_t offset, int rms, int dtype,
                                    void *stream);
 
+/* ---- multi-tensor Adam / AdamW ----------------------------------------- *
+ * Replaces multi_tensor_adam (oslo/torch/_C/csrc/FusedAdamBinder.cpp:1-15 ->
+ * multi_tensor_adam_cuda, oslo/torch/_C/csrc/multi_tensor_adam.cu:112-136,
+ * functor :22-110), called by FusedAdam.step
+ * (oslo/torch/optim/fused_adam.py:96-184).  g, p, m, v are HOST arrays of
+ * ntensors device pointers (gradient, parameter, exp_avg, exp_avg_sq of each
+ * tensor) and sizes the element counts; all tensors share `dtype` (f32, f16,
+ * bf16; the reference dispatches double, float and half), the math is fp32:
+ *   mode 0 (L2):    g += decay * p
+ *   m = b1 m + (1 - b1) g;  v = b2 v + (1 - b2) g g
+ *   update = (m / bc1) / (sqrt(v / bc2) + eps)  [+ decay * p in mode 1, AdamW]
+ *   p -= lr * update
+ * with bc1 = 1 - b1^step, bc2 = 1 - b2^step when bias_correction == 1, else
+ * 1.  p, m, v are updated in place.  The tensor table travels in kernel
+ * arguments (64 tensors per launch); nothing is allocated or copied.  The
+ * reference's chunk_size and noop_flag arguments have no effect on its
+ * result (the flag test is commented out, multi_tensor_adam.cu:29-31) and
+ * are not part of this signature.                                          */
+int oslo_multi_tensor_adam(const void *const *g, void *const *p, void *const *m,
+                           void *const *v, const int64_t *sizes,
+                           int64_t ntensors, float lr, float beta1, float beta2,
+                           float eps, int step, int mode, int bias_correction,
+                           float weight_decay, int dtype, void *stream);
+
 /* ---- test and measurement hooks (no counterpart in the reference) ------ */
 
 /* Writes the keep mask (1 = kept) of n elements as uint8. */
@@ -309,7 +333,7 @@ int oslo_wave_reduce_selftest(float *out4, void *stream);
  * "norm_fwd_vpl", "norm_bwd_vpl", "norm_bwd_blocks_per_cu",
  * "softmax_rows_per_wave", "eltwise_unroll", "eltwise_rowgroups",
  * "eltwise_fwd_steps", "norm_bwd_waves", "norm_fwd_waves",
- * "norm_bwd_prefetch", "norm_fwd_iters";
+ * "norm_bwd_prefetch", "norm_fwd_iters", "adam_unroll";
  * value 0 restores the default.  Process-wide, not thread-safe.            */
 int oslo_tune(const char *key, int value);
 

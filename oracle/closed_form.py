@@ -326,3 +326,37 @@ def bias_dropout_add_norm_bwd(dy, dh_extra, h, mean, invvar, gamma, keep, p, rms
     n2 = dx.shape[-1]
     dbias = round_to(np.asarray(dx, dtype=acc).reshape(-1, n2).sum(axis=0), out)
     return dres, dx, dgamma, dbeta, dbias
+
+
+# ---------------------------------------------------------------------------
+# Adam / AdamW step
+# ---------------------------------------------------------------------------
+def adam_step(g, p, m, v, lr, beta1, beta2, eps, step, mode, bias_correction, weight_decay,
+              out="f64", acc=np.float64):
+    """One Adam update of one tensor; returns the new (p, m, v), each rounded
+    once to the storage type.
+
+    oslo/torch/_C/csrc/multi_tensor_adam.cu:78-96: mode 0 adds decay * p to the
+    gradient (L2), mode 1 adds decay * p to the update (AdamW); the bias
+    corrections 1 - beta^step are formed from the float32 betas and stored as
+    float32 (:120-125); lr, eps, decay and the betas enter as float32 values.
+    """
+    f = lambda x: acc(np.float32(x))
+    b1, b2 = f(beta1), f(beta2)
+    bc1 = bc2 = acc(1.0)
+    if bias_correction:
+        bc1 = acc(np.float32(1.0 - float(np.float32(beta1)) ** step))
+        bc2 = acc(np.float32(1.0 - float(np.float32(beta2)) ** step))
+    g = np.asarray(g, dtype=acc)
+    p = np.asarray(p, dtype=acc)
+    m = np.asarray(m, dtype=acc)
+    v = np.asarray(v, dtype=acc)
+    if mode == 0:
+        g = g + f(weight_decay) * p
+    m = b1 * m + (acc(1.0) - b1) * g
+    v = b2 * v + (acc(1.0) - b2) * g * g
+    update = (m / bc1) / (np.sqrt(v / bc2) + f(eps))
+    if mode != 0:
+        update = update + f(weight_decay) * p
+    p = p - f(lr) * update
+    return round_to(p, out), round_to(m, out), round_to(v, out)

@@ -33,6 +33,7 @@ struct Tuning {
   int norm_fwd_waves;
   int norm_bwd_prefetch;
   int norm_fwd_iters;
+  int adam_unroll;
 };
 extern Tuning g_tune;
 

@@ -90,6 +90,7 @@ int oslo_tune(const char *key, int value) {
       {"norm_fwd_waves", &oslo::g_tune.norm_fwd_waves},
       {"norm_bwd_prefetch", &oslo::g_tune.norm_bwd_prefetch},
       {"norm_fwd_iters", &oslo::g_tune.norm_fwd_iters},
+      {"adam_unroll", &oslo::g_tune.adam_unroll},
   };
   for (const Entry &e : table) {
     if (strcmp(e.name, key) == 0) {

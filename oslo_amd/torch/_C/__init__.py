@@ -110,6 +110,10 @@ _SIGNATURES = {
         [_p, _p, _p, _p, _p, _p, _p, _p, _p, _p, _p, _p, _i64, _i64, _i64, _f32, _u64,
          _u64, _int, _int, _p],
     ),
+    "oslo_multi_tensor_adam": (
+        _int,
+        [_p, _p, _p, _p, _p, _i64, _f32, _f32, _f32, _f32, _int, _int, _int, _f32, _int, _p],
+    ),
     "oslo_philox_mask": (_int, [_p, _i64, _f32, _u64, _u64, _p]),
     "oslo_philox_words": (_int, [_p, _i64, _i64, _u64, _u64, _p]),
     "oslo_copy_probe": (_int, [_p, _p, _i64, _p]),
@@ -834,6 +838,67 @@ def get_softmax_kernel():
     if _softmax_kernel is None:
         _softmax_kernel = _SoftmaxKernel(load_library())
     return _softmax_kernel
+
+
+# ---------------------------------------------------------------------------
+# multi-tensor Adam
+# ---------------------------------------------------------------------------
+class _AdamKernel:
+    """``multi_tensor_adam`` of the reference's ``oslo_fused_adam`` module
+    (``oslo/torch/_C/csrc/FusedAdamBinder.cpp:12-15``), same argument list."""
+
+    def __init__(self, lib):
+        self._lib = lib
+
+    def multi_tensor_adam(
+        self, chunk_size, noop_flag, tensor_lists, lr, beta1, beta2, epsilon, step,
+        mode, bias_correction, weight_decay,
+    ):
+        """``tensor_lists`` = ``[grads, params, exp_avgs, exp_avg_sqs]``, updated in
+        place.  ``chunk_size`` and ``noop_flag`` are accepted for signature
+        compatibility; the reference's kernel does not act on them either
+        (``multi_tensor_adam.cu:29-31``)."""
+        lib = self._lib
+        if len(tensor_lists) != 4:
+            raise RuntimeError("tensor_lists must hold [grads, params, exp_avgs, exp_avg_sqs]")
+        gs, ps, ms, vs = tensor_lists
+        n = len(ps)
+        if not (len(gs) == len(ms) == len(vs) == n):
+            raise RuntimeError("Size mismatch among tensor lists")
+        if n == 0:
+            return
+        ref = ps[0]
+        code = _dtype_code(ref, "params[0]")
+        for i in range(n):
+            sz = ps[i].numel()
+            for name, t in (("grad", gs[i]), ("param", ps[i]), ("exp_avg", ms[i]), ("exp_avg_sq", vs[i])):
+                _check_input(t, "%s %d" % (name, i))
+                if t.dtype != ref.dtype or t.device != ref.device:
+                    raise RuntimeError(
+                        "A tensor was not the same dtype / on the same device as the first tensor"
+                    )
+                if t.numel() != sz:
+                    raise RuntimeError("Size mismatch among tensor lists")
+        arr = ctypes.c_void_p * n
+        sizes = (ctypes.c_int64 * n)(*[t.numel() for t in ps])
+        tables = [arr(*[t.data_ptr() for t in lst]) for lst in (gs, ps, ms, vs)]
+        with torch.cuda.device_of(ref):
+            rc = lib.oslo_multi_tensor_adam(
+                tables[0], tables[1], tables[2], tables[3], sizes, n, float(lr), float(beta1),
+                float(beta2), float(epsilon), int(step), int(mode), int(bias_correction),
+                float(weight_decay), code, _stream(ref),
+            )
+            _check(rc, lib)
+
+
+_adam_kernel = None
+
+
+def get_adam_kernel():
+    global _adam_kernel
+    if _adam_kernel is None:
+        _adam_kernel = _AdamKernel(load_library())
+    return _adam_kernel
 
 
 def get_fused_elementwise_kernel():
