@@ -92,16 +92,22 @@ __device__ __forceinline__ void row_setup(const SoftmaxGeom &g, int64_t r,
   mrow = nullptr;
   visible = g.sk;
   row = r;
+  // 32-bit division where the row count allows it: a 64-bit division costs
+  // about as many instructions as the softmax of a short row itself
+  const bool small = g.rows <= 0x7fffffff;
   if constexpr (MODE == kModeCausal) {
-    const int64_t batch = r / g.sq;
+    const int64_t batch =
+        small ? (int64_t)((uint32_t)r / (uint32_t)g.sq) : r / g.sq;
     const int qi = g.sq - 1 - (int)(r - batch * g.sq);
     row = batch * g.sq + qi;
     int v = qi + 1 + (g.sk - g.sq);
     visible = v < 0 ? 0 : (v > g.sk ? g.sk : v);
   } else if constexpr (MODE == kModeMasked) {
-    const int64_t bh = r / g.sq;
+    const int64_t bh =
+        small ? (int64_t)((uint32_t)r / (uint32_t)g.sq) : r / g.sq;
     const int qi = (int)(r - bh * g.sq);
-    const int64_t bi = bh / g.np;
+    const int64_t bi =
+        small ? (int64_t)((uint32_t)bh / (uint32_t)g.np) : bh / g.np;
     const int64_t mr =
         bi * g.mask_b_stride_rows + (g.mask_per_query ? qi : 0);
     mrow = mask + mr * g.sk;

@@ -85,12 +85,18 @@ def test_bias_gelu_matches_reference_formulas_fp32(device):
     check(db, f64(ref_dx.sum(0)), "dbias vs autograd reduction", atol=2e-4)
 
 
-@pytest.mark.parametrize("rows,cols,dtype", SHAPES)
+# every shape with bias and residual; the operand subsets on three shapes
+BDA_CASES = [
+    (rows, cols, dtype, parts)
+    for (rows, cols, dtype) in SHAPES
+    for parts in ("bias+res", "bias", "res", "none")
+    if parts == "bias+res" or (rows, cols) in [(64, 4096), (9, 100), (5, 768)]
+]
+
+
+@pytest.mark.parametrize("rows,cols,dtype,parts", BDA_CASES)
 @pytest.mark.parametrize("p", [0.0, 0.1, 0.5])
-@pytest.mark.parametrize("parts", ["bias+res", "bias", "res", "none"])
 def test_bias_dropout_add(device, rows, cols, dtype, p, parts):
-    if parts != "bias+res" and (rows, cols) not in [(64, 4096), (9, 100), (5, 768)]:
-        pytest.skip("operand subsets are covered on three shapes")
     seed, offset = 1234, 8
     x = randn((rows, cols), dtype, seed=rows + cols, std=1.0)
     bias = randn((cols,), dtype, seed=1, std=0.02) if "bias" in parts else None
