@@ -1060,6 +1060,22 @@ static int launch_norm_bwd(const void *dy, const void *x, const float *mean,
   return launch_colsum_finalize<V>(part, P, n2, outs[0], outs[1], st, outs[2], na);
 }
 
+// Zero fill of a small parameter-gradient vector (a kernel rather than a
+// memset node, so that a caller may capture the call in a HIP graph).
+__global__ __launch_bounds__(256) void zero_bytes_kernel(uint8_t *p, int64_t nbytes) {
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < nbytes;
+       i += (int64_t)gridDim.x * 256)
+    p[i] = 0;
+}
+
+static int zero_params(void *p, int64_t nbytes, hipStream_t st) {
+  if (p == nullptr || nbytes <= 0) return OSLO_OK;
+  int64_t grid = ceil_div(nbytes, 256);
+  if (grid > 1024) grid = 1024;
+  zero_bytes_kernel<<<dim3((unsigned)grid), 256, 0, st>>>((uint8_t *)p, nbytes);
+  return check_launch("zero_bytes_kernel");
+}
+
 static int check_norm_dtypes(int din, int dout) {
   if (!valid_dtype(din) || !valid_dtype(dout))
     return fail(OSLO_ERR_INVALID_ARGUMENT, "unknown dtype (%d, %d)", din, dout);
@@ -1125,11 +1141,9 @@ static int norm_bwd_entry(bool rms, const void *dy, const void *x,
   if (n1 == 0) {
     // an empty batch still defines zero parameter gradients
     hipStream_t st0 = (hipStream_t)stream;
-    if (dgamma)
-      (void)hipMemsetAsync(dgamma, 0, (size_t)n2 * dtype_size(dout), st0);
-    if (dbeta)
-      (void)hipMemsetAsync(dbeta, 0, (size_t)n2 * dtype_size(dout), st0);
-    return OSLO_OK;
+    int rc0 = zero_params(dgamma, n2 * dtype_size(dout), st0);
+    if (rc0 == OSLO_OK) rc0 = zero_params(dbeta, n2 * dtype_size(dout), st0);
+    return rc0;
   }
   OSLO_REQUIRE(dy && x && invvar && dx, "norm bwd: null tensor pointer");
   OSLO_REQUIRE(rms || mean, "layer norm bwd: null mean pointer");
@@ -1250,11 +1264,11 @@ int oslo_bias_dropout_add_norm_bwd(const void *dy, const void *dh_extra,
                "tensor (dx)");
   hipStream_t st = (hipStream_t)stream;
   if (n1 == 0) {
-    const size_t nb = (size_t)n2 * dtype_size(dtype);
-    if (dgamma) (void)hipMemsetAsync(dgamma, 0, nb, st);
-    if (dbeta && !rms) (void)hipMemsetAsync(dbeta, 0, nb, st);
-    if (dbias) (void)hipMemsetAsync(dbias, 0, nb, st);
-    return OSLO_OK;
+    const int64_t nb = n2 * dtype_size(dtype);
+    rc = zero_params(dgamma, nb, st);
+    if (rc == OSLO_OK && !rms) rc = zero_params(dbeta, nb, st);
+    if (rc == OSLO_OK) rc = zero_params(dbias, nb, st);
+    return rc;
   }
   OSLO_REQUIRE(dy && h && invvar && dres, "fused norm bwd: null tensor pointer");
   OSLO_REQUIRE(rms || mean, "fused layer norm bwd: null mean pointer");
