@@ -411,9 +411,11 @@ struct FuseEpilogue {
   int want_dbias;        // 1: partial rows of the bias gradient are written
 };
 
+// MAXT: largest workgroup the build is launched with (768 leaves a third more
+// registers per lane than 1024, which the 16-elements-per-lane builds need).
 template <typename T, typename V, int VPL, bool RMS, bool EVEN, int PF,
-          bool FUSE = false>
-__global__ __launch_bounds__(1024) void norm_bwd_reg_kernel(
+          bool FUSE = false, int MAXT = 1024>
+__global__ __launch_bounds__(MAXT) void norm_bwd_reg_kernel(
     const V *__restrict__ dy, const T *__restrict__ x,
     const float *__restrict__ mean, const float *__restrict__ invvar,
     const V *__restrict__ gamma, T *__restrict__ dx, float *__restrict__ part,
@@ -1011,11 +1013,11 @@ static int launch_norm_bwd(const void *dy, const void *x, const float *mean,
   // buffers are small (8 elements per lane), else one
   int pf = sp.vpl * E <= 8 ? 2 : 1;
   if (g_tune.norm_bwd_prefetch > 0) pf = g_tune.norm_bwd_prefetch >= 2 ? 2 : 1;
-#define OSLO_BWD_LAUNCH(VPL, EVEN_, PF_)                                   \
+#define OSLO_BWD_LAUNCH_T(VPL, EVEN_, PF_, MAXT_)                          \
   do {                                                                     \
     if constexpr (kCanFuse) {                                              \
       if (fused) {                                                         \
-        norm_bwd_reg_kernel<T, V, VPL, RMS, EVEN_, PF_, true>              \
+        norm_bwd_reg_kernel<T, V, VPL, RMS, EVEN_, PF_, true, MAXT_>       \
             <<<dim3((unsigned)P), threads, lds, st>>>(                     \
                 (const V *)dy, (const T *)x, mean, invvar,                 \
                 (const V *)gamma, (T *)dx, part, n1, (int)n2, sp.wpr,      \
@@ -1023,10 +1025,21 @@ static int launch_norm_bwd(const void *dy, const void *x, const float *mean,
         break;                                                             \
       }                                                                    \
     }                                                                      \
-    norm_bwd_reg_kernel<T, V, VPL, RMS, EVEN_, PF_, false>                 \
+    norm_bwd_reg_kernel<T, V, VPL, RMS, EVEN_, PF_, false, MAXT_>          \
         <<<dim3((unsigned)P), threads, lds, st>>>(                         \
             (const V *)dy, (const T *)x, mean, invvar, (const V *)gamma,   \
             (T *)dx, part, n1, (int)n2, sp.wpr, sp.rpb, fev);              \
+  } while (0)
+  // the 16-elements-per-lane builds exist for 768 threads as well
+#define OSLO_BWD_LAUNCH(VPL, EVEN_, PF_)                                   \
+  do {                                                                     \
+    if constexpr (VPL * E == 16) {                                         \
+      if (threads <= 768) {                                                \
+        OSLO_BWD_LAUNCH_T(VPL, EVEN_, PF_, 768);                           \
+        break;                                                             \
+      }                                                                    \
+    }                                                                      \
+    OSLO_BWD_LAUNCH_T(VPL, EVEN_, PF_, 1024);                              \
   } while (0)
 #define OSLO_BWD_CASE(VPL)                                                 \
   case VPL:                                                                \
@@ -1049,6 +1062,7 @@ static int launch_norm_bwd(const void *dy, const void *x, const float *mean,
       return fail(OSLO_ERR_UNSUPPORTED, "norm bwd: no kernel for vpl=%d", sp.vpl);
   }
 #undef OSLO_BWD_LAUNCH
+#undef OSLO_BWD_LAUNCH_T
 #undef OSLO_BWD_CASE
   int rc = check_launch("norm_bwd_reg_kernel");
   if (rc != OSLO_OK || !want_params) return rc;
