@@ -148,6 +148,25 @@ __device__ __forceinline__ void store_chunk(T *p, const float *f) {
     st16_stream(p + v * io<T>::EPV, io<T>::pack(f + v * io<T>::EPV));
 }
 
+// Stores a chunk (p may be null: nothing is written) and replaces f by the
+// values as stored, taken from the very registers that were written.  Code
+// that accumulates "the tensor as stored" must go through this: rounding f a
+// second time in a separate expression can differ in the last place, because
+// the compiler may fuse the arithmetic that produced f into one of the two
+// conversions (a mixed-precision fma rounds once, a product followed by a
+// conversion rounds twice).
+template <typename T, int E>
+__device__ __forceinline__ void store_chunk_readback(T *p, float *f) {
+  constexpr int NV = E * (int)sizeof(T) / 16;
+  static_assert(NV >= 1, "chunk smaller than one vector");
+#pragma unroll
+  for (int v = 0; v < NV; ++v) {
+    const u32x4 r = io<T>::pack(f + v * io<T>::EPV);
+    if (p != nullptr) st16_stream(p + v * io<T>::EPV, r);
+    io<T>::unpack(r, f + v * io<T>::EPV);
+  }
+}
+
 // A chunk kept in its packed storage form, for loads issued one iteration
 // ahead of their use (software prefetch): E * sizeof(T) / 4 registers.
 template <typename T, int E> struct RawChunk {

@@ -173,11 +173,10 @@ __global__ __launch_bounds__(256) void bias_gelu_bwd_kernel(
         if (r < g.rows) {
           float o[kE];
 #pragma unroll
-          for (int e = 0; e < kE; ++e) {
-            o[e] = gelu_bwd(v[u][e] + b[e]) * gv[u][e];
-            acc[e] += io<T>::round(o[e]);  // sum of dx as stored
-          }
-          store_chunk<T, kE>(dx + r * g.cols + coff, o);
+          for (int e = 0; e < kE; ++e) o[e] = gelu_bwd(v[u][e] + b[e]) * gv[u][e];
+          store_chunk_readback<T, kE>(dx + r * g.cols + coff, o);
+#pragma unroll
+          for (int e = 0; e < kE; ++e) acc[e] += o[e];  // sum of dx as stored
         }
       }
     }
@@ -284,9 +283,10 @@ __global__ __launch_bounds__(256) void bias_dropout_add_bwd_kernel(
             float t = gv[u][e];
             if constexpr (DROP) t = (keep >> e) & 1u ? t * d.scale : 0.f;
             o[e] = t;
-            acc[e] += io<T>::round(t);
           }
-          if (dx != nullptr) store_chunk<T, kE>(dx + r * g.cols + coff, o);
+          store_chunk_readback<T, kE>(dx != nullptr ? dx + r * g.cols + coff : nullptr, o);
+#pragma unroll
+          for (int e = 0; e < kE; ++e) acc[e] += o[e];  // sum of dx as stored
         }
       }
     }

@@ -559,19 +559,27 @@ __global__ __launch_bounds__(MAXT) void norm_bwd_reg_kernel(
 #pragma unroll
             for (int e = 0; e < E; ++e) o[e] += extra[k][e];
           }
-          store_chunk<T, E>(dxr + (int64_t)c * E, o);
-          if constexpr (FUSE) {
-            // gradient of x of the prologue, from the unrounded gradient of h
-            if (fe.drop) {
-              const uint32_t keep = chunk_keep_bits<E>(row, n2, c, fe.d);
+          if constexpr (!FUSE) {
+            store_chunk<T, E>(dxr + (int64_t)c * E, o);
+          } else if (fe.drop) {
+            // gradient of x of the prologue: masked and scaled from the
+            // unrounded gradient of h, then rounded once
+            store_chunk<T, E>(dxr + (int64_t)c * E, o);
+            const uint32_t keep = chunk_keep_bits<E>(row, n2, c, fe.d);
 #pragma unroll
-              for (int e = 0; e < E; ++e)
-                o[e] = (keep >> e) & 1u ? o[e] * fe.d.scale : 0.f;
-            }
+            for (int e = 0; e < E; ++e)
+              o[e] = (keep >> e) & 1u ? o[e] * fe.d.scale : 0.f;
+            store_chunk_readback<T, E>(
+                fdrop != nullptr ? fdrop + row * n2 + (int64_t)c * E : nullptr, o);
+#pragma unroll
+            for (int e = 0; e < E; ++e) acc_d[k][e] += o[e];  // dx as stored
+          } else {
+            // no dropout: the gradient of x is the gradient of h as stored
+            store_chunk_readback<T, E>(dxr + (int64_t)c * E, o);
             if (fdrop != nullptr)
               store_chunk<T, E>(fdrop + row * n2 + (int64_t)c * E, o);
 #pragma unroll
-            for (int e = 0; e < E; ++e) acc_d[k][e] += io<T>::round(o[e]);
+            for (int e = 0; e < E; ++e) acc_d[k][e] += o[e];
           }
         }
       }

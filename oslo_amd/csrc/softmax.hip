@@ -208,14 +208,16 @@ __global__ __launch_bounds__(1024) void softmax_fwd_kernel(
       if (all_visible[j][k]) {
 #pragma unroll
         for (int e = 0; e < E; ++e) {
-          const float t = v[j][k][e] * c2;
+          // (rounded product, never fused into the later subtraction: the
+          //  backward pass of the dropout variant recomputes it bit for bit)
+          const float t = __fmul_rn(v[j][k][e], c2);
           v[j][k][e] = t;
           m = fmaxf(m, t);
         }
       } else {
 #pragma unroll
         for (int e = 0; e < E; ++e) {
-          const float t = (mbits[j][k] >> e) & 1u ? ninf : v[j][k][e] * c2;
+          const float t = (mbits[j][k] >> e) & 1u ? ninf : __fmul_rn(v[j][k][e], c2);
           v[j][k][e] = t;
           m = fmaxf(m, t);
         }
@@ -239,7 +241,7 @@ __global__ __launch_bounds__(1024) void softmax_fwd_kernel(
       if (none_visible[j][k]) continue;
 #pragma unroll
       for (int e = 0; e < E; ++e) {
-        const float p = __builtin_amdgcn_exp2f(v[j][k][e] - off);
+        const float p = __builtin_amdgcn_exp2f(__fsub_rn(v[j][k][e], off));
         v[j][k][e] = p;  // exp2(-inf) == 0 for masked keys
         s += p;
       }
@@ -391,7 +393,10 @@ __global__ __launch_bounds__(1024) void softmax_dropout_bwd_kernel(
           mbits[j][k] != kAll ? chunk_keep_bits<E>(row[j], g.sk, c, d) : 0u;
 #pragma unroll
       for (int e = 0; e < E; ++e) {
-        float p = __builtin_amdgcn_exp2f(fmaf(yv[j][k][e], c2, -rmax[j])) * rinv[j];
+        // the product is rounded before the subtraction, exactly as the
+        // forward pass formed its exponent (no fused multiply-add here)
+        float p =
+            __builtin_amdgcn_exp2f(__fsub_rn(__fmul_rn(yv[j][k][e], c2), rmax[j])) * rinv[j];
         if (empty) p = -rinv[j];
         if ((mbits[j][k] >> e) & 1u) p = 0.f;
         const float dp = (keep >> e) & 1u ? gv[j][k][e] * d.scale : 0.f;
@@ -576,6 +581,9 @@ __global__ __launch_bounds__(256) void softmax_fwd_generic_kernel(
     DropArgs d) {
   __shared__ float sh[4];
   const float ninf = -__builtin_inff();
+  // log2-domain logits t = x * (scale * log2 e), the same rounded products
+  // and differences as in the register kernel
+  const float c2 = scale * kLog2e;
   for (int64_t r = blockIdx.x; r < g.rows; r += gridDim.x) {
     int64_t row;
     int visible;
@@ -586,7 +594,7 @@ __global__ __launch_bounds__(256) void softmax_fwd_generic_kernel(
     float m = ninf;
     for (int i = threadIdx.x; i < g.sk; i += 256) {
       const bool hidden = MODE == kModeCausal ? i >= visible : mrow[i] != 0;
-      if (!hidden) m = fmaxf(m, io<T>::from_scalar(xr[i]) * scale);
+      if (!hidden) m = fmaxf(m, __fmul_rn(io<T>::from_scalar(xr[i]), c2));
     }
     m = block_reduce_256(m, sh, true);
     const bool empty = m == ninf;
@@ -594,8 +602,8 @@ __global__ __launch_bounds__(256) void softmax_fwd_generic_kernel(
     for (int i = threadIdx.x; i < g.sk; i += 256) {
       const bool hidden = MODE == kModeCausal ? i >= visible : mrow[i] != 0;
       if (!hidden)
-        s += __builtin_amdgcn_exp2f((io<T>::from_scalar(xr[i]) * scale - m) *
-                                    kLog2e);
+        s += __builtin_amdgcn_exp2f(
+            __fsub_rn(__fmul_rn(io<T>::from_scalar(xr[i]), c2), m));
     }
     s = block_reduce_256(s, sh, false);
     const float inv = empty ? 0.f : 1.0f / s;
@@ -604,8 +612,8 @@ __global__ __launch_bounds__(256) void softmax_fwd_generic_kernel(
       const bool hidden = MODE == kModeCausal ? i >= visible : mrow[i] != 0;
       float p = 0.f;
       if (!hidden)
-        p = __builtin_amdgcn_exp2f((io<T>::from_scalar(xr[i]) * scale - m) *
-                                   kLog2e);
+        p = __builtin_amdgcn_exp2f(
+            __fsub_rn(__fmul_rn(io<T>::from_scalar(xr[i]), c2), m));
       float o = p * inv + fill;
       if constexpr (DROP)
         o = keep_element(row * g.sk + i, d) ? o * d.scale : 0.f;
@@ -613,8 +621,7 @@ __global__ __launch_bounds__(256) void softmax_fwd_generic_kernel(
     }
     if constexpr (DROP) {
       if (threadIdx.x == 0) {
-        // statistics in the log2 domain, as the register kernel stores them
-        stats[2 * row] = empty ? 0.f : m * kLog2e;
+        stats[2 * row] = empty ? 0.f : m;
         stats[2 * row + 1] = empty ? -fill : inv;
       }
     }
@@ -642,7 +649,9 @@ __global__ __launch_bounds__(256) void softmax_dropout_bwd_generic_kernel(
       if (empty) return -inv;
       const bool hidden = MODE == kModeCausal ? i >= visible : mrow[i] != 0;
       if (hidden) return 0.f;
-      return __builtin_amdgcn_exp2f(fmaf(io<T>::from_scalar(xr[i]), c2, -m)) * inv;
+      return __builtin_amdgcn_exp2f(
+                 __fsub_rn(__fmul_rn(io<T>::from_scalar(xr[i]), c2), m)) *
+             inv;
     };
     auto dprob = [&](int i) {
       return keep_element(row * g.sk + i, d) ? io<T>::from_scalar(gr[i]) * d.scale

@@ -160,3 +160,28 @@ def test_argument_checks(device):
     assert (out == 0).all()
     y = k.bias_gelu_forward(torch.zeros(0, 16, device=device), None)
     assert y.shape == (0, 16)
+
+
+@pytest.mark.parametrize("dtype", [F16, BF16, F32])
+def test_dbias_is_the_sum_of_dx_as_stored(device, dtype):
+    """With one row the bias gradient must equal dx bit for bit: the kernels
+    accumulate the values they stored, not a second rounding of them."""
+    n2 = 1 << 18
+    x = randn((1, n2), dtype, 3, std=1.5)
+    g = randn((1, n2), dtype, 4)
+    bias = randn((n2,), dtype, 5, std=0.3)
+    k = _C.get_fused_elementwise_kernel()
+    dx, db = k.bias_gelu_backward(g.to(device), x.to(device), bias.to(device))
+    assert torch.equal(dx[0], db)
+    ddx, ddb = k.bias_dropout_add_backward(g.to(device), 0.3, 5, 0)
+    assert torch.equal(ddx[0], ddb)
+    ln = _C.get_layernorm_kernel()
+    n2 = 4096
+    h = randn((1, n2), dtype, 6)
+    dy = randn((1, n2), dtype, 7)
+    gamma = randn((n2,), dtype, 8, std=0.1, mean=1.0)
+    y, mean, invvar = ln.layer_norm_forward_affine(h.to(device), (n2,), gamma.to(device), gamma.to(device), 1e-5)
+    for p in (0.0, 0.3):
+        g_res, g_in, _, _, g_bias = ln.bias_dropout_add_norm_backward(
+            False, dy.to(device), None, h.to(device), mean, invvar, (n2,), gamma.to(device), p, 5, 0)
+        assert torch.equal(g_in[0], g_bias)

@@ -1,0 +1,212 @@
+"""Seeded random sweep over shapes, dtypes and option combinations of every op,
+against the float64 oracle: ragged and odd row lengths, lengths around the
+register-path limits, single rows, rows far apart in size, optional operands
+on and off.  Complements the hand-picked cases of the other GPU test files."""
+import numpy as np
+import pytest
+import torch
+
+from helpers import NP_NAME, check, f64, randn
+from oracle import closed_form as cf
+from oracle import philox
+from oslo_amd.torch import _C
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = [torch.float32, torch.float16, torch.bfloat16]
+TRICKY = [1, 2, 3, 4, 7, 8, 9, 15, 16, 17, 31, 32, 33, 63, 64, 65, 127, 128, 129, 255, 256, 257, 511, 512, 513,
+          520, 768, 1000, 1023, 1024, 1025, 1280, 1600, 2047, 2048, 2056, 4095, 4096, 4104, 5120, 8184, 8192,
+          8200, 12288, 16376, 16384, 16392, 20000, 32768, 32776, 40000]
+
+
+def draw_cases(seed, count):
+    r = np.random.default_rng(seed)
+    cases = []
+    for i in range(count):
+        n2 = int(r.choice(TRICKY)) if r.random() < 0.7 else int(r.integers(1, 9000))
+        n1 = int(r.choice([1, 2, 3, 5, 8, 17, 33])) if n2 > 4096 else int(r.integers(1, 70))
+        cases.append((i, n1, n2, DTYPES[int(r.integers(0, 3))], [bool(b) for b in r.integers(0, 2, size=4)]))
+    return cases
+
+
+@pytest.mark.parametrize("i,n1,n2,dtype,flags", draw_cases(101, 60))
+def test_norms(device, i, n1, n2, dtype, flags):
+    rms, affine = flags[0], flags[1]
+    x = randn((n1, n2), dtype, 7 * i, std=1.5, mean=0.3)
+    dy = randn((n1, n2), dtype, 7 * i + 1)
+    gamma = randn((n2,), dtype, 7 * i + 2, std=0.1, mean=1.0) if affine else None
+    beta = randn((n2,), dtype, 7 * i + 3, std=0.1) if affine and not rms else None
+    k = _C.get_layernorm_kernel()
+    name = NP_NAME[dtype]
+    D = lambda t: None if t is None else t.to(device)
+    col = 1e-5 * np.sqrt(n1) + 1e-6
+    if rms:
+        if affine:
+            y, invvar = k.rms_norm_forward_affine(D(x), (n2,), D(gamma), 1e-5)
+        else:
+            y, invvar = k.rms_norm_forward(D(x), (n2,), 1e-5)
+        oy, oinv = cf.rms_norm_fwd(f64(x), None if gamma is None else f64(gamma), 1e-5, name)
+        check(y, oy, "rms fwd", atol=2e-6, max_ulp=2, min_exact=0.99)
+        assert np.allclose(f64(invvar), oinv, rtol=3e-6)
+        odx, odg = cf.rms_norm_bwd(f64(dy), f64(x), f64(invvar), None if gamma is None else f64(gamma))
+        if affine:
+            dx, dg = k.rms_norm_backward_affine(D(dy), invvar, D(x), (n2,), D(gamma), 1e-5)
+            check(dg, odg, "rms dgamma", atol=col, min_exact=0.97, max_ulp=2)
+        else:
+            dx = k.rms_norm_backward(D(dy), invvar, D(x), (n2,), 1e-5)
+        check(dx, odx, "rms dx", atol=4e-6)
+    else:
+        if affine:
+            y, mean, invvar = k.layer_norm_forward_affine(D(x), (n2,), D(gamma), D(beta), 1e-5)
+        else:
+            y, mean, invvar = k.layer_norm_forward(D(x), (n2,), 1e-5)
+        oy, omean, oinv = cf.layer_norm_fwd(f64(x), None if gamma is None else f64(gamma),
+                                            None if beta is None else f64(beta), 1e-5)
+        # a row of one element (or of equal elements) normalises to ~0: absolute floor
+        check(y, oy, "ln fwd", atol=2e-5)
+        assert np.allclose(f64(mean), omean, rtol=1e-5, atol=2e-6)
+        if n2 > 1:
+            assert np.allclose(f64(invvar), oinv, rtol=1e-4)
+        odx, odg, odb = cf.layer_norm_bwd(f64(dy), f64(x), f64(mean), f64(invvar),
+                                          None if gamma is None else f64(gamma))
+        if affine:
+            dx, dg, db = k.layer_norm_backward_affine(D(dy), mean, invvar, D(x), (n2,), D(gamma), D(beta), 1e-5)
+            check(dg, odg, "ln dgamma", atol=col * 3, min_exact=0.97, max_ulp=2)
+            check(db, odb, "ln dbeta", atol=col, min_exact=0.97, max_ulp=2)
+        else:
+            dx = k.layer_norm_backward(D(dy), mean, invvar, D(x), (n2,), 1e-5)
+        check(dx, odx, "ln dx", atol=2e-5)
+
+
+@pytest.mark.parametrize("i,n1,n2,dtype,flags", draw_cases(202, 50))
+def test_fused_residual_norm(device, i, n1, n2, dtype, flags):
+    rms, has_bias, has_res, has_extra = flags
+    p = [0.0, 0.1, 0.5][i % 3]
+    seed, offset = 1000 + i, 4 * i
+    x = randn((n1, n2), dtype, 11 * i)
+    bias = randn((n2,), dtype, 11 * i + 1, std=0.1) if has_bias else None
+    res = randn((n1, n2), dtype, 11 * i + 2) if has_res else None
+    gamma = randn((n2,), dtype, 11 * i + 3, std=0.1, mean=1.0)
+    beta = None if rms else randn((n2,), dtype, 11 * i + 4, std=0.1)
+    dy = randn((n1, n2), dtype, 11 * i + 5)
+    dh = randn((n1, n2), dtype, 11 * i + 6) if has_extra else None
+    k = _C.get_layernorm_kernel()
+    name = NP_NAME[dtype]
+    D = lambda t: None if t is None else t.to(device)
+    F = lambda t: None if t is None else f64(t)
+    y, h, mean, invvar = k.bias_dropout_add_norm_forward(
+        rms, D(x), D(bias), D(res), (n2,), D(gamma), D(beta), 1e-5, p, seed, offset)
+    keep = philox.keep_mask(n1 * n2, p, seed, offset).reshape(n1, n2).astype(bool) if p > 0 else None
+    # (three fp32 roundings before the store: ties fall the other way a little
+    # more often than the default 0.2 %)
+    check(h, cf.bias_dropout_add_fwd(f64(x), F(bias), F(res), keep, p), "fused h", atol=1e-6, min_exact=0.99)
+    if rms:
+        oy, _ = cf.rms_norm_fwd(f64(h), f64(gamma), 1e-5, name)
+    else:
+        oy, _, _ = cf.layer_norm_fwd(f64(h), f64(gamma), f64(beta), 1e-5, name)
+    check(y, oy, "fused y", atol=2e-5, max_ulp=2, min_exact=0.99)
+    g_res, g_in, g_gamma, g_beta, g_bias = k.bias_dropout_add_norm_backward(
+        rms, D(dy), D(dh), h, mean, invvar, (n2,), D(gamma), p, seed, offset, need_bias_grad=has_bias)
+    odres, odx, odg, odb, _ = cf.bias_dropout_add_norm_bwd(
+        f64(dy), F(dh), f64(h), None if rms else f64(mean), f64(invvar), f64(gamma), keep, p, rms, name)
+    check(g_res, odres, "fused dres", atol=2e-5)
+    check(g_in, odx, "fused dx", atol=2e-5)
+    col = 1e-5 * np.sqrt(n1) + 1e-6
+    check(g_gamma, odg, "fused dgamma", atol=3 * col, min_exact=0.97, max_ulp=2)
+    if has_bias:
+        check(g_bias, f64(g_in).sum(0), "fused dbias", atol=3 * col, min_exact=0.97, max_ulp=2)
+
+
+def draw_softmax(seed, count):
+    r = np.random.default_rng(seed)
+    out = []
+    for i in range(count):
+        sk = int(r.choice([1, 5, 8, 16, 31, 64, 100, 128, 256, 257, 512, 1000, 1024, 2048, 2050, 4096, 8192, 9000,
+                           16384, 20000]))
+        sq = int(r.integers(1, 40)) if r.random() < 0.6 else min(sk, 48)
+        b, np_ = int(r.integers(1, 4)), int(r.integers(1, 4))
+        out.append((i, b, np_, sq, sk, DTYPES[int(r.integers(0, 3))], int(r.integers(0, 5))))
+    return out
+
+
+@pytest.mark.parametrize("i,b,np_,sq,sk,dtype,kind", draw_softmax(303, 60))
+def test_softmax_with_and_without_dropout(device, i, b, np_, sq, sk, dtype, kind):
+    """kind 0: causal; 1: key padding; 2: per-query mask; 3: shared mask; 4: rows fully masked."""
+    r = np.random.default_rng(1000 + i)
+    scale = float(r.choice([0.125, 0.5, 1.0]))
+    p = float(r.choice([0.0, 0.1, 0.3]))
+    seed, offset = 50 + i, 4 * i
+    x = randn((b, np_, sq, sk), dtype, 13 * i, std=2.0)
+    g = randn((b, np_, sq, sk), dtype, 13 * i + 1)
+    k = _C.get_softmax_kernel()
+    if kind == 0:
+        hidden = cf.causal_hidden(sq, sk)
+        mask = None
+        xin, gin = x.view(b * np_, sq, sk), g.view(b * np_, sq, sk)
+    else:
+        if kind == 1:
+            valid = r.integers(1, sk + 1, size=b)
+            m = np.arange(sk)[None, :] >= valid[:, None]
+            mask = torch.from_numpy(m).view(b, 1, 1, sk)
+        elif kind == 2:
+            m = r.random((b, 1, sq, sk)) < 0.4
+            m[..., 0] = False
+            mask = torch.from_numpy(m)
+        elif kind == 3:
+            m = r.random((1, 1, sq, sk)) < 0.4
+            m[..., 0] = False
+            mask = torch.from_numpy(m)
+        else:
+            m = r.random((b, 1, sq, sk)) < 0.3
+            m[:, :, ::2, :] = True
+            mask = torch.from_numpy(m)
+        hidden = mask.numpy()
+        xin, gin = x, g
+    xd, gd = xin.to(device), gin.to(device)
+    md = None if mask is None else mask.to(device)
+    xv, gv = f64(xin), f64(gin)
+    if p == 0.0:
+        if mask is None:
+            y = k.fused_scaled_upper_triang_masked_softmax_forward(xd, scale)
+            dx = k.fused_scaled_upper_triang_masked_softmax_backward(gd, y, scale)
+        else:
+            y = k.fused_scaled_masked_softmax_forward(xd, md, scale)
+            dx = k.fused_scaled_masked_softmax_backward(gd, y, scale, mask=md)
+        check(y, cf.softmax_masked_fwd(xv, hidden, scale), "softmax fwd", atol=1e-9)
+        check(dx, cf.softmax_bwd(gv, f64(y), scale), "softmax bwd", atol=2e-7)
+    else:
+        out, stats = k.softmax_dropout_forward(xd, md, scale, p, seed, offset)
+        keep = philox.keep_mask(x.numel(), p, seed, offset).reshape(xv.shape).astype(bool)
+        check(out, cf.softmax_dropout_fwd(xv, hidden, scale, keep, p), "softmax dropout fwd", atol=1e-9)
+        dx = k.softmax_dropout_backward(gd, xd, stats, md, scale, p, seed, offset)
+        check(dx, cf.softmax_dropout_bwd(gv, xv, hidden, scale, keep, p), "softmax dropout bwd", atol=3e-7)
+
+
+@pytest.mark.parametrize("i,n1,n2,dtype,flags", draw_cases(404, 50))
+def test_elementwise(device, i, n1, n2, dtype, flags):
+    has_bias, has_res = flags[0], flags[1]
+    p = [0.0, 0.1, 0.6][i % 3]
+    seed, offset = 9 + i, 4 * i
+    x = randn((n1, n2), dtype, 17 * i, std=1.5)
+    g = randn((n1, n2), dtype, 17 * i + 1)
+    bias = randn((n2,), dtype, 17 * i + 2, std=0.3) if has_bias else None
+    res = randn((n1, n2), dtype, 17 * i + 3) if has_res else None
+    k = _C.get_fused_elementwise_kernel()
+    name = NP_NAME[dtype]
+    D = lambda t: None if t is None else t.to(device)
+    F = lambda t: None if t is None else f64(t)
+    col = 1e-5 * np.sqrt(n1) + 1e-6
+    y = k.bias_gelu_forward(D(x), D(bias))
+    check(y, cf.bias_gelu_fwd(f64(x), F(bias)), "gelu fwd", atol=1e-6)
+    dx, db = k.bias_gelu_backward(D(g), D(x), D(bias), need_bias_grad=has_bias)
+    odx, _ = cf.bias_gelu_bwd(f64(g), f64(x), F(bias), out=name)
+    check(dx, cf.bias_gelu_bwd(f64(g), f64(x), F(bias))[0], "gelu bwd", atol=1e-6)
+    if has_bias:
+        check(db, f64(dx).sum(0), "gelu dbias", atol=3 * col, min_exact=0.97, max_ulp=2)
+    out = k.bias_dropout_add_forward(D(x), D(bias), D(res), p, seed, offset)
+    keep = philox.keep_mask(n1 * n2, p, seed, offset).reshape(n1, n2).astype(bool) if p > 0 else None
+    check(out, cf.bias_dropout_add_fwd(f64(x), F(bias), F(res), keep, p), "bda fwd", atol=1e-6, min_exact=0.99)
+    ddx, ddb = k.bias_dropout_add_backward(D(g), p, seed, offset, need_bias_grad=has_bias)
+    check(ddx, cf.bias_dropout_add_bwd(f64(g), keep, p)[0], "bda bwd", atol=1e-6)
+    if has_bias:
+        check(ddb, f64(ddx).sum(0), "bda dbias", atol=3 * col, min_exact=0.97, max_ulp=2)
