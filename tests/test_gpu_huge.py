@@ -1,0 +1,105 @@
+"""Tensors of more than 2^31 elements: every kernel family indexes with 64-bit
+offsets.  Inputs are generated on the GPU; rows from the far end of each tensor
+(beyond the 32-bit element range) are checked against the oracle."""
+import numpy as np
+import pytest
+import torch
+
+from helpers import check, f64
+from oracle import closed_form as cf
+from oracle import philox
+from oslo_amd.torch import _C
+from test_gpu_fullsize import gpu_randn
+
+pytestmark = pytest.mark.gpu
+
+BF16 = torch.bfloat16
+
+
+def far_rows(n1, n2):
+    """Row indices whose elements start beyond 2^31 and beyond 2^32 where present."""
+    rows = {0, n1 - 1, n1 - 2}
+    for limit in (2 ** 31, 2 ** 32):
+        r = limit // n2 + 1
+        if r < n1:
+            rows.update((r, min(n1 - 1, r + 7)))
+    return torch.tensor(sorted(rows))
+
+
+def test_norm_and_elementwise_beyond_2_31_elements(device):
+    n1, n2 = 140000, 32768  # 4.59e9 elements: beyond 2^32 as well
+    assert n1 * n2 > 2 ** 32
+    x = gpu_randn((n1, n2), BF16, 1, device)
+    gamma = gpu_randn((n2,), BF16, 2, device, std=0.1, mean=1.0)
+    beta = gpu_randn((n2,), BF16, 3, device, std=0.1)
+    ln = _C.get_layernorm_kernel()
+    ek = _C.get_fused_elementwise_kernel()
+    rows = far_rows(n1, n2)
+    sel = rows.to(device)
+    # LayerNorm forward + backward (the backward reuses x as the upstream gradient)
+    y, mean, invvar = ln.layer_norm_forward_affine(x, (n2,), gamma, beta, 1e-5)
+    oy, omean, oinv = cf.layer_norm_fwd(f64(x[sel]), f64(gamma), f64(beta), 1e-5)
+    check(y[sel], oy, "huge ln fwd", atol=1e-5)
+    assert np.allclose(f64(mean[sel]), omean, atol=1e-5)
+    dx, dg, db = ln.layer_norm_backward_affine(y, mean, invvar, x, (n2,), gamma, beta, 1e-5)
+    odx, _, _ = cf.layer_norm_bwd(f64(y[sel]), f64(x[sel]), f64(mean[sel]), f64(invvar[sel]), f64(gamma))
+    check(dx[sel], odx, "huge ln bwd", atol=1e-5)
+    assert torch.isfinite(dg.float()).all() and torch.isfinite(db.float()).all()
+    del dx
+    # bias-dropout-add forward into y's storage is not allowed (no aliasing): fresh output
+    p, seed, offset = 0.1, 11, 4
+    out = ek.bias_dropout_add_forward(x, beta, y, p, seed, offset)
+    keep = np.stack([philox.keep_mask(n2, p, seed, offset, first_element=int(r) * n2) for r in rows]).astype(bool)
+    check(out[sel], cf.bias_dropout_add_fwd(f64(x[sel]), f64(beta), f64(y[sel]), keep, p), "huge bda fwd", atol=1e-6,
+          min_exact=0.99)
+    del out
+    act = ek.bias_gelu_forward(x, beta)
+    check(act[sel], cf.bias_gelu_fwd(f64(x[sel]), f64(beta)), "huge gelu fwd", atol=1e-6)
+    dact, dbias = ek.bias_gelu_backward(y, x, beta)
+    check(dact[sel], cf.bias_gelu_bwd(f64(y[sel]), f64(x[sel]), f64(beta))[0], "huge gelu bwd", atol=1e-6)
+    assert torch.isfinite(dbias.float()).all()
+
+
+def test_softmax_beyond_2_31_elements(device):
+    ab, s = 18, 11008  # 2.18e9 elements
+    assert ab * s * s > 2 ** 31
+    x = gpu_randn((ab, s, s), BF16, 5, device)
+    sm = _C.get_softmax_kernel()
+    scale, p, seed, offset = 0.125, 0.1, 21, 8
+    rows = far_rows(ab * s, s)
+    sel = rows.to(device)
+    qi = (rows % s).numpy()
+    hidden = np.arange(s)[None, :] > qi[:, None]
+    y = sm.fused_scaled_upper_triang_masked_softmax_forward(x, scale)
+    check(y.view(-1, s)[sel], cf.softmax_masked_fwd(f64(x.view(-1, s)[sel]), hidden, scale), "huge softmax fwd",
+          atol=1e-9)
+    dx = sm.fused_scaled_upper_triang_masked_softmax_backward(x, y, scale)
+    check(dx.view(-1, s)[sel], cf.softmax_bwd(f64(x.view(-1, s)[sel]), f64(y.view(-1, s)[sel]), scale),
+          "huge softmax bwd", atol=2e-7)
+    del dx, y
+    out, stats = sm.softmax_dropout_forward(x, None, scale, p, seed, offset)
+    keep = np.stack([philox.keep_mask(s, p, seed, offset, first_element=int(r) * s) for r in rows]).astype(bool)
+    check(out.view(-1, s)[sel], cf.softmax_dropout_fwd(f64(x.view(-1, s)[sel]), hidden, scale, keep, p),
+          "huge softmax dropout fwd", atol=1e-9)
+    ddx = sm.softmax_dropout_backward(out, x, stats, None, scale, p, seed, offset)
+    check(ddx.view(-1, s)[sel],
+          cf.softmax_dropout_bwd(f64(out.view(-1, s)[sel]), f64(x.view(-1, s)[sel]), hidden, scale, keep, p),
+          "huge softmax dropout bwd", atol=3e-7)
+
+
+def test_adam_on_a_tensor_beyond_2_31_elements(device):
+    n = 2 ** 31 + 4099
+    g = torch.empty(n, device=device, dtype=BF16).normal_()
+    p = torch.empty(n, device=device, dtype=BF16).normal_()
+    m = torch.zeros(n, device=device, dtype=BF16)
+    v = torch.zeros(n, device=device, dtype=BF16)
+    tail = slice(n - 5000, n)
+    head = slice(0, 5000)
+    p0 = [f64(p[head]), f64(p[tail])]
+    g0 = [f64(g[head]), f64(g[tail])]
+    _C.get_adam_kernel().multi_tensor_adam(0, None, [[g], [p], [m], [v]], 1e-2, 0.9, 0.999, 1e-8, 1, 1, 1, 0.01)
+    for sl, pp, gg in ((head, p0[0], g0[0]), (tail, p0[1], g0[1])):
+        want = cf.adam_step(gg, pp, np.zeros_like(pp), np.zeros_like(pp), 1e-2, 0.9, 0.999, 1e-8, 1, 1, True, 0.01)
+        check(p[sl], want[0], "huge adam p", atol=5e-7, min_exact=0.99)
+        check(m[sl], want[1], "huge adam m", atol=1e-7, min_exact=0.99)
+        check(v[sl], want[2], "huge adam v", atol=1e-8, min_exact=0.99)
