@@ -37,6 +37,7 @@ extern "C" {
 #define OSLO_DTYPE_F32 0
 #define OSLO_DTYPE_F16 1
 #define OSLO_DTYPE_BF16 2
+#define OSLO_DTYPE_F64 3 /* LayerNorm / RMSNorm entry points only */
 
 /* ops for oslo_workspace_bytes */
 #define OSLO_OP_LN_BWD 1
@@ -62,8 +63,11 @@ int64_t oslo_workspace_bytes(int op, int64_t n1, int64_t n2);
 /* ---- LayerNorm / RMSNorm ----------------------------------------------- *
  * x is [n1, n2] of dtype_in; y, gamma, beta have dtype_out; mean / invvar are
  * fp32 [n1].  Allowed (dtype_in, dtype_out): (f32,f32) (f32,f16) (f32,bf16)
- * (f16,f16) (bf16,bf16) -- the matrix of
- * oslo/torch/_C/csrc/includes/type_shim.h:128-237 without fp64.
+ * (f16,f16) (bf16,bf16) (f64,f64) -- the matrix of
+ * oslo/torch/_C/csrc/includes/type_shim.h:128-237.  For (f64,f64) every
+ * tensor, mean and invvar included, is double and accumulation is double
+ * (type_shim.h:172-186: U = double); the workspace is not used.  That pair is
+ * a plain two-pass kernel meant for checking, not for throughput.
  * gamma == NULL (then beta must be NULL too) selects the non-affine form.  */
 
 /* Replaces layer_norm_forward, layer_norm_forward_affine and
@@ -72,7 +76,7 @@ int64_t oslo_workspace_bytes(int op, int64_t n1, int64_t n2);
  * cuda_layer_norm, fused_layer_norm.cu:771-788).
  * y = (x - mean) * invvar * gamma + beta evaluated in fp32, rounded once.  */
 int oslo_ln_fwd(const void *x, const void *gamma, const void *beta, void *y,
-                float *mean, float *invvar, int64_t n1, int64_t n2, double eps,
+                void *mean, void *invvar, int64_t n1, int64_t n2, double eps,
                 int dtype_in, int dtype_out, void *stream);
 
 /* Replaces layer_norm_backward and layer_norm_backward_affine
@@ -80,8 +84,8 @@ int oslo_ln_fwd(const void *x, const void *gamma, const void *beta, void *y,
  * fused_layer_norm.cu:908-935; three launches there, one pass + a finalize
  * here).  dy, gamma, dgamma, dbeta have dtype_out; x, dx have dtype_in.
  * dgamma / dbeta may be NULL only when gamma is NULL.                      */
-int oslo_ln_bwd(const void *dy, const void *x, const float *mean,
-                const float *invvar, const void *gamma, void *dx, void *dgamma,
+int oslo_ln_bwd(const void *dy, const void *x, const void *mean,
+                const void *invvar, const void *gamma, void *dx, void *dgamma,
                 void *dbeta, void *workspace, int64_t workspace_bytes,
                 int64_t n1, int64_t n2, int dtype_in, int dtype_out,
                 void *stream);
@@ -92,14 +96,14 @@ int oslo_ln_bwd(const void *dy, const void *x, const float *mean,
  * y = gamma * round_out(x * invvar): the normalised value is rounded to
  * dtype_out before the scale, as fused_layer_norm.cu:338 and
  * oslo/torch/nn/modules/layer_norm.py:27-30 both do.                       */
-int oslo_rms_fwd(const void *x, const void *gamma, void *y, float *invvar,
+int oslo_rms_fwd(const void *x, const void *gamma, void *y, void *invvar,
                  int64_t n1, int64_t n2, double eps, int dtype_in,
                  int dtype_out, void *stream);
 
 /* Replaces rms_norm_backward and rms_norm_backward_affine
  * (FusedLayerNormBinder.cpp:360-402 -> cuda_rms_norm_gradient,
  * fused_layer_norm.cu:937-963).                                            */
-int oslo_rms_bwd(const void *dy, const void *x, const float *invvar,
+int oslo_rms_bwd(const void *dy, const void *x, const void *invvar,
                  const void *gamma, void *dx, void *dgamma, void *workspace,
                  int64_t workspace_bytes, int64_t n1, int64_t n2, int dtype_in,
                  int dtype_out, void *stream);

@@ -45,9 +45,21 @@ inline bool valid_dtype(int d) {
   return d == OSLO_DTYPE_F32 || d == OSLO_DTYPE_F16 || d == OSLO_DTYPE_BF16;
 }
 
-inline int dtype_size(int d) { return d == OSLO_DTYPE_F32 ? 4 : 2; }
+inline int dtype_size(int d) {
+  return d == OSLO_DTYPE_F64 ? 8 : d == OSLO_DTYPE_F32 ? 4 : 2;
+}
 
 inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
+// Double-precision LayerNorm / RMSNorm (norm_f64.hip); every pointer is to
+// double data.
+int launch_norm_f64_fwd(bool rms, const void *x, const void *gamma,
+                        const void *beta, void *y, void *mean, void *invvar,
+                        int64_t n1, int64_t n2, double eps, hipStream_t st);
+int launch_norm_f64_bwd(bool rms, const void *dy, const void *x,
+                        const void *mean, const void *invvar,
+                        const void *gamma, void *dx, void *dgamma, void *dbeta,
+                        int64_t n1, int64_t n2, hipStream_t st);
 
 // Column-partial workspace layout shared by the backward kernels and the
 // finalize kernel: `narrays` fp32 arrays of [parts, cols].

@@ -1099,6 +1099,13 @@ static int zero_params(void *p, int64_t nbytes, hipStream_t st) {
 }
 
 static int check_norm_dtypes(int din, int dout) {
+  if (din == OSLO_DTYPE_F64 || dout == OSLO_DTYPE_F64) {
+    if (din == dout) return OSLO_OK;
+    return fail(OSLO_ERR_UNSUPPORTED,
+                "dtype pair (in=%d, out=%d) unsupported: double input and "
+                "double output go together",
+                din, dout);
+  }
   if (!valid_dtype(din) || !valid_dtype(dout))
     return fail(OSLO_ERR_INVALID_ARGUMENT, "unknown dtype (%d, %d)", din, dout);
   if (din != OSLO_DTYPE_F32 && din != dout)
@@ -1123,8 +1130,8 @@ static int check_norm_dtypes(int din, int dout) {
   } while (0)
 
 static int norm_fwd_entry(bool rms, const void *x, const void *gamma,
-                          const void *beta, void *y, float *mean,
-                          float *invvar, int64_t n1, int64_t n2, double eps,
+                          const void *beta, void *y, void *mean_,
+                          void *invvar_, int64_t n1, int64_t n2, double eps,
                           int din, int dout, void *stream) {
   int rc = check_norm_dtypes(din, dout);
   if (rc != OSLO_OK) return rc;
@@ -1132,12 +1139,17 @@ static int norm_fwd_entry(bool rms, const void *x, const void *gamma,
                (long long)n1, (long long)n2);
   OSLO_REQUIRE(n2 <= 0x7fffffff, "norm fwd: n2 too large");
   if (n1 == 0) return OSLO_OK;
-  OSLO_REQUIRE(x && y && invvar, "norm fwd: null tensor pointer");
-  OSLO_REQUIRE(rms || mean, "layer norm fwd: null mean pointer");
+  OSLO_REQUIRE(x && y && invvar_, "norm fwd: null tensor pointer");
+  OSLO_REQUIRE(rms || mean_, "layer norm fwd: null mean pointer");
   OSLO_REQUIRE(rms || (gamma == nullptr) == (beta == nullptr),
                "layer norm fwd: gamma and beta must both be given or both be "
                "NULL");
   hipStream_t st = (hipStream_t)stream;
+  if (din == OSLO_DTYPE_F64)
+    return launch_norm_f64_fwd(rms, x, gamma, beta, y, mean_, invvar_, n1, n2,
+                               eps, st);
+  float *mean = static_cast<float *>(mean_);
+  float *invvar = static_cast<float *>(invvar_);
   if (rms)
     OSLO_NORM_DISPATCH(din, dout, true, launch_norm_fwd, x, gamma, nullptr, y,
                        nullptr, invvar, n1, n2, (float)eps, st);
@@ -1146,7 +1158,7 @@ static int norm_fwd_entry(bool rms, const void *x, const void *gamma,
 }
 
 static int norm_bwd_entry(bool rms, const void *dy, const void *x,
-                          const float *mean, const float *invvar,
+                          const void *mean_, const void *invvar_,
                           const void *gamma, void *dx, void *dgamma,
                           void *dbeta, void *ws, int64_t ws_bytes, int64_t n1,
                           int64_t n2, int din, int dout, void *stream) {
@@ -1167,9 +1179,14 @@ static int norm_bwd_entry(bool rms, const void *dy, const void *x,
     if (rc0 == OSLO_OK) rc0 = zero_params(dbeta, n2 * dtype_size(dout), st0);
     return rc0;
   }
-  OSLO_REQUIRE(dy && x && invvar && dx, "norm bwd: null tensor pointer");
-  OSLO_REQUIRE(rms || mean, "layer norm bwd: null mean pointer");
+  OSLO_REQUIRE(dy && x && invvar_ && dx, "norm bwd: null tensor pointer");
+  OSLO_REQUIRE(rms || mean_, "layer norm bwd: null mean pointer");
   hipStream_t st = (hipStream_t)stream;
+  if (din == OSLO_DTYPE_F64)
+    return launch_norm_f64_bwd(rms, dy, x, mean_, invvar_, gamma, dx, dgamma,
+                               dbeta, n1, n2, st);
+  const float *mean = static_cast<const float *>(mean_);
+  const float *invvar = static_cast<const float *>(invvar_);
   if (rms)
     OSLO_NORM_DISPATCH(din, dout, true, launch_norm_bwd, dy, x, nullptr, invvar,
                        gamma, dx, dgamma, nullptr, ws, ws_bytes, n1, n2, st);
@@ -1182,21 +1199,21 @@ static int norm_bwd_entry(bool rms, const void *dy, const void *x,
 extern "C" {
 
 int oslo_ln_fwd(const void *x, const void *gamma, const void *beta, void *y,
-                float *mean, float *invvar, int64_t n1, int64_t n2, double eps,
+                void *mean, void *invvar, int64_t n1, int64_t n2, double eps,
                 int dtype_in, int dtype_out, void *stream) {
   return oslo::norm_fwd_entry(false, x, gamma, beta, y, mean, invvar, n1, n2,
                               eps, dtype_in, dtype_out, stream);
 }
 
-int oslo_rms_fwd(const void *x, const void *gamma, void *y, float *invvar,
+int oslo_rms_fwd(const void *x, const void *gamma, void *y, void *invvar,
                  int64_t n1, int64_t n2, double eps, int dtype_in,
                  int dtype_out, void *stream) {
   return oslo::norm_fwd_entry(true, x, gamma, nullptr, y, nullptr, invvar, n1,
                               n2, eps, dtype_in, dtype_out, stream);
 }
 
-int oslo_ln_bwd(const void *dy, const void *x, const float *mean,
-                const float *invvar, const void *gamma, void *dx, void *dgamma,
+int oslo_ln_bwd(const void *dy, const void *x, const void *mean,
+                const void *invvar, const void *gamma, void *dx, void *dgamma,
                 void *dbeta, void *workspace, int64_t workspace_bytes,
                 int64_t n1, int64_t n2, int dtype_in, int dtype_out,
                 void *stream) {
@@ -1205,7 +1222,7 @@ int oslo_ln_bwd(const void *dy, const void *x, const float *mean,
                               dtype_in, dtype_out, stream);
 }
 
-int oslo_rms_bwd(const void *dy, const void *x, const float *invvar,
+int oslo_rms_bwd(const void *dy, const void *x, const void *invvar,
                  const void *gamma, void *dx, void *dgamma, void *workspace,
                  int64_t workspace_bytes, int64_t n1, int64_t n2, int dtype_in,
                  int dtype_out, void *stream) {

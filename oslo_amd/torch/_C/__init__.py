@@ -34,6 +34,7 @@ OSLO_OP_BIAS_DROPOUT_ADD_NORM_BWD = 5
 ABI_VERSION = 1
 
 _DTYPE_CODE = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}
+OSLO_DTYPE_F64 = 3  # LayerNorm / RMSNorm only
 
 _lib = None
 _lib_lock = threading.Lock()
@@ -182,14 +183,23 @@ def _stream(t):
     return torch.cuda.current_stream(t.device).cuda_stream
 
 
-def _dtype_code(t, what):
+def _dtype_code(t, what, allow_f64=False):
+    if allow_f64 and t.dtype == torch.float64:
+        return OSLO_DTYPE_F64
     try:
         return _DTYPE_CODE[t.dtype]
     except KeyError:
         raise RuntimeError(
             "%s: dtype %s is not supported by the HIP kernels "
-            "(float32, float16 and bfloat16 are)" % (what, t.dtype)
+            "(float32, float16 and bfloat16 are%s)"
+            % (what, t.dtype, "" if allow_f64 else "; float64 only by the norms")
         ) from None
+
+
+def _stat_dtype(t):
+    # FusedLayerNormBinder.cpp:146-152: the statistics are fp32 for 16-bit
+    # inputs and have the input's type otherwise
+    return torch.float64 if t.dtype == torch.float64 else torch.float32
 
 
 def _check_input(t, name):
@@ -265,9 +275,9 @@ class _LayerNormKernel:
         if gamma is not None:
             _check_param(gamma, normalized_shape, "gamma")
             _check_param(beta, normalized_shape, "beta")
-        din = _dtype_code(input, "input")
+        din = _dtype_code(input, "input", allow_f64=True)
         output = torch.empty_like(input, dtype=out_dtype)
-        dout = _dtype_code(output, "output")
+        dout = _dtype_code(output, "output", allow_f64=True)
         for name, t in (("gamma", gamma), ("beta", beta)):
             if t is not None:
                 _check_input(t, name)
@@ -276,7 +286,7 @@ class _LayerNormKernel:
                         "%s has dtype %s but the output dtype is %s"
                         % (name, t.dtype, out_dtype)
                     )
-        invvar = torch.empty(n1, dtype=torch.float32, device=input.device)
+        invvar = torch.empty(n1, dtype=_stat_dtype(input), device=input.device)
         with torch.cuda.device_of(input):
             if rms:
                 rc = lib.oslo_rms_fwd(
@@ -285,7 +295,7 @@ class _LayerNormKernel:
                 )
                 _check(rc, lib)
                 return [output, invvar]
-            mean = torch.empty(n1, dtype=torch.float32, device=input.device)
+            mean = torch.empty(n1, dtype=_stat_dtype(input), device=input.device)
             rc = lib.oslo_ln_fwd(
                 _ptr(input), _ptr(gamma), _ptr(beta), _ptr(output), _ptr(mean),
                 _ptr(invvar), n1, n2, float(eps), din, dout, _stream(input),
@@ -324,8 +334,13 @@ class _LayerNormKernel:
                 "dout of size %s does not match input of size %s"
                 % (list(dout.shape), list(input.shape))
             )
-        din = _dtype_code(input, "input")
-        dcode = _dtype_code(dout, "dout")
+        din = _dtype_code(input, "input", allow_f64=True)
+        dcode = _dtype_code(dout, "dout", allow_f64=True)
+        for name, t in (("invvar", invvar), ("mean", mean)):
+            if t is not None and t.dtype != _stat_dtype(input):
+                raise RuntimeError(
+                    "%s has dtype %s, expected %s" % (name, t.dtype, _stat_dtype(input))
+                )
         grad_input = torch.empty_like(input)
         grad_gamma = grad_beta = None
         ws, ws_bytes = None, 0
