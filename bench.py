@@ -184,6 +184,9 @@ def kernel_table(L, dev, iters):
     for cfg, ab, s, tdt, code, esz, scale in (
         ("cfg1", 48, 512, torch.float32, F32, 4, 0.125),
         ("cfg5", 256, 2048, torch.bfloat16, BF16, 2, 1.0 / math.sqrt(96.0)),
+        # short rows (batch 256 x 12 heads at sequence length 128): several
+        # rows lie side by side in one wavefront
+        ("seq128", 3072, 128, torch.bfloat16, BF16, 2, 0.125),
     ):
         T = ab * s * s * esz
         f = (s + 1) / (2.0 * s)

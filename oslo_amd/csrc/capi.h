@@ -26,6 +26,8 @@ struct Tuning {
   int norm_bwd_vpl;
   int norm_bwd_blocks_per_cu;
   int softmax_rows_per_wave;
+  int softmax_lanes_per_row;
+  int softmax_fwd_elems;
   int eltwise_unroll;
   int eltwise_rowgroups;
   int eltwise_fwd_steps;

@@ -338,6 +338,20 @@ template <typename Op> __device__ __forceinline__ float row16_allreduce(float v)
   return readlane(v, 0);
 }
 
+// Reduction within each group of LPR (8, 16 or 32) consecutive lanes; every
+// lane of a group receives its group's result (each step is symmetric, so the
+// lanes of a group hold the same bits).
+template <typename Op, int LPR>
+__device__ __forceinline__ float group_allreduce(float v) {
+  static_assert(LPR == 8 || LPR == 16 || LPR == 32, "group size");
+  v = Op::apply(v, dpp_mov<kDppQuadSwap1>(v));
+  v = Op::apply(v, dpp_mov<kDppQuadSwap2>(v));
+  v = Op::apply(v, dpp_mov<kDppRowHalfMirror>(v));
+  if constexpr (LPR >= 16) v = Op::apply(v, dpp_mov<kDppRowMirror>(v));
+  if constexpr (LPR >= 32) v = Op::apply(v, __shfl_xor(v, 16));
+  return v;
+}
+
 // Reduction over the WPR consecutive waves that share one row.  `red` is LDS
 // scratch of at least (waves in block) floats, `slot` selects one of two such
 // areas so that back-to-back reductions need only one barrier each.

@@ -3,7 +3,9 @@
 //
 // A row of sk keys is held in registers by `wpr` wavefronts (one wavefront
 // for sk <= 64 * VPL * E); a wavefront processes RPW rows at once so that
-// short rows still keep several 128-bit loads in flight per lane.  Keys that
+// short rows still keep several 128-bit loads in flight per lane, and rows of
+// at most 32 chunks (256 16-bit keys) lie side by side in a wavefront, 8, 16
+// or 32 lanes each, so that no lane idles.  Keys that
 // are masked out are never loaded: the causal kernels stop at the diagonal,
 // the masked kernels read the mask bytes of a chunk first and skip the chunk
 // when all of them are set.  Probabilities of masked keys are written as
@@ -35,9 +37,13 @@ struct SoftmaxGeom {
 
 // Reductions over the wpr (<= 16) consecutive waves of a row: lane 0 of each
 // wave publishes its wave's value in LDS, lane l < wpr then reads the value of
-// wave first + l and one DPP row reduction combines them.
+// wave first + l and one DPP row reduction combines them.  With LPR < 64 a
+// row belongs to LPR consecutive lanes of one wave (wpr == 1) and the
+// reduction stays inside that group.
+template <int LPR = kWave>
 __device__ __forceinline__ float row_reduce_sum(float a, float *red, int wave,
                                                 int first, int wpr, int lane) {
+  if constexpr (LPR < kWave) return group_allreduce<OpSum, LPR>(a);
   a = wave_sum(a);
   if (wpr > 1) {
     if (lane == 0) red[wave] = a;
@@ -48,8 +54,10 @@ __device__ __forceinline__ float row_reduce_sum(float a, float *red, int wave,
   }
   return a;
 }
+template <int LPR = kWave>
 __device__ __forceinline__ float row_reduce_max(float a, float *red, int wave,
                                                 int first, int wpr, int lane) {
+  if constexpr (LPR < kWave) return group_allreduce<OpMax, LPR>(a);
   a = wave_max(a);
   if (wpr > 1) {
     if (lane == 0) red[wave] = a;
@@ -120,7 +128,11 @@ __device__ __forceinline__ void row_setup(const SoftmaxGeom &g, int64_t r,
 // statistics {max of the log2-domain logits, 1 / sum} go to stats[row], from
 // which the backward pass recomputes the probabilities.  A row without a
 // visible key stores {0, -1 / sk}.
-template <typename T, int VPL, int RPW, int MODE, bool DROP>
+//
+// LPR lanes hold a row: 64 (a row takes whole waves), or 8 / 16 / 32 for rows
+// of at most LPR chunks, where a wave works on 64 / LPR rows side by side
+// (then VPL == 1 and wpr == 1).
+template <typename T, int VPL, int RPW, int MODE, bool DROP, int LPR = kWave>
 __global__ __launch_bounds__(1024) void softmax_fwd_kernel(
     const T *__restrict__ x, const uint8_t *__restrict__ mask,
     T *__restrict__ y, float *__restrict__ stats, SoftmaxGeom g, float scale,
@@ -135,11 +147,15 @@ __global__ __launch_bounds__(1024) void softmax_fwd_kernel(
   const int first = rslot * g.wpr;
   const int nchunks = g.sk / E;
   const int cstride = kWave * g.wpr;
-  const int c0 = (wave - first) * kWave + lane;
+  constexpr int SUB = kWave / LPR;  // rows side by side in a wave
+  const int sl = LPR == kWave ? lane : (lane & (LPR - 1));
+  const int c0 = (wave - first) * kWave + sl;
   const float ninf = -__builtin_inff();
 
+  // first row of this lane: the wave's first row plus the lane group's index
   const int64_t rbase =
-      ((int64_t)blockIdx.x * g.rpb + rslot) * RPW;  // first row of this wave
+      ((int64_t)blockIdx.x * g.rpb + rslot) * (RPW * SUB) +
+      (LPR == kWave ? 0 : lane / LPR);
 
   float v[RPW][VPL][E];
   uint32_t mbits[RPW][VPL];  // bit e set: key masked out
@@ -148,7 +164,7 @@ __global__ __launch_bounds__(1024) void softmax_fwd_kernel(
 
 #pragma unroll
   for (int j = 0; j < RPW; ++j) {
-    const int64_t r = rbase + j;
+    const int64_t r = rbase + j * SUB;
     rvalid[j] = r < g.rows;
     int visible = 0;
     const uint8_t *mrow = nullptr;
@@ -227,7 +243,7 @@ __global__ __launch_bounds__(1024) void softmax_fwd_kernel(
   }
 #pragma unroll
   for (int j = 0; j < RPW; ++j)
-    mx[j] = row_reduce_max(mx[j], red[0], wave, first, g.wpr, lane);
+    mx[j] = row_reduce_max<LPR>(mx[j], red[0], wave, first, g.wpr, lane);
   // (one barrier separates the two LDS areas; RPW > 1 implies wpr == 1,
   //  where LDS is not used at all)
 
@@ -250,7 +266,7 @@ __global__ __launch_bounds__(1024) void softmax_fwd_kernel(
   }
 #pragma unroll
   for (int j = 0; j < RPW; ++j)
-    sm[j] = row_reduce_sum(sm[j], red[1], wave, first, g.wpr, lane);
+    sm[j] = row_reduce_sum<LPR>(sm[j], red[1], wave, first, g.wpr, lane);
 
 #pragma unroll
   for (int j = 0; j < RPW; ++j) {
@@ -298,7 +314,7 @@ __global__ __launch_bounds__(1024) void softmax_fwd_kernel(
 // recomputed as exp2(x * scale * log2 e - stats[row][0]) * stats[row][1], the
 // keep bits are regenerated from (seed, offset), and
 // dx = scale * y * (dp - sum_k dp_k y_k) with dp = keep * dy / (1 - p).
-template <typename T, int VPL, int RPW, int MODE>
+template <typename T, int VPL, int RPW, int MODE, int LPR = kWave>
 __global__ __launch_bounds__(1024) void softmax_dropout_bwd_kernel(
     const T *__restrict__ dy, const T *__restrict__ x,
     const float *__restrict__ stats, const uint8_t *__restrict__ mask,
@@ -312,8 +328,11 @@ __global__ __launch_bounds__(1024) void softmax_dropout_bwd_kernel(
   const int first = rslot * g.wpr;
   const int nchunks = g.sk / E;
   const int cstride = kWave * g.wpr;
-  const int c0 = (wave - first) * kWave + lane;
-  const int64_t rbase = ((int64_t)blockIdx.x * g.rpb + rslot) * RPW;
+  constexpr int SUB = kWave / LPR;
+  const int sl = LPR == kWave ? lane : (lane & (LPR - 1));
+  const int c0 = (wave - first) * kWave + sl;
+  const int64_t rbase = ((int64_t)blockIdx.x * g.rpb + rslot) * (RPW * SUB) +
+                        (LPR == kWave ? 0 : lane / LPR);
   const float c2 = scale * kLog2e;
 
   float yv[RPW][VPL][E], gv[RPW][VPL][E];
@@ -324,7 +343,7 @@ __global__ __launch_bounds__(1024) void softmax_dropout_bwd_kernel(
 
 #pragma unroll
   for (int j = 0; j < RPW; ++j) {
-    const int64_t r = rbase + j;
+    const int64_t r = rbase + j * SUB;
     rvalid[j] = r < g.rows;
     int visible = 0;
     const uint8_t *mrow = nullptr;
@@ -409,7 +428,7 @@ __global__ __launch_bounds__(1024) void softmax_dropout_bwd_kernel(
   }
 #pragma unroll
   for (int j = 0; j < RPW; ++j)
-    s[j] = row_reduce_sum(s[j], red, wave, first, g.wpr, lane);
+    s[j] = row_reduce_sum<LPR>(s[j], red, wave, first, g.wpr, lane);
 
 #pragma unroll
   for (int j = 0; j < RPW; ++j) {
@@ -434,7 +453,7 @@ __global__ __launch_bounds__(1024) void softmax_dropout_bwd_kernel(
   }
 }
 
-template <typename T, int VPL, int RPW, int MODE>
+template <typename T, int VPL, int RPW, int MODE, int LPR = kWave>
 __global__ __launch_bounds__(1024) void softmax_bwd_kernel(
     const T *__restrict__ dy, const T *__restrict__ y,
     const uint8_t *__restrict__ mask, T *__restrict__ dx, SoftmaxGeom g,
@@ -449,9 +468,12 @@ __global__ __launch_bounds__(1024) void softmax_bwd_kernel(
   const int first = rslot * g.wpr;
   const int nchunks = g.sk / E;
   const int cstride = kWave * g.wpr;
-  const int c0 = (wave - first) * kWave + lane;
+  constexpr int SUB = kWave / LPR;
+  const int sl = LPR == kWave ? lane : (lane & (LPR - 1));
+  const int c0 = (wave - first) * kWave + sl;
 
-  const int64_t rbase = ((int64_t)blockIdx.x * g.rpb + rslot) * RPW;
+  const int64_t rbase = ((int64_t)blockIdx.x * g.rpb + rslot) * (RPW * SUB) +
+                        (LPR == kWave ? 0 : lane / LPR);
 
   float yv[RPW][VPL][E], gv[RPW][VPL][E];
   bool skip[RPW][VPL];
@@ -460,7 +482,7 @@ __global__ __launch_bounds__(1024) void softmax_bwd_kernel(
 
 #pragma unroll
   for (int j = 0; j < RPW; ++j) {
-    const int64_t r = rbase + j;
+    const int64_t r = rbase + j * SUB;
     rvalid[j] = r < g.rows;
     int visible = 0;
     const uint8_t *mrow = nullptr;
@@ -485,7 +507,7 @@ __global__ __launch_bounds__(1024) void softmax_bwd_kernel(
     }
     if constexpr (MODE != kModeDense) {
       // a row with no visible key holds the uniform distribution: read it all
-      anyvis = row_reduce_max(anyvis, red[0], wave, first, g.wpr, lane);
+      anyvis = row_reduce_max<LPR>(anyvis, red[0], wave, first, g.wpr, lane);
       if (g.wpr > 1) __syncthreads();
       if (anyvis == 0.f) {
 #pragma unroll
@@ -535,7 +557,7 @@ __global__ __launch_bounds__(1024) void softmax_bwd_kernel(
   }
 #pragma unroll
   for (int j = 0; j < RPW; ++j)
-    s[j] = row_reduce_sum(s[j], red[1], wave, first, g.wpr, lane);
+    s[j] = row_reduce_sum<LPR>(s[j], red[1], wave, first, g.wpr, lane);
 
 #pragma unroll
   for (int j = 0; j < RPW; ++j) {
@@ -690,13 +712,14 @@ __global__ __launch_bounds__(256) void softmax_bwd_generic_kernel(
 // ---------------------------------------------------------------------------
 struct SoftmaxPlan {
   int vpl, rpw, wpr, rpb;
+  int lpr;  // lanes that hold a row: 64, or 8 / 16 / 32 for short rows
   bool ok;
 };
 
 // max_elems: elements of one operand a lane may hold (register budget).
 static SoftmaxPlan plan_softmax(int64_t sk, int E, int max_elems,
-                                int default_rpw) {
-  SoftmaxPlan p{0, 1, 1, 1, false};
+                                int default_rpw, int one_chunk_rpw) {
+  SoftmaxPlan p{0, 1, 1, 1, kWave, false};
   if (sk % E != 0) return p;
   const int64_t nchunks = sk / E;
   const int maxvpl = max_elems / E;  // 8 or 4 for 16-bit types, 16 or 8 for fp32
@@ -705,11 +728,21 @@ static SoftmaxPlan plan_softmax(int64_t sk, int E, int max_elems,
   const int64_t need = ceil_div(nchunks, kWave * wpr);
   int vpl = need <= 1 ? 1 : need <= 2 ? 2 : need <= 4 ? 4 : 8;
   int rpw = 1;
+  // short rows: several rows side by side in a wave instead of idle lanes
+  if (nchunks <= 32 && g_tune.softmax_lanes_per_row != kWave) {
+    p.lpr = nchunks <= 8 ? 8 : nchunks <= 16 ? 16 : 32;
+    if (g_tune.softmax_lanes_per_row == 8 || g_tune.softmax_lanes_per_row == 16 ||
+        g_tune.softmax_lanes_per_row == 32)
+      if (g_tune.softmax_lanes_per_row >= p.lpr) p.lpr = g_tune.softmax_lanes_per_row;
+  }
   if (wpr == 1) {
-    // rows a wave handles at once; measured best on MI355X: one, or two
-    // for the forward with a mask tensor (its loads wait for the mask bytes)
-    int want = g_tune.softmax_rows_per_wave > 0 ? g_tune.softmax_rows_per_wave
-                                                : default_rpw;
+    // row sets a wave handles at once; measured best on MI355X: one, or two
+    // for the forward with a mask tensor (its loads wait for the mask bytes);
+    // a forward that holds one chunk per lane (rows of up to 512 16-bit
+    // keys) wants four, which hides its two dependent reductions
+    int want = g_tune.softmax_rows_per_wave > 0
+                   ? g_tune.softmax_rows_per_wave
+                   : (vpl == 1 ? one_chunk_rpw : default_rpw);
     rpw = want >= 4 ? 4 : (want >= 2 ? 2 : 1);
     while (rpw > 1 && (rpw * vpl * E > max_elems || rpw * vpl > 8)) rpw >>= 1;
   }
@@ -725,25 +758,39 @@ static SoftmaxPlan plan_softmax(int64_t sk, int E, int max_elems,
 constexpr int kFwdMaxElems = 64;  // one operand resident
 constexpr int kBwdMaxElems = 32;  // two operands resident
 
-#define OSLO_SM_CASES(LAUNCH)        \
-  if (pl.vpl == 1 && pl.rpw == 1) {  \
-    LAUNCH(1, 1);                    \
+#define OSLO_SM_CASES_LPR(LAUNCH, LPR_)    \
+  if (pl.rpw == 1) {                       \
+    LAUNCH(1, 1, LPR_);                    \
+  } else if (pl.rpw == 2) {                \
+    LAUNCH(1, 2, LPR_);                    \
+  } else {                                 \
+    LAUNCH(1, 4, LPR_);                    \
+  }
+#define OSLO_SM_CASES(LAUNCH)              \
+  if (pl.lpr == 8) {                       \
+    OSLO_SM_CASES_LPR(LAUNCH, 8)           \
+  } else if (pl.lpr == 16) {               \
+    OSLO_SM_CASES_LPR(LAUNCH, 16)          \
+  } else if (pl.lpr == 32) {               \
+    OSLO_SM_CASES_LPR(LAUNCH, 32)          \
+  } else if (pl.vpl == 1 && pl.rpw == 1) { \
+    LAUNCH(1, 1, kWave);                   \
   } else if (pl.vpl == 1 && pl.rpw == 2) { \
-    LAUNCH(1, 2);                    \
+    LAUNCH(1, 2, kWave);                   \
   } else if (pl.vpl == 1 && pl.rpw == 4) { \
-    LAUNCH(1, 4);                    \
+    LAUNCH(1, 4, kWave);                   \
   } else if (pl.vpl == 2 && pl.rpw == 1) { \
-    LAUNCH(2, 1);                    \
+    LAUNCH(2, 1, kWave);                   \
   } else if (pl.vpl == 2 && pl.rpw == 2) { \
-    LAUNCH(2, 2);                    \
+    LAUNCH(2, 2, kWave);                   \
   } else if (pl.vpl == 2 && pl.rpw == 4) { \
-    LAUNCH(2, 4);                    \
+    LAUNCH(2, 4, kWave);                   \
   } else if (pl.vpl == 4 && pl.rpw == 1) { \
-    LAUNCH(4, 1);                    \
+    LAUNCH(4, 1, kWave);                   \
   } else if (pl.vpl == 4 && pl.rpw == 2) { \
-    LAUNCH(4, 2);                    \
-  } else {                           \
-    LAUNCH(8, 1);                    \
+    LAUNCH(4, 2, kWave);                   \
+  } else {                                 \
+    LAUNCH(8, 1, kWave);                   \
   }
 
 // stats != nullptr selects the dropout variant (d is ignored otherwise).
@@ -753,8 +800,13 @@ static int launch_softmax_fwd(const void *x, const uint8_t *mask, void *y,
                               float scale, hipStream_t st) {
   constexpr int E = io<T>::EPV;
   const bool drop = stats != nullptr;
-  SoftmaxPlan pl =
-      plan_softmax(g.sk, E, kFwdMaxElems, MODE == kModeMasked ? 2 : 1);
+  // 32 elements per lane measure 10-25 % faster than 64 (rows of 4096 and
+  // more 16-bit keys then take two or more waves); 64 only where a row would
+  // otherwise not fit one workgroup
+  const int cap = g_tune.softmax_fwd_elems > 0 ? g_tune.softmax_fwd_elems : 32;
+  SoftmaxPlan pl = plan_softmax(g.sk, E, cap, MODE == kModeMasked ? 2 : 1, 4);
+  if (!pl.ok && cap < kFwdMaxElems)
+    pl = plan_softmax(g.sk, E, kFwdMaxElems, MODE == kModeMasked ? 2 : 1, 4);
   const bool vec_ok = pl.ok && aligned16(x) && aligned16(y) &&
                       (MODE != kModeMasked ||
                        (reinterpret_cast<uintptr_t>(mask) % E) == 0);
@@ -775,16 +827,17 @@ static int launch_softmax_fwd(const void *x, const uint8_t *mask, void *y,
   g.wpr = pl.wpr;
   g.rpb = pl.rpb;
   const int threads = kWave * pl.wpr * pl.rpb;
-  const int64_t grid = ceil_div(g.rows, (int64_t)pl.rpb * pl.rpw);
+  const int64_t grid =
+      ceil_div(g.rows, (int64_t)pl.rpb * pl.rpw * (kWave / pl.lpr));
   OSLO_REQUIRE(grid <= 0x7fffffff, "softmax fwd: too many rows");
-#define OSLO_SM_FWD(VPL, RPW)                                        \
+#define OSLO_SM_FWD(VPL, RPW, LPR_)                                  \
   if constexpr (VPL * RPW * E <= kFwdMaxElems) {                     \
     if (drop)                                                        \
-      softmax_fwd_kernel<T, VPL, RPW, MODE, true>                    \
+      softmax_fwd_kernel<T, VPL, RPW, MODE, true, LPR_>              \
           <<<dim3((unsigned)grid), threads, 0, st>>>(                \
               (const T *)x, mask, (T *)y, stats, g, scale, d);       \
     else                                                             \
-      softmax_fwd_kernel<T, VPL, RPW, MODE, false>                   \
+      softmax_fwd_kernel<T, VPL, RPW, MODE, false, LPR_>             \
           <<<dim3((unsigned)grid), threads, 0, st>>>(                \
               (const T *)x, mask, (T *)y, nullptr, g, scale, d);     \
   }
@@ -798,7 +851,7 @@ static int launch_softmax_bwd(const void *dy, const void *y,
                               const uint8_t *mask, void *dx, SoftmaxGeom g,
                               float scale, hipStream_t st) {
   constexpr int E = io<T>::EPV;
-  SoftmaxPlan pl = plan_softmax(g.sk, E, kBwdMaxElems, 1);
+  SoftmaxPlan pl = plan_softmax(g.sk, E, kBwdMaxElems, 1, 1);
   const bool vec_ok = pl.ok && aligned16(dy) && aligned16(y) &&
                       aligned16(dx) &&
                       (MODE != kModeMasked ||
@@ -814,11 +867,12 @@ static int launch_softmax_bwd(const void *dy, const void *y,
   g.wpr = pl.wpr;
   g.rpb = pl.rpb;
   const int threads = kWave * pl.wpr * pl.rpb;
-  const int64_t grid = ceil_div(g.rows, (int64_t)pl.rpb * pl.rpw);
+  const int64_t grid =
+      ceil_div(g.rows, (int64_t)pl.rpb * pl.rpw * (kWave / pl.lpr));
   OSLO_REQUIRE(grid <= 0x7fffffff, "softmax bwd: too many rows");
-#define OSLO_SM_BWD(VPL, RPW)                              \
+#define OSLO_SM_BWD(VPL, RPW, LPR_)                        \
   if constexpr (VPL * RPW * E <= kBwdMaxElems)             \
-    softmax_bwd_kernel<T, VPL, RPW, MODE>                  \
+    softmax_bwd_kernel<T, VPL, RPW, MODE, LPR_>            \
         <<<dim3((unsigned)grid), threads, 0, st>>>(        \
             (const T *)dy, (const T *)y, mask, (T *)dx, g, scale)
   OSLO_SM_CASES(OSLO_SM_BWD)
@@ -832,7 +886,7 @@ static int launch_softmax_dropout_bwd(const void *dy, const void *x,
                                       void *dx, DropArgs d, SoftmaxGeom g,
                                       float scale, hipStream_t st) {
   constexpr int E = io<T>::EPV;
-  SoftmaxPlan pl = plan_softmax(g.sk, E, kBwdMaxElems, 1);
+  SoftmaxPlan pl = plan_softmax(g.sk, E, kBwdMaxElems, 1, 1);
   const bool vec_ok = pl.ok && aligned16(dy) && aligned16(x) && aligned16(dx) &&
                       (MODE != kModeMasked ||
                        (reinterpret_cast<uintptr_t>(mask) % E) == 0);
@@ -849,11 +903,12 @@ static int launch_softmax_dropout_bwd(const void *dy, const void *x,
   g.wpr = pl.wpr;
   g.rpb = pl.rpb;
   const int threads = kWave * pl.wpr * pl.rpb;
-  const int64_t grid = ceil_div(g.rows, (int64_t)pl.rpb * pl.rpw);
+  const int64_t grid =
+      ceil_div(g.rows, (int64_t)pl.rpb * pl.rpw * (kWave / pl.lpr));
   OSLO_REQUIRE(grid <= 0x7fffffff, "softmax dropout bwd: too many rows");
-#define OSLO_SM_DBWD(VPL, RPW)                                      \
+#define OSLO_SM_DBWD(VPL, RPW, LPR_)                                \
   if constexpr (VPL * RPW * E <= kBwdMaxElems)                      \
-    softmax_dropout_bwd_kernel<T, VPL, RPW, MODE>                   \
+    softmax_dropout_bwd_kernel<T, VPL, RPW, MODE, LPR_>             \
         <<<dim3((unsigned)grid), threads, 0, st>>>(                 \
             (const T *)dy, (const T *)x, stats, mask, (T *)dx, g,   \
             scale, d)
@@ -975,9 +1030,10 @@ int oslo_softmax_batch_per_block(int64_t sq, int64_t sk, int64_t b,
                 "softmax_batch_per_block: bad shape");
   // rows per workgroup of the 16-bit masked kernel (the reference's shim only
   // admits fp16 / bf16); rows that do not vectorise run one row per workgroup
-  SoftmaxPlan pl = plan_softmax(sk, 8, kFwdMaxElems, 2);
+  SoftmaxPlan pl = plan_softmax(sk, 8, 32, 2, 4);
+  if (!pl.ok) pl = plan_softmax(sk, 8, kFwdMaxElems, 2, 4);
   if (!pl.ok) return 1;
-  return pl.rpb * pl.rpw;
+  return pl.rpb * pl.rpw * (kWave / pl.lpr);
 }
 
 
