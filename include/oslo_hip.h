@@ -336,7 +336,7 @@ int oslo_wave_reduce_selftest(float *out4, void *stream);
 /* Overrides a launch heuristic (for tuning sweeps): key is one of
  * "norm_fwd_vpl", "norm_bwd_vpl", "norm_bwd_blocks_per_cu",
  * "softmax_rows_per_wave", "softmax_lanes_per_row" (64 switches the
- * side-by-side short rows off), "softmax_fwd_elems", "eltwise_unroll", "eltwise_rowgroups",
+ * side-by-side short rows off), "softmax_fwd_elems", "norm_lanes_per_row", "eltwise_unroll", "eltwise_rowgroups",
  * "eltwise_fwd_steps", "norm_bwd_waves", "norm_fwd_waves",
  * "norm_bwd_prefetch", "norm_fwd_iters", "adam_unroll";
  * value 0 restores the default.  Process-wide, not thread-safe.            */

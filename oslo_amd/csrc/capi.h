@@ -28,6 +28,7 @@ struct Tuning {
   int softmax_rows_per_wave;
   int softmax_lanes_per_row;
   int softmax_fwd_elems;
+  int norm_lanes_per_row;
   int eltwise_unroll;
   int eltwise_rowgroups;
   int eltwise_fwd_steps;

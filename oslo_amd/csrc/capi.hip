@@ -85,6 +85,7 @@ int oslo_tune(const char *key, int value) {
       {"softmax_rows_per_wave", &oslo::g_tune.softmax_rows_per_wave},
       {"softmax_lanes_per_row", &oslo::g_tune.softmax_lanes_per_row},
       {"softmax_fwd_elems", &oslo::g_tune.softmax_fwd_elems},
+      {"norm_lanes_per_row", &oslo::g_tune.norm_lanes_per_row},
       {"eltwise_unroll", &oslo::g_tune.eltwise_unroll},
       {"eltwise_rowgroups", &oslo::g_tune.eltwise_rowgroups},
       {"eltwise_fwd_steps", &oslo::g_tune.eltwise_fwd_steps},

@@ -30,9 +30,17 @@ namespace oslo {
 // the sum of wave first + l and one DPP row reduction combines them, which
 // costs a fixed dozen instructions instead of a loop over wpr.
 // Two simultaneous row sums sharing one barrier.  red is [2][16] floats.
+// With LPR < 64 a row belongs to LPR consecutive lanes of one wave (wpr == 1)
+// and the sums stay inside that lane group.
+template <int LPR = kWave>
 __device__ __forceinline__ void row_sum2(float &a, float &b, float *red,
                                          int wave, int first, int wpr,
                                          int lane) {
+  if constexpr (LPR < kWave) {
+    a = group_allreduce<OpSum, LPR>(a);
+    b = group_allreduce<OpSum, LPR>(b);
+    return;
+  }
   a = wave_sum(a);
   b = wave_sum(b);
   if (wpr > 1) {
@@ -49,8 +57,10 @@ __device__ __forceinline__ void row_sum2(float &a, float &b, float *red,
   }
 }
 
+template <int LPR = kWave>
 __device__ __forceinline__ float row_sum1(float a, float *red, int wave,
                                           int first, int wpr, int lane) {
+  if constexpr (LPR < kWave) return group_allreduce<OpSum, LPR>(a);
   a = wave_sum(a);
   if (wpr > 1) {
     if (lane == 0) red[wave] = a;
@@ -68,9 +78,28 @@ __device__ __forceinline__ float row_sum1(float a, float *red, int wave,
 // sum_w (M2_w + c (mean_w - mean)^2).  red holds two areas of 48 floats;
 // `parity` alternates between them from one call to the next so that a
 // single barrier per call suffices.
+template <int LPR = kWave>
 __device__ __forceinline__ Welford row_welford(Welford w, float *red, int wave,
                                                int first, int wpr, int lane,
                                                int parity) {
+  if constexpr (LPR < kWave) {
+    // pairwise merges inside the lane group; every merge is symmetric, so
+    // the lanes of a group end with the same bits
+    float mean = w.mean, m2 = w.m2;
+    const float c = w.n;
+    merge_equal(mean, m2, dpp_mov<kDppQuadSwap1>(mean), dpp_mov<kDppQuadSwap1>(m2), c);
+    merge_equal(mean, m2, dpp_mov<kDppQuadSwap2>(mean), dpp_mov<kDppQuadSwap2>(m2), 2.f * c);
+    merge_equal(mean, m2, dpp_mov<kDppRowHalfMirror>(mean), dpp_mov<kDppRowHalfMirror>(m2),
+                4.f * c);
+    if constexpr (LPR >= 16)
+      merge_equal(mean, m2, dpp_mov<kDppRowMirror>(mean), dpp_mov<kDppRowMirror>(m2), 8.f * c);
+    if constexpr (LPR >= 32)
+      merge_equal(mean, m2, __shfl_xor(mean, 16), __shfl_xor(m2, 16), 16.f * c);
+    w.mean = mean;
+    w.m2 = m2;
+    w.n = c * (float)LPR;
+    return w;
+  }
   w = wave_welford_equal(w.mean, w.m2, w.n);
   if (wpr > 1) {
     float *area = red + parity * 48;
@@ -111,8 +140,11 @@ struct FusePrologue {
 
 // EVEN: every lane holds exactly VPL chunks of its row (no column guards;
 // LayerNorm then merges equal-sized Welford partials).
+// LPR: lanes that hold a row.  64: a row takes wpr whole waves.  8, 16, 32:
+// rows of at most LPR chunks lie side by side in a wave (VPL == 1, wpr == 1,
+// and rpb counts the rows of all lane groups of the workgroup).
 template <typename T, typename V, int VPL, bool RMS, bool EVEN, int MAXT,
-          bool FUSE = false>
+          bool FUSE = false, int LPR = kWave>
 __global__ __launch_bounds__(MAXT) void norm_fwd_reg_kernel(
     const T *__restrict__ x, const V *__restrict__ gamma,
     const V *__restrict__ beta, V *__restrict__ y, float *__restrict__ mean,
@@ -120,15 +152,17 @@ __global__ __launch_bounds__(MAXT) void norm_fwd_reg_kernel(
     int rpb, int iters, FusePrologue fp) {
   constexpr int E = chunk_elems<T, V>::value;
   static_assert(!FUSE || sizeof(T) == sizeof(V), "fused prologue: one dtype");
+  static_assert(LPR == kWave || (VPL == 1 && !FUSE), "side-by-side rows: one chunk per lane");
   __shared__ float red[2][48];
   const int lane = threadIdx.x & 63;
   // the wave index is uniform: keep it (and the row arithmetic) in scalar registers
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int rslot = wave / wpr;
-  const int first = rslot * wpr;
+  constexpr int SUB = kWave / LPR;
+  const int first = (wave / wpr) * wpr;
+  const int rslot = LPR == kWave ? wave / wpr : wave * SUB + lane / LPR;
   const int nchunks = n2 / E;
   const int cstride = kWave * wpr;
-  const int c0 = (wave - first) * kWave + lane;
+  const int c0 = LPR == kWave ? (wave - first) * kWave + lane : (lane & (LPR - 1));
   const float fn = (float)n2;
   int parity = 0;
 
@@ -250,7 +284,7 @@ __global__ __launch_bounds__(MAXT) void norm_fwd_reg_kernel(
           const float d = v[k][e] - w.mean;
           w.m2 += d * d;
         }
-      w = row_welford(w, &red[0][0], wave, first, wpr, lane, parity);
+      w = row_welford<LPR>(w, &red[0][0], wave, first, wpr, lane, parity);
       parity ^= 1;
       mu = w.mean;
       q = w.m2;
@@ -262,7 +296,7 @@ __global__ __launch_bounds__(MAXT) void norm_fwd_reg_kernel(
       for (int k = 0; k < VPL; ++k)
 #pragma unroll
         for (int e = 0; e < E; ++e) s += v[k][e];
-      s = row_sum1(s, &red[0][0], wave, first, wpr, lane);
+      s = row_sum1<LPR>(s, &red[0][0], wave, first, wpr, lane);
       mu = s / fn;
 #pragma unroll
       for (int k = 0; k < VPL; ++k) {
@@ -274,13 +308,13 @@ __global__ __launch_bounds__(MAXT) void norm_fwd_reg_kernel(
           }
         }
       }
-      q = row_sum1(q, &red[1][0], wave, first, wpr, lane);
+      q = row_sum1<LPR>(q, &red[1][0], wave, first, wpr, lane);
     } else {
 #pragma unroll
       for (int k = 0; k < VPL; ++k)
 #pragma unroll
         for (int e = 0; e < E; ++e) q += v[k][e] * v[k][e];
-      q = row_sum1(q, red[parity], wave, first, wpr, lane);
+      q = row_sum1<LPR>(q, red[parity], wave, first, wpr, lane);
       parity ^= 1;
     }
     const float rs = rsqrt_refined(q / fn + eps);
@@ -413,8 +447,9 @@ struct FuseEpilogue {
 
 // MAXT: largest workgroup the build is launched with (768 leaves a third more
 // registers per lane than 1024, which the 16-elements-per-lane builds need).
+// LPR: as in the forward kernel (rows side by side in a wave when < 64).
 template <typename T, typename V, int VPL, bool RMS, bool EVEN, int PF,
-          bool FUSE = false, int MAXT = 1024>
+          bool FUSE = false, int MAXT = 1024, int LPR = kWave>
 __global__ __launch_bounds__(MAXT) void norm_bwd_reg_kernel(
     const V *__restrict__ dy, const T *__restrict__ x,
     const float *__restrict__ mean, const float *__restrict__ invvar,
@@ -422,16 +457,21 @@ __global__ __launch_bounds__(MAXT) void norm_bwd_reg_kernel(
     int64_t n1, int n2, int wpr, int rpb, FuseEpilogue fe) {
   constexpr int E = chunk_elems<T, V>::value;
   static_assert(!FUSE || sizeof(T) == sizeof(V), "fused epilogue: one dtype");
+  static_assert(LPR == kWave || (VPL == 1 && !FUSE), "side-by-side rows: one chunk per lane");
   extern __shared__ float xslot[];  // [n2] when rpb > 1
   __shared__ float red[2][32];
   const int lane = threadIdx.x & 63;
   // the wave index is uniform: keep it (and the row arithmetic) in scalar registers
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int rslot = wave / wpr;
-  const int first = rslot * wpr;
+  constexpr int SUB = kWave / LPR;
+  const int first = (wave / wpr) * wpr;
+  // row slot of this lane; wslot is the wave's slot when its lane groups
+  // have been folded into one
+  const int wslot = wave / wpr;
+  const int rslot = LPR == kWave ? wslot : wave * SUB + lane / LPR;
   const int nchunks = n2 / E;
   const int cstride = kWave * wpr;
-  const int c0 = (wave - first) * kWave + lane;
+  const int c0 = LPR == kWave ? (wave - first) * kWave + lane : (lane & (LPR - 1));
   const float fn = (float)n2;
   const bool affine = gamma != nullptr;
 
@@ -535,10 +575,10 @@ __global__ __launch_bounds__(MAXT) void norm_bwd_reg_kernel(
       }
     }
     if constexpr (RMS) {
-      s2 = row_sum1(s2, red[parity], wave, first, wpr, lane);
+      s2 = row_sum1<LPR>(s2, red[parity], wave, first, wpr, lane);
       s1 = 0.f;
     } else {
-      row_sum2(s1, s2, red[parity], wave, first, wpr, lane);
+      row_sum2<LPR>(s1, s2, red[parity], wave, first, wpr, lane);
     }
     parity ^= 1;
     // dx = invvar / n2 * (n2 * dy * gamma - s1 - xhat * s2), regrouped as
@@ -611,10 +651,25 @@ __global__ __launch_bounds__(MAXT) void norm_bwd_reg_kernel(
   const int64_t P = gridDim.x;
   // (a lambda over one accumulator array at a time keeps the arrays in
   // registers: none of them is indexed by a run-time value)
+  const int wslots = LPR == kWave ? rpb : rpb / SUB;  // wave-level row slots
+  const bool lead = LPR == kWave || lane < LPR;        // first lane group
   auto fold_and_store = [&](auto &acc, int a) {
-    for (int s = 1; s < rpb; ++s) {
+    if constexpr (LPR < kWave) {
+      // the lane groups of a wave hold the same columns: sum them into the
+      // first group
+#pragma unroll
+      for (int k = 0; k < VPL; ++k)
+#pragma unroll
+        for (int e = 0; e < E; ++e) {
+          float t = acc[k][e];
+#pragma unroll
+          for (int o = LPR; o < kWave; o <<= 1) t += __shfl_xor(t, o);
+          acc[k][e] = t;
+        }
+    }
+    for (int s = 1; s < wslots; ++s) {
       __syncthreads();
-      if (rslot == s) {
+      if (wslot == s && lead) {
 #pragma unroll
         for (int k = 0; k < VPL; ++k) {
           const int c = c0 + k * cstride;
@@ -625,7 +680,7 @@ __global__ __launch_bounds__(MAXT) void norm_bwd_reg_kernel(
         }
       }
       __syncthreads();
-      if (rslot == 0) {
+      if (wslot == 0 && lead) {
 #pragma unroll
         for (int k = 0; k < VPL; ++k) {
           const int c = c0 + k * cstride;
@@ -636,7 +691,7 @@ __global__ __launch_bounds__(MAXT) void norm_bwd_reg_kernel(
         }
       }
     }
-    if (rslot == 0) {
+    if (wslot == 0 && lead) {
       float *prow = part + ((int64_t)a * P + blockIdx.x) * n2;
 #pragma unroll
       for (int k = 0; k < VPL; ++k) {
@@ -764,6 +819,16 @@ static RowSplit split_row(int64_t nchunks, int cap, const int *allowed,
   return r;
 }
 
+// Lanes that hold a row of `nchunks` chunks: 64, or 8 / 16 / 32 when the row
+// is short enough for several rows to lie side by side in a wave.
+static int lanes_per_row(int64_t nchunks) {
+  if (nchunks > 32 || g_tune.norm_lanes_per_row == kWave) return kWave;
+  int lpr = nchunks <= 8 ? 8 : nchunks <= 16 ? 16 : 32;
+  const int t = g_tune.norm_lanes_per_row;
+  if ((t == 8 || t == 16 || t == 32) && t >= lpr) lpr = t;
+  return lpr;
+}
+
 int64_t colsum_parts_norm(int64_t n1, int64_t n2) {
   (void)n2;
   int bpc = g_tune.norm_bwd_blocks_per_cu > 0 ? g_tune.norm_bwd_blocks_per_cu : 1;
@@ -843,6 +908,34 @@ static int launch_norm_fwd(const void *x, const void *gamma, const void *beta,
   int64_t grid = ceil_div(ceil_div(n1, sp.rpb), iters);
   const int64_t maxgrid = (int64_t)device_cu_count() * 64;
   if (grid > maxgrid) grid = maxgrid;
+  // short rows side by side in a wave
+  const int lpr = (!fused && sp.wpr == 1 && sp.vpl == 1) ? lanes_per_row(n2 / E) : kWave;
+  if (lpr < kWave) {
+    const int rpb_eff = sp.rpb * (kWave / lpr);
+    const bool even_l = (n2 / E) == lpr;
+    int64_t grid_l = ceil_div(ceil_div(n1, rpb_eff), iters);
+    if (grid_l > maxgrid) grid_l = maxgrid;
+#define OSLO_FWD_LPR(LPR_)                                                   \
+  case LPR_:                                                                 \
+    if (even_l)                                                              \
+      norm_fwd_reg_kernel<T, V, 1, RMS, true, 256, false, LPR_>              \
+          <<<dim3((unsigned)grid_l), threads, 0, st>>>(                      \
+              (const T *)x, (const V *)gamma, (const V *)beta, (V *)y, mean, \
+              invvar, n1, (int)n2, eps, 1, rpb_eff, iters, FusePrologue{});  \
+    else                                                                     \
+      norm_fwd_reg_kernel<T, V, 1, RMS, false, 256, false, LPR_>             \
+          <<<dim3((unsigned)grid_l), threads, 0, st>>>(                      \
+              (const T *)x, (const V *)gamma, (const V *)beta, (V *)y, mean, \
+              invvar, n1, (int)n2, eps, 1, rpb_eff, iters, FusePrologue{});  \
+    break;
+    switch (lpr) {
+      OSLO_FWD_LPR(8)
+      OSLO_FWD_LPR(16)
+      OSLO_FWD_LPR(32)
+    }
+#undef OSLO_FWD_LPR
+    return check_launch("norm_fwd_reg_kernel (side-by-side rows)");
+  }
   if constexpr (kCanFuse) {
     if (fused) {
 #define OSLO_FWD_FUSED_L(VPL, EVEN_, MAXT_)                                 \
@@ -997,6 +1090,10 @@ static int launch_norm_bwd(const void *dy, const void *x, const float *mean,
             (V *)dbeta, n1, n2);
     return check_launch("norm_bwd_param_generic_kernel");
   }
+  // short rows side by side in a wave: the row slots of a workgroup multiply
+  const int lpr = (!fused && sp.wpr == 1 && sp.vpl == 1) ? lanes_per_row(n2 / E) : kWave;
+  const int wave_slots = sp.rpb;  // row slots at wave granularity
+  if (lpr < kWave) sp.rpb *= kWave / lpr;
   int64_t P = colsum_parts_norm(n1, n2);
   if (P > ceil_div(n1, sp.rpb)) P = ceil_div(n1, sp.rpb);
   float *part = nullptr;
@@ -1014,12 +1111,14 @@ static int launch_norm_bwd(const void *dy, const void *x, const float *mean,
                   (long long)need, (long long)ws_bytes);
     part = (float *)ws;
   }
-  const int threads = kWave * sp.wpr * sp.rpb;
-  const size_t lds = sp.rpb > 1 ? (size_t)n2 * sizeof(float) : 0;
-  const bool even = (n2 / E) == (int64_t)sp.vpl * kWave * sp.wpr;
+  const int threads = kWave * sp.wpr * wave_slots;
+  const size_t lds = wave_slots > 1 ? (size_t)n2 * sizeof(float) : 0;
+  const bool even = lpr < kWave ? (n2 / E) == lpr
+                                : (n2 / E) == (int64_t)sp.vpl * kWave * sp.wpr;
   // rows in flight ahead of the one being reduced: two while the packed row
-  // buffers are small (8 elements per lane), else one
-  int pf = sp.vpl * E <= 8 ? 2 : 1;
+  // buffers are small (8 elements per lane) and a row spans several waves,
+  // else one (a wave that owns whole rows measures 6 % slower with two)
+  int pf = sp.vpl * E <= 8 && sp.wpr >= 2 ? 2 : 1;
   if (g_tune.norm_bwd_prefetch > 0) pf = g_tune.norm_bwd_prefetch >= 2 ? 2 : 1;
 #define OSLO_BWD_LAUNCH_T(VPL, EVEN_, PF_, MAXT_)                          \
   do {                                                                     \
@@ -1062,6 +1161,27 @@ static int launch_norm_bwd(const void *dy, const void *x, const float *mean,
         OSLO_BWD_LAUNCH(VPL, false, 1);                                    \
     }                                                                      \
     break;
+  if (lpr < kWave) {
+#define OSLO_BWD_LPR(LPR_)                                                  \
+  case LPR_:                                                                \
+    if (even)                                                               \
+      norm_bwd_reg_kernel<T, V, 1, RMS, true, 1, false, 1024, LPR_>         \
+          <<<dim3((unsigned)P), threads, lds, st>>>(                        \
+              (const V *)dy, (const T *)x, mean, invvar, (const V *)gamma,  \
+              (T *)dx, part, n1, (int)n2, 1, sp.rpb, fev);                  \
+    else                                                                    \
+      norm_bwd_reg_kernel<T, V, 1, RMS, false, 1, false, 1024, LPR_>        \
+          <<<dim3((unsigned)P), threads, lds, st>>>(                        \
+              (const V *)dy, (const T *)x, mean, invvar, (const V *)gamma,  \
+              (T *)dx, part, n1, (int)n2, 1, sp.rpb, fev);                  \
+    break;
+    switch (lpr) {
+      OSLO_BWD_LPR(8)
+      OSLO_BWD_LPR(16)
+      OSLO_BWD_LPR(32)
+    }
+#undef OSLO_BWD_LPR
+  } else
   switch (sp.vpl) {
     OSLO_BWD_CASE(1)
     OSLO_BWD_CASE(2)
