@@ -334,11 +334,14 @@ int oslo_copy_probe(const void *src, void *dst, int64_t bytes, void *stream);
 int oslo_wave_reduce_selftest(float *out4, void *stream);
 
 /* Overrides a launch heuristic (for tuning sweeps): key is one of
- * "norm_fwd_vpl", "norm_bwd_vpl", "norm_bwd_blocks_per_cu",
- * "softmax_rows_per_wave", "softmax_lanes_per_row" (64 switches the
- * side-by-side short rows off), "softmax_fwd_elems", "norm_lanes_per_row", "eltwise_unroll", "eltwise_rowgroups",
- * "eltwise_fwd_steps", "norm_bwd_waves", "norm_fwd_waves",
- * "norm_bwd_prefetch", "norm_fwd_iters", "adam_unroll";
+ * "norm_fwd_vpl", "norm_bwd_vpl", "norm_bwd_blocks_per_cu", "norm_bwd_waves",
+ * "norm_fwd_waves", "norm_bwd_prefetch", "norm_fwd_iters",
+ * "norm_lanes_per_row", "softmax_lanes_per_row" (64 switches the
+ * side-by-side short rows off), "softmax_rows_per_wave",
+ * "softmax_fwd_elems", "eltwise_unroll", "eltwise_rowgroups",
+ * "eltwise_fwd_steps", "eltwise_tile_max", "eltwise_tile_min" (lanes along
+ * the columns of an element-wise tile; 64 as the minimum restores whole-wave
+ * tiles), "adam_unroll";
  * value 0 restores the default.  Process-wide, not thread-safe.            */
 int oslo_tune(const char *key, int value);
 

@@ -29,6 +29,8 @@ struct Tuning {
   int softmax_lanes_per_row;
   int softmax_fwd_elems;
   int norm_lanes_per_row;
+  int eltwise_tile_max;
+  int eltwise_tile_min;
   int eltwise_unroll;
   int eltwise_rowgroups;
   int eltwise_fwd_steps;

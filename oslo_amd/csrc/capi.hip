@@ -86,6 +86,8 @@ int oslo_tune(const char *key, int value) {
       {"softmax_lanes_per_row", &oslo::g_tune.softmax_lanes_per_row},
       {"softmax_fwd_elems", &oslo::g_tune.softmax_fwd_elems},
       {"norm_lanes_per_row", &oslo::g_tune.norm_lanes_per_row},
+      {"eltwise_tile_max", &oslo::g_tune.eltwise_tile_max},
+      {"eltwise_tile_min", &oslo::g_tune.eltwise_tile_min},
       {"eltwise_unroll", &oslo::g_tune.eltwise_unroll},
       {"eltwise_rowgroups", &oslo::g_tune.eltwise_rowgroups},
       {"eltwise_fwd_steps", &oslo::g_tune.eltwise_fwd_steps},

@@ -446,14 +446,32 @@ static inline int eltwise_unroll(int dflt) {
   return u == 1 || u == 2 || u == 4 ? u : dflt;
 }
 
-// Tile shape for `cols`: tx lanes wide (power of two, 64..256), ty rows tall.
+// Tile shape for `cols`: tx lanes wide (a power of two up to 256), ty = 256 /
+// tx rows tall.  The widest tile that leaves at most 1/32 of its lanes
+// without a chunk is taken (384 chunks -> three tiles of 128 rather than two
+// of 256; 8 chunks -> 8 lanes and 32 rows side by side), else the one with the
+// fewest idle lanes.
 static inline void eltwise_tile(int64_t cols, int *tx, int *ty, int *tiles) {
   const int64_t nchunks = ceil_div(cols, kE);
-  int t = 64;
-  while (t < 256 && t < nchunks) t *= 2;
-  *tx = t;
-  *ty = 256 / t;
-  *tiles = (int)ceil_div(nchunks, t);
+  int best = 256;
+  int64_t best_waste = -1;
+  const int tmax = g_tune.eltwise_tile_max > 0 ? g_tune.eltwise_tile_max : 256;
+  const int tmin = g_tune.eltwise_tile_min > 0 ? g_tune.eltwise_tile_min : 1;
+  for (int t = tmax; t >= tmin; t >>= 1) {
+    const int64_t waste = ceil_div(nchunks, t) * t - nchunks;
+    if (waste * 32 <= nchunks) {
+      best = t;
+      best_waste = waste;
+      break;
+    }
+    if (best_waste < 0 || waste < best_waste) {
+      best = t;
+      best_waste = waste;
+    }
+  }
+  *tx = best;
+  *ty = 256 / best;
+  *tiles = (int)ceil_div(nchunks, best);
 }
 
 // Backward: workgroups per column tile = fp32 partial rows.  Two workgroups
