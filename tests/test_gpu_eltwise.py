@@ -27,6 +27,14 @@ SHAPES = [
     (9, 100, F16),        # cols % 8 != 0: scalar kernels
     (7, 1, F32),
     (2051, 64, BF16),
+    # tile widths below a wavefront and tiles that divide odd chunk counts
+    (4099, 8, F16),       # 1 lane x 256 rows
+    (1031, 16, BF16),     # 2 lanes
+    (777, 40, BF16),      # 5 chunks in 8 lanes
+    (515, 136, F16),      # 17 chunks: 32 lanes, or 1 lane x 17 tiles
+    (301, 3072, BF16),    # 384 chunks: three tiles of 128 lanes
+    (67, 11008, BF16),    # 1376 chunks: 43 tiles of 32 lanes
+    (129, 96, F32),
 ]
 
 
