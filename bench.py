@@ -16,7 +16,10 @@ Prints ONE JSON line.  Beside the contract's keys it carries
   cpu_baseline  the reference's unfused torch path (oracle/torch_path.py) on
                 the host cores, same workload,
   kernels       achieved GB/s and fraction of the 8 TB/s HBM peak for every
-                fused kernel of BASELINE.json's five configurations.
+                fused kernel of BASELINE.json's five configurations,
+  cpu_path      the reference's unfused torch path, forward + backward, for
+                the other four configurations on bounded samples, with the
+                GPU rate of the same pair and their ratio.
 """
 import argparse
 import json
@@ -442,6 +445,117 @@ def cpu_baseline(n1, n2, reps):
     }
 
 
+def cpu_path_table(gpu_rows, budget_s=3.0):
+    """The reference's unfused torch path, forward + backward, for every
+    configuration, on the host cores and on a BOUNDED sample of the rows (the
+    CPU rate does not depend on the row count at these sizes); each entry
+    carries the GPU rate of the same forward + backward pair from the kernel
+    table and their ratio.  At most `budget_s` seconds of timed work per entry."""
+    import torch
+
+    from oracle import torch_path as tp
+
+    threads = min(os.cpu_count() or 1, 16)
+    torch.set_num_threads(threads)
+    g = torch.Generator().manual_seed(0)
+
+    def rnd(shape, dtype, std=1.0):
+        return (std * torch.randn(shape, generator=g)).to(dtype)
+
+    def gpu_rate(names, cfg, **match):
+        rows = [r for r in gpu_rows if r["kernel"] in names and r["config"] == cfg
+                and all(r.get(k) == v for k, v in match.items())]
+        if len(rows) != len(names):
+            return None
+        return sum(r["algorithmic_MB"] for r in rows) / sum(r["us"] for r in rows) * 1e3
+
+    def timed(fn):
+        fn()
+        times, spent = [], 0.0
+        while len(times) < 3 and spent < budget_s:
+            t0 = time.perf_counter()
+            fn()
+            times.append(time.perf_counter() - t0)
+            spent += times[-1]
+        times.sort()
+        return times[len(times) // 2]
+
+    BF16, F16, F32 = torch.bfloat16, torch.float16, torch.float32
+    out = []
+
+    def entry(name, cfg, sample, nbytes, fn, gpu):
+        t = timed(fn)
+        cpu = nbytes / t / 1e9
+        out.append({
+            "kernel": name, "config": cfg, "sample": sample, "cores": threads,
+            "cpu_ms": round(t * 1e3, 1), "cpu_GBps": round(cpu, 2),
+            "gpu_GBps": None if gpu is None else round(gpu, 1),
+            "speedup": None if gpu is None else round(gpu / cpu, 1),
+        })
+
+    def causal(cfg, ab, s, dtype, scale, esz):
+        x, dy = rnd((ab, s, s), dtype), rnd((ab, s, s), dtype)
+        f = (s + 1) / (2.0 * s)
+
+        def fn():
+            xr = x.clone().requires_grad_()
+            tp.causal_softmax(xr, scale).backward(dy)
+        entry("softmax_causal fwd+bwd", cfg, "[%d,%d,%d] %s" % (ab, s, s, str(dtype).split(".")[-1]),
+              (2 + 3 * f) * ab * s * s * esz, fn,
+              gpu_rate(("softmax_causal_fwd", "softmax_causal_bwd"), cfg))
+
+    def norm_ln(cfg, n1, n2):
+        x, dy = rnd((n1, n2), BF16), rnd((n1, n2), BF16)
+        gamma, beta = rnd((n2,), BF16, 0.02) + 1, rnd((n2,), BF16, 0.02)
+
+        def fn():
+            xr = x.clone().requires_grad_()
+            w, b = gamma.clone().requires_grad_(), beta.clone().requires_grad_()
+            tp.layer_norm(xr, w, b, 1e-5).backward(dy)
+        entry("layer_norm fwd+bwd", cfg, "[%d,%d] bf16" % (n1, n2), 5 * n1 * n2 * 2, fn,
+              gpu_rate(("ln_fwd", "ln_bwd"), cfg))
+
+    def gelu(cfg, n1, n2):
+        x, dy, b = rnd((n1, n2), BF16), rnd((n1, n2), BF16), rnd((n2,), BF16, 0.02)
+
+        def fn():
+            xr, br = x.clone().requires_grad_(), b.clone().requires_grad_()
+            tp.bias_gelu(xr, br).backward(dy)
+        entry("bias_gelu fwd+bwd", cfg, "[%d,%d] bf16" % (n1, n2), 5 * n1 * n2 * 2, fn,
+              gpu_rate(("bias_gelu_fwd", "bias_gelu_bwd"), cfg))
+
+    def bda(cfg, n1, n2):
+        x, res, dy, b = rnd((n1, n2), BF16), rnd((n1, n2), BF16), rnd((n1, n2), BF16), rnd((n2,), BF16, 0.02)
+
+        def fn():
+            xr, br = x.clone().requires_grad_(), b.clone().requires_grad_()
+            tp.bias_dropout_add(xr, br, res, 0.1, True).backward(dy)
+        entry("bias_dropout_add fwd+bwd (p=0.1)", cfg, "[%d,%d] bf16" % (n1, n2), 5 * n1 * n2 * 2, fn,
+              gpu_rate(("bias_dropout_add_fwd", "bias_dropout_add_bwd"), cfg, p=0.1))
+
+    causal("cfg1", 48, 512, F32, 0.125, 4)
+    # cfg3: two of the sixteen batch entries
+    b_, h, s = 2, 16, 1024
+    x, dy = rnd((b_, h, s, s), F16, 2.0), rnd((b_, h, s, s), F16)
+    valid = torch.tensor([1024, 640])
+    pad = torch.arange(s)[None, :] >= valid[:, None]
+    r = float(valid.double().mean()) / s
+
+    def masked():
+        xr = x.clone().requires_grad_()
+        tp.padding_softmax(xr, pad, 0.125).backward(dy)
+    entry("softmax_masked fwd+bwd", "cfg3", "[2,16,1024,1024] fp16 of batch 16", (2 + 3 * r) * x.numel() * 2,
+          masked, gpu_rate(("softmax_masked_fwd", "softmax_masked_bwd"), "cfg3"))
+    del x, dy
+    gelu("cfg4", 2048, 16384)
+    bda("cfg4", 4096, 4096)
+    norm_ln("cfg5", 8192, 6144)  # whole: a smaller sample would stay in the host caches
+    causal("cfg5", 8, 2048, BF16, 1.0 / math.sqrt(96.0), 2)
+    gelu("cfg5", 1024, 24576)
+    bda("cfg5", 2048, 6144)
+    return out
+
+
 def main():
     args = parse_args()
     if args.gpus != 1:
@@ -540,6 +654,8 @@ def main():
         cb = cpu_baseline(n1, n2, args.cpu_reps)
         cb["speedup_gpu_over_cpu"] = round(value / cb["value"], 1) if cb["value"] > 0 else None
         out["cpu_baseline"] = cb
+        if "kernels" in out:
+            out["cpu_path"] = cpu_path_table(out["kernels"])
     print(json.dumps(out))
 
 
