@@ -23,7 +23,9 @@
 
 namespace oslo {
 
-constexpr int kE = 8;  // chunk = dropout group = 8 elements for every dtype
+// A chunk is one 128-bit vector: 8 elements of a 16-bit type, 4 of fp32 (kE
+// inside the kernels).  The dropout groups are 8 consecutive elements of the
+// flattened tensor for every dtype: an fp32 chunk takes half a group.
 
 // -2 * log2(e) * 0.79788456 and that times 0.044715: exp(-2 z) = exp2(u * (K1 + K2 u^2))
 constexpr float kGeluK1 = -2.0f * 1.4426950408889634f * 0.79788456f;
@@ -78,6 +80,7 @@ template <typename T, int U, bool HAS_BIAS>
 __global__ __launch_bounds__(256) void bias_gelu_fwd_kernel(
     const T *__restrict__ x, const T *__restrict__ bias, T *__restrict__ y,
     EltGeom g) {
+  constexpr int kE = io<T>::EPV;
   const EltPos ps = elt_pos(g);
   if (ps.cc >= g.nchunks) return;
   float b[kE];
@@ -106,7 +109,8 @@ __global__ __launch_bounds__(256) void bias_gelu_fwd_kernel(
 }
 
 // Folds the per-lane column sums of the ty rows of the workgroup and writes
-// the partial row of this slot.  sh is [ty][8][tx] floats (8 KB).
+// the partial row of this slot.  sh is [ty][kE][tx] floats (at most 8 KB).
+template <int kE>
 __device__ __forceinline__ void write_col_partials(const float *acc, float *sh,
                                                    float *__restrict__ part,
                                                    const EltGeom &g,
@@ -133,6 +137,7 @@ __global__ __launch_bounds__(256) void bias_gelu_bwd_kernel(
     const T *__restrict__ gr, const T *__restrict__ x,
     const T *__restrict__ bias, T *__restrict__ dx, float *__restrict__ part,
     EltGeom g) {
+  constexpr int kE = io<T>::EPV;
   __shared__ float sh[256 * kE];
   const EltPos ps = elt_pos(g);
   float b[kE], acc[kE];
@@ -181,7 +186,7 @@ __global__ __launch_bounds__(256) void bias_gelu_bwd_kernel(
       }
     }
   }
-  if (part != nullptr) write_col_partials(acc, sh, part, g, ps);
+  if (part != nullptr) write_col_partials<kE>(acc, sh, part, g, ps);
 }
 
 // ---------------------------------------------------------------------------
@@ -193,6 +198,7 @@ __global__ __launch_bounds__(256) void bias_dropout_add_fwd_kernel(
     const T *__restrict__ x, const T *__restrict__ bias,
     const T *__restrict__ res, T *__restrict__ out,
     uint8_t *__restrict__ mask_out, EltGeom g, DropArgs d) {
+  constexpr int kE = io<T>::EPV;
   const EltPos ps = elt_pos(g);
   if (ps.cc >= g.nchunks) return;
   float b[kE];
@@ -215,8 +221,7 @@ __global__ __launch_bounds__(256) void bias_dropout_add_fwd_kernel(
       if (r < g.rows) {
         uint32_t keep = 0xffu;
         if constexpr (DROP)
-          keep = dropout_keep_bits((uint64_t)r * (uint64_t)g.nchunks + ps.cc,
-                                   d.seed, d.offset, d.threshold);
+          keep = chunk_keep_bits<kE>(r, (int)g.cols, ps.cc, d);
         float o[kE];
 #pragma unroll
         for (int e = 0; e < kE; ++e) {
@@ -231,9 +236,12 @@ __global__ __launch_bounds__(256) void bias_dropout_add_fwd_kernel(
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
             m.x |= ((keep >> e) & 1u) << (8 * e);
-            m.y |= ((keep >> (4 + e)) & 1u) << (8 * e);
+            if constexpr (kE == 8) m.y |= ((keep >> (4 + e)) & 1u) << (8 * e);
           }
-          *reinterpret_cast<u32x2 *>(mask_out + r * g.cols + coff) = m;
+          if constexpr (kE == 8)
+            *reinterpret_cast<u32x2 *>(mask_out + r * g.cols + coff) = m;
+          else
+            *reinterpret_cast<uint32_t *>(mask_out + r * g.cols + coff) = m.x;
         }
       }
     }
@@ -244,6 +252,7 @@ template <typename T, int U, bool DROP>
 __global__ __launch_bounds__(256) void bias_dropout_add_bwd_kernel(
     const T *__restrict__ gr, T *__restrict__ dx, float *__restrict__ part,
     EltGeom g, DropArgs d) {
+  constexpr int kE = io<T>::EPV;
   __shared__ float sh[256 * kE];
   const EltPos ps = elt_pos(g);
   float acc[kE];
@@ -275,8 +284,7 @@ __global__ __launch_bounds__(256) void bias_dropout_add_bwd_kernel(
         if (r < g.rows) {
           uint32_t keep = 0xffu;
           if constexpr (DROP)
-            keep = dropout_keep_bits((uint64_t)r * (uint64_t)g.nchunks + ps.cc,
-                                     d.seed, d.offset, d.threshold);
+            keep = chunk_keep_bits<kE>(r, (int)g.cols, ps.cc, d);
           float o[kE];
 #pragma unroll
           for (int e = 0; e < kE; ++e) {
@@ -291,7 +299,7 @@ __global__ __launch_bounds__(256) void bias_dropout_add_bwd_kernel(
       }
     }
   }
-  if (part != nullptr) write_col_partials(acc, sh, part, g, ps);
+  if (part != nullptr) write_col_partials<kE>(acc, sh, part, g, ps);
 }
 
 // ---------------------------------------------------------------------------
@@ -451,8 +459,8 @@ static inline int eltwise_unroll(int dflt) {
 // without a chunk is taken (384 chunks -> three tiles of 128 rather than two
 // of 256; 8 chunks -> 8 lanes and 32 rows side by side), else the one with the
 // fewest idle lanes.
-static inline void eltwise_tile(int64_t cols, int *tx, int *ty, int *tiles) {
-  const int64_t nchunks = ceil_div(cols, kE);
+static inline void eltwise_tile(int64_t cols, int E, int *tx, int *ty, int *tiles) {
+  const int64_t nchunks = ceil_div(cols, E);
   int best = 256;
   int64_t best_waste = -1;
   const int tmax = g_tune.eltwise_tile_max > 0 ? g_tune.eltwise_tile_max : 256;
@@ -479,9 +487,9 @@ static inline void eltwise_tile(int64_t cols, int *tx, int *ty, int *tiles) {
 // advance through the rows in step, every lane keeps four chunks per operand
 // in flight plus the prefetch of the next step, and the partial rows stay
 // below one percent of the tensor traffic.
-int64_t colsum_parts_eltwise(int64_t rows, int64_t cols) {
+static int64_t colsum_parts_eltwise_e(int64_t rows, int64_t cols, int E) {
   int tx, ty, tiles;
-  eltwise_tile(cols, &tx, &ty, &tiles);
+  eltwise_tile(cols, E, &tx, &ty, &tiles);
   int64_t parts = g_tune.eltwise_rowgroups > 0
                       ? g_tune.eltwise_rowgroups
                       : ((int64_t)device_cu_count() * 2) / tiles;  // never more than two per CU
@@ -493,24 +501,31 @@ int64_t colsum_parts_eltwise(int64_t rows, int64_t cols) {
   return parts;
 }
 
-static inline EltGeom eltwise_geom_bwd(int64_t rows, int64_t cols, int unroll) {
+// Upper bound over the chunk widths (the workspace query knows no dtype).
+int64_t colsum_parts_eltwise(int64_t rows, int64_t cols) {
+  const int64_t a = colsum_parts_eltwise_e(rows, cols, 8);
+  const int64_t b = colsum_parts_eltwise_e(rows, cols, 4);
+  return a > b ? a : b;
+}
+
+static inline EltGeom eltwise_geom_bwd(int64_t rows, int64_t cols, int unroll, int E) {
   EltGeom g;
   g.rows = rows;
   g.cols = cols;
-  g.nchunks = (int)(cols / kE);
-  eltwise_tile(cols, &g.tx, &g.ty, &g.tiles);
+  g.nchunks = (int)(cols / E);
+  eltwise_tile(cols, E, &g.tx, &g.ty, &g.tiles);
   const int64_t nsteps = ceil_div(rows, (int64_t)g.ty * unroll);
-  g.slots = colsum_parts_eltwise(rows, cols);
+  g.slots = colsum_parts_eltwise_e(rows, cols, E);
   if (g.slots > nsteps) g.slots = nsteps;
   return g;
 }
 
-static inline EltGeom eltwise_geom_fwd(int64_t rows, int64_t cols, int unroll) {
+static inline EltGeom eltwise_geom_fwd(int64_t rows, int64_t cols, int unroll, int E) {
   EltGeom g;
   g.rows = rows;
   g.cols = cols;
-  g.nchunks = (int)(cols / kE);
-  eltwise_tile(cols, &g.tx, &g.ty, &g.tiles);
+  g.nchunks = (int)(cols / E);
+  eltwise_tile(cols, E, &g.tx, &g.ty, &g.tiles);
   const int steps = g_tune.eltwise_fwd_steps > 0 ? g_tune.eltwise_fwd_steps : 1;
   g.slots = ceil_div(ceil_div(rows, (int64_t)g.ty * unroll), steps);
   return g;
@@ -535,7 +550,8 @@ static inline int64_t flat_grid(int64_t n) {
 template <typename T>
 static int run_bias_gelu_fwd(const void *x, const void *bias, void *y,
                              int64_t rows, int64_t cols, hipStream_t st) {
-  const bool vec_ok = cols % kE == 0 && aligned16(x) && aligned16(y) &&
+  constexpr int kE = io<T>::EPV;
+  const bool vec_ok = cols % kE == 0 && cols <= 0x7fffffff && aligned16(x) && aligned16(y) &&
                       aligned16(bias) && cols / kE <= 0x7fffffff;
   if (!vec_ok) {
     const int64_t n = rows * cols;
@@ -544,7 +560,7 @@ static int run_bias_gelu_fwd(const void *x, const void *bias, void *y,
     return check_launch("bias_gelu_fwd_generic_kernel");
   }
   const int unroll = eltwise_unroll(2);
-  const EltGeom g = eltwise_geom_fwd(rows, cols, unroll);
+  const EltGeom g = eltwise_geom_fwd(rows, cols, unroll, kE);
   const int64_t nblocks = g.slots * g.tiles;
   OSLO_REQUIRE(nblocks <= 0x7fffffff, "bias_gelu fwd: too many workgroups");
   const dim3 grid((unsigned)nblocks);
@@ -563,7 +579,8 @@ template <typename T>
 static int run_bias_gelu_bwd(const void *gr, const void *x, const void *bias,
                              void *dx, void *dbias, void *ws, int64_t ws_bytes,
                              int64_t rows, int64_t cols, hipStream_t st) {
-  const bool vec_ok = cols % kE == 0 && aligned16(x) && aligned16(gr) &&
+  constexpr int kE = io<T>::EPV;
+  const bool vec_ok = cols % kE == 0 && cols <= 0x7fffffff && aligned16(x) && aligned16(gr) &&
                       aligned16(dx) && aligned16(bias) && aligned16(ws) &&
                       cols / kE <= 0x7fffffff;
   if (!vec_ok) {
@@ -577,7 +594,7 @@ static int run_bias_gelu_bwd(const void *gr, const void *x, const void *bias,
     return check_launch("colsum_generic_kernel");
   }
   const int unroll = eltwise_unroll(4);
-  const EltGeom g = eltwise_geom_bwd(rows, cols, unroll);
+  const EltGeom g = eltwise_geom_bwd(rows, cols, unroll, kE);
   const int64_t parts = g.slots;
   const int64_t nblocks = parts * g.tiles;
   OSLO_REQUIRE(nblocks <= 0x7fffffff, "bias_gelu bwd: too many workgroups");
@@ -611,7 +628,8 @@ static int run_bda_fwd(const void *x, const void *bias, const void *res,
                        hipStream_t st) {
   const DropArgs d = make_drop(p, seed, offset);
   const bool drop = p > 0.f;
-  const bool vec_ok = cols % kE == 0 && aligned16(x) && aligned16(out) &&
+  constexpr int kE = io<T>::EPV;
+  const bool vec_ok = cols % kE == 0 && cols <= 0x7fffffff && aligned16(x) && aligned16(out) &&
                       aligned16(bias) && aligned16(res) &&
                       (reinterpret_cast<uintptr_t>(mask_out) & 7u) == 0 &&
                       cols / kE <= 0x7fffffff;
@@ -624,7 +642,7 @@ static int run_bda_fwd(const void *x, const void *bias, const void *res,
     return check_launch("bias_dropout_add_fwd_generic_kernel");
   }
   const int unroll = eltwise_unroll(2) > 2 ? 2 : eltwise_unroll(2);
-  const EltGeom g = eltwise_geom_fwd(rows, cols, unroll);
+  const EltGeom g = eltwise_geom_fwd(rows, cols, unroll, kE);
   const int64_t nblocks = g.slots * g.tiles;
   OSLO_REQUIRE(nblocks <= 0x7fffffff, "bias_dropout_add fwd: too many workgroups");
   const dim3 grid((unsigned)nblocks);
@@ -654,7 +672,8 @@ static int run_bda_bwd(const void *gr, void *dx, void *dbias, void *ws,
                        uint64_t seed, uint64_t offset, hipStream_t st) {
   const DropArgs d = make_drop(p, seed, offset);
   const bool drop = p > 0.f;
-  const bool vec_ok = cols % kE == 0 && aligned16(gr) && aligned16(dx) &&
+  constexpr int kE = io<T>::EPV;
+  const bool vec_ok = cols % kE == 0 && cols <= 0x7fffffff && aligned16(gr) && aligned16(dx) &&
                       aligned16(ws) && cols / kE <= 0x7fffffff;
   if (!vec_ok) {
     if (dx == nullptr) {
@@ -674,7 +693,7 @@ static int run_bda_bwd(const void *gr, void *dx, void *dbias, void *ws,
     return check_launch("colsum_generic_kernel");
   }
   const int unroll = eltwise_unroll(4);
-  const EltGeom g = eltwise_geom_bwd(rows, cols, unroll);
+  const EltGeom g = eltwise_geom_bwd(rows, cols, unroll, kE);
   const int64_t parts = g.slots;
   const int64_t nblocks = parts * g.tiles;
   OSLO_REQUIRE(nblocks <= 0x7fffffff, "bias_dropout_add bwd: too many workgroups");

@@ -35,6 +35,11 @@ SHAPES = [
     (301, 3072, BF16),    # 384 chunks: three tiles of 128 lanes
     (67, 11008, BF16),    # 1376 chunks: 43 tiles of 32 lanes
     (129, 96, F32),
+    # fp32 chunks are 4 elements = half a dropout group; with cols % 8 == 4
+    # every other row starts in the middle of a group
+    (513, 36, F32),
+    (77, 100, F32),
+    (33, 4, F32),
 ]
 
 
