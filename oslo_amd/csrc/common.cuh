@@ -338,6 +338,20 @@ template <typename Op> __device__ __forceinline__ float row16_allreduce(float v)
   return readlane(v, 0);
 }
 
+// A product / difference that is rounded on its own and never fused with a
+// neighbouring operation into a multiply-add.  Two kernels that must
+// reproduce the same bits (a forward pass and the backward pass that
+// recomputes it) cannot leave that choice to the optimiser; the header's
+// __fmul_rn / __fsub_rn are plain operators here and do get fused.
+__device__ __forceinline__ float mul_rn(float a, float b) {
+#pragma clang fp contract(off)
+  return a * b;
+}
+__device__ __forceinline__ float sub_rn(float a, float b) {
+#pragma clang fp contract(off)
+  return a - b;
+}
+
 // Reduction within each group of LPR (8, 16 or 32) consecutive lanes; every
 // lane of a group receives its group's result (each step is symmetric, so the
 // lanes of a group hold the same bits).

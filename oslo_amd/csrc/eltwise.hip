@@ -446,9 +446,40 @@ __global__ __launch_bounds__(64) void wave_reduce_selftest_kernel(float *out) {
   }
 }
 
+// Functor of the generic column sum: the value dx would hold, rounded to the
+// storage type, without storing it.
+template <typename T> struct DroppedGradient {
+  const T *gr;
+  int64_t cols;
+  DropArgs d;
+  bool drop;
+  __device__ __forceinline__ void operator()(int64_t r, int64_t c, float *acc) const {
+    const int64_t i = r * cols + c;
+    float t = io<T>::from_scalar(gr[i]);
+    if (drop) t = keep_element(i, d) ? t * d.scale : 0.f;
+    acc[0] += io<T>::round(t);
+  }
+};
+
 // ---------------------------------------------------------------------------
 // host side
 // ---------------------------------------------------------------------------
+// Column sum of a stored [rows, cols] tensor on the generic path: row slices
+// through the workspace when it can be used, else one thread per column.
+template <typename T>
+static int generic_colsum_of_stored(const void *a, void *out, void *ws,
+                                    int64_t ws_bytes, int64_t rows,
+                                    int64_t cols, hipStream_t st) {
+  const int64_t S = generic_colsum_slices(ws, ws_bytes, 1, rows, cols);
+  if (S > 0) {
+    StoredValue<T> f{(const T *)a, cols};
+    return launch_generic_colsum<1, T>(f, ws, S, rows, cols, out, nullptr, st);
+  }
+  colsum_generic_kernel<T><<<dim3((unsigned)ceil_div(cols, 256)), 256, 0, st>>>(
+      (const T *)a, (T *)out, rows, cols);
+  return check_launch("colsum_generic_kernel");
+}
+
 static inline int eltwise_unroll(int dflt) {
   const int u = g_tune.eltwise_unroll;
   return u == 1 || u == 2 || u == 4 ? u : dflt;
@@ -589,9 +620,7 @@ static int run_bias_gelu_bwd(const void *gr, const void *x, const void *bias,
         (const T *)gr, (const T *)x, (const T *)bias, (T *)dx, n, cols);
     int rc = check_launch("bias_gelu_bwd_generic_kernel");
     if (rc != OSLO_OK || dbias == nullptr) return rc;
-    colsum_generic_kernel<T><<<dim3((unsigned)ceil_div(cols, 256)), 256, 0, st>>>(
-        (const T *)dx, (T *)dbias, rows, cols);
-    return check_launch("colsum_generic_kernel");
+    return generic_colsum_of_stored<T>(dx, dbias, ws, ws_bytes, rows, cols, st);
   }
   const int unroll = eltwise_unroll(4);
   const EltGeom g = eltwise_geom_bwd(rows, cols, unroll, kE);
@@ -677,6 +706,11 @@ static int run_bda_bwd(const void *gr, void *dx, void *dbias, void *ws,
                       aligned16(ws) && cols / kE <= 0x7fffffff;
   if (!vec_ok) {
     if (dx == nullptr) {
+      const int64_t S = generic_colsum_slices(ws, ws_bytes, 1, rows, cols);
+      if (S > 0) {
+        DroppedGradient<T> f{(const T *)gr, cols, d, drop};
+        return launch_generic_colsum<1, T>(f, ws, S, rows, cols, dbias, nullptr, st);
+      }
       bias_dropout_add_dbias_generic_kernel<T>
           <<<dim3((unsigned)ceil_div(cols, 256)), 256, 0, st>>>(
               (const T *)gr, (T *)dbias, rows, cols, d, drop);
@@ -688,9 +722,7 @@ static int run_bda_bwd(const void *gr, void *dx, void *dbias, void *ws,
                                                        n, d, drop);
     int rc = check_launch("bias_dropout_add_bwd_generic_kernel");
     if (rc != OSLO_OK || dbias == nullptr) return rc;
-    colsum_generic_kernel<T><<<dim3((unsigned)ceil_div(cols, 256)), 256, 0, st>>>(
-        (const T *)dx, (T *)dbias, rows, cols);
-    return check_launch("colsum_generic_kernel");
+    return generic_colsum_of_stored<T>(dx, dbias, ws, ws_bytes, rows, cols, st);
   }
   const int unroll = eltwise_unroll(4);
   const EltGeom g = eltwise_geom_bwd(rows, cols, unroll, kE);

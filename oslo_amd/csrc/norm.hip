@@ -785,6 +785,21 @@ __global__ __launch_bounds__(256) void norm_bwd_param_generic_kernel(
   if constexpr (!RMS) dbeta[col] = io<V>::to_scalar(ab);
 }
 
+// Functor of the generic column sums: dgamma (and dbeta) contributions.
+template <typename T, typename V, bool RMS> struct NormParamGrad {
+  const V *dy;
+  const T *x;
+  const float *mean;
+  const float *invvar;
+  int64_t n2;
+  __device__ __forceinline__ void operator()(int64_t r, int64_t c, float *acc) const {
+    const float mu = RMS ? 0.f : mean[r];
+    const float d = io<V>::from_scalar(dy[r * n2 + c]);
+    acc[0] += d * (io<T>::from_scalar(x[r * n2 + c]) - mu) * invvar[r];
+    if constexpr (!RMS) acc[1] += d;
+  }
+};
+
 // ---------------------------------------------------------------------------
 // host side
 // ---------------------------------------------------------------------------
@@ -1075,15 +1090,31 @@ static int launch_norm_bwd(const void *dy, const void *x, const float *mean,
           if (fe->drop && fe->dx_drop == nullptr)
             return fail(OSLO_ERR_INVALID_ARGUMENT,
                         "fused norm bwd: dbias with dropout needs dx_drop");
-          norm_colsum_generic_kernel<T>
-              <<<dim3((unsigned)ceil_div(n2, 256)), 256, 0, st>>>(
-                  (const T *)src, (T *)dbias, n1, n2);
-          rc = check_launch("norm_colsum_generic_kernel");
+          const int64_t S = generic_colsum_slices(ws, ws_bytes, 1, n1, n2);
+          if (S > 0) {
+            StoredValue<T> f{(const T *)src, n2};
+            rc = launch_generic_colsum<1, T>(f, ws, S, n1, n2, dbias, nullptr, st);
+          } else {
+            norm_colsum_generic_kernel<T>
+                <<<dim3((unsigned)ceil_div(n2, 256)), 256, 0, st>>>(
+                    (const T *)src, (T *)dbias, n1, n2);
+            rc = check_launch("norm_colsum_generic_kernel");
+          }
           if (rc != OSLO_OK) return rc;
         }
       }
     }
     if (dgamma == nullptr) return rc;
+    {
+      // (stream order: the partial rows of a bias gradient above have been
+      //  consumed by their own finalize before these overwrite them)
+      constexpr int NA = RMS ? 1 : 2;
+      const int64_t S = generic_colsum_slices(ws, ws_bytes, NA, n1, n2);
+      if (S > 0) {
+        NormParamGrad<T, V, RMS> f{(const V *)dy, (const T *)x, mean, invvar, n2};
+        return launch_generic_colsum<NA, V>(f, ws, S, n1, n2, dgamma, dbeta, st);
+      }
+    }
     norm_bwd_param_generic_kernel<T, V, RMS>
         <<<dim3((unsigned)ceil_div(n2, 256)), 256, 0, st>>>(
             (const V *)dy, (const T *)x, mean, invvar, (V *)dgamma,

@@ -226,14 +226,14 @@ __global__ __launch_bounds__(1024) void softmax_fwd_kernel(
         for (int e = 0; e < E; ++e) {
           // (rounded product, never fused into the later subtraction: the
           //  backward pass of the dropout variant recomputes it bit for bit)
-          const float t = __fmul_rn(v[j][k][e], c2);
+          const float t = mul_rn(v[j][k][e], c2);
           v[j][k][e] = t;
           m = fmaxf(m, t);
         }
       } else {
 #pragma unroll
         for (int e = 0; e < E; ++e) {
-          const float t = (mbits[j][k] >> e) & 1u ? ninf : __fmul_rn(v[j][k][e], c2);
+          const float t = (mbits[j][k] >> e) & 1u ? ninf : mul_rn(v[j][k][e], c2);
           v[j][k][e] = t;
           m = fmaxf(m, t);
         }
@@ -257,7 +257,7 @@ __global__ __launch_bounds__(1024) void softmax_fwd_kernel(
       if (none_visible[j][k]) continue;
 #pragma unroll
       for (int e = 0; e < E; ++e) {
-        const float p = __builtin_amdgcn_exp2f(__fsub_rn(v[j][k][e], off));
+        const float p = __builtin_amdgcn_exp2f(sub_rn(v[j][k][e], off));
         v[j][k][e] = p;  // exp2(-inf) == 0 for masked keys
         s += p;
       }
@@ -415,10 +415,10 @@ __global__ __launch_bounds__(1024) void softmax_dropout_bwd_kernel(
         // the product is rounded before the subtraction, exactly as the
         // forward pass formed its exponent (no fused multiply-add here)
         float p =
-            __builtin_amdgcn_exp2f(__fsub_rn(__fmul_rn(yv[j][k][e], c2), rmax[j])) * rinv[j];
+            __builtin_amdgcn_exp2f(sub_rn(mul_rn(yv[j][k][e], c2), rmax[j])) * rinv[j];
         if (empty) p = -rinv[j];
         if ((mbits[j][k] >> e) & 1u) p = 0.f;
-        const float dp = (keep >> e) & 1u ? gv[j][k][e] * d.scale : 0.f;
+        const float dp = (keep >> e) & 1u ? mul_rn(gv[j][k][e], d.scale) : 0.f;
         yv[j][k][e] = p;
         gv[j][k][e] = dp;
         a += p * dp;
@@ -616,7 +616,7 @@ __global__ __launch_bounds__(256) void softmax_fwd_generic_kernel(
     float m = ninf;
     for (int i = threadIdx.x; i < g.sk; i += 256) {
       const bool hidden = MODE == kModeCausal ? i >= visible : mrow[i] != 0;
-      if (!hidden) m = fmaxf(m, __fmul_rn(io<T>::from_scalar(xr[i]), c2));
+      if (!hidden) m = fmaxf(m, mul_rn(io<T>::from_scalar(xr[i]), c2));
     }
     m = block_reduce_256(m, sh, true);
     const bool empty = m == ninf;
@@ -625,7 +625,7 @@ __global__ __launch_bounds__(256) void softmax_fwd_generic_kernel(
       const bool hidden = MODE == kModeCausal ? i >= visible : mrow[i] != 0;
       if (!hidden)
         s += __builtin_amdgcn_exp2f(
-            __fsub_rn(__fmul_rn(io<T>::from_scalar(xr[i]), c2), m));
+            sub_rn(mul_rn(io<T>::from_scalar(xr[i]), c2), m));
     }
     s = block_reduce_256(s, sh, false);
     const float inv = empty ? 0.f : 1.0f / s;
@@ -635,7 +635,7 @@ __global__ __launch_bounds__(256) void softmax_fwd_generic_kernel(
       float p = 0.f;
       if (!hidden)
         p = __builtin_amdgcn_exp2f(
-            __fsub_rn(__fmul_rn(io<T>::from_scalar(xr[i]), c2), m));
+            sub_rn(mul_rn(io<T>::from_scalar(xr[i]), c2), m));
       float o = p * inv + fill;
       if constexpr (DROP)
         o = keep_element(row * g.sk + i, d) ? o * d.scale : 0.f;
@@ -672,12 +672,13 @@ __global__ __launch_bounds__(256) void softmax_dropout_bwd_generic_kernel(
       const bool hidden = MODE == kModeCausal ? i >= visible : mrow[i] != 0;
       if (hidden) return 0.f;
       return __builtin_amdgcn_exp2f(
-                 __fsub_rn(__fmul_rn(io<T>::from_scalar(xr[i]), c2), m)) *
+                 sub_rn(mul_rn(io<T>::from_scalar(xr[i]), c2), m)) *
              inv;
     };
     auto dprob = [&](int i) {
-      return keep_element(row * g.sk + i, d) ? io<T>::from_scalar(gr[i]) * d.scale
-                                             : 0.f;
+      return keep_element(row * g.sk + i, d)
+                 ? mul_rn(io<T>::from_scalar(gr[i]), d.scale)
+                 : 0.f;
     };
     float s = 0.f;
     for (int i = threadIdx.x; i < g.sk; i += 256) s += prob(i) * dprob(i);
@@ -705,6 +706,168 @@ __global__ __launch_bounds__(256) void softmax_bwd_generic_kernel(
       dxr[i] = io<T>::to_scalar(scale * (yy * (io<T>::from_scalar(gr[i]) - s)));
     }
   }
+}
+
+// ---------------------------------------------------------------------------
+// generic rows of at most kWaveRowMax keys: one wavefront per row, the row in
+// registers (lane l holds keys l, l + 64, ...), scalar accesses, no LDS and no
+// barrier.  Any length and alignment; the arithmetic is that of the kernels
+// above, term for term.
+// ---------------------------------------------------------------------------
+constexpr int kWaveRowMax = 1024;
+
+template <typename T, int MODE, bool DROP>
+__global__ __launch_bounds__(256) void softmax_fwd_wave_kernel(
+    const T *__restrict__ x, const uint8_t *__restrict__ mask,
+    T *__restrict__ y, float *__restrict__ stats, SoftmaxGeom g, float scale,
+    DropArgs d) {
+  constexpr int K = kWaveRowMax / kWave;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const float ninf = -__builtin_inff();
+  const float c2 = scale * kLog2e;
+  for (int64_t r = (int64_t)blockIdx.x * 4 + wave; r < g.rows;
+       r += (int64_t)gridDim.x * 4) {
+    int64_t row;
+    int visible;
+    const uint8_t *mrow;
+    row_setup<MODE>(g, r, mask, row, visible, mrow);
+    const T *xr = x + row * g.sk;
+    T *yr = y + row * g.sk;
+    float v[K];
+    float m = ninf;
+#pragma unroll
+    for (int k = 0; k < K; ++k) {
+      const int i = lane + kWave * k;
+      v[k] = ninf;
+      if (i < g.sk) {
+        const bool hidden = MODE == kModeCausal ? i >= visible : mrow[i] != 0;
+        if (!hidden) v[k] = mul_rn(io<T>::from_scalar(xr[i]), c2);
+      }
+      m = fmaxf(m, v[k]);
+    }
+    m = wave_max(m);
+    const bool empty = m == ninf;
+    const float off = empty ? 0.f : m;
+    float s = 0.f;
+#pragma unroll
+    for (int k = 0; k < K; ++k) {
+      const float p = __builtin_amdgcn_exp2f(sub_rn(v[k], off));  // 0 for hidden keys
+      v[k] = p;
+      s += p;
+    }
+    s = wave_sum(s);
+    const float inv = empty ? 0.f : 1.0f / s;
+    const float fill = empty ? 1.0f / (float)g.sk : 0.f;
+#pragma unroll
+    for (int k = 0; k < K; ++k) {
+      const int i = lane + kWave * k;
+      if (i < g.sk) {
+        float o = v[k] * inv + fill;
+        if constexpr (DROP)
+          o = keep_element(row * g.sk + i, d) ? o * d.scale : 0.f;
+        yr[i] = io<T>::to_scalar(o);
+      }
+    }
+    if constexpr (DROP) {
+      if (lane == 0) {
+        stats[2 * row] = empty ? 0.f : m;
+        stats[2 * row + 1] = empty ? -fill : inv;
+      }
+    }
+  }
+}
+
+template <typename T, int MODE>
+__global__ __launch_bounds__(256) void softmax_dropout_bwd_wave_kernel(
+    const T *__restrict__ dy, const T *__restrict__ x,
+    const float *__restrict__ stats, const uint8_t *__restrict__ mask,
+    T *__restrict__ dx, SoftmaxGeom g, float scale, DropArgs d) {
+  constexpr int K = kWaveRowMax / kWave;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const float c2 = scale * kLog2e;
+  for (int64_t r = (int64_t)blockIdx.x * 4 + wave; r < g.rows;
+       r += (int64_t)gridDim.x * 4) {
+    int64_t row;
+    int visible;
+    const uint8_t *mrow;
+    row_setup<MODE>(g, r, mask, row, visible, mrow);
+    const T *xr = x + row * g.sk;
+    const T *gr = dy + row * g.sk;
+    T *dxr = dx + row * g.sk;
+    const float m = stats[2 * row], inv = stats[2 * row + 1];
+    const bool empty = inv < 0.f;
+    float pv[K], gv[K];
+    float s = 0.f;
+#pragma unroll
+    for (int k = 0; k < K; ++k) {
+      const int i = lane + kWave * k;
+      pv[k] = 0.f;
+      gv[k] = 0.f;
+      if (i < g.sk) {
+        const bool hidden = MODE == kModeCausal ? i >= visible : mrow[i] != 0;
+        float p = 0.f;
+        if (empty)
+          p = -inv;
+        else if (!hidden)
+          p = __builtin_amdgcn_exp2f(
+                  sub_rn(mul_rn(io<T>::from_scalar(xr[i]), c2), m)) *
+              inv;
+        pv[k] = p;
+        // (a rounded product: fused into the subtraction below it would
+        //  leave the product's rounding error where an exact zero belongs)
+        gv[k] = keep_element(row * g.sk + i, d)
+                    ? mul_rn(io<T>::from_scalar(gr[i]), d.scale)
+                    : 0.f;
+      }
+      s += pv[k] * gv[k];
+    }
+    s = wave_sum(s);
+#pragma unroll
+    for (int k = 0; k < K; ++k) {
+      const int i = lane + kWave * k;
+      if (i < g.sk) dxr[i] = io<T>::to_scalar(scale * (pv[k] * (gv[k] - s)));
+    }
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void softmax_bwd_wave_kernel(
+    const T *__restrict__ dy, const T *__restrict__ y, T *__restrict__ dx,
+    int64_t rows, int sk, float scale) {
+  constexpr int K = kWaveRowMax / kWave;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  for (int64_t r = (int64_t)blockIdx.x * 4 + wave; r < rows;
+       r += (int64_t)gridDim.x * 4) {
+    const T *yr = y + r * sk;
+    const T *gr = dy + r * sk;
+    T *dxr = dx + r * sk;
+    float yv[K], gv[K];
+    float s = 0.f;
+#pragma unroll
+    for (int k = 0; k < K; ++k) {
+      const int i = lane + kWave * k;
+      yv[k] = 0.f;
+      gv[k] = 0.f;
+      if (i < sk) {
+        yv[k] = io<T>::from_scalar(yr[i]);
+        gv[k] = io<T>::from_scalar(gr[i]);
+      }
+      s += yv[k] * gv[k];
+    }
+    s = wave_sum(s);
+#pragma unroll
+    for (int k = 0; k < K; ++k) {
+      const int i = lane + kWave * k;
+      if (i < sk) dxr[i] = io<T>::to_scalar(scale * (yv[k] * (gv[k] - s)));
+    }
+  }
+}
+
+// workgroups of a wave-per-row launch (four rows each)
+static inline int64_t wave_row_grid(int64_t rows) {
+  const int64_t want = ceil_div(rows, 4);
+  const int64_t cap = (int64_t)device_cu_count() * 64;
+  return want < cap ? want : cap;
 }
 
 // ---------------------------------------------------------------------------
@@ -814,6 +977,16 @@ static int launch_softmax_fwd(const void *x, const uint8_t *mask, void *y,
     const int64_t grid = g.rows < (int64_t)device_cu_count() * 32
                              ? g.rows
                              : (int64_t)device_cu_count() * 32;
+    if (g.sk <= kWaveRowMax) {
+      const dim3 wgrid((unsigned)wave_row_grid(g.rows));
+      if (drop)
+        softmax_fwd_wave_kernel<T, MODE, true><<<wgrid, 256, 0, st>>>(
+            (const T *)x, mask, (T *)y, stats, g, scale, d);
+      else
+        softmax_fwd_wave_kernel<T, MODE, false><<<wgrid, 256, 0, st>>>(
+            (const T *)x, mask, (T *)y, nullptr, g, scale, d);
+      return check_launch("softmax_fwd_wave_kernel");
+    }
     if (drop)
       softmax_fwd_generic_kernel<T, MODE, true>
           <<<dim3((unsigned)grid), 256, 0, st>>>((const T *)x, mask, (T *)y,
@@ -860,6 +1033,11 @@ static int launch_softmax_bwd(const void *dy, const void *y,
     const int64_t grid = g.rows < (int64_t)device_cu_count() * 32
                              ? g.rows
                              : (int64_t)device_cu_count() * 32;
+    if (g.sk <= kWaveRowMax) {
+      softmax_bwd_wave_kernel<T><<<dim3((unsigned)wave_row_grid(g.rows)), 256, 0, st>>>(
+          (const T *)dy, (const T *)y, (T *)dx, g.rows, g.sk, scale);
+      return check_launch("softmax_bwd_wave_kernel");
+    }
     softmax_bwd_generic_kernel<T><<<dim3((unsigned)grid), 256, 0, st>>>(
         (const T *)dy, (const T *)y, (T *)dx, g.rows, g.sk, scale);
     return check_launch("softmax_bwd_generic_kernel");
@@ -894,6 +1072,12 @@ static int launch_softmax_dropout_bwd(const void *dy, const void *x,
     const int64_t grid = g.rows < (int64_t)device_cu_count() * 32
                              ? g.rows
                              : (int64_t)device_cu_count() * 32;
+    if (g.sk <= kWaveRowMax) {
+      softmax_dropout_bwd_wave_kernel<T, MODE>
+          <<<dim3((unsigned)wave_row_grid(g.rows)), 256, 0, st>>>(
+              (const T *)dy, (const T *)x, stats, mask, (T *)dx, g, scale, d);
+      return check_launch("softmax_dropout_bwd_wave_kernel");
+    }
     softmax_dropout_bwd_generic_kernel<T, MODE>
         <<<dim3((unsigned)grid), 256, 0, st>>>((const T *)dy, (const T *)x,
                                                stats, mask, (T *)dx, g, scale,

@@ -38,6 +38,11 @@ CASES = [
     (17, 8, BF16, BF16),
     (1, 4096, BF16, BF16),
     (300, 2048, F32, F32),
+    # lengths that are no multiple of the vector width, many rows: scalar row
+    # kernels and the two-step column sums through the workspace
+    (3001, 100, BF16, BF16),
+    (300, 4100, F16, F16),
+    (2000, 37, F32, F32),
 ]
 
 

@@ -28,6 +28,13 @@ CAUSAL_CASES = [
     (2, 33, 33, F32, 0.7),          # odd length: scalar kernel
     (2, 9, 100000, BF16, 1.0),      # beyond the register path
     (1, 1, 8, F32, 2.0),
+    # lengths that are no multiple of the vector width: one wavefront per row
+    # up to 1024 keys, one workgroup per row beyond
+    (3, 50, 50, BF16, 0.5),
+    (2, 197, 197, F16, 0.125),
+    (2, 40, 1001, BF16, 0.25),
+    (2, 7, 1027, F16, 0.25),
+    (5, 3, 1, BF16, 1.0),
 ]
 
 

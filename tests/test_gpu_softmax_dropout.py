@@ -36,6 +36,10 @@ CAUSAL_CASES = [
     (2, 5, 100000, BF16, 1.0, 0.1),       # beyond the register path
     (1, 1, 8, F32, 2.0, 0.3),
     (2, 16, 64, BF16, 1.0, 1.0),          # p = 1: everything dropped
+    (3, 50, 50, BF16, 0.5, 0.1),          # one wavefront per row, scalar accesses
+    (2, 197, 197, F16, 0.125, 0.2),
+    (2, 9, 1001, BF16, 0.25, 0.1),
+    (4, 5, 1, F32, 1.0, 0.3),             # one key: the gradient is exactly zero
 ]
 
 
