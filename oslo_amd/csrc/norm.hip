@@ -152,7 +152,7 @@ __global__ __launch_bounds__(MAXT) void norm_fwd_reg_kernel(
     int rpb, int iters, FusePrologue fp) {
   constexpr int E = chunk_elems<T, V>::value;
   static_assert(!FUSE || sizeof(T) == sizeof(V), "fused prologue: one dtype");
-  static_assert(LPR == kWave || (VPL == 1 && !FUSE), "side-by-side rows: one chunk per lane");
+  static_assert(LPR == kWave || VPL == 1, "side-by-side rows: one chunk per lane");
   __shared__ float red[2][48];
   const int lane = threadIdx.x & 63;
   // the wave index is uniform: keep it (and the row arithmetic) in scalar registers
@@ -457,7 +457,7 @@ __global__ __launch_bounds__(MAXT) void norm_bwd_reg_kernel(
     int64_t n1, int n2, int wpr, int rpb, FuseEpilogue fe) {
   constexpr int E = chunk_elems<T, V>::value;
   static_assert(!FUSE || sizeof(T) == sizeof(V), "fused epilogue: one dtype");
-  static_assert(LPR == kWave || (VPL == 1 && !FUSE), "side-by-side rows: one chunk per lane");
+  static_assert(LPR == kWave || VPL == 1, "side-by-side rows: one chunk per lane");
   extern __shared__ float xslot[];  // [n2] when rpb > 1
   __shared__ float red[2][32];
   const int lane = threadIdx.x & 63;
@@ -887,7 +887,7 @@ static int launch_norm_fwd(const void *x, const void *gamma, const void *beta,
   }
   // The fused build holds two more packed operands per chunk: at most 16
   // elements per lane.  Measured on MI355X: 16 per lane while a row then fits
-  // four waves, else 8 per lane over up to sixteen waves, else 16 per lane.
+  // four waves, else 8 per lane over up to twelve waves, else 16 per lane.
   bool fused_big = false;
   if (fused && vec_ok) {
     const int waves = g_tune.norm_fwd_waves > 0 ? g_tune.norm_fwd_waves : 4;
@@ -897,8 +897,15 @@ static int launch_norm_fwd(const void *x, const void *gamma, const void *beta,
     } else {
       sp = split_row(n2 / E, 16 / E, kVpl, 4, waves);
       if (!sp.ok || sp.wpr > 4) {
+        // (8 per lane measures 20 % slower once it needs 14 or more waves:
+        //  rows of 7168 and 8192 16-bit elements)
         const RowSplit narrow = split_row(n2 / E, 8 / E, kVpl, 4, waves);
-        if (narrow.ok) sp = narrow;
+        if (sp.ok && sp.wpr == 5)
+          // rows of 5120 16-bit elements: three rows of five waves per
+          // workgroup measure 8 % faster than ten waves at 8 per lane
+          sp = split_row(n2 / E, 16 / E, kVpl, 4, 16);
+        else if (narrow.ok && (!sp.ok || narrow.wpr <= 12))
+          sp = narrow;
       }
     }
     if (sp.ok && sp.vpl * E > 16) sp.ok = false;
@@ -924,12 +931,36 @@ static int launch_norm_fwd(const void *x, const void *gamma, const void *beta,
   const int64_t maxgrid = (int64_t)device_cu_count() * 64;
   if (grid > maxgrid) grid = maxgrid;
   // short rows side by side in a wave
-  const int lpr = (!fused && sp.wpr == 1 && sp.vpl == 1) ? lanes_per_row(n2 / E) : kWave;
+  const int lpr = (sp.wpr == 1 && sp.vpl == 1) ? lanes_per_row(n2 / E) : kWave;
   if (lpr < kWave) {
     const int rpb_eff = sp.rpb * (kWave / lpr);
     const bool even_l = (n2 / E) == lpr;
     int64_t grid_l = ceil_div(ceil_div(n1, rpb_eff), iters);
     if (grid_l > maxgrid) grid_l = maxgrid;
+    if constexpr (kCanFuse) {
+      if (fused) {
+#define OSLO_FWD_LPR_FUSED(LPR_)                                             \
+  case LPR_:                                                                 \
+    if (even_l)                                                              \
+      norm_fwd_reg_kernel<T, V, 1, RMS, true, 256, true, LPR_>               \
+          <<<dim3((unsigned)grid_l), threads, 0, st>>>(                      \
+              (const T *)x, (const V *)gamma, (const V *)beta, (V *)y, mean, \
+              invvar, n1, (int)n2, eps, 1, rpb_eff, iters, *fp);             \
+    else                                                                     \
+      norm_fwd_reg_kernel<T, V, 1, RMS, false, 256, true, LPR_>              \
+          <<<dim3((unsigned)grid_l), threads, 0, st>>>(                      \
+              (const T *)x, (const V *)gamma, (const V *)beta, (V *)y, mean, \
+              invvar, n1, (int)n2, eps, 1, rpb_eff, iters, *fp);             \
+    break;
+        switch (lpr) {
+          OSLO_FWD_LPR_FUSED(8)
+          OSLO_FWD_LPR_FUSED(16)
+          OSLO_FWD_LPR_FUSED(32)
+        }
+#undef OSLO_FWD_LPR_FUSED
+        return check_launch("norm_fwd_reg_kernel (fused, side-by-side rows)");
+      }
+    }
 #define OSLO_FWD_LPR(LPR_)                                                   \
   case LPR_:                                                                 \
     if (even_l)                                                              \
@@ -1122,7 +1153,7 @@ static int launch_norm_bwd(const void *dy, const void *x, const float *mean,
     return check_launch("norm_bwd_param_generic_kernel");
   }
   // short rows side by side in a wave: the row slots of a workgroup multiply
-  const int lpr = (!fused && sp.wpr == 1 && sp.vpl == 1) ? lanes_per_row(n2 / E) : kWave;
+  const int lpr = (sp.wpr == 1 && sp.vpl == 1) ? lanes_per_row(n2 / E) : kWave;
   const int wave_slots = sp.rpb;  // row slots at wave granularity
   if (lpr < kWave) sp.rpb *= kWave / lpr;
   int64_t P = colsum_parts_norm(n1, n2);
@@ -1195,6 +1226,23 @@ static int launch_norm_bwd(const void *dy, const void *x, const float *mean,
   if (lpr < kWave) {
 #define OSLO_BWD_LPR(LPR_)                                                  \
   case LPR_:                                                                \
+    if constexpr (kCanFuse) {                                               \
+      if (fused) {                                                          \
+        if (even)                                                           \
+          norm_bwd_reg_kernel<T, V, 1, RMS, true, 1, true, 1024, LPR_>      \
+              <<<dim3((unsigned)P), threads, lds, st>>>(                    \
+                  (const V *)dy, (const T *)x, mean, invvar,                \
+                  (const V *)gamma, (T *)dx, part, n1, (int)n2, 1, sp.rpb,  \
+                  fev);                                                     \
+        else                                                                \
+          norm_bwd_reg_kernel<T, V, 1, RMS, false, 1, true, 1024, LPR_>     \
+              <<<dim3((unsigned)P), threads, lds, st>>>(                    \
+                  (const V *)dy, (const T *)x, mean, invvar,                \
+                  (const V *)gamma, (T *)dx, part, n1, (int)n2, 1, sp.rpb,  \
+                  fev);                                                     \
+        break;                                                              \
+      }                                                                     \
+    }                                                                       \
     if (even)                                                               \
       norm_bwd_reg_kernel<T, V, 1, RMS, true, 1, false, 1024, LPR_>         \
           <<<dim3((unsigned)P), threads, lds, st>>>(                        \

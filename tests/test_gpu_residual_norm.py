@@ -30,6 +30,13 @@ CASES = [
     (7, 100, F32, 0.1),         # vector path needs n2 % 4 == 0: ok; 25 chunks
     (6, 1001, BF16, 0.1),       # odd length: composed scalar path
     (4, 40000, BF16, 0.1),      # beyond the register path: composed path
+    # short rows side by side in a wavefront (8 / 16 / 32 lanes per row)
+    (1003, 256, BF16, 0.1),
+    (517, 128, F16, 0.2),
+    (2050, 64, BF16, 0.1),
+    (333, 40, BF16, 0.1),       # 5 chunks in 8 lanes
+    (700, 100, F32, 0.1),       # 25 fp32 chunks in 32 lanes
+    (90, 7168, BF16, 0.1),      # 16 elements per lane over seven waves
     (1, 8, F32, 0.5),
     (12, 2048, BF16, 0.0),      # no dropout
     (12, 2048, BF16, 1.0),      # everything dropped
