@@ -710,18 +710,83 @@ __global__ __launch_bounds__(256) void softmax_bwd_generic_kernel(
 
 // ---------------------------------------------------------------------------
 // generic rows of at most kWaveRowMax keys: one wavefront per row, the row in
-// registers (lane l holds keys l, l + 64, ...), scalar accesses, no LDS and no
-// barrier.  Any length and alignment; the arithmetic is that of the kernels
-// above, term for term.
+// registers, no LDS and no barrier.  A lane accesses EW consecutive keys at a
+// time (lane l holds keys EW * (l + 64 k) ...): EW = 4 or 2 when the row
+// length and the pointers allow 8- or 4-byte accesses, else 1 (any length and
+// alignment).  The arithmetic is that of the kernels above, term for term.
 // ---------------------------------------------------------------------------
 constexpr int kWaveRowMax = 1024;
 
-template <typename T, int MODE, bool DROP>
+template <typename T, int EW>
+__device__ __forceinline__ void ld_small(const T *p, float *f) {
+  if constexpr (EW == 1) {
+    f[0] = io<T>::from_scalar(p[0]);
+  } else {
+    T t[EW];
+    if constexpr (EW * sizeof(T) == 4) {
+      const uint32_t raw = *reinterpret_cast<const uint32_t *>(p);
+      __builtin_memcpy(t, &raw, 4);
+    } else {
+      static_assert(EW * sizeof(T) == 8, "at most 8 bytes per access");
+      const u32x2 raw = *reinterpret_cast<const u32x2 *>(p);
+      __builtin_memcpy(t, &raw, 8);
+    }
+#pragma unroll
+    for (int e = 0; e < EW; ++e) f[e] = io<T>::from_scalar(t[e]);
+  }
+}
+
+template <typename T, int EW>
+__device__ __forceinline__ void st_small(T *p, const float *f) {
+  if constexpr (EW == 1) {
+    p[0] = io<T>::to_scalar(f[0]);
+  } else {
+    T t[EW];
+#pragma unroll
+    for (int e = 0; e < EW; ++e) t[e] = io<T>::to_scalar(f[e]);
+    if constexpr (EW * sizeof(T) == 4) {
+      uint32_t raw;
+      __builtin_memcpy(&raw, t, 4);
+      *reinterpret_cast<uint32_t *>(p) = raw;
+    } else {
+      u32x2 raw;
+      __builtin_memcpy(&raw, t, 8);
+      *reinterpret_cast<u32x2 *>(p) = raw;
+    }
+  }
+}
+
+// bit e set: key i0 + e is masked out (EW consecutive mask bytes, EW-aligned)
+template <int EW>
+__device__ __forceinline__ uint32_t ld_mask_small(const uint8_t *p) {
+  if constexpr (EW == 1) {
+    return p[0] != 0 ? 1u : 0u;
+  } else if constexpr (EW == 2) {
+    const uint32_t m = *reinterpret_cast<const uint16_t *>(p);
+    return ((m & 0xffu) ? 1u : 0u) | ((m >> 8) ? 2u : 0u);
+  } else {
+    const uint32_t m = *reinterpret_cast<const uint32_t *>(p);
+    uint32_t bits = 0;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) bits |= ((m >> (8 * e)) & 0xffu) ? (1u << e) : 0u;
+    return bits;
+  }
+}
+
+// keep bits of the EW consecutive elements that start at flat index `flat`
+// (a multiple of EW, so they lie inside one dropout group)
+template <int EW>
+__device__ __forceinline__ uint32_t keep_small(int64_t flat, const DropArgs &d) {
+  return dropout_keep_bits((uint64_t)flat >> 3, d.seed, d.offset, d.threshold) >>
+         (uint32_t)(flat & 7);
+}
+
+template <typename T, int MODE, bool DROP, int EW>
 __global__ __launch_bounds__(256) void softmax_fwd_wave_kernel(
     const T *__restrict__ x, const uint8_t *__restrict__ mask,
     T *__restrict__ y, float *__restrict__ stats, SoftmaxGeom g, float scale,
     DropArgs d) {
-  constexpr int K = kWaveRowMax / kWave;
+  constexpr int K = kWaveRowMax / kWave / EW;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const float ninf = -__builtin_inff();
   const float c2 = scale * kLog2e;
@@ -733,39 +798,61 @@ __global__ __launch_bounds__(256) void softmax_fwd_wave_kernel(
     row_setup<MODE>(g, r, mask, row, visible, mrow);
     const T *xr = x + row * g.sk;
     T *yr = y + row * g.sk;
-    float v[K];
+    float v[K][EW];
     float m = ninf;
 #pragma unroll
     for (int k = 0; k < K; ++k) {
-      const int i = lane + kWave * k;
-      v[k] = ninf;
-      if (i < g.sk) {
-        const bool hidden = MODE == kModeCausal ? i >= visible : mrow[i] != 0;
-        if (!hidden) v[k] = mul_rn(io<T>::from_scalar(xr[i]), c2);
+      const int i0 = (lane + kWave * k) * EW;
+#pragma unroll
+      for (int e = 0; e < EW; ++e) v[k][e] = ninf;
+      if (i0 < g.sk) {
+        // keys beyond the diagonal are not loaded; with a mask tensor the
+        // logits are requested together with the mask bytes (waiting for the
+        // mask first measures 30 % slower than the loads it can save)
+        uint32_t hid = 0;
+        if constexpr (MODE != kModeCausal) hid = ld_mask_small<EW>(mrow + i0);
+        const bool none = MODE == kModeCausal ? i0 >= visible : false;
+        if (!none) {
+          float t[EW];
+          ld_small<T, EW>(xr + i0, t);
+#pragma unroll
+          for (int e = 0; e < EW; ++e) {
+            const bool hidden =
+                MODE == kModeCausal ? i0 + e >= visible : ((hid >> e) & 1u) != 0;
+            if (!hidden) v[k][e] = mul_rn(t[e], c2);
+            m = fmaxf(m, v[k][e]);
+          }
+        }
       }
-      m = fmaxf(m, v[k]);
     }
     m = wave_max(m);
     const bool empty = m == ninf;
     const float off = empty ? 0.f : m;
     float s = 0.f;
 #pragma unroll
-    for (int k = 0; k < K; ++k) {
-      const float p = __builtin_amdgcn_exp2f(sub_rn(v[k], off));  // 0 for hidden keys
-      v[k] = p;
-      s += p;
-    }
+    for (int k = 0; k < K; ++k)
+#pragma unroll
+      for (int e = 0; e < EW; ++e) {
+        const float p = __builtin_amdgcn_exp2f(sub_rn(v[k][e], off));  // 0 for hidden keys
+        v[k][e] = p;
+        s += p;
+      }
     s = wave_sum(s);
     const float inv = empty ? 0.f : 1.0f / s;
     const float fill = empty ? 1.0f / (float)g.sk : 0.f;
 #pragma unroll
     for (int k = 0; k < K; ++k) {
-      const int i = lane + kWave * k;
-      if (i < g.sk) {
-        float o = v[k] * inv + fill;
-        if constexpr (DROP)
-          o = keep_element(row * g.sk + i, d) ? o * d.scale : 0.f;
-        yr[i] = io<T>::to_scalar(o);
+      const int i0 = (lane + kWave * k) * EW;
+      if (i0 < g.sk) {
+        float o[EW];
+        uint32_t keep = 0xffu;
+        if constexpr (DROP) keep = keep_small<EW>(row * g.sk + i0, d);
+#pragma unroll
+        for (int e = 0; e < EW; ++e) {
+          o[e] = v[k][e] * inv + fill;
+          if constexpr (DROP) o[e] = (keep >> e) & 1u ? o[e] * d.scale : 0.f;
+        }
+        st_small<T, EW>(yr + i0, o);
       }
     }
     if constexpr (DROP) {
@@ -777,12 +864,12 @@ __global__ __launch_bounds__(256) void softmax_fwd_wave_kernel(
   }
 }
 
-template <typename T, int MODE>
+template <typename T, int MODE, int EW>
 __global__ __launch_bounds__(256) void softmax_dropout_bwd_wave_kernel(
     const T *__restrict__ dy, const T *__restrict__ x,
     const float *__restrict__ stats, const uint8_t *__restrict__ mask,
     T *__restrict__ dx, SoftmaxGeom g, float scale, DropArgs d) {
-  constexpr int K = kWaveRowMax / kWave;
+  constexpr int K = kWaveRowMax / kWave / EW;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const float c2 = scale * kLog2e;
   for (int64_t r = (int64_t)blockIdx.x * 4 + wave; r < g.rows;
@@ -796,71 +883,118 @@ __global__ __launch_bounds__(256) void softmax_dropout_bwd_wave_kernel(
     T *dxr = dx + row * g.sk;
     const float m = stats[2 * row], inv = stats[2 * row + 1];
     const bool empty = inv < 0.f;
-    float pv[K], gv[K];
+    float pv[K][EW], gv[K][EW];
     float s = 0.f;
 #pragma unroll
     for (int k = 0; k < K; ++k) {
-      const int i = lane + kWave * k;
-      pv[k] = 0.f;
-      gv[k] = 0.f;
-      if (i < g.sk) {
-        const bool hidden = MODE == kModeCausal ? i >= visible : mrow[i] != 0;
-        float p = 0.f;
-        if (empty)
-          p = -inv;
-        else if (!hidden)
-          p = __builtin_amdgcn_exp2f(
-                  sub_rn(mul_rn(io<T>::from_scalar(xr[i]), c2), m)) *
-              inv;
-        pv[k] = p;
-        // (a rounded product: fused into the subtraction below it would
-        //  leave the product's rounding error where an exact zero belongs)
-        gv[k] = keep_element(row * g.sk + i, d)
-                    ? mul_rn(io<T>::from_scalar(gr[i]), d.scale)
-                    : 0.f;
+      const int i0 = (lane + kWave * k) * EW;
+#pragma unroll
+      for (int e = 0; e < EW; ++e) {
+        pv[k][e] = 0.f;
+        gv[k][e] = 0.f;
       }
-      s += pv[k] * gv[k];
+      uint32_t hid = 0;
+      bool none = true;
+      if (i0 < g.sk) {
+        if constexpr (MODE != kModeCausal) hid = ld_mask_small<EW>(mrow + i0);
+        // keys beyond the diagonal contribute nothing and are not loaded
+        // (a row without a visible key is uniform: every key counts)
+        none = !empty && (MODE == kModeCausal ? i0 >= visible : false);
+      }
+      if (!none) {
+        float xt[EW], gt[EW];
+        ld_small<T, EW>(xr + i0, xt);
+        ld_small<T, EW>(gr + i0, gt);
+        const uint32_t keep = keep_small<EW>(row * g.sk + i0, d);
+#pragma unroll
+        for (int e = 0; e < EW; ++e) {
+          const bool hidden =
+              MODE == kModeCausal ? i0 + e >= visible : ((hid >> e) & 1u) != 0;
+          float p = 0.f;
+          if (empty)
+            p = -inv;
+          else if (!hidden)
+            p = __builtin_amdgcn_exp2f(sub_rn(mul_rn(xt[e], c2), m)) * inv;
+          pv[k][e] = p;
+          // (a rounded product: fused into the subtraction below it would
+          //  leave the product's rounding error where an exact zero belongs)
+          gv[k][e] = (keep >> e) & 1u ? mul_rn(gt[e], d.scale) : 0.f;
+          s += pv[k][e] * gv[k][e];
+        }
+      }
     }
     s = wave_sum(s);
 #pragma unroll
     for (int k = 0; k < K; ++k) {
-      const int i = lane + kWave * k;
-      if (i < g.sk) dxr[i] = io<T>::to_scalar(scale * (pv[k] * (gv[k] - s)));
+      const int i0 = (lane + kWave * k) * EW;
+      if (i0 < g.sk) {
+        float o[EW];
+#pragma unroll
+        for (int e = 0; e < EW; ++e) o[e] = scale * (pv[k][e] * (gv[k][e] - s));
+        st_small<T, EW>(dxr + i0, o);
+      }
     }
   }
 }
 
-template <typename T>
+template <typename T, int EW>
 __global__ __launch_bounds__(256) void softmax_bwd_wave_kernel(
     const T *__restrict__ dy, const T *__restrict__ y, T *__restrict__ dx,
     int64_t rows, int sk, float scale) {
-  constexpr int K = kWaveRowMax / kWave;
+  constexpr int K = kWaveRowMax / kWave / EW;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   for (int64_t r = (int64_t)blockIdx.x * 4 + wave; r < rows;
        r += (int64_t)gridDim.x * 4) {
     const T *yr = y + r * sk;
     const T *gr = dy + r * sk;
     T *dxr = dx + r * sk;
-    float yv[K], gv[K];
+    float yv[K][EW], gv[K][EW];
     float s = 0.f;
 #pragma unroll
     for (int k = 0; k < K; ++k) {
-      const int i = lane + kWave * k;
-      yv[k] = 0.f;
-      gv[k] = 0.f;
-      if (i < sk) {
-        yv[k] = io<T>::from_scalar(yr[i]);
-        gv[k] = io<T>::from_scalar(gr[i]);
+      const int i0 = (lane + kWave * k) * EW;
+#pragma unroll
+      for (int e = 0; e < EW; ++e) {
+        yv[k][e] = 0.f;
+        gv[k][e] = 0.f;
       }
-      s += yv[k] * gv[k];
+      if (i0 < sk) {
+        ld_small<T, EW>(yr + i0, yv[k]);
+        ld_small<T, EW>(gr + i0, gv[k]);
+      }
+#pragma unroll
+      for (int e = 0; e < EW; ++e) s += yv[k][e] * gv[k][e];
     }
     s = wave_sum(s);
 #pragma unroll
     for (int k = 0; k < K; ++k) {
-      const int i = lane + kWave * k;
-      if (i < sk) dxr[i] = io<T>::to_scalar(scale * (yv[k] * (gv[k] - s)));
+      const int i0 = (lane + kWave * k) * EW;
+      if (i0 < sk) {
+        float o[EW];
+#pragma unroll
+        for (int e = 0; e < EW; ++e) o[e] = scale * (yv[k][e] * (gv[k][e] - s));
+        st_small<T, EW>(dxr + i0, o);
+      }
     }
   }
+}
+
+// Elements per access of the wave-per-row kernels: the widest of 4, 2, 1 for
+// which the row length divides, an access stays within 8 bytes and every
+// pointer (and the mask) is aligned to the access.
+template <typename T>
+static inline int wave_row_ew(int64_t sk, const void *a, const void *b,
+                              const void *c, const uint8_t *mask) {
+  for (int ew = 4; ew > 1; ew >>= 1) {
+    const uintptr_t bytes = (uintptr_t)ew * sizeof(T);
+    if (bytes > 8 || sk % ew != 0) continue;
+    const uintptr_t all = reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b) |
+                          reinterpret_cast<uintptr_t>(c);
+    if ((all & (bytes - 1)) != 0) continue;
+    if (mask != nullptr && (reinterpret_cast<uintptr_t>(mask) & (uintptr_t)(ew - 1)) != 0) continue;
+    return ew;
+  }
+  return 1;
 }
 
 // workgroups of a wave-per-row launch (four rows each)
@@ -979,12 +1113,22 @@ static int launch_softmax_fwd(const void *x, const uint8_t *mask, void *y,
                              : (int64_t)device_cu_count() * 32;
     if (g.sk <= kWaveRowMax) {
       const dim3 wgrid((unsigned)wave_row_grid(g.rows));
-      if (drop)
-        softmax_fwd_wave_kernel<T, MODE, true><<<wgrid, 256, 0, st>>>(
-            (const T *)x, mask, (T *)y, stats, g, scale, d);
-      else
-        softmax_fwd_wave_kernel<T, MODE, false><<<wgrid, 256, 0, st>>>(
-            (const T *)x, mask, (T *)y, nullptr, g, scale, d);
+      const int ew = wave_row_ew<T>(g.sk, x, y, nullptr, MODE == kModeMasked ? mask : nullptr);
+#define OSLO_SM_WAVE_FWD(EW_)                                              \
+  do {                                                                     \
+    if constexpr (EW_ * sizeof(T) <= 8) {                                  \
+      if (drop)                                                            \
+        softmax_fwd_wave_kernel<T, MODE, true, EW_><<<wgrid, 256, 0, st>>>(  \
+            (const T *)x, mask, (T *)y, stats, g, scale, d);               \
+      else                                                                 \
+        softmax_fwd_wave_kernel<T, MODE, false, EW_><<<wgrid, 256, 0, st>>>( \
+            (const T *)x, mask, (T *)y, nullptr, g, scale, d);             \
+    }                                                                      \
+  } while (0)
+      if (ew == 4) OSLO_SM_WAVE_FWD(4);
+      else if (ew == 2) OSLO_SM_WAVE_FWD(2);
+      else OSLO_SM_WAVE_FWD(1);
+#undef OSLO_SM_WAVE_FWD
       return check_launch("softmax_fwd_wave_kernel");
     }
     if (drop)
@@ -1034,8 +1178,18 @@ static int launch_softmax_bwd(const void *dy, const void *y,
                              ? g.rows
                              : (int64_t)device_cu_count() * 32;
     if (g.sk <= kWaveRowMax) {
-      softmax_bwd_wave_kernel<T><<<dim3((unsigned)wave_row_grid(g.rows)), 256, 0, st>>>(
-          (const T *)dy, (const T *)y, (T *)dx, g.rows, g.sk, scale);
+      const dim3 wgrid((unsigned)wave_row_grid(g.rows));
+      const int ew = wave_row_ew<T>(g.sk, dy, y, dx, nullptr);
+#define OSLO_SM_WAVE_BWD(EW_)                                              \
+  do {                                                                     \
+    if constexpr (EW_ * sizeof(T) <= 8)                                    \
+      softmax_bwd_wave_kernel<T, EW_><<<wgrid, 256, 0, st>>>(              \
+          (const T *)dy, (const T *)y, (T *)dx, g.rows, g.sk, scale);      \
+  } while (0)
+      if (ew == 4) OSLO_SM_WAVE_BWD(4);
+      else if (ew == 2) OSLO_SM_WAVE_BWD(2);
+      else OSLO_SM_WAVE_BWD(1);
+#undef OSLO_SM_WAVE_BWD
       return check_launch("softmax_bwd_wave_kernel");
     }
     softmax_bwd_generic_kernel<T><<<dim3((unsigned)grid), 256, 0, st>>>(
@@ -1073,9 +1227,18 @@ static int launch_softmax_dropout_bwd(const void *dy, const void *x,
                              ? g.rows
                              : (int64_t)device_cu_count() * 32;
     if (g.sk <= kWaveRowMax) {
-      softmax_dropout_bwd_wave_kernel<T, MODE>
-          <<<dim3((unsigned)wave_row_grid(g.rows)), 256, 0, st>>>(
-              (const T *)dy, (const T *)x, stats, mask, (T *)dx, g, scale, d);
+      const dim3 wgrid((unsigned)wave_row_grid(g.rows));
+      const int ew = wave_row_ew<T>(g.sk, dy, x, dx, MODE == kModeMasked ? mask : nullptr);
+#define OSLO_SM_WAVE_DBWD(EW_)                                             \
+  do {                                                                     \
+    if constexpr (EW_ * sizeof(T) <= 8)                                    \
+      softmax_dropout_bwd_wave_kernel<T, MODE, EW_><<<wgrid, 256, 0, st>>>( \
+          (const T *)dy, (const T *)x, stats, mask, (T *)dx, g, scale, d); \
+  } while (0)
+      if (ew == 4) OSLO_SM_WAVE_DBWD(4);
+      else if (ew == 2) OSLO_SM_WAVE_DBWD(2);
+      else OSLO_SM_WAVE_DBWD(1);
+#undef OSLO_SM_WAVE_DBWD
       return check_launch("softmax_dropout_bwd_wave_kernel");
     }
     softmax_dropout_bwd_generic_kernel<T, MODE>

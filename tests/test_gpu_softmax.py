@@ -35,6 +35,10 @@ CAUSAL_CASES = [
     (2, 40, 1001, BF16, 0.25),
     (2, 7, 1027, F16, 0.25),
     (5, 3, 1, BF16, 1.0),
+    (2, 36, 36, F16, 0.5),          # 8-byte accesses (length a multiple of 4)
+    (2, 20, 1004, BF16, 0.25),
+    (2, 30, 50, F32, 0.5),          # fp32: 8-byte accesses for even lengths
+    (2, 10, 998, F16, 0.25),        # 4-byte accesses
 ]
 
 
@@ -87,6 +91,12 @@ MASKED_CASES = [
     (2, 1, 5, 37, F32, 0.5, "full"),             # scalar kernel
     (2, 2, 16, 64, F16, 1.0, "rows_fully_masked"),
     (2, 2, 16, 64, BF16, 1.0, "none_masked"),
+    # scalar kernels with 8-, 4- and 2-byte accesses (mask bytes read 4, 2, 1 at a time)
+    (2, 2, 9, 100, F16, 0.5, "full"),
+    (2, 2, 9, 50, BF16, 0.5, "padding"),
+    (2, 2, 9, 50, BF16, 0.5, "rows_fully_masked"),
+    (2, 1, 6, 203, F16, 0.5, "full"),
+    (2, 1, 6, 1030, BF16, 0.5, "padding"),   # one workgroup per row
 ]
 
 

@@ -77,6 +77,10 @@ MASKED_CASES = [
     (2, 2, 7, 50, F16, 0.5, "full", 0.1),            # scalar kernel
     (1, 2, 4, 8192, BF16, 1.0, "padding", 0.1),
     (3, 1, 9, 128, F32, 0.3, "none", 0.4),
+    (2, 2, 12, 100, F16, 0.5, "full", 0.1),          # scalar kernel, 8-byte accesses
+    (2, 2, 12, 50, BF16, 0.5, "padding", 0.2),       # 4-byte accesses
+    (2, 2, 12, 50, F32, 0.5, "full", 0.1),           # fp32, 8-byte accesses
+    (2, 2, 12, 77, BF16, 0.5, "rows_fully_masked", 0.1),
 ]
 
 
