@@ -715,7 +715,7 @@ __global__ __launch_bounds__(256) void softmax_bwd_generic_kernel(
 // length and the pointers allow 8- or 4-byte accesses, else 1 (any length and
 // alignment).  The arithmetic is that of the kernels above, term for term.
 // ---------------------------------------------------------------------------
-constexpr int kWaveRowMax = 1024;
+constexpr int kWaveRowMax = 2048;  // 32 elements per lane and operand; builds for 256, 1024, 2048
 
 template <typename T, int EW>
 __device__ __forceinline__ void ld_small(const T *p, float *f) {
@@ -781,12 +781,12 @@ __device__ __forceinline__ uint32_t keep_small(int64_t flat, const DropArgs &d) 
          (uint32_t)(flat & 7);
 }
 
-template <typename T, int MODE, bool DROP, int EW>
+template <typename T, int MODE, bool DROP, int EW, int ROWMAX>
 __global__ __launch_bounds__(256) void softmax_fwd_wave_kernel(
     const T *__restrict__ x, const uint8_t *__restrict__ mask,
     T *__restrict__ y, float *__restrict__ stats, SoftmaxGeom g, float scale,
     DropArgs d) {
-  constexpr int K = kWaveRowMax / kWave / EW;
+  constexpr int K = ROWMAX / kWave / EW;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const float ninf = -__builtin_inff();
   const float c2 = scale * kLog2e;
@@ -864,12 +864,12 @@ __global__ __launch_bounds__(256) void softmax_fwd_wave_kernel(
   }
 }
 
-template <typename T, int MODE, int EW>
+template <typename T, int MODE, int EW, int ROWMAX>
 __global__ __launch_bounds__(256) void softmax_dropout_bwd_wave_kernel(
     const T *__restrict__ dy, const T *__restrict__ x,
     const float *__restrict__ stats, const uint8_t *__restrict__ mask,
     T *__restrict__ dx, SoftmaxGeom g, float scale, DropArgs d) {
-  constexpr int K = kWaveRowMax / kWave / EW;
+  constexpr int K = ROWMAX / kWave / EW;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const float c2 = scale * kLog2e;
   for (int64_t r = (int64_t)blockIdx.x * 4 + wave; r < g.rows;
@@ -937,11 +937,11 @@ __global__ __launch_bounds__(256) void softmax_dropout_bwd_wave_kernel(
   }
 }
 
-template <typename T, int EW>
+template <typename T, int EW, int ROWMAX>
 __global__ __launch_bounds__(256) void softmax_bwd_wave_kernel(
     const T *__restrict__ dy, const T *__restrict__ y, T *__restrict__ dx,
     int64_t rows, int sk, float scale) {
-  constexpr int K = kWaveRowMax / kWave / EW;
+  constexpr int K = ROWMAX / kWave / EW;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   for (int64_t r = (int64_t)blockIdx.x * 4 + wave; r < rows;
        r += (int64_t)gridDim.x * 4) {
@@ -1114,21 +1114,28 @@ static int launch_softmax_fwd(const void *x, const uint8_t *mask, void *y,
     if (g.sk <= kWaveRowMax) {
       const dim3 wgrid((unsigned)wave_row_grid(g.rows));
       const int ew = wave_row_ew<T>(g.sk, x, y, nullptr, MODE == kModeMasked ? mask : nullptr);
-#define OSLO_SM_WAVE_FWD(EW_)                                              \
+#define OSLO_SM_WAVE_FWD_R(EW_, RM_)                                       \
   do {                                                                     \
     if constexpr (EW_ * sizeof(T) <= 8) {                                  \
       if (drop)                                                            \
-        softmax_fwd_wave_kernel<T, MODE, true, EW_><<<wgrid, 256, 0, st>>>(  \
+        softmax_fwd_wave_kernel<T, MODE, true, EW_, RM_><<<wgrid, 256, 0, st>>>(  \
             (const T *)x, mask, (T *)y, stats, g, scale, d);               \
       else                                                                 \
-        softmax_fwd_wave_kernel<T, MODE, false, EW_><<<wgrid, 256, 0, st>>>( \
+        softmax_fwd_wave_kernel<T, MODE, false, EW_, RM_><<<wgrid, 256, 0, st>>>( \
             (const T *)x, mask, (T *)y, nullptr, g, scale, d);             \
     }                                                                      \
+  } while (0)
+#define OSLO_SM_WAVE_FWD(EW_)                                              \
+  do {                                                                     \
+    if (g.sk <= 256) OSLO_SM_WAVE_FWD_R(EW_, 256);                         \
+    else if (g.sk <= 1024) OSLO_SM_WAVE_FWD_R(EW_, 1024);                  \
+    else OSLO_SM_WAVE_FWD_R(EW_, 2048);                                    \
   } while (0)
       if (ew == 4) OSLO_SM_WAVE_FWD(4);
       else if (ew == 2) OSLO_SM_WAVE_FWD(2);
       else OSLO_SM_WAVE_FWD(1);
 #undef OSLO_SM_WAVE_FWD
+#undef OSLO_SM_WAVE_FWD_R
       return check_launch("softmax_fwd_wave_kernel");
     }
     if (drop)
@@ -1180,16 +1187,23 @@ static int launch_softmax_bwd(const void *dy, const void *y,
     if (g.sk <= kWaveRowMax) {
       const dim3 wgrid((unsigned)wave_row_grid(g.rows));
       const int ew = wave_row_ew<T>(g.sk, dy, y, dx, nullptr);
-#define OSLO_SM_WAVE_BWD(EW_)                                              \
+#define OSLO_SM_WAVE_BWD_R(EW_, RM_)                                       \
   do {                                                                     \
     if constexpr (EW_ * sizeof(T) <= 8)                                    \
-      softmax_bwd_wave_kernel<T, EW_><<<wgrid, 256, 0, st>>>(              \
+      softmax_bwd_wave_kernel<T, EW_, RM_><<<wgrid, 256, 0, st>>>(         \
           (const T *)dy, (const T *)y, (T *)dx, g.rows, g.sk, scale);      \
+  } while (0)
+#define OSLO_SM_WAVE_BWD(EW_)                                              \
+  do {                                                                     \
+    if (g.sk <= 256) OSLO_SM_WAVE_BWD_R(EW_, 256);                         \
+    else if (g.sk <= 1024) OSLO_SM_WAVE_BWD_R(EW_, 1024);                  \
+    else OSLO_SM_WAVE_BWD_R(EW_, 2048);                                    \
   } while (0)
       if (ew == 4) OSLO_SM_WAVE_BWD(4);
       else if (ew == 2) OSLO_SM_WAVE_BWD(2);
       else OSLO_SM_WAVE_BWD(1);
 #undef OSLO_SM_WAVE_BWD
+#undef OSLO_SM_WAVE_BWD_R
       return check_launch("softmax_bwd_wave_kernel");
     }
     softmax_bwd_generic_kernel<T><<<dim3((unsigned)grid), 256, 0, st>>>(
@@ -1229,16 +1243,23 @@ static int launch_softmax_dropout_bwd(const void *dy, const void *x,
     if (g.sk <= kWaveRowMax) {
       const dim3 wgrid((unsigned)wave_row_grid(g.rows));
       const int ew = wave_row_ew<T>(g.sk, dy, x, dx, MODE == kModeMasked ? mask : nullptr);
-#define OSLO_SM_WAVE_DBWD(EW_)                                             \
+#define OSLO_SM_WAVE_DBWD_R(EW_, RM_)                                      \
   do {                                                                     \
     if constexpr (EW_ * sizeof(T) <= 8)                                    \
-      softmax_dropout_bwd_wave_kernel<T, MODE, EW_><<<wgrid, 256, 0, st>>>( \
+      softmax_dropout_bwd_wave_kernel<T, MODE, EW_, RM_><<<wgrid, 256, 0, st>>>( \
           (const T *)dy, (const T *)x, stats, mask, (T *)dx, g, scale, d); \
+  } while (0)
+#define OSLO_SM_WAVE_DBWD(EW_)                                             \
+  do {                                                                     \
+    if (g.sk <= 256) OSLO_SM_WAVE_DBWD_R(EW_, 256);                        \
+    else if (g.sk <= 1024) OSLO_SM_WAVE_DBWD_R(EW_, 1024);                 \
+    else OSLO_SM_WAVE_DBWD_R(EW_, 2048);                                   \
   } while (0)
       if (ew == 4) OSLO_SM_WAVE_DBWD(4);
       else if (ew == 2) OSLO_SM_WAVE_DBWD(2);
       else OSLO_SM_WAVE_DBWD(1);
 #undef OSLO_SM_WAVE_DBWD
+#undef OSLO_SM_WAVE_DBWD_R
       return check_launch("softmax_dropout_bwd_wave_kernel");
     }
     softmax_dropout_bwd_generic_kernel<T, MODE>

@@ -29,11 +29,13 @@ CAUSAL_CASES = [
     (2, 9, 100000, BF16, 1.0),      # beyond the register path
     (1, 1, 8, F32, 2.0),
     # lengths that are no multiple of the vector width: one wavefront per row
-    # up to 1024 keys, one workgroup per row beyond
+    # up to 2048 keys, one workgroup per row beyond
     (3, 50, 50, BF16, 0.5),
     (2, 197, 197, F16, 0.125),
     (2, 40, 1001, BF16, 0.25),
     (2, 7, 1027, F16, 0.25),
+    (2, 5, 2049, BF16, 0.25),
+    (2, 6, 2044, F16, 0.25),
     (5, 3, 1, BF16, 1.0),
     (2, 36, 36, F16, 0.5),          # 8-byte accesses (length a multiple of 4)
     (2, 20, 1004, BF16, 0.25),
@@ -96,7 +98,8 @@ MASKED_CASES = [
     (2, 2, 9, 50, BF16, 0.5, "padding"),
     (2, 2, 9, 50, BF16, 0.5, "rows_fully_masked"),
     (2, 1, 6, 203, F16, 0.5, "full"),
-    (2, 1, 6, 1030, BF16, 0.5, "padding"),   # one workgroup per row
+    (2, 1, 6, 1030, BF16, 0.5, "padding"),
+    (2, 1, 6, 2050, BF16, 0.5, "padding"),   # one workgroup per row
 ]
 
 

@@ -39,6 +39,8 @@ CAUSAL_CASES = [
     (3, 50, 50, BF16, 0.5, 0.1),          # one wavefront per row, scalar accesses
     (2, 197, 197, F16, 0.125, 0.2),
     (2, 9, 1001, BF16, 0.25, 0.1),
+    (2, 5, 2046, F16, 0.25, 0.1),
+    (2, 5, 2051, BF16, 0.25, 0.1),        # one workgroup per row
     (4, 5, 1, F32, 1.0, 0.3),             # one key: the gradient is exactly zero
 ]
 
