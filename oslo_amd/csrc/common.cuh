@@ -323,7 +323,10 @@ __device__ __forceinline__ Welford wave_welford_equal(float mean, float m2,
 __device__ __forceinline__ float rsqrt_refined(float a) {
   float y = __builtin_amdgcn_rsqf(a);
   const float h = 0.5f * a * y;
-  return fmaf(y, 0.5f - h * y, y);
+  const float r = fmaf(y, 0.5f - h * y, y);
+  // a = inf gives 0 and a = 0 gives inf, as rsqrt does; the Newton step would
+  // turn both into NaN (inf * 0)
+  return a > 0.f && a < __builtin_inff() ? r : y;
 }
 
 // Reduction of the values held by lanes 0..15 (one DPP row), returned to every
