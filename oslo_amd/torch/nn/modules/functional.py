@@ -149,6 +149,16 @@ def _next_philox_state(device):
     """(seed, offset) from torch's generator of `device`; advances the offset."""
     index = device.index if device.index is not None else torch.cuda.current_device()
     gen = torch.cuda.default_generators[index]
+    if torch.cuda.is_current_stream_capturing():
+        # torch keeps the generator state on the device while a graph is being
+        # captured and refuses host reads; a pair baked into the graph would
+        # also repeat the same mask on every replay
+        raise RuntimeError(
+            "dropout with p > 0 cannot be captured in a CUDA/HIP graph through this "
+            "layer: (seed, offset) come from torch's generator on the host. Capture in "
+            "eval mode or with p = 0, or call the kernels of oslo_amd.torch._C with an "
+            "explicit (seed, offset) per replay."
+        )
     seed = gen.initial_seed()
     offset = gen.get_offset()
     gen.set_offset(offset + 4)

@@ -73,3 +73,22 @@ def test_captured_layer_chain_replays(device):
             assert torch.equal(a, b), "output %d differs on replay %d" % (i, rep)
         for a, b in zip(gp + gm + gv, ep + em + ev):
             assert torch.equal(a, b), "optimizer state differs on replay %d" % rep
+
+
+def test_dropout_from_the_generator_refuses_capture_with_a_message(device):
+    from oslo_amd.torch.nn.modules import functional as F_
+
+    x = randn((8, 64), BF16, 1).to(device)
+    b = torch.zeros(64, dtype=BF16, device=device)
+    F_.fused_bias_dropout_add(x, b, None, 0.5, True)  # eager: fine
+    graph = torch.cuda.CUDAGraph()
+    with pytest.raises(RuntimeError, match="cannot be captured"):
+        with torch.cuda.graph(graph):
+            F_.fused_bias_dropout_add(x, b, None, 0.5, True)
+    # p = 0 captures (nothing is drawn)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        out = F_.fused_bias_dropout_add(x, b, None, 0.0, True)
+    graph.replay()
+    torch.cuda.synchronize()
+    assert torch.equal(out, x)
