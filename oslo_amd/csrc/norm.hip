@@ -142,7 +142,9 @@ struct FusePrologue {
 // LayerNorm then merges equal-sized Welford partials).
 // LPR: lanes that hold a row.  64: a row takes wpr whole waves.  8, 16, 32:
 // rows of at most LPR chunks lie side by side in a wave (VPL == 1, wpr == 1,
-// and rpb counts the rows of all lane groups of the workgroup).
+// and rpb counts the rows of all lane groups of the workgroup); rows of
+// exactly 3 * LPR chunks (768 16-bit elements = 96 chunks = 32 lanes x 3)
+// take VPL == 3.
 template <typename T, typename V, int VPL, bool RMS, bool EVEN, int MAXT,
           bool FUSE = false, int LPR = kWave>
 __global__ __launch_bounds__(MAXT) void norm_fwd_reg_kernel(
@@ -152,7 +154,7 @@ __global__ __launch_bounds__(MAXT) void norm_fwd_reg_kernel(
     int rpb, int iters, FusePrologue fp) {
   constexpr int E = chunk_elems<T, V>::value;
   static_assert(!FUSE || sizeof(T) == sizeof(V), "fused prologue: one dtype");
-  static_assert(LPR == kWave || VPL == 1, "side-by-side rows: one chunk per lane");
+  static_assert(LPR == kWave || VPL == 1 || VPL == 3, "side-by-side rows: one or three chunks per lane");
   __shared__ float red[2][48];
   const int lane = threadIdx.x & 63;
   // the wave index is uniform: keep it (and the row arithmetic) in scalar registers
@@ -161,7 +163,7 @@ __global__ __launch_bounds__(MAXT) void norm_fwd_reg_kernel(
   const int first = (wave / wpr) * wpr;
   const int rslot = LPR == kWave ? wave / wpr : wave * SUB + lane / LPR;
   const int nchunks = n2 / E;
-  const int cstride = kWave * wpr;
+  const int cstride = LPR == kWave ? kWave * wpr : LPR;
   const int c0 = LPR == kWave ? (wave - first) * kWave + lane : (lane & (LPR - 1));
   const float fn = (float)n2;
   int parity = 0;
@@ -457,7 +459,7 @@ __global__ __launch_bounds__(MAXT) void norm_bwd_reg_kernel(
     int64_t n1, int n2, int wpr, int rpb, FuseEpilogue fe) {
   constexpr int E = chunk_elems<T, V>::value;
   static_assert(!FUSE || sizeof(T) == sizeof(V), "fused epilogue: one dtype");
-  static_assert(LPR == kWave || VPL == 1, "side-by-side rows: one chunk per lane");
+  static_assert(LPR == kWave || VPL == 1 || VPL == 3, "side-by-side rows: one or three chunks per lane");
   extern __shared__ float xslot[];  // [n2] when rpb > 1
   __shared__ float red[2][32];
   const int lane = threadIdx.x & 63;
@@ -470,7 +472,7 @@ __global__ __launch_bounds__(MAXT) void norm_bwd_reg_kernel(
   const int wslot = wave / wpr;
   const int rslot = LPR == kWave ? wslot : wave * SUB + lane / LPR;
   const int nchunks = n2 / E;
-  const int cstride = kWave * wpr;
+  const int cstride = LPR == kWave ? kWave * wpr : LPR;
   const int c0 = LPR == kWave ? (wave - first) * kWave + lane : (lane & (LPR - 1));
   const float fn = (float)n2;
   const bool affine = gamma != nullptr;
@@ -844,6 +846,14 @@ static int lanes_per_row(int64_t nchunks) {
   return lpr;
 }
 
+// Rows of exactly 3 * 8, 3 * 16 or 3 * 32 chunks (hidden sizes 192, 384, 768
+// in a 16-bit type): lanes per row for the three-chunks-per-lane builds, else 0.
+static int lanes_per_row_x3(int64_t nchunks) {
+  if (g_tune.norm_lanes_per_row == kWave || nchunks % 3 != 0) return 0;
+  const int64_t q = nchunks / 3;
+  return q == 8 || q == 16 || q == 32 ? (int)q : 0;
+}
+
 int64_t colsum_parts_norm(int64_t n1, int64_t n2) {
   (void)n2;
   int bpc = g_tune.norm_bwd_blocks_per_cu > 0 ? g_tune.norm_bwd_blocks_per_cu : 1;
@@ -930,6 +940,37 @@ static int launch_norm_fwd(const void *x, const void *gamma, const void *beta,
   int64_t grid = ceil_div(ceil_div(n1, sp.rpb), iters);
   const int64_t maxgrid = (int64_t)device_cu_count() * 64;
   if (grid > maxgrid) grid = maxgrid;
+  // rows of 3 x 8 / 16 / 32 chunks: three chunks per lane, two or more rows
+  // side by side in a wave, no idle lane and no barrier
+  if (const int l3 = lanes_per_row_x3(n2 / E)) {
+    const int threads3 = 256;
+    const int rpb3 = (threads3 / kWave) * (kWave / l3);
+    int64_t grid3 = ceil_div(ceil_div(n1, rpb3), iters);
+    if (grid3 > maxgrid) grid3 = maxgrid;
+#define OSLO_FWD_X3(LPR_)                                                    \
+  case LPR_:                                                                 \
+    if constexpr (kCanFuse) {                                                \
+      if (fused) {                                                           \
+        norm_fwd_reg_kernel<T, V, 3, RMS, true, 256, true, LPR_>             \
+            <<<dim3((unsigned)grid3), threads3, 0, st>>>(                    \
+                (const T *)x, (const V *)gamma, (const V *)beta, (V *)y,     \
+                mean, invvar, n1, (int)n2, eps, 1, rpb3, iters, *fp);        \
+        break;                                                               \
+      }                                                                      \
+    }                                                                        \
+    norm_fwd_reg_kernel<T, V, 3, RMS, true, 256, false, LPR_>                \
+        <<<dim3((unsigned)grid3), threads3, 0, st>>>(                        \
+            (const T *)x, (const V *)gamma, (const V *)beta, (V *)y, mean,   \
+            invvar, n1, (int)n2, eps, 1, rpb3, iters, FusePrologue{});       \
+    break;
+    switch (l3) {
+      OSLO_FWD_X3(8)
+      OSLO_FWD_X3(16)
+      OSLO_FWD_X3(32)
+    }
+#undef OSLO_FWD_X3
+    return check_launch("norm_fwd_reg_kernel (three chunks per lane)");
+  }
   // short rows side by side in a wave
   const int lpr = (sp.wpr == 1 && sp.vpl == 1) ? lanes_per_row(n2 / E) : kWave;
   if (lpr < kWave) {
@@ -1153,6 +1194,9 @@ static int launch_norm_bwd(const void *dy, const void *x, const float *mean,
     return check_launch("norm_bwd_param_generic_kernel");
   }
   // short rows side by side in a wave: the row slots of a workgroup multiply
+  // (the three-chunks-per-lane mapping of the forward kernel does not pay
+  //  here: its 24 elements per lane and operand need a 512-thread workgroup,
+  //  and eight waves per CU measure 2 % slower than whole-wave rows)
   const int lpr = (sp.wpr == 1 && sp.vpl == 1) ? lanes_per_row(n2 / E) : kWave;
   const int wave_slots = sp.rpb;  // row slots at wave granularity
   if (lpr < kWave) sp.rpb *= kWave / lpr;

@@ -22,6 +22,9 @@ ROWS = [
     (4, F32, F32), (32, F32, F32), (36, F32, F32), (64, F32, F32),
     (100, F32, F32), (128, F32, F32),
     (64, F32, BF16), (128, F32, F16),                         # fp32 input, 16-bit output
+    # exactly 3 x 8 / 16 / 32 chunks: three chunks per lane, rows side by side
+    (192, BF16, BF16), (384, F16, F16), (768, BF16, BF16), (768, F16, F16),
+    (96, F32, F32), (192, F32, F32), (384, F32, F32), (768, F32, BF16),
 ]
 N1 = [1, 37, 5003]
 

@@ -37,6 +37,10 @@ CASES = [
     (333, 40, BF16, 0.1),       # 5 chunks in 8 lanes
     (700, 100, F32, 0.1),       # 25 fp32 chunks in 32 lanes
     (90, 7168, BF16, 0.1),      # 16 elements per lane over seven waves
+    (1001, 768, BF16, 0.1),     # three chunks per lane, two rows per wave
+    (515, 384, F16, 0.2),
+    (260, 192, BF16, 0.1),
+    (300, 384, F32, 0.1),
     (1, 8, F32, 0.5),
     (12, 2048, BF16, 0.0),      # no dropout
     (12, 2048, BF16, 1.0),      # everything dropped
