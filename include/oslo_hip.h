@@ -199,6 +199,21 @@ int oslo_softmax_masked_dropout_bwd(const void *dout, const void *x,
                                     float scale, float p, uint64_t seed,
                                     uint64_t offset, int dtype, void *stream);
 
+/* ---- dropout state in device memory ------------------------------------- *
+ * No counterpart in the reference.  For callers that capture launches in a
+ * HIP graph: a (seed, offset) pair passed by value is frozen into the graph
+ * and every replay would draw the same mask.  After
+ * oslo_rng_from_device(state), the dropout entry points called NEXT ON THE
+ * SAME HOST THREAD (bias-dropout-add, its fusion into the norm, softmax with
+ * dropout; forward and backward) ignore their `seed` argument and make their
+ * kernels read, when they run, seed = state[0] and offset = state[1] + the
+ * `offset` argument from device memory.  oslo_rng_from_device(NULL) restores
+ * the by-value behaviour.  `state` points to two uint64 in device memory that
+ * the caller owns and updates (e.g. state[1] += 4 between calls, in a kernel
+ * of its own that is captured too); the setting itself is per host thread
+ * and is not part of any graph.                                            */
+int oslo_rng_from_device(const uint64_t *state);
+
 /* ---- bias-GeLU (tanh approximation) ------------------------------------ *
  * x, y, g, dx are [rows, cols]; bias, dbias are [cols]; one dtype for all. */
 

@@ -17,6 +17,11 @@ int fail(int code, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
 // hipGetLastError() after a launch -> OSLO_OK or OSLO_ERR_LAUNCH.
 int check_launch(const char *what);
 
+// Device pointer to {seed, offset} that the *_rng entry points put in place
+// for the duration of their call on the calling thread (null otherwise).
+const uint64_t *current_rng_state();
+void set_current_rng_state(const uint64_t *state);
+
 // Number of compute units of the current device (cached per device id).
 int device_cu_count();
 

@@ -7,6 +7,10 @@
 namespace oslo {
 
 static thread_local char t_err[512] = "";
+static thread_local const uint64_t *t_rng_state = nullptr;
+
+const uint64_t *current_rng_state() { return t_rng_state; }
+void set_current_rng_state(const uint64_t *state) { t_rng_state = state; }
 
 int fail(int code, const char *fmt, ...) {
   va_list ap;
@@ -42,6 +46,11 @@ Tuning g_tune = {0, 0, 0, 0, 0, 0, 0, 0, 0};
 }  // namespace oslo
 
 extern "C" {
+
+int oslo_rng_from_device(const uint64_t *state) {
+  oslo::set_current_rng_state(state);
+  return OSLO_OK;
+}
 
 const char *oslo_hip_last_error(void) { return oslo::t_err; }
 

@@ -447,7 +447,20 @@ struct DropArgs {
   uint64_t seed, offset;
   uint32_t threshold;  // keep when the 16-bit draw >= threshold
   float scale;         // 1 / (1 - p), 0 when p >= 1
+  // non-null: {seed, offset} are read from device memory when the kernel
+  // runs (seed = dev[0], offset = dev[1] + offset), so that a launch captured
+  // in a graph draws a new mask on every replay
+  const uint64_t *dev;
 };
+
+// The (seed, offset) pair a kernel works with; uniform over the launch.
+__device__ __forceinline__ DropArgs resolve_drop(DropArgs d) {
+  if (d.dev != nullptr) {
+    d.seed = d.dev[0];
+    d.offset += d.dev[1];
+  }
+  return d;
+}
 
 __device__ __host__ __forceinline__ bool keep_element(int64_t i, const DropArgs &d) {
   const uint32_t bits =
@@ -459,6 +472,7 @@ static inline DropArgs make_drop(float p, uint64_t seed, uint64_t offset) {
   DropArgs d;
   d.seed = seed;
   d.offset = offset;
+  d.dev = current_rng_state();  // set by the *_rng entry points, else null
   double t = (double)p * 65536.0 + 0.5;
   d.threshold = t >= 65536.0 ? 65536u : (uint32_t)t;
   d.scale = p < 1.0f ? 1.0f / (1.0f - p) : 0.f;

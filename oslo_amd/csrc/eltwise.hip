@@ -199,6 +199,7 @@ __global__ __launch_bounds__(256) void bias_dropout_add_fwd_kernel(
     const T *__restrict__ res, T *__restrict__ out,
     uint8_t *__restrict__ mask_out, EltGeom g, DropArgs d) {
   constexpr int kE = io<T>::EPV;
+  d = resolve_drop(d);
   const EltPos ps = elt_pos(g);
   if (ps.cc >= g.nchunks) return;
   float b[kE];
@@ -253,6 +254,7 @@ __global__ __launch_bounds__(256) void bias_dropout_add_bwd_kernel(
     const T *__restrict__ gr, T *__restrict__ dx, float *__restrict__ part,
     EltGeom g, DropArgs d) {
   constexpr int kE = io<T>::EPV;
+  d = resolve_drop(d);
   __shared__ float sh[256 * kE];
   const EltPos ps = elt_pos(g);
   float acc[kE];
@@ -337,6 +339,7 @@ __global__ __launch_bounds__(256) void bias_dropout_add_fwd_generic_kernel(
     const T *__restrict__ res, T *__restrict__ out,
     uint8_t *__restrict__ mask_out, int64_t n, int64_t cols, DropArgs d,
     bool drop) {
+  d = resolve_drop(d);
   for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n;
        i += (int64_t)gridDim.x * 256) {
     float t = io<T>::from_scalar(x[i]);
@@ -353,6 +356,7 @@ template <typename T>
 __global__ __launch_bounds__(256) void bias_dropout_add_bwd_generic_kernel(
     const T *__restrict__ gr, T *__restrict__ dx, int64_t n, DropArgs d,
     bool drop) {
+  d = resolve_drop(d);
   for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n;
        i += (int64_t)gridDim.x * 256) {
     float t = io<T>::from_scalar(gr[i]);
@@ -367,6 +371,7 @@ template <typename T>
 __global__ __launch_bounds__(256) void bias_dropout_add_dbias_generic_kernel(
     const T *__restrict__ gr, T *__restrict__ dbias, int64_t rows,
     int64_t cols, DropArgs d, bool drop) {
+  d = resolve_drop(d);
   const int64_t col = (int64_t)blockIdx.x * 256 + threadIdx.x;
   if (col >= cols) return;
   float s = 0.f;
@@ -392,6 +397,7 @@ __global__ __launch_bounds__(256) void colsum_generic_kernel(
 
 __global__ __launch_bounds__(256) void philox_mask_kernel(
     uint8_t *__restrict__ mask_out, int64_t n, DropArgs d) {
+  d = resolve_drop(d);
   const int64_t ngroups = (n + 7) / 8;
   for (int64_t grp = (int64_t)blockIdx.x * 256 + threadIdx.x; grp < ngroups;
        grp += (int64_t)gridDim.x * 256) {
@@ -456,7 +462,10 @@ template <typename T> struct DroppedGradient {
   __device__ __forceinline__ void operator()(int64_t r, int64_t c, float *acc) const {
     const int64_t i = r * cols + c;
     float t = io<T>::from_scalar(gr[i]);
-    if (drop) t = keep_element(i, d) ? t * d.scale : 0.f;
+    if (drop) {
+      const DropArgs dd = resolve_drop(d);
+      t = keep_element(i, dd) ? t * dd.scale : 0.f;
+    }
     acc[0] += io<T>::round(t);
   }
 };

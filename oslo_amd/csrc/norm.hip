@@ -154,6 +154,7 @@ __global__ __launch_bounds__(MAXT) void norm_fwd_reg_kernel(
     int rpb, int iters, FusePrologue fp) {
   constexpr int E = chunk_elems<T, V>::value;
   static_assert(!FUSE || sizeof(T) == sizeof(V), "fused prologue: one dtype");
+  if constexpr (FUSE) fp.d = resolve_drop(fp.d);
   static_assert(LPR == kWave || VPL == 1 || VPL == 3, "side-by-side rows: one or three chunks per lane");
   __shared__ float red[2][48];
   const int lane = threadIdx.x & 63;
@@ -459,6 +460,7 @@ __global__ __launch_bounds__(MAXT) void norm_bwd_reg_kernel(
     int64_t n1, int n2, int wpr, int rpb, FuseEpilogue fe) {
   constexpr int E = chunk_elems<T, V>::value;
   static_assert(!FUSE || sizeof(T) == sizeof(V), "fused epilogue: one dtype");
+  if constexpr (FUSE) fe.d = resolve_drop(fe.d);
   static_assert(LPR == kWave || VPL == 1 || VPL == 3, "side-by-side rows: one or three chunks per lane");
   extern __shared__ float xslot[];  // [n2] when rpb > 1
   __shared__ float red[2][32];
@@ -721,6 +723,7 @@ __global__ __launch_bounds__(256) void norm_bwd_dx_generic_kernel(
     FuseEpilogue fe) {
   // fe: the fused epilogue (all-null for the plain backward): dh_extra is added
   // before the single rounding, dx_drop receives the masked, scaled gradient
+  fe.d = resolve_drop(fe.d);
   const T *extra = static_cast<const T *>(fe.dh_extra);
   T *dx_drop = static_cast<T *>(fe.dx_drop);
   __shared__ float sh[2][4];

@@ -137,6 +137,7 @@ __global__ __launch_bounds__(1024) void softmax_fwd_kernel(
     const T *__restrict__ x, const uint8_t *__restrict__ mask,
     T *__restrict__ y, float *__restrict__ stats, SoftmaxGeom g, float scale,
     DropArgs d) {
+  d = resolve_drop(d);
   constexpr int E = io<T>::EPV;
   constexpr uint32_t kAll = (1u << E) - 1u;
   __shared__ float red[2][16];
@@ -319,6 +320,7 @@ __global__ __launch_bounds__(1024) void softmax_dropout_bwd_kernel(
     const T *__restrict__ dy, const T *__restrict__ x,
     const float *__restrict__ stats, const uint8_t *__restrict__ mask,
     T *__restrict__ dx, SoftmaxGeom g, float scale, DropArgs d) {
+  d = resolve_drop(d);
   constexpr int E = io<T>::EPV;
   constexpr uint32_t kAll = (1u << E) - 1u;
   __shared__ float red[16];
@@ -601,6 +603,7 @@ __global__ __launch_bounds__(256) void softmax_fwd_generic_kernel(
     const T *__restrict__ x, const uint8_t *__restrict__ mask,
     T *__restrict__ y, float *__restrict__ stats, SoftmaxGeom g, float scale,
     DropArgs d) {
+  d = resolve_drop(d);
   __shared__ float sh[4];
   const float ninf = -__builtin_inff();
   // log2-domain logits t = x * (scale * log2 e), the same rounded products
@@ -655,6 +658,7 @@ __global__ __launch_bounds__(256) void softmax_dropout_bwd_generic_kernel(
     const T *__restrict__ dy, const T *__restrict__ x,
     const float *__restrict__ stats, const uint8_t *__restrict__ mask,
     T *__restrict__ dx, SoftmaxGeom g, float scale, DropArgs d) {
+  d = resolve_drop(d);
   __shared__ float sh[4];
   const float c2 = scale * kLog2e;
   for (int64_t r = blockIdx.x; r < g.rows; r += gridDim.x) {
@@ -786,6 +790,7 @@ __global__ __launch_bounds__(256) void softmax_fwd_wave_kernel(
     const T *__restrict__ x, const uint8_t *__restrict__ mask,
     T *__restrict__ y, float *__restrict__ stats, SoftmaxGeom g, float scale,
     DropArgs d) {
+  d = resolve_drop(d);
   constexpr int K = ROWMAX / kWave / EW;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const float ninf = -__builtin_inff();
@@ -869,6 +874,7 @@ __global__ __launch_bounds__(256) void softmax_dropout_bwd_wave_kernel(
     const T *__restrict__ dy, const T *__restrict__ x,
     const float *__restrict__ stats, const uint8_t *__restrict__ mask,
     T *__restrict__ dx, SoftmaxGeom g, float scale, DropArgs d) {
+  d = resolve_drop(d);
   constexpr int K = ROWMAX / kWave / EW;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const float c2 = scale * kLog2e;

@@ -115,6 +115,7 @@ _SIGNATURES = {
         _int,
         [_p, _p, _p, _p, _p, _i64, _f32, _f32, _f32, _f32, _int, _int, _int, _f32, _int, _p],
     ),
+    "oslo_rng_from_device": (_int, [_p]),
     "oslo_philox_mask": (_int, [_p, _i64, _f32, _u64, _u64, _p]),
     "oslo_philox_words": (_int, [_p, _i64, _i64, _u64, _u64, _p]),
     "oslo_copy_probe": (_int, [_p, _p, _i64, _p]),
@@ -215,6 +216,33 @@ def _workspace(lib, op, n1, n2, device):
     if nbytes < 0:
         _check(int(nbytes), lib)
     return torch.empty(max(int(nbytes), 16), dtype=torch.uint8, device=device), int(nbytes)
+
+
+class device_rng:
+    """Within the block, the dropout entry points called on this host thread
+    read (seed, offset) from ``state`` -- two 64-bit integers in device memory --
+    when their kernels run, and add their ``offset`` argument to it; their
+    ``seed`` argument is ignored.  ``state`` None makes the block a no-op.
+    Launches captured in a graph then draw a new mask on every replay."""
+
+    def __init__(self, state):
+        if state is not None:
+            if not (state.is_cuda and state.is_contiguous() and state.numel() == 2
+                    and state.element_size() == 8):
+                raise RuntimeError("device_rng: two 64-bit integers on the GPU expected")
+        self._state = state
+
+    def __enter__(self):
+        if self._state is not None:
+            lib = load_library()
+            _check(lib.oslo_rng_from_device(self._state.data_ptr()), lib)
+        return self
+
+    def __exit__(self, *exc):
+        if self._state is not None:
+            lib = load_library()
+            lib.oslo_rng_from_device(None)
+        return False
 
 
 def tune(key, value):

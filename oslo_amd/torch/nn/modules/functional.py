@@ -116,15 +116,16 @@ class _FusedBiasDropoutAddFunction(torch.autograd.Function):
     def forward(ctx, input, bias, residual, p, seed, offset, inplace):
         kernel = get_fused_elementwise_kernel()
         input_ = input.contiguous()
-        out = kernel.bias_dropout_add_forward(
-            input_,
-            None if bias is None else bias.contiguous(),
-            None if residual is None else residual.contiguous(),
-            p,
-            seed,
-            offset,
-            out=input_ if (inplace and input_ is input) else None,
-        )
+        with _rng(seed):
+            out = kernel.bias_dropout_add_forward(
+                input_,
+                None if bias is None else bias.contiguous(),
+                None if residual is None else residual.contiguous(),
+                p,
+                _seed_arg(seed),
+                offset,
+                out=input_ if (inplace and input_ is input) else None,
+            )
         if inplace and input_ is input:
             ctx.mark_dirty(input)
         ctx.p, ctx.seed, ctx.offset = p, seed, offset
@@ -138,31 +139,76 @@ class _FusedBiasDropoutAddFunction(torch.autograd.Function):
         need_x = ctx.needs_input_grad[0]
         need_b = ctx.has_bias and ctx.needs_input_grad[1]
         need_r = ctx.has_residual and ctx.needs_input_grad[2]
-        grad_input, grad_bias = get_fused_elementwise_kernel().bias_dropout_add_backward(
-            grad_output, ctx.p, ctx.seed, ctx.offset,
-            need_input_grad=need_x, need_bias_grad=need_b,
-        )
+        with _rng(ctx.seed):
+            grad_input, grad_bias = get_fused_elementwise_kernel().bias_dropout_add_backward(
+                grad_output, ctx.p, _seed_arg(ctx.seed), ctx.offset,
+                need_input_grad=need_x, need_bias_grad=need_b,
+            )
         return grad_input, grad_bias, (grad_output if need_r else None), None, None, None, None
 
 
+# Dropout state in device memory, one per device, for launches captured in a
+# graph: {seed, offset} as two int64.  Created by the first eager dropout call
+# on the device (a host-to-device copy cannot be captured) and re-seeded when
+# torch's seed changes; its offsets start 2^40 above the generator's so that the
+# two sequences stay apart.
+_graph_rng = {}
+
+
+def _as_i64(v):
+    v &= (1 << 64) - 1
+    return v - (1 << 64) if v >= (1 << 63) else v
+
+
+def _graph_rng_state(index, seed, offset):
+    entry = _graph_rng.get(index)
+    if entry is None or entry[0] != seed:
+        state = torch.tensor([_as_i64(seed), _as_i64(offset + (1 << 40))], dtype=torch.int64,
+                             device=torch.device("cuda", index))
+        _graph_rng[index] = (seed, state)
+        return state
+    return entry[1]
+
+
 def _next_philox_state(device):
-    """(seed, offset) from torch's generator of `device`; advances the offset."""
+    """(seed, offset) for one dropout call.
+
+    Eager: the pair comes from torch's generator of `device`, whose offset
+    advances by 4.  During stream capture the host cannot read the generator
+    (and a pair baked into the graph would repeat one mask on every replay):
+    ``seed`` is then a snapshot of the device-resident state -- a tensor that
+    the kernels read when they run -- and that state advances by a captured
+    add, so every replay draws new masks.  Backward takes the same pair."""
     index = device.index if device.index is not None else torch.cuda.current_device()
-    gen = torch.cuda.default_generators[index]
     if torch.cuda.is_current_stream_capturing():
-        # torch keeps the generator state on the device while a graph is being
-        # captured and refuses host reads; a pair baked into the graph would
-        # also repeat the same mask on every replay
-        raise RuntimeError(
-            "dropout with p > 0 cannot be captured in a CUDA/HIP graph through this "
-            "layer: (seed, offset) come from torch's generator on the host. Capture in "
-            "eval mode or with p = 0, or call the kernels of oslo_amd.torch._C with an "
-            "explicit (seed, offset) per replay."
-        )
+        entry = _graph_rng.get(index)
+        if entry is None:
+            raise RuntimeError(
+                "dropout with p > 0 is being captured in a graph before any eager dropout "
+                "call on this device: run one eager step first (it creates the dropout "
+                "state in device memory that captured launches read)."
+            )
+        state = entry[1]
+        snapshot = state.clone()
+        state[1:2].add_(4)
+        return snapshot, 0
+    gen = torch.cuda.default_generators[index]
     seed = gen.initial_seed()
     offset = gen.get_offset()
     gen.set_offset(offset + 4)
+    _graph_rng_state(index, seed, offset)
     return seed, offset
+
+
+def _rng(seed):
+    """Context for a kernel call: a tensor `seed` is the device-resident pair."""
+    from oslo_amd.torch._C import device_rng
+
+    return device_rng(seed if isinstance(seed, torch.Tensor) else None)
+
+
+def _seed_arg(seed):
+    return 0 if isinstance(seed, torch.Tensor) else seed
 
 
 def _norm_forward(ctx, rms, mixed, input, weight, bias, normalized_shape, eps):
@@ -292,16 +338,17 @@ class _FusedBiasDropoutAddNormFunction(torch.autograd.Function):
     def forward(ctx, input, bias, residual, weight, norm_bias, normalized_shape, eps,
                 p, seed, offset, rms):
         kernel = get_layernorm_kernel()
-        y, h, mean, invvar = kernel.bias_dropout_add_norm_forward(
-            rms,
-            input.contiguous(),
-            None if bias is None else bias.contiguous(),
-            None if residual is None else residual.contiguous(),
-            normalized_shape,
-            None if weight is None else weight.contiguous(),
-            None if norm_bias is None else norm_bias.contiguous(),
-            eps, p, seed, offset,
-        )
+        with _rng(seed):
+            y, h, mean, invvar = kernel.bias_dropout_add_norm_forward(
+                rms,
+                input.contiguous(),
+                None if bias is None else bias.contiguous(),
+                None if residual is None else residual.contiguous(),
+                normalized_shape,
+                None if weight is None else weight.contiguous(),
+                None if norm_bias is None else norm_bias.contiguous(),
+                eps, p, _seed_arg(seed), offset,
+            )
         ctx.rms, ctx.p, ctx.seed, ctx.offset = rms, p, seed, offset
         ctx.normalized_shape = normalized_shape
         ctx.has = (bias is not None, residual is not None, weight is not None,
@@ -322,14 +369,15 @@ class _FusedBiasDropoutAddNormFunction(torch.autograd.Function):
         has_bias, has_res, has_weight, has_nbias = ctx.has
         weight = saved[-1] if has_weight else None
         need_b = has_bias and ctx.needs_input_grad[1]
-        g_res, g_in, g_gamma, g_beta, g_bias = (
-            get_layernorm_kernel().bias_dropout_add_norm_backward(
-                ctx.rms, grad_y.contiguous(),
-                None if grad_h is None else grad_h.contiguous(),
-                h, mean, invvar, ctx.normalized_shape, weight,
-                ctx.p, ctx.seed, ctx.offset, need_bias_grad=need_b,
+        with _rng(ctx.seed):
+            g_res, g_in, g_gamma, g_beta, g_bias = (
+                get_layernorm_kernel().bias_dropout_add_norm_backward(
+                    ctx.rms, grad_y.contiguous(),
+                    None if grad_h is None else grad_h.contiguous(),
+                    h, mean, invvar, ctx.normalized_shape, weight,
+                    ctx.p, _seed_arg(ctx.seed), ctx.offset, need_bias_grad=need_b,
+                )
             )
-        )
         return (
             g_in,
             g_bias if need_b else None,
@@ -413,9 +461,10 @@ class _ScaledMaskedSoftmaxDropout(torch.autograd.Function):
     def forward(ctx, inputs, mask, scale, p, seed, offset):
         scale = float(scale)
         inputs = inputs.contiguous()
-        out, stats = get_softmax_kernel().softmax_dropout_forward(
-            inputs, mask, scale, p, seed, offset
-        )
+        with _rng(seed):
+            out, stats = get_softmax_kernel().softmax_dropout_forward(
+                inputs, mask, scale, p, _seed_arg(seed), offset
+            )
         ctx.scale, ctx.p, ctx.seed, ctx.offset = scale, p, seed, offset
         ctx.has_mask = mask is not None
         if mask is not None:
@@ -430,10 +479,11 @@ class _ScaledMaskedSoftmaxDropout(torch.autograd.Function):
             inputs, stats, mask = ctx.saved_tensors
         else:
             (inputs, stats), mask = ctx.saved_tensors, None
-        input_grads = get_softmax_kernel().softmax_dropout_backward(
-            output_grads.contiguous(), inputs, stats, mask, ctx.scale, ctx.p,
-            ctx.seed, ctx.offset,
-        )
+        with _rng(ctx.seed):
+            input_grads = get_softmax_kernel().softmax_dropout_backward(
+                output_grads.contiguous(), inputs, stats, mask, ctx.scale, ctx.p,
+                _seed_arg(ctx.seed), ctx.offset,
+            )
         return input_grads, None, None, None, None, None
 
 

@@ -75,20 +75,87 @@ def test_captured_layer_chain_replays(device):
             assert torch.equal(a, b), "optimizer state differs on replay %d" % rep
 
 
-def test_dropout_from_the_generator_refuses_capture_with_a_message(device):
+def test_captured_dropout_draws_a_new_mask_on_every_replay(device):
+    """Through the Python layer: during capture the kernels read (seed, offset)
+    from device memory, a captured add advances the offset, and backward takes
+    the forward's pair; every replay must equal the integer Philox oracle for
+    the pair that the state held when the replay started."""
+    import numpy as np
+
+    from oracle import philox
     from oslo_amd.torch.nn.modules import functional as F_
 
-    x = randn((8, 64), BF16, 1).to(device)
-    b = torch.zeros(64, dtype=BF16, device=device)
-    F_.fused_bias_dropout_add(x, b, None, 0.5, True)  # eager: fine
+    n1, n2, p = 64, 256, 0.25
+    x = randn((n1, n2), BF16, 1).to(device)
+    b = torch.zeros(n2, dtype=BF16, device=device)
+    dy = torch.ones(n1, n2, dtype=BF16, device=device)
+    sc = randn((2, 64, 64), BF16, 2).to(device)
+
+    # before any eager call on the device there is no state to read
+    F_._graph_rng.clear()
     graph = torch.cuda.CUDAGraph()
-    with pytest.raises(RuntimeError, match="cannot be captured"):
+    with pytest.raises(RuntimeError, match="eager step first"):
         with torch.cuda.graph(graph):
-            F_.fused_bias_dropout_add(x, b, None, 0.5, True)
-    # p = 0 captures (nothing is drawn)
+            F_.fused_bias_dropout_add(x, b, None, p, True)
+
+    torch.manual_seed(1234)
+    F_.fused_bias_dropout_add(x, b, None, p, True)  # eager: creates the state
+    index = device.index if device.index is not None else torch.cuda.current_device()
+    state = F_._graph_rng[index][1]
+
+    xg = x.clone().requires_grad_()
+    scg = sc.clone().requires_grad_()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):  # warm-up of the autograd machinery
+        F_.fused_bias_dropout_add(xg, b, None, p, True).backward(dy)
+    torch.cuda.current_stream().wait_stream(side)
+    xg.grad = None
     graph = torch.cuda.CUDAGraph()
     with torch.cuda.graph(graph):
-        out = F_.fused_bias_dropout_add(x, b, None, 0.0, True)
+        out = F_.fused_bias_dropout_add(xg, b, None, p, True)
+        gx, = torch.autograd.grad(out, xg, dy)
+        probs = F_.scaled_upper_triang_masked_softmax_dropout(scg, 0.5, p, True)
+        gs, = torch.autograd.grad(probs, scg, torch.ones_like(probs))
+    masks = []
+    for rep in range(3):
+        seed, offset = (int(v) for v in state.cpu())
+        graph.replay()
+        torch.cuda.synchronize()
+        keep = philox.keep_mask(n1 * n2, p, seed % 2 ** 64, offset % 2 ** 64).reshape(n1, n2).astype(bool)
+        got = (out != 0).cpu().numpy() | (x == 0).cpu().numpy()
+        assert np.array_equal(got, keep | (x == 0).cpu().numpy()), "forward mask differs from the oracle"
+        # backward used the forward's pair: dx = keep / (1 - p)
+        assert np.array_equal((gx != 0).cpu().numpy(), keep)
+        # the softmax call was captured second: its pair is 4 further
+        keep2 = philox.keep_mask(sc.numel(), p, seed % 2 ** 64, (offset + 4) % 2 ** 64).reshape(sc.shape).astype(bool)
+        visible = np.tril(np.ones((64, 64), dtype=bool))[None]
+        assert np.array_equal((probs != 0).cpu().numpy(), keep2 & visible)
+        assert torch.isfinite(gs).all()
+        masks.append(keep)
+        assert int(state.cpu()[1]) == offset + 8, "two captured calls advance the offset by 8"
+    assert not np.array_equal(masks[0], masks[1]) and not np.array_equal(masks[1], masks[2])
+    # the fusion into the norm reads the same state (prologue and epilogue)
+    w = torch.ones(n2, dtype=BF16, device=device)
+    res = torch.zeros(n1, n2, dtype=BF16, device=device)
+    xg2 = x.clone().requires_grad_()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        y, h = F_.fused_bias_dropout_add_layer_norm(xg2, b, res, w, b, (n2,), 1e-5, p, True,
+                                                    return_sum=True)
+        gx2, = torch.autograd.grad(y, xg2, dy)
+    for rep in range(2):
+        seed, offset = (int(v) for v in state.cpu())
+        graph.replay()
+        torch.cuda.synchronize()
+        keep = philox.keep_mask(n1 * n2, p, seed % 2 ** 64, offset % 2 ** 64).reshape(n1, n2).astype(bool)
+        assert np.array_equal((h != 0).cpu().numpy() | (x == 0).cpu().numpy(),
+                              keep | (x == 0).cpu().numpy())
+        assert ((gx2 == 0).cpu().numpy() | keep).all(), "dropped elements get no gradient"
+    # p = 0 captures without touching the state
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        same = F_.fused_bias_dropout_add(x, b, None, 0.0, True)
     graph.replay()
     torch.cuda.synchronize()
-    assert torch.equal(out, x)
+    assert torch.equal(same, x)
