@@ -72,6 +72,28 @@ __device__ __forceinline__ float row_sum1(float a, float *red, int wave,
   return a;
 }
 
+// The same sums when a row is a whole number of half-waves ("units" of 32
+// lanes, `upr` of them per row; rows of 96 or 160 chunks then leave no lane
+// idle): reduction inside the unit, one value per unit through LDS, then every
+// lane adds the upr values of its row.  red is [2][32] floats.
+__device__ __forceinline__ void unit_sum2(float &a, float &b, float *red,
+                                          int unit, int first, int upr,
+                                          int ulane) {
+  a = group_allreduce<OpSum, 32>(a);
+  b = group_allreduce<OpSum, 32>(b);
+  if (ulane == 0) {
+    red[unit] = a;
+    red[32 + unit] = b;
+  }
+  __syncthreads();
+  a = 0.f;
+  b = 0.f;
+  for (int u = 0; u < upr; ++u) {
+    a += red[first + u];
+    b += red[32 + first + u];
+  }
+}
+
 // Welford partials of equal size (every lane holds w.n values) merged over
 // the wave and then over the wpr waves of a row.  The waves hold equal
 // counts c, so the row's mean is the average of the wave means and its M2 is
@@ -451,8 +473,10 @@ struct FuseEpilogue {
 // MAXT: largest workgroup the build is launched with (768 leaves a third more
 // registers per lane than 1024, which the 16-elements-per-lane builds need).
 // LPR: as in the forward kernel (rows side by side in a wave when < 64).
+// UNIT: 64, or 32 when a row is `wpr` half-waves (then "wave" below means
+// such a unit of 32 lanes; LPR == 64, VPL == 1, EVEN).
 template <typename T, typename V, int VPL, bool RMS, bool EVEN, int PF,
-          bool FUSE = false, int MAXT = 1024, int LPR = kWave>
+          bool FUSE = false, int MAXT = 1024, int LPR = kWave, int UNIT = kWave>
 __global__ __launch_bounds__(MAXT) void norm_bwd_reg_kernel(
     const V *__restrict__ dy, const T *__restrict__ x,
     const float *__restrict__ mean, const float *__restrict__ invvar,
@@ -462,11 +486,14 @@ __global__ __launch_bounds__(MAXT) void norm_bwd_reg_kernel(
   static_assert(!FUSE || sizeof(T) == sizeof(V), "fused epilogue: one dtype");
   if constexpr (FUSE) fe.d = resolve_drop(fe.d);
   static_assert(LPR == kWave || VPL == 1 || VPL == 3, "side-by-side rows: one or three chunks per lane");
+  static_assert(UNIT == kWave || (UNIT == 32 && LPR == kWave && VPL == 1 && EVEN),
+                "half-wave units: whole-unit rows, one chunk per lane");
   extern __shared__ float xslot[];  // [n2] when rpb > 1
-  __shared__ float red[2][32];
-  const int lane = threadIdx.x & 63;
+  __shared__ float red[2][64];
+  const int lane = UNIT == kWave ? (threadIdx.x & 63) : (threadIdx.x & 31);
   // the wave index is uniform: keep it (and the row arithmetic) in scalar registers
-  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int wave = UNIT == kWave ? __builtin_amdgcn_readfirstlane(threadIdx.x >> 6)
+                                 : (int)(threadIdx.x >> 5);
   constexpr int SUB = kWave / LPR;
   const int first = (wave / wpr) * wpr;
   // row slot of this lane; wslot is the wave's slot when its lane groups
@@ -474,8 +501,8 @@ __global__ __launch_bounds__(MAXT) void norm_bwd_reg_kernel(
   const int wslot = wave / wpr;
   const int rslot = LPR == kWave ? wslot : wave * SUB + lane / LPR;
   const int nchunks = n2 / E;
-  const int cstride = LPR == kWave ? kWave * wpr : LPR;
-  const int c0 = LPR == kWave ? (wave - first) * kWave + lane : (lane & (LPR - 1));
+  const int cstride = LPR == kWave ? UNIT * wpr : LPR;
+  const int c0 = LPR == kWave ? (wave - first) * UNIT + lane : (lane & (LPR - 1));
   const float fn = (float)n2;
   const bool affine = gamma != nullptr;
 
@@ -578,7 +605,10 @@ __global__ __launch_bounds__(MAXT) void norm_bwd_reg_kernel(
         d[k][e] = dg;  // only dy * gamma is needed from here on
       }
     }
-    if constexpr (RMS) {
+    if constexpr (UNIT == 32) {
+      unit_sum2(s1, s2, red[parity], wave, first, wpr, lane);
+      if constexpr (RMS) s1 = 0.f;
+    } else if constexpr (RMS) {
       s2 = row_sum1<LPR>(s2, red[parity], wave, first, wpr, lane);
       s1 = 0.f;
     } else {
@@ -1196,6 +1226,19 @@ static int launch_norm_bwd(const void *dy, const void *x, const float *mean,
             (V *)dbeta, n1, n2);
     return check_launch("norm_bwd_param_generic_kernel");
   }
+  // rows that are a whole number of half-waves but not of waves (96, 160 or
+  // 224 chunks: 768, 1280, 1792 16-bit elements): units of 32 lanes, so that
+  // no lane idles
+  int upr = 0;
+  if (E == 8 && g_tune.norm_lanes_per_row != kWave && sp.vpl == 1) {
+    const int64_t nch = n2 / E;
+    if (nch % 32 == 0 && nch % 64 != 0 && (nch == 96 || nch == 160 || nch == 224))
+      upr = (int)(nch / 32);
+  }
+  if (upr > 0) {
+    sp.wpr = upr;
+    sp.rpb = 32 / upr;
+  }
   // short rows side by side in a wave: the row slots of a workgroup multiply
   // (the three-chunks-per-lane mapping of the forward kernel does not pay
   //  here: its 24 elements per lane and operand need a 512-thread workgroup,
@@ -1220,9 +1263,10 @@ static int launch_norm_bwd(const void *dy, const void *x, const float *mean,
                   (long long)need, (long long)ws_bytes);
     part = (float *)ws;
   }
-  const int threads = kWave * sp.wpr * wave_slots;
+  const int threads = (upr > 0 ? 32 : kWave) * sp.wpr * wave_slots;
   const size_t lds = wave_slots > 1 ? (size_t)n2 * sizeof(float) : 0;
-  const bool even = lpr < kWave ? (n2 / E) == lpr
+  const bool even = upr > 0 ? true
+                  : lpr < kWave ? (n2 / E) == lpr
                                 : (n2 / E) == (int64_t)sp.vpl * kWave * sp.wpr;
   // rows in flight ahead of the one being reduced: two while the packed row
   // buffers are small (8 elements per lane) and a row spans several waves,
@@ -1270,7 +1314,30 @@ static int launch_norm_bwd(const void *dy, const void *x, const float *mean,
         OSLO_BWD_LAUNCH(VPL, false, 1);                                    \
     }                                                                      \
     break;
-  if (lpr < kWave) {
+  if (upr > 0) {
+#define OSLO_BWD_UNIT(PF_)                                                  \
+  do {                                                                      \
+    if constexpr (kCanFuse) {                                               \
+      if (fused) {                                                          \
+        norm_bwd_reg_kernel<T, V, 1, RMS, true, PF_, true, 1024, kWave, 32> \
+            <<<dim3((unsigned)P), threads, lds, st>>>(                      \
+                (const V *)dy, (const T *)x, mean, invvar,                  \
+                (const V *)gamma, (T *)dx, part, n1, (int)n2, sp.wpr,       \
+                sp.rpb, fev);                                               \
+        break;                                                              \
+      }                                                                     \
+    }                                                                       \
+    norm_bwd_reg_kernel<T, V, 1, RMS, true, PF_, false, 1024, kWave, 32>    \
+        <<<dim3((unsigned)P), threads, lds, st>>>(                          \
+            (const V *)dy, (const T *)x, mean, invvar, (const V *)gamma,    \
+            (T *)dx, part, n1, (int)n2, sp.wpr, sp.rpb, fev);               \
+  } while (0)
+    if constexpr (E == 8) {
+      if (pf == 2) OSLO_BWD_UNIT(2);
+      else OSLO_BWD_UNIT(1);
+    }
+#undef OSLO_BWD_UNIT
+  } else if (lpr < kWave) {
 #define OSLO_BWD_LPR(LPR_)                                                  \
   case LPR_:                                                                \
     if constexpr (kCanFuse) {                                               \

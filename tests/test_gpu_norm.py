@@ -43,6 +43,12 @@ CASES = [
     (3001, 100, BF16, BF16),
     (300, 4100, F16, F16),
     (2000, 37, F32, F32),
+    # rows of a whole number of half-waves (96, 160, 224 chunks): the backward
+    # works in units of 32 lanes
+    (1003, 768, BF16, BF16),
+    (517, 1280, F16, F16),
+    (260, 1792, BF16, BF16),
+    (129, 384, F32, F32),     # 96 fp32 chunks: whole waves
 ]
 
 
