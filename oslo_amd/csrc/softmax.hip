@@ -147,7 +147,7 @@ __global__ __launch_bounds__(1024) void softmax_fwd_kernel(
   const int rslot = wave / g.wpr;
   const int first = rslot * g.wpr;
   const int nchunks = g.sk / E;
-  const int cstride = kWave * g.wpr;
+  const int cstride = LPR == kWave ? kWave * g.wpr : LPR;
   constexpr int SUB = kWave / LPR;  // rows side by side in a wave
   const int sl = LPR == kWave ? lane : (lane & (LPR - 1));
   const int c0 = (wave - first) * kWave + sl;
@@ -329,7 +329,7 @@ __global__ __launch_bounds__(1024) void softmax_dropout_bwd_kernel(
   const int rslot = wave / g.wpr;
   const int first = rslot * g.wpr;
   const int nchunks = g.sk / E;
-  const int cstride = kWave * g.wpr;
+  const int cstride = LPR == kWave ? kWave * g.wpr : LPR;
   constexpr int SUB = kWave / LPR;
   const int sl = LPR == kWave ? lane : (lane & (LPR - 1));
   const int c0 = (wave - first) * kWave + sl;
@@ -469,7 +469,7 @@ __global__ __launch_bounds__(1024) void softmax_bwd_kernel(
   const int rslot = wave / g.wpr;
   const int first = rslot * g.wpr;
   const int nchunks = g.sk / E;
-  const int cstride = kWave * g.wpr;
+  const int cstride = LPR == kWave ? kWave * g.wpr : LPR;
   constexpr int SUB = kWave / LPR;
   const int sl = LPR == kWave ? lane : (lane & (LPR - 1));
   const int c0 = (wave - first) * kWave + sl;
@@ -1021,7 +1021,8 @@ struct SoftmaxPlan {
 
 // max_elems: elements of one operand a lane may hold (register budget).
 static SoftmaxPlan plan_softmax(int64_t sk, int E, int max_elems,
-                                int default_rpw, int one_chunk_rpw) {
+                                int default_rpw, int one_chunk_rpw,
+                                bool two_chunk_groups = false) {
   SoftmaxPlan p{0, 1, 1, 1, kWave, false};
   if (sk % E != 0) return p;
   const int64_t nchunks = sk / E;
@@ -1037,6 +1038,37 @@ static SoftmaxPlan plan_softmax(int64_t sk, int E, int max_elems,
     if (g_tune.softmax_lanes_per_row == 8 || g_tune.softmax_lanes_per_row == 16 ||
         g_tune.softmax_lanes_per_row == 32)
       if (g_tune.softmax_lanes_per_row >= p.lpr) p.lpr = g_tune.softmax_lanes_per_row;
+  }
+  // rows of exactly 3 x 8 / 16 / 32 / 64 chunks (192, 384, 768, 1536 16-bit
+  // keys): three chunks per lane, no idle lane
+  if (nchunks % 3 == 0 && g_tune.softmax_lanes_per_row != kWave && 3 * E <= max_elems) {
+    const int64_t q = nchunks / 3;
+    if (q == 8 || q == 16 || q == 32 || q == 64) {
+      p.vpl = 3;
+      p.rpw = 1;
+      p.wpr = 1;
+      p.rpb = 4;
+      p.lpr = (int)q;
+      p.ok = true;
+      return p;
+    }
+  }
+  // forward: rows of exactly 2 x 8 / 16 / 32 chunks (128, 256, 512 16-bit
+  // keys) as two chunks per lane in a lane group
+  if (two_chunk_groups && nchunks % 2 == 0 && g_tune.softmax_lanes_per_row != kWave &&
+      g_tune.softmax_lanes_per_row != 1) {
+    const int64_t q = nchunks / 2;
+    if (q == 8 || q == 16 || q == 32) {
+      // one row set per wave without a mask tensor, two with one (measured)
+      int want = g_tune.softmax_rows_per_wave > 0 ? g_tune.softmax_rows_per_wave : default_rpw;
+      p.vpl = 2;
+      p.rpw = want >= 2 && 2 * 2 * E <= max_elems ? 2 : 1;
+      p.wpr = 1;
+      p.rpb = 4;
+      p.lpr = (int)q;
+      p.ok = true;
+      return p;
+    }
   }
   if (wpr == 1) {
     // row sets a wave handles at once; measured best on MI355X: one, or two
@@ -1070,7 +1102,27 @@ constexpr int kBwdMaxElems = 32;  // two operands resident
     LAUNCH(1, 4, LPR_);                    \
   }
 #define OSLO_SM_CASES(LAUNCH)              \
-  if (pl.lpr == 8) {                       \
+  if (pl.vpl == 3 && pl.lpr == 8) {        \
+    LAUNCH(3, 1, 8);                       \
+  } else if (pl.vpl == 3 && pl.lpr == 16) { \
+    LAUNCH(3, 1, 16);                      \
+  } else if (pl.vpl == 3 && pl.lpr == 32) { \
+    LAUNCH(3, 1, 32);                      \
+  } else if (pl.vpl == 3) {                \
+    LAUNCH(3, 1, kWave);                   \
+  } else if (pl.vpl == 2 && pl.lpr == 8 && pl.rpw == 1) {  \
+    LAUNCH(2, 1, 8);                       \
+  } else if (pl.vpl == 2 && pl.lpr == 8) { \
+    LAUNCH(2, 2, 8);                       \
+  } else if (pl.vpl == 2 && pl.lpr == 16 && pl.rpw == 1) { \
+    LAUNCH(2, 1, 16);                      \
+  } else if (pl.vpl == 2 && pl.lpr == 16) { \
+    LAUNCH(2, 2, 16);                      \
+  } else if (pl.vpl == 2 && pl.lpr == 32 && pl.rpw == 1) { \
+    LAUNCH(2, 1, 32);                      \
+  } else if (pl.vpl == 2 && pl.lpr == 32) { \
+    LAUNCH(2, 2, 32);                      \
+  } else if (pl.lpr == 8) {                \
     OSLO_SM_CASES_LPR(LAUNCH, 8)           \
   } else if (pl.lpr == 16) {               \
     OSLO_SM_CASES_LPR(LAUNCH, 16)          \
@@ -1107,7 +1159,7 @@ static int launch_softmax_fwd(const void *x, const uint8_t *mask, void *y,
   // more 16-bit keys then take two or more waves); 64 only where a row would
   // otherwise not fit one workgroup
   const int cap = g_tune.softmax_fwd_elems > 0 ? g_tune.softmax_fwd_elems : 32;
-  SoftmaxPlan pl = plan_softmax(g.sk, E, cap, MODE == kModeMasked ? 2 : 1, 4);
+  SoftmaxPlan pl = plan_softmax(g.sk, E, cap, MODE == kModeMasked ? 2 : 1, 4, true);
   if (!pl.ok && cap < kFwdMaxElems)
     pl = plan_softmax(g.sk, E, kFwdMaxElems, MODE == kModeMasked ? 2 : 1, 4);
   const bool vec_ok = pl.ok && aligned16(x) && aligned16(y) &&

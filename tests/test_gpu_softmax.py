@@ -41,6 +41,13 @@ CAUSAL_CASES = [
     (2, 20, 1004, BF16, 0.25),
     (2, 30, 50, F32, 0.5),          # fp32: 8-byte accesses for even lengths
     (2, 10, 998, F16, 0.25),        # 4-byte accesses
+    # rows of exactly 3 x 8 / 16 / 32 / 64 chunks: three chunks per lane
+    (3, 192, 192, BF16, 0.25),
+    (2, 384, 384, F16, 0.125),
+    (2, 768, 768, BF16, 0.125),
+    (1, 200, 1536, F16, 0.25),
+    (2, 96, 96, F32, 0.5),
+    (2, 50, 384, F32, 0.25),
 ]
 
 
@@ -100,6 +107,9 @@ MASKED_CASES = [
     (2, 1, 6, 203, F16, 0.5, "full"),
     (2, 1, 6, 1030, BF16, 0.5, "padding"),
     (2, 1, 6, 2050, BF16, 0.5, "padding"),   # one workgroup per row
+    (2, 2, 16, 384, F16, 0.125, "padding"),  # three chunks per lane
+    (2, 2, 16, 768, BF16, 0.125, "full"),
+    (2, 2, 9, 192, F32, 0.25, "rows_fully_masked"),
 ]
 
 

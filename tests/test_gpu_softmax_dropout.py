@@ -42,6 +42,9 @@ CAUSAL_CASES = [
     (2, 5, 2046, F16, 0.25, 0.1),
     (2, 5, 2051, BF16, 0.25, 0.1),        # one workgroup per row
     (4, 5, 1, F32, 1.0, 0.3),             # one key: the gradient is exactly zero
+    (2, 384, 384, BF16, 0.125, 0.1),      # three chunks per lane
+    (2, 100, 768, F16, 0.125, 0.2),
+    (2, 60, 192, F32, 0.25, 0.1),
 ]
 
 
@@ -83,6 +86,8 @@ MASKED_CASES = [
     (2, 2, 12, 50, BF16, 0.5, "padding", 0.2),       # 4-byte accesses
     (2, 2, 12, 50, F32, 0.5, "full", 0.1),           # fp32, 8-byte accesses
     (2, 2, 12, 77, BF16, 0.5, "rows_fully_masked", 0.1),
+    (2, 2, 12, 768, F16, 0.125, "full", 0.1),        # three chunks per lane
+    (2, 2, 12, 1536, BF16, 0.125, "padding", 0.1),
 ]
 
 
