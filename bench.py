@@ -36,7 +36,7 @@ HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published
 METRIC = "achieved HBM GB/s (% of MI355X peak) per fused fwd+bwd kernel; speedup vs CPU path"
 # HBM traffic of one LayerNorm-backward call on bf16 [16384, 4096], measured with
 # rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE and calibrated against a 1 GiB copy:
-# main kernel 270.6 MB read + 140.4 MB written, finalize 8.4 MB read
+# main kernel 270.9 MB read + 142.5 MB written, finalize 8.4 MB read
 # (summary: profiles/bench_all_kernels_hbm_traffic.txt).  Algorithmic: 402.7 MB.
 LN_BWD_TRAFFIC_BYTES = 421.9e6
 
