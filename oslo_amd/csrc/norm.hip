@@ -488,7 +488,7 @@ __global__ __launch_bounds__(MAXT) void norm_bwd_reg_kernel(
   static_assert(LPR == kWave || VPL == 1 || VPL == 3, "side-by-side rows: one or three chunks per lane");
   static_assert(UNIT == kWave || (UNIT == 32 && LPR == kWave && VPL == 1 && EVEN),
                 "half-wave units: whole-unit rows, one chunk per lane");
-  extern __shared__ float xslot[];  // [n2] when rpb > 1
+  extern __shared__ __align__(16) float xslot[];  // [n2] when rpb > 1
   __shared__ float red[2][64];
   const int lane = UNIT == kWave ? (threadIdx.x & 63) : (threadIdx.x & 31);
   // the wave index is uniform: keep it (and the row arithmetic) in scalar registers
@@ -506,17 +506,31 @@ __global__ __launch_bounds__(MAXT) void norm_bwd_reg_kernel(
   const float fn = (float)n2;
   const bool affine = gamma != nullptr;
 
-  // gamma stays packed (half the registers) and is unpacked once per row
-  RawChunk<V, E> gmraw[VPL];
+  // gamma stays packed (half the registers) and is unpacked once per row.
+  // With 16 elements per lane the registers run out: all but GREG chunks of
+  // gamma then live in LDS, each lane reading back what it wrote (no barrier).
+  constexpr int GREG = VPL * E >= 16 ? (sizeof(V) == 4 ? 1 : 0) : VPL;
+  RawChunk<V, E> gmraw[GREG > 0 ? GREG : 1];
+  RawChunk<V, E> *const gslot =
+      reinterpret_cast<RawChunk<V, E> *>(xslot + (rpb > SUB ? n2 : 0));
   float acc_g[VPL][E], acc_b[VPL][E];
   float acc_d[FUSE ? VPL : 1][E];  // bias gradient of the fused epilogue
 #pragma unroll
   for (int k = 0; k < VPL; ++k) {
     const int c = c0 + k * cstride;
+    RawChunk<V, E> g;
     if (affine && c < nchunks)
-      gmraw[k].load_cached(gamma + (int64_t)c * E);
+      g.load_cached(gamma + (int64_t)c * E);
     else
-      gmraw[k].zero();
+      g.zero();
+    if constexpr (GREG == VPL) {
+      gmraw[k] = g;
+    } else {
+      if (k < GREG)
+        gmraw[k < GREG ? k : 0] = g;
+      else
+        gslot[(k - GREG) * blockDim.x + threadIdx.x] = g;
+    }
 #pragma unroll
     for (int e = 0; e < E; ++e) {
       acc_g[k][e] = 0.f;
@@ -591,7 +605,10 @@ __global__ __launch_bounds__(MAXT) void norm_bwd_reg_kernel(
 #pragma unroll
     for (int k = 0; k < VPL; ++k) {
       float gm[E];
-      gmraw[k].unpack(gm);
+      if (k < GREG)
+        gmraw[k < GREG ? k : 0].unpack(gm);
+      else
+        gslot[(k - GREG) * blockDim.x + threadIdx.x].unpack(gm);
 #pragma unroll
       for (int e = 0; e < E; ++e) {
         // normalised input; subtract first: exact when x is close to the mean
@@ -917,9 +934,16 @@ static int launch_norm_fwd(const void *x, const void *gamma, const void *beta,
   RowSplit sp{0, 1, 1, false};
   if (vec_ok) {
     // measured fastest on MI355X: up to four chunks per lane; LayerNorm,
-    // whose kernel holds more live registers, takes two while the row then
-    // still fits four waves
-    int cap = (!RMS && n2 / E <= kWave * 2 * 4) ? 2 : 4;
+    // whose kernel holds more live registers, takes two in rows of up to four
+    // waves that four per lane would not fill evenly (3072 16-bit elements:
+    // three waves of two chunks rather than two waves of three), and so do
+    // rows of 1536 eight-element chunks (12288 elements: twelve waves measure
+    // 5 % faster than six)
+    const int64_t nch = n2 / E;
+    int cap = (!RMS && nch <= kWave * 2 * 4 && nch % (kWave * 4) != 0) ? 2 : 4;
+    if (E == 8 && nch == 1536) cap = 2;
+    // fp32 rows of 3072 and 4096 elements: 3 % faster over twice the waves
+    if (E == 4 && (nch == 768 || nch == 1024)) cap = 2;
     if (g_tune.norm_fwd_vpl > 0) cap = g_tune.norm_fwd_vpl;
     const int waves = g_tune.norm_fwd_waves > 0 ? g_tune.norm_fwd_waves : 4;
     sp = split_row(n2 / E, cap > 8 ? 8 : cap, kVpl, 4, waves);
@@ -969,7 +993,8 @@ static int launch_norm_fwd(const void *x, const void *gamma, const void *beta,
   // are spread over that many rows
   // (LayerNorm: two groups, the second one prefetched; RMSNorm is fastest
   // with short-lived workgroups)
-  int iters = g_tune.norm_fwd_iters > 0 ? g_tune.norm_fwd_iters : (RMS ? 1 : 2);
+  int iters = g_tune.norm_fwd_iters > 0 ? g_tune.norm_fwd_iters
+              : (RMS && !(E == 8 && n2 / E == 1536)) ? 1 : 2;
   int64_t grid = ceil_div(ceil_div(n1, sp.rpb), iters);
   const int64_t maxgrid = (int64_t)device_cu_count() * 64;
   if (grid > maxgrid) grid = maxgrid;
@@ -1264,7 +1289,12 @@ static int launch_norm_bwd(const void *dy, const void *x, const float *mean,
     part = (float *)ws;
   }
   const int threads = (upr > 0 ? 32 : kWave) * sp.wpr * wave_slots;
-  const size_t lds = wave_slots > 1 ? (size_t)n2 * sizeof(float) : 0;
+  // LDS: one row of column partials when a workgroup holds several row
+  // slots, and behind it the chunks of gamma that 16 elements per lane move
+  // out of the registers (one of four with 4-byte parameters, else all)
+  size_t lds = wave_slots > 1 ? (size_t)n2 * sizeof(float) : 0;
+  if (sp.vpl * E >= 16)
+    lds += (size_t)(sp.vpl - (sizeof(V) == 4 ? 1 : 0)) * threads * E * sizeof(V);
   const bool even = upr > 0 ? true
                   : lpr < kWave ? (n2 / E) == lpr
                                 : (n2 / E) == (int64_t)sp.vpl * kWave * sp.wpr;

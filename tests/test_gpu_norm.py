@@ -49,6 +49,13 @@ CASES = [
     (517, 1280, F16, F16),
     (260, 1792, BF16, BF16),
     (129, 384, F32, F32),     # 96 fp32 chunks: whole waves
+    # 16 elements per lane in the backward (part of gamma lives in LDS)
+    (5, 16384, F32, F32),
+    (6, 12288, F32, F32),
+    (5, 16384, F32, BF16),
+    (7, 12288, BF16, BF16),
+    (5, 9000, F16, F16),      # ... with lanes beyond the end of the row
+    (4, 14000, F32, F32),
 ]
 
 
