@@ -1301,7 +1301,10 @@ static int launch_norm_bwd(const void *dy, const void *x, const float *mean,
   // rows in flight ahead of the one being reduced: two while the packed row
   // buffers are small (8 elements per lane) and a row spans several waves,
   // else one (a wave that owns whole rows measures 6 % slower with two)
-  int pf = sp.vpl * E <= 8 && sp.wpr >= 2 ? 2 : 1;
+  // (plain workgroups of twelve waves, rows of 3072 and 6144 16-bit
+  //  elements, measure 2.5 % faster with one; with the fused epilogue 8 %
+  //  slower)
+  int pf = sp.vpl * E <= 8 && sp.wpr >= 2 && (fused || threads != 12 * kWave) ? 2 : 1;
   if (g_tune.norm_bwd_prefetch > 0) pf = g_tune.norm_bwd_prefetch >= 2 ? 2 : 1;
 #define OSLO_BWD_LAUNCH_T(VPL, EVEN_, PF_, MAXT_)                          \
   do {                                                                     \
