@@ -396,6 +396,15 @@ struct Philox4 {
   uint32_t x, y, z, w;
 };
 
+// a ^ b ^ c: one v_bitop3_b32 (truth table 0x96) on the GPU
+__device__ __host__ __forceinline__ uint32_t xor3(uint32_t a, uint32_t b, uint32_t c) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  return __builtin_amdgcn_bitop3_b32(a, b, c, 0x96);
+#else
+  return a ^ b ^ c;
+#endif
+}
+
 __device__ __host__ __forceinline__ Philox4 philox4x32_10(uint32_t c0,
                                                            uint32_t c1,
                                                            uint32_t c2,
@@ -408,9 +417,9 @@ __device__ __host__ __forceinline__ Philox4 philox4x32_10(uint32_t c0,
   for (int r = 0; r < 10; ++r) {
     const uint64_t p0 = (uint64_t)M0 * c0;
     const uint64_t p1 = (uint64_t)M1 * c2;
-    const uint32_t n0 = (uint32_t)(p1 >> 32) ^ c1 ^ k0;
+    const uint32_t n0 = xor3((uint32_t)(p1 >> 32), c1, k0);
     const uint32_t n1 = (uint32_t)p1;
-    const uint32_t n2 = (uint32_t)(p0 >> 32) ^ c3 ^ k1;
+    const uint32_t n2 = xor3((uint32_t)(p0 >> 32), c3, k1);
     const uint32_t n3 = (uint32_t)p0;
     c0 = n0;
     c1 = n1;
