@@ -36,7 +36,7 @@ HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published
 METRIC = "achieved HBM GB/s (% of MI355X peak) per fused fwd+bwd kernel; speedup vs CPU path"
 # HBM traffic of one LayerNorm-backward call on bf16 [16384, 4096], measured with
 # rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE and calibrated against a 1 GiB copy:
-# main kernel 270.9 MB read + 142.5 MB written, finalize 8.4 MB read
+# main kernel 270.9 MB read + 142.6 MB written, finalize 8.4 MB read
 # (summary: profiles/bench_all_kernels_hbm_traffic.txt).  Algorithmic: 402.7 MB.
 LN_BWD_TRAFFIC_BYTES = 421.9e6
 
@@ -48,9 +48,9 @@ def parse_args():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--table-iters", type=int, default=20, help="launches per kernel in the per-kernel table (0 = skip)")
+    ap.add_argument("--table-iters", type=int, default=200, help="launches per kernel in the per-kernel table (0 = skip)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--cpu-reps", type=int, default=3)
+    ap.add_argument("--cpu-reps", type=int, default=15)
     return ap.parse_args()
 
 
@@ -80,7 +80,8 @@ def p(t):
 
 def time_launches(torch, fn, iters, nsets):
     """Average duration in ms of fn(i % nsets), events on the current stream."""
-    for i in range(max(3, nsets)):  # every buffer set is touched before the timed region
+    # warm-up: every buffer set is touched, 20 launches ahead of a long timed region
+    for i in range(max(3, nsets, min(20, iters // 10))):
         fn(i % nsets)
     torch.cuda.synchronize()
     e0 = torch.cuda.Event(enable_timing=True)
