@@ -357,7 +357,15 @@ int oslo_wave_reduce_selftest(float *out4, void *stream);
  * "eltwise_fwd_steps", "eltwise_tile_max", "eltwise_tile_min" (lanes along
  * the columns of an element-wise tile; 64 as the minimum restores whole-wave
  * tiles), "adam_unroll";
- * value 0 restores the default.  Process-wide, not thread-safe.            */
+ * value 0 restores the default.  Other values must be ones the launch code
+ * has a kernel build and a valid workgroup shape for, else
+ * OSLO_ERR_INVALID_ARGUMENT: chunks per lane (*_vpl: 1, 2, 4, forward also 8),
+ * waves per workgroup 1..16, norm_bwd_prefetch 1 or 2, norm_fwd_iters 1..16,
+ * norm_bwd_blocks_per_cu 1..8, lanes per row 8, 16, 32 or 64 (softmax also
+ * 1), softmax_rows_per_wave and the unroll factors 1, 2 or 4,
+ * softmax_fwd_elems 16, 32 or 64, eltwise tile widths powers of two up to
+ * 256, eltwise_rowgroups 1..4096, eltwise_fwd_steps 1..64.
+ * Process-wide, not thread-safe.                                           */
 int oslo_tune(const char *key, int value);
 
 #ifdef __cplusplus

@@ -83,31 +83,45 @@ int64_t oslo_workspace_bytes(int op, int64_t n1, int64_t n2) {
 int oslo_tune(const char *key, int value) {
   if (key == nullptr || value < 0)
     return oslo::fail(OSLO_ERR_INVALID_ARGUMENT, "tune: bad arguments");
+  // 0 restores the built-in choice; any other value must be one the launch
+  // code has a kernel build and a valid workgroup shape for
+  enum Kind { kPow2, kRange, kLanes };
   struct Entry {
     const char *name;
     int *slot;
+    Kind kind;
+    int lo, hi;  // kPow2: powers of two in [lo, hi]; kRange: lo..hi
   };
   const Entry table[] = {
-      {"norm_fwd_vpl", &oslo::g_tune.norm_fwd_vpl},
-      {"norm_bwd_vpl", &oslo::g_tune.norm_bwd_vpl},
-      {"norm_bwd_blocks_per_cu", &oslo::g_tune.norm_bwd_blocks_per_cu},
-      {"softmax_rows_per_wave", &oslo::g_tune.softmax_rows_per_wave},
-      {"softmax_lanes_per_row", &oslo::g_tune.softmax_lanes_per_row},
-      {"softmax_fwd_elems", &oslo::g_tune.softmax_fwd_elems},
-      {"norm_lanes_per_row", &oslo::g_tune.norm_lanes_per_row},
-      {"eltwise_tile_max", &oslo::g_tune.eltwise_tile_max},
-      {"eltwise_tile_min", &oslo::g_tune.eltwise_tile_min},
-      {"eltwise_unroll", &oslo::g_tune.eltwise_unroll},
-      {"eltwise_rowgroups", &oslo::g_tune.eltwise_rowgroups},
-      {"eltwise_fwd_steps", &oslo::g_tune.eltwise_fwd_steps},
-      {"norm_bwd_waves", &oslo::g_tune.norm_bwd_waves},
-      {"norm_fwd_waves", &oslo::g_tune.norm_fwd_waves},
-      {"norm_bwd_prefetch", &oslo::g_tune.norm_bwd_prefetch},
-      {"norm_fwd_iters", &oslo::g_tune.norm_fwd_iters},
-      {"adam_unroll", &oslo::g_tune.adam_unroll},
+      {"norm_fwd_vpl", &oslo::g_tune.norm_fwd_vpl, kPow2, 1, 8},
+      {"norm_bwd_vpl", &oslo::g_tune.norm_bwd_vpl, kPow2, 1, 4},
+      {"norm_bwd_blocks_per_cu", &oslo::g_tune.norm_bwd_blocks_per_cu, kRange, 1, 8},
+      {"softmax_rows_per_wave", &oslo::g_tune.softmax_rows_per_wave, kPow2, 1, 4},
+      {"softmax_lanes_per_row", &oslo::g_tune.softmax_lanes_per_row, kLanes, 1, 64},
+      {"softmax_fwd_elems", &oslo::g_tune.softmax_fwd_elems, kPow2, 16, 64},
+      {"norm_lanes_per_row", &oslo::g_tune.norm_lanes_per_row, kLanes, 8, 64},
+      {"eltwise_tile_max", &oslo::g_tune.eltwise_tile_max, kPow2, 1, 256},
+      {"eltwise_tile_min", &oslo::g_tune.eltwise_tile_min, kPow2, 1, 256},
+      {"eltwise_unroll", &oslo::g_tune.eltwise_unroll, kPow2, 1, 4},
+      {"eltwise_rowgroups", &oslo::g_tune.eltwise_rowgroups, kRange, 1, 4096},
+      {"eltwise_fwd_steps", &oslo::g_tune.eltwise_fwd_steps, kRange, 1, 64},
+      {"norm_bwd_waves", &oslo::g_tune.norm_bwd_waves, kRange, 1, 16},
+      {"norm_fwd_waves", &oslo::g_tune.norm_fwd_waves, kRange, 1, 16},
+      {"norm_bwd_prefetch", &oslo::g_tune.norm_bwd_prefetch, kRange, 1, 2},
+      {"norm_fwd_iters", &oslo::g_tune.norm_fwd_iters, kRange, 1, 16},
+      {"adam_unroll", &oslo::g_tune.adam_unroll, kPow2, 1, 4},
   };
   for (const Entry &e : table) {
     if (strcmp(e.name, key) == 0) {
+      bool ok = value == 0;
+      if (!ok && value >= e.lo && value <= e.hi) {
+        const bool pow2 = (value & (value - 1)) == 0;
+        ok = e.kind == kRange || (e.kind == kPow2 && pow2) ||
+             (e.kind == kLanes && (value == 1 || (pow2 && value >= 8)));
+      }
+      if (!ok)
+        return oslo::fail(OSLO_ERR_INVALID_ARGUMENT,
+                          "tune: %d is no valid value for '%s'", value, key);
       *e.slot = value;
       return OSLO_OK;
     }

@@ -1032,7 +1032,10 @@ static int launch_norm_fwd(const void *x, const void *gamma, const void *beta,
   // short rows side by side in a wave
   const int lpr = (sp.wpr == 1 && sp.vpl == 1) ? lanes_per_row(n2 / E) : kWave;
   if (lpr < kWave) {
-    const int rpb_eff = sp.rpb * (kWave / lpr);
+    // (these builds are bounded to 256 threads: at most four waves)
+    const int waves_l = sp.rpb < 4 ? sp.rpb : 4;
+    const int threads_l = kWave * waves_l;
+    const int rpb_eff = waves_l * (kWave / lpr);
     const bool even_l = (n2 / E) == lpr;
     int64_t grid_l = ceil_div(ceil_div(n1, rpb_eff), iters);
     if (grid_l > maxgrid) grid_l = maxgrid;
@@ -1042,12 +1045,12 @@ static int launch_norm_fwd(const void *x, const void *gamma, const void *beta,
   case LPR_:                                                                 \
     if (even_l)                                                              \
       norm_fwd_reg_kernel<T, V, 1, RMS, true, 256, true, LPR_>               \
-          <<<dim3((unsigned)grid_l), threads, 0, st>>>(                      \
+          <<<dim3((unsigned)grid_l), threads_l, 0, st>>>(                      \
               (const T *)x, (const V *)gamma, (const V *)beta, (V *)y, mean, \
               invvar, n1, (int)n2, eps, 1, rpb_eff, iters, *fp);             \
     else                                                                     \
       norm_fwd_reg_kernel<T, V, 1, RMS, false, 256, true, LPR_>              \
-          <<<dim3((unsigned)grid_l), threads, 0, st>>>(                      \
+          <<<dim3((unsigned)grid_l), threads_l, 0, st>>>(                      \
               (const T *)x, (const V *)gamma, (const V *)beta, (V *)y, mean, \
               invvar, n1, (int)n2, eps, 1, rpb_eff, iters, *fp);             \
     break;
@@ -1064,12 +1067,12 @@ static int launch_norm_fwd(const void *x, const void *gamma, const void *beta,
   case LPR_:                                                                 \
     if (even_l)                                                              \
       norm_fwd_reg_kernel<T, V, 1, RMS, true, 256, false, LPR_>              \
-          <<<dim3((unsigned)grid_l), threads, 0, st>>>(                      \
+          <<<dim3((unsigned)grid_l), threads_l, 0, st>>>(                      \
               (const T *)x, (const V *)gamma, (const V *)beta, (V *)y, mean, \
               invvar, n1, (int)n2, eps, 1, rpb_eff, iters, FusePrologue{});  \
     else                                                                     \
       norm_fwd_reg_kernel<T, V, 1, RMS, false, 256, false, LPR_>             \
-          <<<dim3((unsigned)grid_l), threads, 0, st>>>(                      \
+          <<<dim3((unsigned)grid_l), threads_l, 0, st>>>(                      \
               (const T *)x, (const V *)gamma, (const V *)beta, (V *)y, mean, \
               invvar, n1, (int)n2, eps, 1, rpb_eff, iters, FusePrologue{});  \
     break;

@@ -1222,7 +1222,8 @@ static int launch_softmax_fwd(const void *x, const uint8_t *mask, void *y,
       softmax_fwd_kernel<T, VPL, RPW, MODE, false, LPR_>             \
           <<<dim3((unsigned)grid), threads, 0, st>>>(                \
               (const T *)x, mask, (T *)y, nullptr, g, scale, d);     \
-  }
+  } else                                                             \
+    return fail(OSLO_ERR_UNSUPPORTED, "softmax fwd: no kernel for %d x %d chunks per lane", VPL, RPW)
   OSLO_SM_CASES(OSLO_SM_FWD)
 #undef OSLO_SM_FWD
   return check_launch("softmax_fwd_kernel");
@@ -1278,7 +1279,9 @@ static int launch_softmax_bwd(const void *dy, const void *y,
   if constexpr (VPL * RPW * E <= kBwdMaxElems)             \
     softmax_bwd_kernel<T, VPL, RPW, MODE, LPR_>            \
         <<<dim3((unsigned)grid), threads, 0, st>>>(        \
-            (const T *)dy, (const T *)y, mask, (T *)dx, g, scale)
+            (const T *)dy, (const T *)y, mask, (T *)dx, g, scale); \
+  else                                                     \
+    return fail(OSLO_ERR_UNSUPPORTED, "softmax bwd: no kernel for %d x %d chunks per lane", VPL, RPW)
   OSLO_SM_CASES(OSLO_SM_BWD)
 #undef OSLO_SM_BWD
   return check_launch("softmax_bwd_kernel");
@@ -1337,7 +1340,9 @@ static int launch_softmax_dropout_bwd(const void *dy, const void *x,
     softmax_dropout_bwd_kernel<T, VPL, RPW, MODE, LPR_>             \
         <<<dim3((unsigned)grid), threads, 0, st>>>(                 \
             (const T *)dy, (const T *)x, stats, mask, (T *)dx, g,   \
-            scale, d)
+            scale, d);                                              \
+  else                                                              \
+    return fail(OSLO_ERR_UNSUPPORTED, "softmax dropout bwd: no kernel for %d x %d chunks per lane", VPL, RPW)
   OSLO_SM_CASES(OSLO_SM_DBWD)
 #undef OSLO_SM_DBWD
   return check_launch("softmax_dropout_bwd_kernel");

@@ -58,6 +58,18 @@ def test_invalid_arguments_are_rejected_before_any_launch():
     assert rc == -1
     assert lib.oslo_tune(b"no_such_knob", 1) == -1
     assert lib.oslo_tune(b"norm_fwd_vpl", 0) == 0
+    # values without a kernel build or a valid workgroup shape are refused
+    for key, bad in ((b"norm_fwd_vpl", 3), (b"norm_bwd_vpl", 8), (b"norm_fwd_waves", 17),
+                     (b"norm_bwd_prefetch", 3), (b"softmax_rows_per_wave", 3),
+                     (b"softmax_lanes_per_row", 4), (b"norm_lanes_per_row", 1),
+                     (b"softmax_fwd_elems", 4), (b"eltwise_tile_max", 100),
+                     (b"eltwise_tile_min", 512), (b"eltwise_unroll", 3), (b"adam_unroll", 8),
+                     (b"norm_bwd_blocks_per_cu", -1)):
+        assert lib.oslo_tune(key, bad) == -1, key
+    assert lib.oslo_tune(b"eltwise_tile_max", 100) == -1 and b"no valid value" in lib.oslo_hip_last_error()
+    for key, good in ((b"norm_fwd_vpl", 8), (b"softmax_lanes_per_row", 1), (b"eltwise_tile_min", 64),
+                      (b"norm_bwd_waves", 16)):
+        assert lib.oslo_tune(key, good) == 0 and lib.oslo_tune(key, 0) == 0, key
     # empty problems succeed without touching any pointer
     assert lib.oslo_ln_fwd(None, None, None, None, None, None, 0, 8, 1e-5, 0, 0, None) == 0
     assert lib.oslo_bias_gelu_fwd(None, None, None, 0, 8, 2, None) == 0

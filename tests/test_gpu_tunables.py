@@ -1,0 +1,86 @@
+"""The launch-shape overrides of the softmax, element-wise and Adam kernels
+(oslo_tune) change how the work is split over lanes, waves and workgroups,
+never the result: every override runs the kernels against the float64 oracle
+with the tolerances of the default launch shapes."""
+import pytest
+import torch
+
+from oslo_amd.torch import _C
+from test_gpu_adam import test_multi_tensor_adam_vs_oracle as check_adam
+from test_gpu_adam import test_unaligned_views_and_many_tensors as check_adam_views
+from test_gpu_eltwise import test_bias_dropout_add as check_bias_dropout_add
+from test_gpu_eltwise import test_bias_gelu as check_bias_gelu
+from test_gpu_softmax import test_causal as check_causal
+from test_gpu_softmax import test_masked as check_masked
+from test_gpu_softmax_dropout import test_causal_dropout as check_causal_dropout
+from test_gpu_softmax_dropout import test_masked_dropout as check_masked_dropout
+
+pytestmark = pytest.mark.gpu
+
+F32, F16, BF16 = torch.float32, torch.float16, torch.bfloat16
+
+KEYS = [
+    "softmax_rows_per_wave", "softmax_lanes_per_row", "softmax_fwd_elems",
+    "eltwise_tile_max", "eltwise_tile_min", "eltwise_unroll", "eltwise_rowgroups", "eltwise_fwd_steps",
+    "adam_unroll",
+]
+
+
+@pytest.fixture
+def tuned():
+    yield
+    for key in KEYS:
+        _C.tune(key, 0)
+
+
+SOFTMAX_OVERRIDES = [
+    ("softmax_rows_per_wave", 1), ("softmax_rows_per_wave", 2), ("softmax_rows_per_wave", 4),
+    ("softmax_lanes_per_row", 1), ("softmax_lanes_per_row", 64),
+    ("softmax_fwd_elems", 16), ("softmax_fwd_elems", 32), ("softmax_fwd_elems", 64),
+]
+
+# (sq, sk, dtype): one to eight chunks per lane, one or several waves per row
+SOFTMAX_ROWS = [
+    (40, 128, BF16), (33, 256, F16), (21, 512, BF16), (19, 512, F32), (17, 768, F16),
+    (9, 1024, BF16), (7, 2048, F16), (5, 2048, F32), (5, 4096, BF16), (3, 8192, F16),
+]
+
+
+@pytest.mark.parametrize("key,value", SOFTMAX_OVERRIDES)
+@pytest.mark.parametrize("sq,sk,dtype", SOFTMAX_ROWS)
+def test_softmax_override_keeps_the_result(device, tuned, sq, sk, dtype, key, value):
+    _C.tune(key, value)
+    check_causal(device, 2, sq, sk, dtype, 0.25)
+    check_masked(device, 2, 2, sq, sk, dtype, 0.25, "padding")
+    check_causal_dropout(device, 2, sq, sk, dtype, 0.25, 0.2)
+    check_masked_dropout(device, 2, 2, sq, sk, dtype, 0.25, "full", 0.2)
+
+
+ELTWISE_OVERRIDES = [
+    ("eltwise_tile_max", 64), ("eltwise_tile_max", 8), ("eltwise_tile_max", 1),
+    ("eltwise_tile_min", 64), ("eltwise_tile_min", 256),
+    ("eltwise_unroll", 1), ("eltwise_unroll", 2), ("eltwise_unroll", 4),
+    ("eltwise_rowgroups", 1), ("eltwise_rowgroups", 7), ("eltwise_rowgroups", 1024),
+    ("eltwise_fwd_steps", 2), ("eltwise_fwd_steps", 5),
+]
+
+ELTWISE_SHAPES = [
+    (517, 64, BF16), (301, 3072, BF16), (67, 11008, F16), (1031, 16, BF16), (129, 96, F32),
+    (513, 36, F32), (64, 4096, BF16),
+]
+
+
+@pytest.mark.parametrize("key,value", ELTWISE_OVERRIDES)
+@pytest.mark.parametrize("rows,cols,dtype", ELTWISE_SHAPES)
+def test_eltwise_override_keeps_the_result(device, tuned, rows, cols, dtype, key, value):
+    _C.tune(key, value)
+    check_bias_gelu(device, rows, cols, dtype, True)
+    check_bias_dropout_add(device, rows, cols, dtype, 0.1, "bias+res")
+
+
+@pytest.mark.parametrize("unroll", [1, 2, 4])
+@pytest.mark.parametrize("dtype", [F32, BF16])
+def test_adam_override_keeps_the_result(device, tuned, dtype, unroll):
+    _C.tune("adam_unroll", unroll)
+    check_adam(device, dtype, 1, 1, 0.01)
+    check_adam_views(device)
