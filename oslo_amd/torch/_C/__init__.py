@@ -180,8 +180,33 @@ def _ptr(t):
     return None if t is None else t.data_ptr()
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def _stream(t):
+    """Handle of torch's current stream on the tensor's device."""
+    if _raw_stream is not None:
+        return _raw_stream(t.device.index)
     return torch.cuda.current_stream(t.device).cuda_stream
+
+
+class _SameDevice:
+    def __enter__(self):
+        return None
+
+    def __exit__(self, *exc):
+        return False
+
+
+_SAME_DEVICE = _SameDevice()
+
+
+def _device_of(t):
+    """Context that makes the tensor's device current; nothing to do (and
+    nothing allocated) when it already is."""
+    if t.device.index == torch.cuda.current_device():
+        return _SAME_DEVICE
+    return torch.cuda.device_of(t)
 
 
 def _dtype_code(t, what, allow_f64=False):
@@ -256,6 +281,9 @@ def tune(key, value):
 # ---------------------------------------------------------------------------
 def _compute_n1_n2(input, normalized_shape):
     # check_args / compute_n1_n2 of FusedLayerNormBinder.cpp:19-36, 59-93
+    if len(normalized_shape) == 1 and input.dim() >= 1 and input.shape[-1] == normalized_shape[0]:
+        n2 = int(normalized_shape[0])  # the common case, without building tuples
+        return (input.numel() // n2 if n2 > 0 else 0), n2
     normalized_shape = tuple(int(s) for s in normalized_shape)
     if len(normalized_shape) < 1:
         raise RuntimeError(
@@ -315,7 +343,7 @@ class _LayerNormKernel:
                         % (name, t.dtype, out_dtype)
                     )
         invvar = torch.empty(n1, dtype=_stat_dtype(input), device=input.device)
-        with torch.cuda.device_of(input):
+        with _device_of(input):
             if rms:
                 rc = lib.oslo_rms_fwd(
                     _ptr(input), _ptr(gamma), _ptr(output), _ptr(invvar),
@@ -385,7 +413,7 @@ class _LayerNormKernel:
             ws, ws_bytes = _workspace(
                 lib, OSLO_OP_RMS_BWD if rms else OSLO_OP_LN_BWD, n1, n2, input.device
             )
-        with torch.cuda.device_of(input):
+        with _device_of(input):
             if rms:
                 rc = lib.oslo_rms_bwd(
                     _ptr(dout), _ptr(input), _ptr(invvar), _ptr(gamma), _ptr(grad_input),
@@ -454,7 +482,7 @@ class _LayerNormKernel:
         h = torch.empty_like(input) if want_h else None
         invvar = torch.empty(n1, dtype=torch.float32, device=input.device)
         mean = None if rms else torch.empty(n1, dtype=torch.float32, device=input.device)
-        with torch.cuda.device_of(input):
+        with _device_of(input):
             rc = lib.oslo_bias_dropout_add_norm_fwd(
                 _ptr(input), _ptr(bias), _ptr(residual), _ptr(gamma), _ptr(beta), _ptr(h),
                 _ptr(y), _ptr(mean), _ptr(invvar), n1, n2, float(eps), float(p),
@@ -493,7 +521,7 @@ class _LayerNormKernel:
         ws, ws_bytes = None, 0
         if gamma is not None or need_bias_grad:
             ws, ws_bytes = _workspace(lib, OSLO_OP_BIAS_DROPOUT_ADD_NORM_BWD, n1, n2, h.device)
-        with torch.cuda.device_of(h):
+        with _device_of(h):
             rc = lib.oslo_bias_dropout_add_norm_bwd(
                 _ptr(dout), _ptr(dh_extra), _ptr(h), _ptr(mean), _ptr(invvar), _ptr(gamma),
                 _ptr(grad_res), _ptr(grad_in), _ptr(grad_gamma), _ptr(grad_beta),
@@ -547,7 +575,7 @@ class _SoftmaxKernel:
             )
         m8 = self._mask_u8(mask)
         out = torch.empty_like(input)
-        with torch.cuda.device_of(input):
+        with _device_of(input):
             rc = lib.oslo_softmax_masked_fwd(
                 _ptr(input), _ptr(m8), _ptr(out), b, np_, sq, sk, mb, msq,
                 float(scale_factor), _dtype_code(input, "input"), _stream(input),
@@ -574,7 +602,7 @@ class _SoftmaxKernel:
         # inplace=True overwrites output_grads, as the kernel this shim was
         # written for does
         grad_input = output_grads if inplace else torch.empty_like(output_grads)
-        with torch.cuda.device_of(output_grads):
+        with _device_of(output_grads):
             rc = lib.oslo_softmax_masked_bwd(
                 _ptr(output_grads), _ptr(softmax_results), _ptr(m8), _ptr(grad_input),
                 b, np_, sq, sk, mb, msq, float(scale_factor),
@@ -599,7 +627,7 @@ class _SoftmaxKernel:
         _check_input(input, "input")
         ab, sq, sk = input.shape
         out = torch.empty_like(input)
-        with torch.cuda.device_of(input):
+        with _device_of(input):
             rc = lib.oslo_softmax_causal_fwd(
                 _ptr(input), _ptr(out), ab, sq, sk, float(scale_factor),
                 _dtype_code(input, "input"), _stream(input),
@@ -619,7 +647,7 @@ class _SoftmaxKernel:
             raise RuntimeError("output_grads and softmax_results differ in dtype")
         ab, sq, sk = softmax_results.shape
         grad_input = output_grads if inplace else torch.empty_like(output_grads)
-        with torch.cuda.device_of(output_grads):
+        with _device_of(output_grads):
             rc = lib.oslo_softmax_causal_bwd(
                 _ptr(output_grads), _ptr(softmax_results), _ptr(grad_input), ab, sq, sk,
                 float(scale_factor), _dtype_code(output_grads, "output_grads"),
@@ -656,7 +684,7 @@ class _SoftmaxKernel:
         out = torch.empty_like(input)
         rows = input.numel() // input.shape[-1] if input.numel() else 0
         stats = torch.empty((rows, 2), dtype=torch.float32, device=input.device)
-        with torch.cuda.device_of(input):
+        with _device_of(input):
             if mask is None:
                 if input.dim() != 3:
                     raise RuntimeError("expected 3D tensor")
@@ -691,7 +719,7 @@ class _SoftmaxKernel:
         if stats.dtype != torch.float32 or stats.numel() != 2 * rows:
             raise RuntimeError("stats must be float32 [rows, 2]")
         grad_input = output_grads if inplace else torch.empty_like(output_grads)
-        with torch.cuda.device_of(input):
+        with _device_of(input):
             if mask is None:
                 if input.dim() != 3:
                     raise RuntimeError("expected 3D tensor")
@@ -743,7 +771,7 @@ class _FusedElementwiseKernel:
                 raise RuntimeError("bias and input differ in dtype")
         rows, cols = _rows_cols(input, bias)
         out = torch.empty_like(input)
-        with torch.cuda.device_of(input):
+        with _device_of(input):
             rc = lib.oslo_bias_gelu_fwd(
                 _ptr(input), _ptr(bias), _ptr(out), rows, cols,
                 _dtype_code(input, "input"), _stream(input),
@@ -764,7 +792,7 @@ class _FusedElementwiseKernel:
         if bias is not None and need_bias_grad:
             grad_bias = torch.empty_like(bias)
             ws, ws_bytes = _workspace(lib, OSLO_OP_BIAS_GELU_BWD, rows, cols, input.device)
-        with torch.cuda.device_of(input):
+        with _device_of(input):
             rc = lib.oslo_bias_gelu_bwd(
                 _ptr(grad_output), _ptr(input), _ptr(bias), _ptr(grad_input),
                 _ptr(grad_bias), _ptr(ws), ws_bytes, rows, cols,
@@ -793,7 +821,7 @@ class _FusedElementwiseKernel:
             if return_mask
             else None
         )
-        with torch.cuda.device_of(input):
+        with _device_of(input):
             rc = lib.oslo_bias_dropout_add_fwd(
                 _ptr(input), _ptr(bias), _ptr(residual), _ptr(out), _ptr(mask),
                 rows, cols, float(p), int(seed), int(offset),
@@ -819,7 +847,7 @@ class _FusedElementwiseKernel:
             )
         if grad_input is None and grad_bias is None:
             return None, None
-        with torch.cuda.device_of(grad_output):
+        with _device_of(grad_output):
             rc = lib.oslo_bias_dropout_add_bwd(
                 _ptr(grad_output), _ptr(grad_input), _ptr(grad_bias), _ptr(ws), ws_bytes,
                 rows, cols, float(p), int(seed), int(offset),
@@ -852,7 +880,7 @@ class _FusedElementwiseKernel:
     def copy_probe(self, src, dst):
         lib = self._lib
         nbytes = src.numel() * src.element_size()
-        with torch.cuda.device_of(src):
+        with _device_of(src):
             _check(lib.oslo_copy_probe(_ptr(src), _ptr(dst), nbytes, _stream(src)), lib)
         return dst
 
@@ -925,7 +953,7 @@ class _AdamKernel:
         arr = ctypes.c_void_p * n
         sizes = (ctypes.c_int64 * n)(*[t.numel() for t in ps])
         tables = [arr(*[t.data_ptr() for t in lst]) for lst in (gs, ps, ms, vs)]
-        with torch.cuda.device_of(ref):
+        with _device_of(ref):
             rc = lib.oslo_multi_tensor_adam(
                 tables[0], tables[1], tables[2], tables[3], sizes, n, float(lr), float(beta1),
                 float(beta2), float(epsilon), int(step), int(mode), int(bias_correction),

@@ -36,6 +36,17 @@ def _cast_if_autocast_enabled(*args):
     return tuple(cast(a) for a in args)
 
 
+def _apply_outside_autocast(function, *args):
+    """``function.apply`` on operands cast to the autocast dtype with autocast
+    switched off (functional.py:249-284 of the reference); without an active
+    autocast region neither step does anything and both are skipped."""
+    if not torch.is_autocast_enabled("cuda"):
+        return function.apply(*args)
+    args = _cast_if_autocast_enabled(*args)
+    with torch.amp.autocast("cuda", enabled=False):
+        return function.apply(*args)
+
+
 def _gelu_fwd_torch(x):
     # functional.py:23-25
     return x * 0.5 * (1.0 + torch.tanh(0.79788456 * x * (1 + 0.044715 * x * x)))
@@ -493,41 +504,29 @@ User Functions
 
 
 def fused_layer_norm_affine(input, weight, bias, normalized_shape, eps=1e-6):
-    args = _cast_if_autocast_enabled(input, weight, bias, normalized_shape, eps)
-    with torch.amp.autocast("cuda", enabled=False):
-        return _FusedLayerNormAffineFunction.apply(*args)
+    return _apply_outside_autocast(_FusedLayerNormAffineFunction, input, weight, bias, normalized_shape, eps)
 
 
 def fused_layer_norm(input, normalized_shape, eps=1e-6):
-    args = _cast_if_autocast_enabled(input, normalized_shape, eps)
-    with torch.amp.autocast("cuda", enabled=False):
-        return _FusedLayerNormFunction.apply(*args)
+    return _apply_outside_autocast(_FusedLayerNormFunction, input, normalized_shape, eps)
 
 
 def mixed_dtype_fused_layer_norm_affine(
     input, weight, bias, normalized_shape, eps=1e-6
 ):
-    args = _cast_if_autocast_enabled(input, weight, bias, normalized_shape, eps)
-    with torch.amp.autocast("cuda", enabled=False):
-        return _FusedLayerNormAffineMixedDtypesFunction.apply(*args)
+    return _apply_outside_autocast(_FusedLayerNormAffineMixedDtypesFunction, input, weight, bias, normalized_shape, eps)
 
 
 def fused_rms_norm_affine(input, weight, normalized_shape, eps=1e-6):
-    args = _cast_if_autocast_enabled(input, weight, normalized_shape, eps)
-    with torch.amp.autocast("cuda", enabled=False):
-        return _FusedRMSNormAffineFunction.apply(*args)
+    return _apply_outside_autocast(_FusedRMSNormAffineFunction, input, weight, normalized_shape, eps)
 
 
 def fused_rms_norm(input, normalized_shape, eps=1e-6):
-    args = _cast_if_autocast_enabled(input, normalized_shape, eps)
-    with torch.amp.autocast("cuda", enabled=False):
-        return _FusedRMSNormFunction.apply(*args)
+    return _apply_outside_autocast(_FusedRMSNormFunction, input, normalized_shape, eps)
 
 
 def mixed_dtype_fused_rms_norm_affine(input, weight, normalized_shape, eps=1e-6):
-    args = _cast_if_autocast_enabled(input, weight, normalized_shape, eps)
-    with torch.amp.autocast("cuda", enabled=False):
-        return _FusedRMSNormAffineMixedDtypesFunction.apply(*args)
+    return _apply_outside_autocast(_FusedRMSNormAffineMixedDtypesFunction, input, weight, normalized_shape, eps)
 
 
 def fused_gelu(x):
