@@ -2,6 +2,7 @@
 ``oslo/transformers/kernel_fusion_utils.py`` of the reference."""
 from oslo_amd.transformers.kernel_fusion_utils import (
     fused_attention_forward,
+    fused_bias_dropout_add_layer_norm,
     fused_layer_norm,
     fused_rms_norm,
     fused_scale_mask_softmax,
@@ -10,6 +11,7 @@ from oslo_amd.transformers.kernel_fusion_utils import (
 
 __all__ = [
     "fused_attention_forward",
+    "fused_bias_dropout_add_layer_norm",
     "fused_layer_norm",
     "fused_rms_norm",
     "fused_scale_mask_softmax",

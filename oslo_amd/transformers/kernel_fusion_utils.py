@@ -8,7 +8,13 @@ attention blocks run scale -> mask -> softmax -> dropout unfused
 ``fused_scale_mask_softmax`` routes a Hugging Face model's attention through
 ``FusedScaleMaskSoftmax`` (softmax and attention dropout in one kernel) by
 registering an attention function with the library's attention interface.
+The reference's post-LN output blocks chain ``FusedBiasDropout``, the residual
+add and ``nn.LayerNorm`` (``oslo/transformers/models/bert/modeling_bert.py:337-346,
+440-449``); ``fused_bias_dropout_add_layer_norm`` folds the three into the
+one-kernel op.
 """
+import inspect
+
 import torch
 import torch.nn as nn
 
@@ -54,6 +60,60 @@ def fused_layer_norm(model):
                 continue  # weight without bias: no fused counterpart
             module.__class__ = FusedLayerNorm
             n += 1
+    return n
+
+
+def _is_post_ln_output(module):
+    """``dense`` -> ``dropout`` -> ``LayerNorm(. + input_tensor)``: the shape of
+    BertSelfOutput / BertOutput (modeling_bert.py:337-346, 440-449) and of their
+    copies in the other post-LN encoders."""
+    ln = getattr(module, "LayerNorm", None)
+    if not (
+        isinstance(getattr(module, "dense", None), nn.Linear)
+        and isinstance(getattr(module, "dropout", None), nn.Dropout)
+        and isinstance(ln, (nn.LayerNorm, FusedLayerNorm))
+        and ln.elementwise_affine
+        and ln.bias is not None
+    ):
+        return False
+    try:
+        names = list(inspect.signature(type(module).forward).parameters)
+    except (TypeError, ValueError):
+        return False
+    return names == ["self", "hidden_states", "input_tensor"]
+
+
+def _post_ln_output_forward(self, hidden_states, input_tensor):
+    # the dense layer's bias travels to the fused op (skip_bias_add of the
+    # reference's linear.py:31-35): bias add, dropout, residual add and
+    # LayerNorm are one kernel
+    ln = self.LayerNorm
+    out = nn.functional.linear(hidden_states, self.dense.weight)
+    return onn_f.fused_bias_dropout_add_layer_norm(
+        out, self.dense.bias, input_tensor, ln.weight, ln.bias, ln.normalized_shape,
+        ln.eps, self.dropout.p, self.training,
+    )
+
+
+_POST_LN_CLASSES = {}
+
+
+def fused_bias_dropout_add_layer_norm(model):
+    """Gives every post-LN output block of ``model`` (dense, dropout, residual
+    add, LayerNorm) a forward that runs bias add, dropout, residual add and
+    LayerNorm in one kernel; the parameters stay where they are.  Returns the
+    number of blocks changed."""
+    n = 0
+    for module in model.modules():
+        cls = type(module)
+        if cls in _POST_LN_CLASSES.values() or not _is_post_ln_output(module):
+            continue
+        if cls not in _POST_LN_CLASSES:
+            _POST_LN_CLASSES[cls] = type(
+                "Fused" + cls.__name__, (cls,), {"forward": _post_ln_output_forward}
+            )
+        module.__class__ = _POST_LN_CLASSES[cls]
+        n += 1
     return n
 
 
