@@ -3,6 +3,7 @@
 from oslo_amd.transformers.kernel_fusion_utils import (
     fused_attention_forward,
     fused_bias_dropout_add_layer_norm,
+    fused_bias_gelu,
     fused_layer_norm,
     fused_rms_norm,
     fused_scale_mask_softmax,
@@ -12,6 +13,7 @@ from oslo_amd.transformers.kernel_fusion_utils import (
 __all__ = [
     "fused_attention_forward",
     "fused_bias_dropout_add_layer_norm",
+    "fused_bias_gelu",
     "fused_layer_norm",
     "fused_rms_norm",
     "fused_scale_mask_softmax",

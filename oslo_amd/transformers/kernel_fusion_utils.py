@@ -117,6 +117,125 @@ def fused_bias_dropout_add_layer_norm(model):
     return n
 
 
+def _is_tanh_gelu(act):
+    """True when ``act`` computes the tanh form of GeLU the fused kernel
+    evaluates (functional.py:23-25 of the reference; "gelu_new",
+    "gelu_pytorch_tanh", "gelu_fast" in Hugging Face's table), decided by its
+    values, not by its name."""
+    probe = torch.linspace(-6.0, 6.0, 97)
+    try:
+        out = act(probe)
+    except Exception:
+        return False
+    want = 0.5 * probe * (1.0 + torch.tanh(0.79788456 * probe * (1.0 + 0.044715 * probe * probe)))
+    return (
+        isinstance(out, torch.Tensor)
+        and out.shape == probe.shape
+        and torch.allclose(out.float(), want, atol=2e-6, rtol=0.0)
+    )
+
+
+def _is_projection(layer):
+    # nn.Linear, or transformers' Conv1D (weight stored [in, out], ``nf`` outputs)
+    return isinstance(layer, nn.Linear) or (
+        hasattr(layer, "nf") and isinstance(getattr(layer, "weight", None), nn.Parameter)
+        and layer.weight.dim() == 2
+    )
+
+
+def _project_gelu(layer, x):
+    """gelu(x W + b) with the bias add inside the GeLU kernel."""
+    if isinstance(layer, nn.Linear):
+        out = nn.functional.linear(x, layer.weight)
+    else:
+        out = torch.mm(x.reshape(-1, x.size(-1)), layer.weight).view(x.size()[:-1] + (layer.nf,))
+    if layer.bias is None:
+        return onn_f.fused_gelu(out)
+    return onn_f.fused_bias_gelu(out, layer.bias)
+
+
+# (up projection, down projection or None, activation): GPT-2 / GPT-Neo MLP,
+# GPT-J MLP, BERT-style intermediate block
+_MLP_SHAPES = (
+    ("c_fc", "c_proj", "act"),
+    ("fc_in", "fc_out", "act"),
+    ("dense", None, "intermediate_act_fn"),
+)
+
+
+def _mlp_shape(module):
+    try:
+        names = list(inspect.signature(type(module).forward).parameters)
+    except (TypeError, ValueError):
+        return None
+    if names != ["self", "hidden_states"]:
+        return None
+    children = dict(module.named_children())
+    for up, down, act in _MLP_SHAPES:
+        expected = {up} | ({down, "dropout"} if down else set())
+        others = set(children) - expected - {act}
+        if others or not expected <= set(children):
+            continue
+        if not _is_projection(children[up]) or (down and not _is_projection(children[down])):
+            continue
+        if down and not isinstance(children["dropout"], nn.Dropout):
+            continue
+        fn = getattr(module, act, None)
+        if callable(fn) and _is_tanh_gelu(fn):
+            return up, down
+    return None
+
+
+def _mlp_forward(self, hidden_states):
+    up, down = self._oslo_mlp_shape
+    h = _project_gelu(getattr(self, up), hidden_states)
+    if down is None:
+        return h
+    return self.dropout(getattr(self, down)(h))
+
+
+_MLP_CLASSES = {}
+
+
+def fused_bias_gelu(model):
+    """Gives every MLP (or BERT-style intermediate) block of ``model`` whose
+    activation is the tanh form of GeLU a forward that adds the up projection's
+    bias inside the GeLU kernel (the reference's ``fused_bias_gelu`` over a
+    ``skip_bias_add`` linear, linear.py:31-35).  A block is changed only if its
+    new forward reproduces the old one on a probe input.  Returns the number
+    of blocks changed."""
+    n = 0
+    for module in model.modules():
+        cls = type(module)
+        if cls in _MLP_CLASSES.values():
+            continue
+        shape = _mlp_shape(module)
+        if shape is None:
+            continue
+        if cls not in _MLP_CLASSES:
+            _MLP_CLASSES[cls] = type("Fused" + cls.__name__, (cls,), {"forward": _mlp_forward})
+        up = getattr(module, shape[0])
+        in_features = up.in_features if isinstance(up, nn.Linear) else up.weight.size(0)
+        probe = torch.linspace(-2.0, 2.0, 3 * in_features, device=up.weight.device)
+        probe = probe.view(3, in_features).to(up.weight.dtype)
+        was_training = module.training
+        module.eval()
+        with torch.no_grad():
+            want = module(probe)
+            module._oslo_mlp_shape = shape
+            module.__class__ = _MLP_CLASSES[cls]
+            got = module(probe)
+        module.train(was_training)
+        tol = 1e-4 if want.dtype == torch.float32 else 3e-2
+        scale = want.float().abs().max().item() + 1e-6
+        if (got.float() - want.float()).abs().max().item() > tol * scale:
+            module.__class__ = cls  # not the chain it looked like: leave it alone
+            del module._oslo_mlp_shape
+            continue
+        n += 1
+    return n
+
+
 def _repeat_kv(hidden_states, n_rep):
     if n_rep == 1:
         return hidden_states

@@ -299,3 +299,59 @@ def test_bert_post_ln_dropout_draws_from_the_generator(device):
     d = m(ids, attention_mask=am).last_hidden_state
     e = m(ids, attention_mask=am).last_hidden_state
     assert torch.equal(d, e)
+
+
+def test_bias_gelu_swap_on_cpu_keeps_the_model_output():
+    from oslo_amd.transformers import fused_bias_gelu
+
+    m = tiny_gpt2().eval()  # activation "gelu_new": the tanh form
+    ids, am = inputs()
+    ref = m(ids).logits
+    assert fused_bias_gelu(m) == 2 and fused_bias_gelu(m) == 0
+    assert type(m.transformer.h[0].mlp).__name__ == "FusedGPT2MLP"
+    assert torch.allclose(m(ids).logits, ref, atol=1e-5, rtol=1e-5)
+    # the erf form of GeLU is another function: such blocks stay as they are
+    assert fused_bias_gelu(tiny_bert()) == 0
+    b = tiny_bert(hidden_act="gelu_new").eval()
+    ref = b(ids, attention_mask=am).last_hidden_state
+    assert fused_bias_gelu(b) == 2
+    assert torch.allclose(b(ids, attention_mask=am).last_hidden_state, ref, atol=1e-5, rtol=1e-5)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_gpt2_with_every_swap_outputs_and_gradients(device, dtype, monkeypatch):
+    from oslo_amd.torch import _C
+    from oslo_amd.transformers import fused_bias_gelu
+
+    ids, am = inputs(b=3, s=32)
+    ids, am = ids.to(device), am.to(device)
+    kw = dict(attn_pdrop=0.0, resid_pdrop=0.0, embd_pdrop=0.0)
+    ref = tiny_gpt2(seed=3, **kw).to(device).to(dtype).train()
+    fused = tiny_gpt2(seed=3, **kw).to(device).to(dtype).train()
+    assert fused_bias_gelu(fused) == 2
+    fused_layer_norm(fused)
+    fused_scale_mask_softmax(fused)
+    kernel = _C.get_fused_elementwise_kernel()
+    calls = []
+    fwd = kernel.bias_gelu_forward
+
+    def counted(*a, **k):
+        calls.append(1)
+        return fwd(*a, **k)
+
+    monkeypatch.setattr(kernel, "bias_gelu_forward", counted)
+    lr = ref(ids, attention_mask=am, labels=ids).loss
+    lf = fused(ids, attention_mask=am, labels=ids).loss
+    assert len(calls) == 2  # one bias-GeLU kernel per block
+    assert abs(lr.item() - lf.item()) <= (1e-4 if dtype == torch.float32 else 3e-2)
+    lr.backward()
+    lf.backward()
+    gtol = 2e-3 if dtype == torch.float32 else 8e-2
+    gmax = max(p.grad.float().abs().max().item() for p in ref.parameters() if p.grad is not None)
+    floor = 1e-8 if dtype == torch.float32 else 1e-3 * gmax
+    for (n, pr), (_, pf) in zip(ref.named_parameters(), fused.named_parameters()):
+        if pr.grad is None:
+            continue
+        scale = pr.grad.float().abs().max().item() + floor
+        assert (pr.grad.float() - pf.grad.float()).abs().max().item() <= gtol * scale + 1e-6, n
