@@ -6,7 +6,9 @@ Parity metrics (the tolerances the tests state):
   16-bit outputs (1) against the float64 oracle rounded once to the storage
                  type: at least 99.8 % of the elements bit-identical and no
                  element further than 1 ulp; (2) relative L2 error against the
-                 unrounded float64 oracle <= 2e-3.
+                 unrounded float64 oracle <= 2e-3, or what the correctly
+                 rounded oracle itself reaches where that is more (values that
+                 crowd just above a power of two: up to 2.3e-3 in bf16).
                  (A per-element 2e-3 bound is not meaningful for bf16, whose
                  half-ulp is 3.9e-3: two correct roundings of values 1e-7
                  apart can differ by a full ulp.)
@@ -71,6 +73,11 @@ def check_lowp(actual, truth64, what, min_exact=0.998, max_ulp=1, l2_tol=2e-3, a
     # the L2 bound presumes enough elements to average over; a handful of
     # values can each sit at the half-ulp worst case (2^-9 for bf16)
     l2_bound = l2_tol if actual.numel() >= 256 else 2 * l2_tol
+    # values that crowd just above a power of two (a near-uniform softmax row of
+    # 1024 keys: every probability ~ 2^-10) carry the largest relative rounding
+    # error of the storage type, 2.3e-3 rms in bf16: the bound is never tighter
+    # than what the correctly rounded oracle itself achieves
+    l2_bound = max(l2_bound, 1.02 * rel_l2(f64(expect), truth64))
     assert worst <= max_ulp, "%s: %d ulp off the rounded oracle (exact %.5f)" % (what, worst, exact)
     # a small tensor may hold a few values that sit on a rounding tie
     allowed = max(3.0, (1.0 - min_exact) * actual.numel()) if min_exact < 1.0 else 0.0
