@@ -5,6 +5,7 @@ from oslo_amd.transformers.kernel_fusion_utils import (
     fused_bias_dropout_add_layer_norm,
     fused_bias_gelu,
     fused_layer_norm,
+    fused_pre_ln_block,
     fused_rms_norm,
     fused_scale_mask_softmax,
     register_fused_attention,
@@ -15,6 +16,7 @@ __all__ = [
     "fused_bias_dropout_add_layer_norm",
     "fused_bias_gelu",
     "fused_layer_norm",
+    "fused_pre_ln_block",
     "fused_rms_norm",
     "fused_scale_mask_softmax",
     "register_fused_attention",

@@ -145,10 +145,7 @@ def _is_projection(layer):
 
 def _project_gelu(layer, x):
     """gelu(x W + b) with the bias add inside the GeLU kernel."""
-    if isinstance(layer, nn.Linear):
-        out = nn.functional.linear(x, layer.weight)
-    else:
-        out = torch.mm(x.reshape(-1, x.size(-1)), layer.weight).view(x.size()[:-1] + (layer.nf,))
+    out = _project_no_bias(layer, x)
     if layer.bias is None:
         return onn_f.fused_gelu(out)
     return onn_f.fused_bias_gelu(out, layer.bias)
@@ -232,6 +229,121 @@ def fused_bias_gelu(model):
             module.__class__ = cls  # not the chain it looked like: leave it alone
             del module._oslo_mlp_shape
             continue
+        n += 1
+    return n
+
+
+def _project_no_bias(layer, x):
+    if isinstance(layer, nn.Linear):
+        return nn.functional.linear(x, layer.weight)
+    return torch.mm(x.reshape(-1, x.size(-1)), layer.weight).view(x.size()[:-1] + (layer.nf,))
+
+
+def _no_bias_forward(self, x):
+    return _project_no_bias(self, x)
+
+
+def _identity_forward(self, x):
+    return x
+
+
+_HELPER_CLASSES = {}
+
+
+def _swap_forward(module, suffix, forward):
+    """Rewrites the module's class to a subclass with another forward: the
+    parameters, buffers and state-dict keys stay what they were."""
+    cls = type(module)
+    key = (cls, suffix)
+    if key not in _HELPER_CLASSES:
+        _HELPER_CLASSES[key] = type(cls.__name__ + suffix, (cls,), {"forward": forward})
+    module.__class__ = _HELPER_CLASSES[key]
+    return cls
+
+
+def _is_pre_ln_block(module):
+    """ln_1 -> attn (c_proj, resid_dropout) -> +residual -> ln_2 -> mlp (c_proj,
+    dropout) -> +residual: the GPT-2 block (modeling_gpt2.py:355-400 of the
+    reference), without cross-attention."""
+    attn, mlp = getattr(module, "attn", None), getattr(module, "mlp", None)
+    ln2 = getattr(module, "ln_2", None)
+    return (
+        attn is not None and mlp is not None
+        and isinstance(getattr(module, "ln_1", None), (nn.LayerNorm, FusedLayerNorm))
+        and isinstance(ln2, (nn.LayerNorm, FusedLayerNorm))
+        and ln2.elementwise_affine and ln2.bias is not None
+        and not hasattr(module, "crossattention")
+        and _is_projection(getattr(attn, "c_proj", None))
+        and isinstance(getattr(attn, "resid_dropout", None), nn.Dropout)
+        and _is_projection(getattr(mlp, "c_proj", None))
+        and isinstance(getattr(mlp, "dropout", None), nn.Dropout)
+        and attn.c_proj.bias is not None and mlp.c_proj.bias is not None
+    )
+
+
+def _pre_ln_block_forward(self, hidden_states, *args, **kwargs):
+    # attn and mlp return their raw output projections (bias and dropout
+    # switched off inside them); both bias-dropout-residual steps run fused:
+    # the first one together with ln_2, its sum carried on as the residual
+    if kwargs.get("encoder_hidden_states") is not None:
+        raise ValueError("the fused GPT-2 block has no cross-attention")
+    attn_out = self.attn(self.ln_1(hidden_states), *args, **kwargs)
+    attn_out = attn_out[0] if isinstance(attn_out, tuple) else attn_out
+    ln2 = self.ln_2
+    normed, summed = onn_f.fused_bias_dropout_add_layer_norm(
+        attn_out, self.attn.c_proj.bias, hidden_states, ln2.weight, ln2.bias,
+        ln2.normalized_shape, ln2.eps, self.attn.resid_dropout.p, self.training, True,
+    )
+    mlp_out = self.mlp(normed)
+    return onn_f.fused_bias_dropout_add(
+        mlp_out, self.mlp.c_proj.bias, summed, self.mlp.dropout.p, self.training
+    )
+
+
+def fused_pre_ln_block(model):
+    """Gives every GPT-2 style pre-LN block of ``model`` a forward in which
+    ``dropout(attn_out + bias) + residual`` runs inside the LayerNorm kernel of
+    ``ln_2`` and ``dropout(mlp_out + bias) + residual`` as one kernel
+    (the residual adds of modeling_gpt2.py:369, 396 of the reference folded into
+    its ``FusedBiasDropout``).  A block is changed only if the new forward
+    reproduces the old one on a probe input.  Returns the number of blocks
+    changed."""
+    n = 0
+    for module in model.modules():
+        if getattr(module, "_oslo_pre_ln", False) or not _is_pre_ln_block(module):
+            continue
+        width = module.ln_2.normalized_shape[0]
+        w = module.ln_2.weight
+        probe = torch.linspace(-1.5, 1.5, 2 * 5 * width, device=w.device).view(2, 5, width).to(w.dtype)
+        was_training = module.training
+        module.eval()
+        parts = (module, module.attn.c_proj, module.attn.resid_dropout, module.mlp.c_proj,
+                 module.mlp.dropout)
+        old = None
+        try:
+            with torch.no_grad():
+                want = module(probe)
+                want = want[0] if isinstance(want, tuple) else want
+                old = [
+                    _swap_forward(parts[0], "FusedResiduals", _pre_ln_block_forward),
+                    _swap_forward(parts[1], "NoBias", _no_bias_forward),
+                    _swap_forward(parts[2], "Off", _identity_forward),
+                    _swap_forward(parts[3], "NoBias", _no_bias_forward),
+                    _swap_forward(parts[4], "Off", _identity_forward),
+                ]
+                got = module(probe)
+            tol = 1e-4 if want.dtype == torch.float32 else 3e-2
+            scale = want.float().abs().max().item() + 1e-6
+            ok = got.shape == want.shape and (got.float() - want.float()).abs().max().item() <= tol * scale
+        except Exception:
+            ok = False
+        module.train(was_training)
+        if not ok:
+            if old:  # not the chain it looked like: put everything back
+                for part, cls in zip(parts, old):
+                    part.__class__ = cls
+            continue
+        module._oslo_pre_ln = True
         n += 1
     return n
 

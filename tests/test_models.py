@@ -355,3 +355,84 @@ def test_gpt2_with_every_swap_outputs_and_gradients(device, dtype, monkeypatch):
             continue
         scale = pr.grad.float().abs().max().item() + floor
         assert (pr.grad.float() - pf.grad.float()).abs().max().item() <= gtol * scale + 1e-6, n
+
+
+def test_pre_ln_block_swap_on_cpu_keeps_the_model_output():
+    from oslo_amd.transformers import fused_bias_gelu, fused_pre_ln_block
+
+    ids, am = inputs()
+    for gelu_first in (False, True):
+        m = tiny_gpt2().eval()
+        ref, ref_padded = m(ids).logits, m(ids, attention_mask=am).logits
+        keys = list(m.state_dict())
+        if gelu_first:
+            assert fused_bias_gelu(m) == 2
+        assert fused_pre_ln_block(m) == 2 and fused_pre_ln_block(m) == 0
+        if not gelu_first:
+            assert fused_bias_gelu(m) == 2
+        assert list(m.state_dict()) == keys  # checkpoints keep loading
+        assert torch.allclose(m(ids).logits, ref, atol=1e-5, rtol=1e-5)
+        valid = am.bool()
+        assert torch.allclose(m(ids, attention_mask=am).logits[valid], ref_padded[valid], atol=1e-5, rtol=1e-5)
+        gen = m.generate(ids[:1, :8], max_new_tokens=4, do_sample=False)
+        assert gen.shape == (1, 12)
+    assert fused_pre_ln_block(tiny_bert()) == 0  # post-LN blocks are another shape
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_gpt2_pre_ln_blocks_through_the_fused_kernels(device, dtype, monkeypatch):
+    from oslo_amd.torch import _C
+    from oslo_amd.transformers import fused_bias_gelu, fused_pre_ln_block
+
+    ids, am = inputs(b=3, s=32)
+    ids, am = ids.to(device), am.to(device)
+    kw = dict(attn_pdrop=0.0, resid_pdrop=0.0, embd_pdrop=0.0)
+    ref = tiny_gpt2(seed=3, **kw).to(device).to(dtype).train()
+    fused = tiny_gpt2(seed=3, **kw).to(device).to(dtype).train()
+    assert fused_pre_ln_block(fused) == 2
+    fused_bias_gelu(fused)
+    fused_layer_norm(fused)
+    fused_scale_mask_softmax(fused)
+    norm_kernel, elt_kernel = _C.get_layernorm_kernel(), _C.get_fused_elementwise_kernel()
+    calls = []
+    norm_fwd, bda_fwd = norm_kernel.bias_dropout_add_norm_forward, elt_kernel.bias_dropout_add_forward
+    monkeypatch.setattr(norm_kernel, "bias_dropout_add_norm_forward",
+                        lambda *a, **k: (calls.append("norm"), norm_fwd(*a, **k))[1])
+    monkeypatch.setattr(elt_kernel, "bias_dropout_add_forward",
+                        lambda *a, **k: (calls.append("bda"), bda_fwd(*a, **k))[1])
+    lr = ref(ids, attention_mask=am, labels=ids).loss
+    lf = fused(ids, attention_mask=am, labels=ids).loss
+    assert calls == ["norm", "bda"] * 2  # per block: residual add inside ln_2, then the MLP's
+    assert abs(lr.item() - lf.item()) <= (1e-4 if dtype == torch.float32 else 3e-2)
+    lr.backward()
+    lf.backward()
+    gtol = 2e-3 if dtype == torch.float32 else 8e-2
+    gmax = max(p.grad.float().abs().max().item() for p in ref.parameters() if p.grad is not None)
+    floor = 1e-8 if dtype == torch.float32 else 1e-3 * gmax
+    for (n, pr), (_, pf) in zip(ref.named_parameters(), fused.named_parameters()):
+        if pr.grad is None:
+            continue
+        scale = pr.grad.float().abs().max().item() + floor
+        assert (pr.grad.float() - pf.grad.float()).abs().max().item() <= gtol * scale + 1e-6, n
+
+
+@pytest.mark.gpu
+def test_gpt2_pre_ln_residual_dropout_draws_from_the_generator(device):
+    from oslo_amd.transformers import fused_pre_ln_block
+
+    m = tiny_gpt2(attn_pdrop=0.0, resid_pdrop=0.3, embd_pdrop=0.0).to(device).train()
+    assert fused_pre_ln_block(m) == 2
+    ids, _ = inputs()
+    ids = ids.to(device)
+    gen = torch.cuda.default_generators[torch.device(device).index or 0]
+    torch.manual_seed(7)
+    off = gen.get_offset()
+    a = m(ids).logits
+    assert gen.get_offset() == off + 4 * 4  # two fused dropouts per block
+    torch.manual_seed(7)
+    b = m(ids).logits
+    assert torch.equal(a, b)
+    assert not torch.equal(a, m(ids).logits)
+    m.eval()
+    assert torch.equal(m(ids).logits, m(ids).logits)
