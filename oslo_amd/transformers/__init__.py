@@ -1,6 +1,7 @@
 """Model-level helpers that put the fused ops into existing models, mirroring
 ``oslo/transformers/kernel_fusion_utils.py`` of the reference."""
 from oslo_amd.transformers.kernel_fusion_utils import (
+    fuse_all,
     fused_attention_forward,
     fused_bias_dropout_add_layer_norm,
     fused_bias_gelu,
@@ -12,6 +13,7 @@ from oslo_amd.transformers.kernel_fusion_utils import (
 )
 
 __all__ = [
+    "fuse_all",
     "fused_attention_forward",
     "fused_bias_dropout_add_layer_norm",
     "fused_bias_gelu",

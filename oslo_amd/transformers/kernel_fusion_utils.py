@@ -438,3 +438,24 @@ def fused_scale_mask_softmax(model, name=ATTENTION_NAME):
     else:
         model.config._attn_implementation = name
     return model
+
+
+def fuse_all(model, attention=True):
+    """Applies every swap of this module that fits ``model``; returns how many
+    modules each one changed (``attention`` is True/False: the attention
+    function is a property of the whole model)."""
+    changed = {
+        "fused_pre_ln_block": fused_pre_ln_block(model),
+        "fused_bias_dropout_add_layer_norm": fused_bias_dropout_add_layer_norm(model),
+        "fused_bias_gelu": fused_bias_gelu(model),
+        "fused_layer_norm": fused_layer_norm(model),
+        "fused_rms_norm": fused_rms_norm(model),
+        "fused_scale_mask_softmax": False,
+    }
+    if attention and hasattr(model, "config"):
+        try:
+            fused_scale_mask_softmax(model)
+            changed["fused_scale_mask_softmax"] = True
+        except (ImportError, ValueError):
+            pass  # no pluggable attention in this model / library version
+    return changed

@@ -436,3 +436,23 @@ def test_gpt2_pre_ln_residual_dropout_draws_from_the_generator(device):
     assert not torch.equal(a, m(ids).logits)
     m.eval()
     assert torch.equal(m(ids).logits, m(ids).logits)
+
+
+def test_fuse_all_on_cpu():
+    from oslo_amd.transformers import fuse_all
+
+    ids, am = inputs()
+    m = tiny_gpt2().eval()
+    ref = m(ids, attention_mask=am).logits
+    assert fuse_all(m) == {
+        "fused_pre_ln_block": 2, "fused_bias_dropout_add_layer_norm": 0, "fused_bias_gelu": 2,
+        "fused_layer_norm": 5, "fused_rms_norm": 0, "fused_scale_mask_softmax": True,
+    }
+    valid = am.bool()
+    assert torch.allclose(m(ids, attention_mask=am).logits[valid], ref[valid], atol=1e-5, rtol=1e-5)
+    b = tiny_bert().eval()
+    ref = b(ids, attention_mask=am).last_hidden_state
+    changed = fuse_all(b)
+    assert changed["fused_bias_dropout_add_layer_norm"] == 4 and changed["fused_layer_norm"] == 5
+    assert changed["fused_pre_ln_block"] == 0 and changed["fused_bias_gelu"] == 0
+    assert torch.allclose(b(ids, attention_mask=am).last_hidden_state[valid], ref[valid], atol=1e-5, rtol=1e-5)
