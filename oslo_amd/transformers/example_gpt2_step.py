@@ -48,12 +48,13 @@ def main():
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--vocab", type=int, default=8192)
     ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--only", choices=["eager", "sdpa", "fused"], help="time one variant only")
     args = ap.parse_args()
     from oslo_amd.transformers import fuse_all
 
     ids = torch.randint(0, args.vocab, (args.batch, args.seq), device="cuda:0")
     tokens = args.batch * args.seq
-    for name in ("eager", "sdpa", "fused"):
+    for name in ([args.only] if args.only else ["eager", "sdpa", "fused"]):
         model = build(args, "eager" if name == "fused" else name)
         if name == "fused":
             print("swaps:", fuse_all(model))
