@@ -57,6 +57,5 @@ def test_override_keeps_the_result(device, tuned, n1, n2, tin, tout, key, value)
     _C.tune(key, value)
     check_layer_norm(device, n1, n2, tin, tout, True)
     check_rms_norm(device, n1, n2, tin, tout, True)
-    if tin == tout:  # the bias-dropout-add prologue / epilogue builds
-        check_fused(device, n1, n2, tin, 0.1, False)
-        check_fused(device, n1, n2, tin, 0.1, True)
+    if tin == tout:  # the bias-dropout-add prologue / epilogue builds (LayerNorm or RMSNorm by shape)
+        check_fused(device, n1, n2, tin, 0.1, n1 % 2 == 0)
