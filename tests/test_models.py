@@ -456,3 +456,49 @@ def test_fuse_all_on_cpu():
     assert changed["fused_bias_dropout_add_layer_norm"] == 4 and changed["fused_layer_norm"] == 5
     assert changed["fused_pre_ln_block"] == 0 and changed["fused_bias_gelu"] == 0
     assert torch.allclose(b(ids, attention_mask=am).last_hidden_state[valid], ref[valid], atol=1e-5, rtol=1e-5)
+
+
+def tiny_t5(seed=0):
+    from transformers import T5Config, T5ForConditionalGeneration
+
+    cfg = T5Config(d_model=128, d_kv=32, d_ff=256, num_layers=2, num_decoder_layers=2, num_heads=4,
+                   vocab_size=211, decoder_start_token_id=0, pad_token_id=0, dropout_rate=0.0)
+    torch.manual_seed(seed)
+    return T5ForConditionalGeneration(cfg)
+
+
+def t5_inputs(seed=1):
+    g = torch.Generator().manual_seed(seed)
+    return torch.randint(1, 211, (3, 24), generator=g), torch.randint(1, 211, (3, 10), generator=g)
+
+
+def test_t5_rms_norm_swap_on_cpu_keeps_the_model_output():
+    # the swap the reference ships (kernel_fusion_utils.py:71-87), on a whole model
+    m = tiny_t5().eval()
+    ids, labels = t5_inputs()
+    ref = m(input_ids=ids, labels=labels).logits
+    assert fused_rms_norm(m) == 12  # encoder 2 x 2 + 1, decoder 2 x 3 + 1
+    assert torch.allclose(m(input_ids=ids, labels=labels).logits, ref, atol=1e-5, rtol=1e-5)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_t5_through_the_fused_rms_norm(device, dtype):
+    ids, labels = t5_inputs()
+    ids, labels = ids.to(device), labels.to(device)
+    ref = tiny_t5(seed=2).to(device).to(dtype).train()
+    fused = tiny_t5(seed=2).to(device).to(dtype).train()
+    assert fused_rms_norm(fused) == 12
+    lr = ref(input_ids=ids, labels=labels).loss
+    lf = fused(input_ids=ids, labels=labels).loss
+    assert abs(lr.item() - lf.item()) <= (1e-4 if dtype == torch.float32 else 5e-2)
+    lr.backward()
+    lf.backward()
+    gtol = 2e-3 if dtype == torch.float32 else 1e-1
+    gmax = max(p.grad.float().abs().max().item() for p in ref.parameters() if p.grad is not None)
+    floor = 1e-8 if dtype == torch.float32 else 2e-3 * gmax
+    for (n, pr), (_, pf) in zip(ref.named_parameters(), fused.named_parameters()):
+        if pr.grad is None:
+            continue
+        scale = pr.grad.float().abs().max().item() + floor
+        assert (pr.grad.float() - pf.grad.float()).abs().max().item() <= gtol * scale + 1e-6, n
