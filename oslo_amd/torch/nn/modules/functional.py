@@ -8,7 +8,7 @@ reference evaluates there (its TorchScript bodies ``:23-50, 295-298`` and the
 module fallbacks ``layer_norm.py:17-30, 452-455``).
 """
 import torch
-from torch import Tensor
+from torch import Tensor  # noqa: F401  (named by the type comment of fused_bias_dropout)
 from torch.nn import functional as F
 
 from oslo_amd.torch._C import (

@@ -10,7 +10,6 @@ the norm's parameters and take the dense layer's ``(out, bias)`` pair
 import numbers
 
 import torch
-import torch.nn as nn
 from torch.nn import Parameter, init
 from torch.nn.modules.dropout import _DropoutNd
 

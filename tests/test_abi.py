@@ -1,7 +1,6 @@
 """The C-ABI library loads on a machine without a GPU and exports every symbol
 that include/oslo_hip.h declares; argument validation that needs no device is
 exercised too (no kernel is launched here)."""
-import ctypes
 import os
 import re
 

@@ -1,6 +1,5 @@
 """Multi-tensor Adam / AdamW on the GPU through the C ABI against the float64
 oracle, and FusedAdam against torch.optim on a small model."""
-import numpy as np
 import pytest
 import torch
 

@@ -3,7 +3,6 @@ tests (tests_deprecated/torch/_C/csrc/test_fused_layer_norm.py: the same module
 built twice, once on the CPU = unfused torch path, once on the GPU = fused
 kernels; outputs, input gradients and weight gradients compared), plus
 autocast, strided inputs and the softmax / GeLU / dropout modules."""
-import numpy as np
 import pytest
 import torch
 

@@ -2,7 +2,6 @@
 softmax) or its own element (bias-GeLU, bias-dropout-add) exactly as it does in
 the reference's unfused torch path, and leaves every other row bit-identical to
 the run without it."""
-import numpy as np
 import pytest
 import torch
 

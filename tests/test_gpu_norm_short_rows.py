@@ -7,7 +7,6 @@ import pytest
 import torch
 
 import test_gpu_norm as base
-from helpers import randn
 from oslo_amd.torch import _C
 
 pytestmark = pytest.mark.gpu

@@ -4,7 +4,6 @@ lane-group size and every rows-per-wave setting of those kernels runs here,
 for the causal, masked and dense forms, with and without the fused dropout,
 against the float64 oracle; and the side-by-side layout must agree with one
 row per wavefront up to the order of summation."""
-import numpy as np
 import pytest
 import torch
 
