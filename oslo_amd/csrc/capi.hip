@@ -41,7 +41,7 @@ int device_cu_count() {
   return cached[dev];
 }
 
-Tuning g_tune = {0, 0, 0, 0, 0, 0, 0, 0, 0};
+Tuning g_tune = {};  // all zero: every heuristic at its built-in choice
 
 }  // namespace oslo
 
