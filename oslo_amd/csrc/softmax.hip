@@ -284,6 +284,35 @@ __global__ __launch_bounds__(1024) void softmax_fwd_kernel(
         stats[2 * row[j] + 1] = empty ? -fill : inv;
       }
     }
+    // A 4-element chunk is half a dropout group, and the lanes 2i and 2i + 1
+    // hold the two halves: instead of evaluating every group twice, the even
+    // lane draws the pair's group of chunk slot 2m, the odd lane that of slot
+    // 2m + 1, and one DPP swap hands each lane the other's result.  (Rows of a
+    // multiple of 8 keys, so that groups do not straddle rows; the row and the
+    // conditions below are uniform over the wave, so all lanes are active.)
+    constexpr bool kPairDraw = DROP && E == 4 && LPR == kWave && VPL % 2 == 0;
+    uint32_t keepk[kPairDraw ? VPL : 1];
+    bool paired = false;
+    if constexpr (kPairDraw) {
+      if ((g.sk & 7) == 0) {
+        paired = true;
+        const int odd = lane & 1;
+#pragma unroll
+        for (int m = 0; m < VPL / 2; ++m) {
+          keepk[2 * m] = keepk[2 * m + 1] = 0u;
+          if (none_visible[j][2 * m] && none_visible[j][2 * m + 1] && !empty) continue;
+          const int cpair = (c0 - odd) + (2 * m + odd) * cstride;  // the pair's even chunk
+          const uint64_t flat = (uint64_t)row[j] * (uint64_t)g.sk + (uint64_t)cpair * E;
+          const uint32_t bits = dropout_keep_bits(flat >> 3, d.seed, d.offset, d.threshold);
+          const uint32_t other = (uint32_t)__builtin_amdgcn_update_dpp(
+              0, (int)bits, kDppQuadSwap1, 0xF, 0xF, false);
+          const uint32_t mine = (bits >> (4 * odd)) & 0xFu;     // slot 2m + odd
+          const uint32_t theirs = (other >> (4 * odd)) & 0xFu;  // the other slot
+          keepk[2 * m] = odd ? theirs : mine;
+          keepk[2 * m + 1] = odd ? mine : theirs;
+        }
+      }
+    }
 #pragma unroll
     for (int k = 0; k < VPL; ++k) {
       const int c = c0 + k * cstride;
@@ -299,7 +328,12 @@ __global__ __launch_bounds__(1024) void softmax_fwd_kernel(
         if constexpr (DROP) {
           // exact zeros need no draw (wave-uniform test)
           if (!none_visible[j][k] || empty) {
-            const uint32_t keep = chunk_keep_bits<E>(row[j], g.sk, c, d);
+            uint32_t keep;
+            if constexpr (kPairDraw) {
+              keep = paired ? keepk[k] : chunk_keep_bits<E>(row[j], g.sk, c, d);
+            } else {
+              keep = chunk_keep_bits<E>(row[j], g.sk, c, d);
+            }
 #pragma unroll
             for (int e = 0; e < E; ++e)
               o[e] = (keep >> e) & 1u ? o[e] * d.scale : 0.f;
