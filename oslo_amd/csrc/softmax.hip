@@ -1189,10 +1189,12 @@ static int launch_softmax_fwd(const void *x, const uint8_t *mask, void *y,
                               float scale, hipStream_t st) {
   constexpr int E = io<T>::EPV;
   const bool drop = stats != nullptr;
-  // 32 elements per lane measure 10-25 % faster than 64 (rows of 4096 and
-  // more 16-bit keys then take two or more waves); 64 only where a row would
-  // otherwise not fit one workgroup
-  const int cap = g_tune.softmax_fwd_elems > 0 ? g_tune.softmax_fwd_elems : 32;
+  // 64 bytes of the operand per lane (32 16-bit or 16 fp32 elements) measure
+  // 10-25 % faster than twice that (rows of 4096 and more 16-bit keys then
+  // take two or more waves); 64 elements only where a row would otherwise not
+  // fit one workgroup
+  const int cap = g_tune.softmax_fwd_elems > 0 ? g_tune.softmax_fwd_elems
+                                               : (sizeof(T) == 4 ? 16 : 32);
   SoftmaxPlan pl = plan_softmax(g.sk, E, cap, MODE == kModeMasked ? 2 : 1, 4, true);
   if (!pl.ok && cap < kFwdMaxElems)
     pl = plan_softmax(g.sk, E, kFwdMaxElems, MODE == kModeMasked ? 2 : 1, 4);
