@@ -1270,7 +1270,9 @@ static int launch_softmax_bwd(const void *dy, const void *y,
                               const uint8_t *mask, void *dx, SoftmaxGeom g,
                               float scale, hipStream_t st) {
   constexpr int E = io<T>::EPV;
-  SoftmaxPlan pl = plan_softmax(g.sk, E, kBwdMaxElems, 1, 1);
+  // (fp32: 16 elements of each operand per lane, as in the forward)
+  SoftmaxPlan pl = plan_softmax(g.sk, E, sizeof(T) == 4 ? 16 : kBwdMaxElems, 1, 1);
+  if (!pl.ok && sizeof(T) == 4) pl = plan_softmax(g.sk, E, kBwdMaxElems, 1, 1);
   const bool vec_ok = pl.ok && aligned16(dy) && aligned16(y) &&
                       aligned16(dx) &&
                       (MODE != kModeMasked ||
@@ -1329,7 +1331,9 @@ static int launch_softmax_dropout_bwd(const void *dy, const void *x,
                                       void *dx, DropArgs d, SoftmaxGeom g,
                                       float scale, hipStream_t st) {
   constexpr int E = io<T>::EPV;
-  SoftmaxPlan pl = plan_softmax(g.sk, E, kBwdMaxElems, 1, 1);
+  // (fp32: 16 elements of each operand per lane, as in the forward)
+  SoftmaxPlan pl = plan_softmax(g.sk, E, sizeof(T) == 4 ? 16 : kBwdMaxElems, 1, 1);
+  if (!pl.ok && sizeof(T) == 4) pl = plan_softmax(g.sk, E, kBwdMaxElems, 1, 1);
   const bool vec_ok = pl.ok && aligned16(dy) && aligned16(x) && aligned16(dx) &&
                       (MODE != kModeMasked ||
                        (reinterpret_cast<uintptr_t>(mask) % E) == 0);
