@@ -5,6 +5,15 @@ or fp16 tensor is passed as the float32/float64 array of its values), computes
 in ``acc`` precision (float64 unless stated) and, where ``out`` names a storage
 type, rounds the result to it once at the point where the fused kernel rounds.
 File:line citations are into the reference repository (EleutherAI/oslo).
+
+Pinning: the reference holds no numeric vectors, known answers or fixtures for
+these ops (its tests compare two of its own paths on unseeded data), so none of
+the functions here is pinned by reference-held data.  Each one is pinned
+instead by tests/test_oracle_closed_form.py, test_oracle_philox.py and
+test_oracle_adam.py: torch library routines and torch autograd in float64,
+finite differences, invariants (row sums, shift invariance, exact zeros,
+orthogonality of the norm gradients), brute force on tiny inputs and the
+Random123 known-answer vectors.
 """
 import numpy as np
 
