@@ -90,6 +90,25 @@ int oslo_ln_bwd(const void *dy, const void *x, const void *mean,
                 int64_t n1, int64_t n2, int dtype_in, int dtype_out,
                 void *stream);
 
+/* oslo_ln_bwd without a workspace argument and without any allocation.  It
+ * has no counterpart in the reference; it is for callers that cannot
+ * allocate device memory around the call: code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc.  The fp32 partial
+ * rows of dgamma / dbeta go to an array of
+ * OSLO_LN_BWD_STATIC_SCRATCH_BYTES bytes that is part of the library's device
+ * code (each GPU the library runs on holds its copy until the process ends).
+ * A problem whose oslo_workspace_bytes(OSLO_OP_LN_BWD, n1, n2) exceeds that
+ * size is refused with OSLO_ERR_WORKSPACE (n2 up to 8192 fits at any n1 on a
+ * 256-CU part).  Results equal oslo_ln_bwd's bit for bit.  All calls on one
+ * GPU share the array: calls that may overlap there (different streams or
+ * host threads without ordering between them) race and must use oslo_ln_bwd
+ * with their own workspaces instead.                                        */
+#define OSLO_LN_BWD_STATIC_SCRATCH_BYTES (16 * 1024 * 1024)
+int oslo_ln_bwd_static(const void *dy, const void *x, const void *mean,
+                       const void *invvar, const void *gamma, void *dx,
+                       void *dgamma, void *dbeta, int64_t n1, int64_t n2,
+                       int dtype_in, int dtype_out, void *stream);
+
 /* Replaces rms_norm_forward, rms_norm_forward_affine and
  * rms_norm_forward_affine_mixed_dtypes (FusedLayerNormBinder.cpp:285-358 ->
  * cuda_rms_norm, fused_layer_norm.cu:790-806).

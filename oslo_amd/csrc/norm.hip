@@ -16,6 +16,7 @@
 //
 // Formulas follow oslo/torch/_C/csrc/fused_layer_norm.cu:310-359 (forward)
 // and :594-741 (grad input), :458-591 (grad gamma/beta) of the reference.
+#include <atomic>
 #include <type_traits>
 
 #include "capi.h"
@@ -1549,6 +1550,40 @@ static int norm_bwd_entry(bool rms, const void *dy, const void *x,
                      gamma, dx, dgamma, dbeta, ws, ws_bytes, n1, n2, st);
 }
 
+// ---------------------------------------------------------------------------
+// LayerNorm backward without a workspace argument: the fp32 partial rows of
+// dgamma / dbeta live in a file-scope device array.  Every GPU holds its own
+// copy of the array at its own address; in host code the array's name is only
+// a handle for hipGetSymbolAddress, never a device address.
+// ---------------------------------------------------------------------------
+constexpr int64_t kStaticScratchBytes = OSLO_LN_BWD_STATIC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+constexpr int kMaxDevices = 64;
+static std::atomic<void *> g_scratch_ptr[kMaxDevices];
+
+// Device address of `scratch` on the current device, looked up once per
+// device (threads that race here obtain the same address).
+static int static_scratch(void **out) {
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess)
+    return fail(OSLO_ERR_LAUNCH, "ln bwd static: hipGetDevice: %s", hipGetErrorString(e));
+  if (dev < 0 || dev >= kMaxDevices)
+    return fail(OSLO_ERR_UNSUPPORTED, "ln bwd static: device index %d beyond %d", dev,
+                kMaxDevices - 1);
+  void *ptr = g_scratch_ptr[dev].load(std::memory_order_acquire);
+  if (ptr == nullptr) {
+    e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || ptr == nullptr)
+      return fail(OSLO_ERR_LAUNCH, "ln bwd static: hipGetSymbolAddress: %s",
+                  hipGetErrorString(e));
+    g_scratch_ptr[dev].store(ptr, std::memory_order_release);
+  }
+  *out = ptr;
+  return OSLO_OK;
+}
+
 }  // namespace oslo
 
 extern "C" {
@@ -1584,6 +1619,34 @@ int oslo_rms_bwd(const void *dy, const void *x, const void *invvar,
   return oslo::norm_bwd_entry(true, dy, x, nullptr, invvar, gamma, dx, dgamma,
                               nullptr, workspace, workspace_bytes, n1, n2,
                               dtype_in, dtype_out, stream);
+}
+
+int oslo_ln_bwd_static(const void *dy, const void *x, const void *mean,
+                       const void *invvar, const void *gamma, void *dx,
+                       void *dgamma, void *dbeta, int64_t n1, int64_t n2,
+                       int dtype_in, int dtype_out, void *stream) {
+  using namespace oslo;
+  OSLO_REQUIRE(n1 >= 0 && n2 >= 1, "ln bwd static: bad shape [%lld, %lld]",
+               (long long)n1, (long long)n2);
+  void *ws = nullptr;
+  if (dgamma != nullptr && n1 > 0 && dtype_in != OSLO_DTYPE_F64) {
+    const int64_t need = oslo_workspace_bytes(OSLO_OP_LN_BWD, n1, n2);
+    if (need < 0) return (int)need;
+    if (need > kStaticScratchBytes)
+      return fail(OSLO_ERR_WORKSPACE,
+                  "ln bwd static: [%lld, %lld] needs %lld bytes of partial rows, "
+                  "the static scratch holds %lld; use oslo_ln_bwd with a "
+                  "workspace",
+                  (long long)n1, (long long)n2, (long long)need,
+                  (long long)kStaticScratchBytes);
+    const int rc = static_scratch(&ws);
+    if (rc != OSLO_OK) return rc;
+  }
+  // The partial rows are written in full before the finalize kernel reads
+  // them: nothing in the array has to start at zero.
+  return norm_bwd_entry(false, dy, x, mean, invvar, gamma, dx, dgamma, dbeta, ws,
+                        ws != nullptr ? kStaticScratchBytes : 0, n1, n2,
+                        dtype_in, dtype_out, stream);
 }
 
 int oslo_bias_dropout_add_norm_fwd(const void *x, const void *bias,

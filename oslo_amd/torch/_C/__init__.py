@@ -35,6 +35,7 @@ ABI_VERSION = 1
 
 _DTYPE_CODE = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}
 OSLO_DTYPE_F64 = 3  # LayerNorm / RMSNorm only
+OSLO_LN_BWD_STATIC_SCRATCH_BYTES = 16 * 1024 * 1024
 
 _lib = None
 _lib_lock = threading.Lock()
@@ -56,6 +57,10 @@ _SIGNATURES = {
     "oslo_ln_bwd": (
         _int,
         [_p, _p, _p, _p, _p, _p, _p, _p, _p, _i64, _i64, _i64, _int, _int, _p],
+    ),
+    "oslo_ln_bwd_static": (
+        _int,
+        [_p, _p, _p, _p, _p, _p, _p, _p, _i64, _i64, _int, _int, _p],
     ),
     "oslo_rms_fwd": (_int, [_p, _p, _p, _p, _i64, _i64, _f64, _int, _int, _p]),
     "oslo_rms_bwd": (
