@@ -381,7 +381,9 @@ int oslo_wave_reduce_selftest(float *out4, void *stream);
  * OSLO_ERR_INVALID_ARGUMENT: chunks per lane (*_vpl: 1, 2, 4, forward also 8),
  * waves per workgroup 1..16, norm_bwd_prefetch 1 or 2, norm_fwd_iters 1..16,
  * norm_bwd_blocks_per_cu 1..8, lanes per row 8, 16, 32 or 64 (softmax also
- * 1), softmax_rows_per_wave and the unroll factors 1, 2 or 4,
+ * 1), softmax_rows_per_wave and the unroll factors 1, 2 or 4 (eltwise_unroll
+ * also 8, which only the bias-GeLU backward has a build for; the other
+ * element-wise kernels then keep their default),
  * softmax_fwd_elems 16, 32 or 64, eltwise tile widths powers of two up to
  * 256, eltwise_rowgroups 1..4096, eltwise_fwd_steps 1..64.
  * Process-wide, not thread-safe.                                           */

@@ -102,7 +102,7 @@ int oslo_tune(const char *key, int value) {
       {"norm_lanes_per_row", &oslo::g_tune.norm_lanes_per_row, kLanes, 8, 64},
       {"eltwise_tile_max", &oslo::g_tune.eltwise_tile_max, kPow2, 1, 256},
       {"eltwise_tile_min", &oslo::g_tune.eltwise_tile_min, kPow2, 1, 256},
-      {"eltwise_unroll", &oslo::g_tune.eltwise_unroll, kPow2, 1, 4},
+      {"eltwise_unroll", &oslo::g_tune.eltwise_unroll, kPow2, 1, 8},
       {"eltwise_rowgroups", &oslo::g_tune.eltwise_rowgroups, kRange, 1, 4096},
       {"eltwise_fwd_steps", &oslo::g_tune.eltwise_fwd_steps, kRange, 1, 64},
       {"norm_bwd_waves", &oslo::g_tune.norm_bwd_waves, kRange, 1, 16},

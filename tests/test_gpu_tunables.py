@@ -59,7 +59,7 @@ def test_softmax_override_keeps_the_result(device, tuned, sq, sk, dtype, key, va
 ELTWISE_OVERRIDES = [
     ("eltwise_tile_max", 64), ("eltwise_tile_max", 8), ("eltwise_tile_max", 1),
     ("eltwise_tile_min", 64), ("eltwise_tile_min", 256),
-    ("eltwise_unroll", 1), ("eltwise_unroll", 2), ("eltwise_unroll", 4),
+    ("eltwise_unroll", 1), ("eltwise_unroll", 2), ("eltwise_unroll", 4), ("eltwise_unroll", 8),
     ("eltwise_rowgroups", 1), ("eltwise_rowgroups", 7), ("eltwise_rowgroups", 1024),
     ("eltwise_fwd_steps", 2), ("eltwise_fwd_steps", 5),
 ]
