@@ -3,28 +3,39 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W]
 
-Headline workload (BASELINE.json configs[1]): LayerNorm and RMSNorm forward +
-backward on a bf16 [16384, 4096] activation.  One step = LN fwd, LN bwd, RMS
-fwd, RMS bwd over one batch, called through the C ABI with every buffer
-resident in HBM and pre-allocated; buffer sets rotate so the 256 MB Infinity
-Cache cannot serve the reads.  `value` = algorithmic bytes of a step (10 T,
-T = 134.2 MB) / wall time per step.
+Headline workload (BASELINE.json configs[4], the largest that fits one GPU):
+the non-GEMM chain of one GPT-NeoX-20B-shaped layer, bf16, batch 4, sequence
+2048, hidden 6144, 64 heads.  One step = eight launches through the C ABI,
+    ln_fwd, ln_bwd                  [8192, 6144]
+    softmax_causal_fwd, _bwd        [256, 2048, 2048], scale 1/sqrt(96)
+    bias_gelu_fwd, _bwd             [8192, 24576]
+    bias_dropout_add_fwd, _bwd      [8192, 6144], p = 0.1
+every buffer resident in HBM and pre-allocated; each stage has its own
+synthetic input (the GEMMs between the stages are not part of the path).
+`value` = algorithmic bytes of a step (10 537.7 MB) / wall time per step.
 
 Prints ONE JSON line.  Beside the contract's keys it carries
-  roofline      the dominant launch (LN backward), timed with events on the
-                launch stream inside the timed region,
-  cpu_baseline  the reference's unfused torch path (oracle/torch_path.py) on
-                the host cores, same workload,
-  kernels       achieved GB/s and fraction of the 8 TB/s HBM peak for every
-                fused kernel of BASELINE.json's five configurations,
-  cpu_path      the reference's unfused torch path, forward + backward, for
-                the other four configurations on bounded samples, with the
-                GPU rate of the same pair and their ratio.
+  roofline      the dominant launch of the step (causal softmax backward,
+                4 296.0 MB), timed with events on the launch stream inside the
+                timed region; `traffic` is read from the rocprofv3 counter
+                summary under profiles/,
+  cpu_baseline  the same chain through the reference's unfused torch path
+                (oracle/torch_path.py) on the host cores, on a bounded sample,
+  kernels       a compact table (cols / rows) of achieved GB/s and fraction of
+                the 8 TB/s HBM peak for every fused kernel of BASELINE.json's
+                five configurations, with mean / median / minimum times, the
+                time per launch inside a captured HIP graph for the backward
+                kernels that end in a second (finalize) launch, and plain
+                copies of matching sizes,
+  cpu_path      the reference's unfused torch path, forward + backward, per
+                configuration on bounded samples, with the GPU rate of the
+                same pair and their ratio.
 """
 import argparse
 import json
 import math
 import os
+import re
 import sys
 import time
 
@@ -34,11 +45,7 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published
 METRIC = "achieved HBM GB/s (% of MI355X peak) per fused fwd+bwd kernel; speedup vs CPU path"
-# HBM traffic of one LayerNorm-backward call on bf16 [16384, 4096], measured with
-# rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE and calibrated against a 1 GiB copy:
-# main kernel 270.9 MB read + 142.6 MB written, finalize 8.4 MB read
-# (summary: profiles/bench_all_kernels_hbm_traffic.txt).  Algorithmic: 402.7 MB.
-LN_BWD_TRAFFIC_BYTES = 421.9e6
+TRAFFIC_SUMMARY = os.path.join(ROOT, "profiles", "bench_all_kernels_hbm_traffic.txt")
 
 F32, F16, BF16 = 0, 1, 2
 
@@ -46,11 +53,11 @@ F32, F16, BF16 = 0, 1, 2
 def parse_args():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=100)
-    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--steps", type=int, default=30)
+    ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--table-iters", type=int, default=200, help="launches per kernel in the per-kernel table (0 = skip)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--cpu-reps", type=int, default=15)
+    ap.add_argument("--no-graph-column", action="store_true", help="skip the captured-graph timings of the table")
     return ap.parse_args()
 
 
@@ -78,20 +85,71 @@ def p(t):
     return None if t is None else t.data_ptr()
 
 
+WARM_MS = 30.0  # launches before a timed region: the clocks of an idle GPU take this long to settle
+BATCHES = 10    # event pairs per table row: mean over all launches, median and minimum over the batches
+
+
 def time_launches(torch, fn, iters, nsets):
-    """Average duration in ms of fn(i % nsets), events on the current stream."""
-    # warm-up: every buffer set is touched, 20 launches ahead of a long timed region
-    for i in range(max(3, nsets, min(20, iters // 10))):
-        fn(i % nsets)
-    torch.cuda.synchronize()
+    """Times fn(i % nsets) with events on the current stream: `iters` launches
+    in BATCHES batches, each between one pair of events.  Returns (mean,
+    median of the batch means, smallest batch mean) in ms per launch."""
     e0 = torch.cuda.Event(enable_timing=True)
     e1 = torch.cuda.Event(enable_timing=True)
-    e0.record()
-    for i in range(iters):
-        fn(i % nsets)
-    e1.record()
+    # warm-up: every buffer set is touched, and the GPU is kept busy for WARM_MS
+    n = max(3, nsets)
+    spent = 0.0
+    while spent < WARM_MS:
+        e0.record()
+        for i in range(n):
+            fn(i % nsets)
+        e1.record()
+        torch.cuda.synchronize()
+        spent += e0.elapsed_time(e1)
+        n = min(4 * n, 400)
+    per = max(1, iters // BATCHES)
+    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(BATCHES)]
+    k = 0
+    for a, b in evs:
+        a.record()
+        for _ in range(per):
+            fn(k % nsets)
+            k += 1
+        b.record()
     torch.cuda.synchronize()
-    return e0.elapsed_time(e1) / iters
+    times = sorted(a.elapsed_time(b) / per for a, b in evs)
+    return sum(times) / len(times), times[len(times) // 2], times[0]
+
+
+def time_in_graph(torch, fn, nsets, launches=24, replays=8):
+    """ms per launch of fn inside a captured HIP graph (the dependent launches
+    of one call follow each other without host dispatch); None if capture fails."""
+    try:
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.stream(side):
+            for i in range(nsets):
+                fn(i)
+            torch.cuda.synchronize()
+            with torch.cuda.graph(graph, stream=side):
+                for i in range(launches):
+                    fn(i % nsets)
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        for _ in range(3):
+            graph.replay()
+        torch.cuda.synchronize()
+        e0 = torch.cuda.Event(enable_timing=True)
+        e1 = torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(replays):
+            graph.replay()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / (replays * launches)
+    except Exception as exc:  # noqa: BLE001 - a timing column, never fatal
+        sys.stderr.write("bench.py: graph timing skipped (%s)\n" % (exc,))
+        return None
 
 
 def norm_buffers(torch, dev, n1, n2, nsets, seed):
@@ -145,13 +203,107 @@ def make_norm_calls(L, dev, n1, n2, nsets, seed=0):
     return {"ln_fwd": ln_fwd, "ln_bwd": ln_bwd, "rms_fwd": rms_fwd, "rms_bwd": rms_bwd, "_keep": keep}
 
 
-def table_row(name, cfg, shape, dtype, nbytes, ms):
-    gbps = nbytes / (ms * 1e-3) / 1e9
-    return {
-        "kernel": name, "config": cfg, "shape": shape, "io_dtype": dtype,
-        "algorithmic_MB": round(nbytes / 1e6, 1), "us": round(ms * 1e3, 2),
-        "GBps": round(gbps, 1), "frac_of_peak": round(gbps / HBM_PEAK_GBPS, 4),
-    }
+# ---------------------------------------------------------------------------
+# the headline step: BASELINE.json configs[4]
+# ---------------------------------------------------------------------------
+CHAIN = {
+    "tokens": 8192, "hidden": 6144, "attn_batches": 256, "seq": 2048, "ffn": 24576,
+    "scale": 1.0 / math.sqrt(96.0), "p": 0.1,
+}
+
+
+def chain_bytes():
+    """Algorithmic bytes of each launch of the step (bf16: 2 bytes per element)."""
+    c = CHAIN
+    t_ln = c["tokens"] * c["hidden"] * 2
+    t_sm = c["attn_batches"] * c["seq"] * c["seq"] * 2
+    t_ff = c["tokens"] * c["ffn"] * 2
+    f = (c["seq"] + 1) / (2.0 * c["seq"])
+    return [
+        ("ln_fwd", 2 * t_ln), ("ln_bwd", 3 * t_ln),
+        ("softmax_causal_fwd", (1 + f) * t_sm), ("softmax_causal_bwd", (1 + 2 * f) * t_sm),
+        ("bias_gelu_fwd", 2 * t_ff), ("bias_gelu_bwd", 3 * t_ff),
+        ("bias_dropout_add_fwd", 3 * t_ln), ("bias_dropout_add_bwd", 2 * t_ln),
+    ]
+
+
+def make_chain(L, dev):
+    """Pre-allocates every buffer of the step and returns its eight launches in
+    order (the order of the reference's layer: LayerNorm, attention softmax,
+    feed-forward activation, output dropout + residual), each as fn()."""
+    torch = L.torch
+    lib = L.lib
+    c = CHAIN
+    n1, h, ab, s, ff = c["tokens"], c["hidden"], c["attn_batches"], c["seq"], c["ffn"]
+    g = torch.Generator(device=dev).manual_seed(0)
+    bf = torch.bfloat16
+
+    def rnd(*shape, std=1.0, mean=0.0):
+        return (mean + std * torch.randn(*shape, generator=g, device=dev)).to(bf)
+
+    ln = {"x": rnd(n1, h), "dy": rnd(n1, h), "y": torch.empty(n1, h, device=dev, dtype=bf),
+          "dx": torch.empty(n1, h, device=dev, dtype=bf), "mean": torch.empty(n1, device=dev),
+          "invvar": torch.empty(n1, device=dev), "gamma": rnd(h, std=0.02, mean=1.0), "beta": rnd(h, std=0.02)}
+    ln["dgamma"], ln["dbeta"] = torch.empty_like(ln["gamma"]), torch.empty_like(ln["beta"])
+    ws_ln, ws_ln_b = L.ws(L._C.OSLO_OP_LN_BWD, n1, h, dev)
+    sm = {"x": rnd(ab, s, s), "dy": rnd(ab, s, s)}
+    sm["y"], sm["dx"] = torch.empty_like(sm["x"]), torch.empty_like(sm["x"])
+    ge = {"x": rnd(n1, ff), "g": rnd(n1, ff), "bias": rnd(ff, std=0.02)}
+    ge["y"], ge["dx"], ge["dbias"] = torch.empty_like(ge["x"]), torch.empty_like(ge["x"]), torch.empty_like(ge["bias"])
+    ws_ge, ws_ge_b = L.ws(L._C.OSLO_OP_BIAS_GELU_BWD, n1, ff, dev)
+    bd = {"x": rnd(n1, h), "res": rnd(n1, h), "g": rnd(n1, h), "bias": rnd(h, std=0.02)}
+    bd["out"], bd["dx"], bd["dbias"] = torch.empty_like(bd["x"]), torch.empty_like(bd["x"]), torch.empty_like(bd["bias"])
+    ws_bd, ws_bd_b = L.ws(L._C.OSLO_OP_BIAS_DROPOUT_ADD_BWD, n1, h, dev)
+    keep = (ln, sm, ge, bd, ws_ln, ws_ge, ws_bd)
+    st = L.stream
+
+    calls = [
+        lambda: L.ok(lib.oslo_ln_fwd(p(ln["x"]), p(ln["gamma"]), p(ln["beta"]), p(ln["y"]), p(ln["mean"]),
+                                     p(ln["invvar"]), n1, h, 1e-5, BF16, BF16, st())),
+        lambda: L.ok(lib.oslo_ln_bwd(p(ln["dy"]), p(ln["x"]), p(ln["mean"]), p(ln["invvar"]), p(ln["gamma"]),
+                                     p(ln["dx"]), p(ln["dgamma"]), p(ln["dbeta"]), p(ws_ln), ws_ln_b, n1, h,
+                                     BF16, BF16, st())),
+        lambda: L.ok(lib.oslo_softmax_causal_fwd(p(sm["x"]), p(sm["y"]), ab, s, s, c["scale"], BF16, st())),
+        lambda: L.ok(lib.oslo_softmax_causal_bwd(p(sm["dy"]), p(sm["y"]), p(sm["dx"]), ab, s, s, c["scale"], BF16,
+                                                 st())),
+        lambda: L.ok(lib.oslo_bias_gelu_fwd(p(ge["x"]), p(ge["bias"]), p(ge["y"]), n1, ff, BF16, st())),
+        lambda: L.ok(lib.oslo_bias_gelu_bwd(p(ge["g"]), p(ge["x"]), p(ge["bias"]), p(ge["dx"]), p(ge["dbias"]),
+                                            p(ws_ge), ws_ge_b, n1, ff, BF16, st())),
+        lambda: L.ok(lib.oslo_bias_dropout_add_fwd(p(bd["x"]), p(bd["bias"]), p(bd["res"]), p(bd["out"]), None, n1, h,
+                                                   c["p"], 1234, 0, BF16, st())),
+        lambda: L.ok(lib.oslo_bias_dropout_add_bwd(p(bd["g"]), p(bd["dx"]), p(bd["dbias"]), p(ws_bd), ws_bd_b, n1, h,
+                                                   c["p"], 1234, 0, BF16, st())),
+    ]
+    return calls, keep
+
+
+def traffic_from_profile(kernel, blocks, wg):
+    """HBM bytes per launch of `kernel` at launch shape blocks x wg, from the
+    committed rocprofv3 FETCH_SIZE / WRITE_SIZE summary (columns: kernel,
+    template, blocks, wg, FETCH KiB, WRITE KiB, read MB, write MB)."""
+    try:
+        text = open(TRAFFIC_SUMMARY).read()
+    except OSError as exc:
+        raise RuntimeError("bench.py: counter summary %s is missing (%s)" % (TRAFFIC_SUMMARY, exc))
+    for line in text.splitlines():
+        f = line.split()
+        if len(f) >= 8 and f[0] == kernel and f[-6] == str(blocks) and f[-5] == str(wg):
+            try:
+                return (float(f[-2]) + float(f[-1])) * 1e6
+            except ValueError:
+                continue
+    raise RuntimeError("bench.py: no row for %s at %d x %d in %s" % (kernel, blocks, wg, TRAFFIC_SUMMARY))
+
+
+TABLE_COLS = ["kernel", "cfg", "MB", "us", "us_med", "us_min", "GBps", "frac", "graph_us", "note"]
+
+
+def table_row(name, cfg, nbytes, t, graph_ms=None, note=""):
+    mean, med, mn = t
+    gbps = nbytes / (mean * 1e-3) / 1e9
+    return [name, cfg, round(nbytes / 1e6, 1), round(mean * 1e3, 2), round(med * 1e3, 2), round(mn * 1e3, 2),
+            round(gbps, 1), round(gbps / HBM_PEAK_GBPS, 4),
+            None if graph_ms is None else round(graph_ms * 1e3, 2), note]
 
 
 def nsets_for(total_bytes_per_set):
@@ -159,7 +311,7 @@ def nsets_for(total_bytes_per_set):
     return max(1, min(8, math.ceil(1.0e9 / max(total_bytes_per_set, 1))))
 
 
-def kernel_table(L, dev, iters):
+def kernel_table(L, dev, iters, graph_column=True):
     """Every fused kernel at the shapes of BASELINE.json's five configurations."""
     torch = L.torch
     lib = L.lib
@@ -167,6 +319,9 @@ def kernel_table(L, dev, iters):
 
     def timed(fn, nsets):
         return time_launches(torch, fn, iters, nsets)
+
+    def graphed(fn, nsets):
+        return time_in_graph(torch, fn, nsets) if graph_column else None
 
     # ---- LayerNorm / RMSNorm: cfg2 and cfg5 ----
     for cfg, n1, n2 in (("cfg2", 16384, 4096), ("cfg5", 8192, 6144)):
@@ -177,10 +332,10 @@ def kernel_table(L, dev, iters):
             if cfg == "cfg5" and name.startswith("rms"):
                 continue
             if name.endswith("bwd"):
-                calls[name.replace("bwd", "fwd")](0)
                 for i in range(ns):
                     calls[name.replace("bwd", "fwd")](i)
-            rows.append(table_row(name, cfg, [n1, n2], "bf16", mult * T, timed(calls[name], ns)))
+            rows.append(table_row(name, cfg, mult * T, timed(calls[name], ns),
+                                  graphed(calls[name], ns) if name.endswith("bwd") else None))
         del calls
         torch.cuda.empty_cache()
 
@@ -210,8 +365,8 @@ def kernel_table(L, dev, iters):
             x, y, dy, dx = bufs[i]
             L.ok(lib.oslo_softmax_causal_bwd(p(dy), p(y), p(dx), ab, s, s, scale, code, L.stream()))
 
-        rows.append(table_row("softmax_causal_fwd", cfg, [ab, s, s], str(tdt).split(".")[-1], (1 + f) * T, timed(fwd, ns)))
-        rows.append(table_row("softmax_causal_bwd", cfg, [ab, s, s], str(tdt).split(".")[-1], (1 + 2 * f) * T, timed(bwd, ns)))
+        rows.append(table_row("softmax_causal_fwd", cfg, (1 + f) * T, timed(fwd, ns)))
+        rows.append(table_row("softmax_causal_bwd", cfg, (1 + 2 * f) * T, timed(bwd, ns)))
 
         # softmax with the attention dropout (p = 0.1) fused in: the same
         # compulsory bytes (backward reads the logits instead of the
@@ -226,10 +381,8 @@ def kernel_table(L, dev, iters):
             x, y, dy, dx = bufs[i]
             L.ok(lib.oslo_softmax_causal_dropout_bwd(p(dy), p(x), p(stats), p(dx), ab, s, s, scale, 0.1, 1234, 0, code, L.stream()))
 
-        for name, fn, nbytes in (("softmax_causal_dropout_fwd", dfwd, (1 + f) * T), ("softmax_causal_dropout_bwd", dbwd, (1 + 2 * f) * T)):
-            row = table_row(name, cfg, [ab, s, s], str(tdt).split(".")[-1], nbytes, timed(fn, ns))
-            row["p"] = 0.1
-            rows.append(row)
+        rows.append(table_row("softmax_causal_dropout_fwd", cfg, (1 + f) * T, timed(dfwd, ns), note="p=0.1"))
+        rows.append(table_row("softmax_causal_dropout_bwd", cfg, (1 + 2 * f) * T, timed(dbwd, ns), note="p=0.1"))
         del bufs, stats
         torch.cuda.empty_cache()
 
@@ -255,14 +408,12 @@ def kernel_table(L, dev, iters):
         x, y, dy, dx = bufs[i]
         L.ok(lib.oslo_softmax_masked_bwd(p(dy), p(y), p(mask), p(dx), b, h, s, s, b, 1, 0.125, F16, L.stream()))
 
-    row = table_row("softmax_masked_fwd", "cfg3", [b, h, s, s], "float16", (r + 1) * T, timed(mfwd, ns))
-    row["valid_fraction"] = round(r, 4)
-    row["dense_equiv_GBps"] = round(2 * T / (row["us"] * 1e-6) / 1e9, 1)
-    rows.append(row)
-    row = table_row("softmax_masked_bwd", "cfg3", [b, h, s, s], "float16", (2 * r + 1) * T, timed(mbwd, ns))
-    row["valid_fraction"] = round(r, 4)
-    row["dense_equiv_GBps"] = round(3 * T / (row["us"] * 1e-6) / 1e9, 1)
-    rows.append(row)
+    t = timed(mfwd, ns)
+    rows.append(table_row("softmax_masked_fwd", "cfg3", (r + 1) * T, t,
+                          note="valid %.4f, dense-equivalent %.0f GB/s" % (r, 2 * T / (t[0] * 1e-3) / 1e9)))
+    t = timed(mbwd, ns)
+    rows.append(table_row("softmax_masked_bwd", "cfg3", (2 * r + 1) * T, t,
+                          note="valid %.4f, dense-equivalent %.0f GB/s" % (r, 3 * T / (t[0] * 1e-3) / 1e9)))
     del bufs
     torch.cuda.empty_cache()
 
@@ -288,8 +439,8 @@ def kernel_table(L, dev, iters):
             x, y, gg, dx = bufs[i]
             L.ok(lib.oslo_bias_gelu_bwd(p(gg), p(x), p(bias), p(dx), p(dbias), p(ws), wsb, n1, n2, BF16, L.stream()))
 
-        rows.append(table_row("bias_gelu_fwd", cfg, [n1, n2], "bf16", 2 * T, timed(gfwd, ns)))
-        rows.append(table_row("bias_gelu_bwd", cfg, [n1, n2], "bf16", 3 * T, timed(gbwd, ns)))
+        rows.append(table_row("bias_gelu_fwd", cfg, 2 * T, timed(gfwd, ns)))
+        rows.append(table_row("bias_gelu_bwd", cfg, 3 * T, timed(gbwd, ns), graphed(gbwd, ns)))
         del bufs
         torch.cuda.empty_cache()
 
@@ -319,10 +470,8 @@ def kernel_table(L, dev, iters):
                                                L.stream()))
 
         tag = "p=%.1f" % pdrop
-        r1 = table_row("bias_dropout_add_fwd", cfg, [n1, n2], "bf16", 3 * T, timed(dfwd, ns))
-        r2 = table_row("bias_dropout_add_bwd", cfg, [n1, n2], "bf16", 2 * T, timed(dbwd, ns))
-        r1["p"] = r2["p"] = pdrop
-        rows += [r1, r2]
+        rows.append(table_row("bias_dropout_add_fwd", cfg, 3 * T, timed(dfwd, ns), note=tag))
+        rows.append(table_row("bias_dropout_add_bwd", cfg, 2 * T, timed(dbwd, ns), graphed(dbwd, ns), note=tag))
 
         # the same op fused into the LayerNorm that follows it (post-LN block):
         # forward reads x, residual and writes h, y (4T instead of 3T + 2T);
@@ -349,12 +498,10 @@ def kernel_table(L, dev, iters):
                                                         p(extra[i][1]), p(dx), p(dgamma), p(dbeta), p(dbias), p(ws2),
                                                         wsb2, n1, n2, pdrop, 1234, 0, 0, BF16, L.stream()))
 
-            r3 = table_row("bias_dropout_add_ln_fwd", cfg, [n1, n2], "bf16", 4 * T, timed(ffwd, ns))
+            rows.append(table_row("bias_dropout_add_ln_fwd", cfg, 4 * T, timed(ffwd, ns), note=tag))
             for i in range(ns):
                 ffwd(i)
-            r4 = table_row("bias_dropout_add_ln_bwd", cfg, [n1, n2], "bf16", 4 * T, timed(fbwd, ns))
-            r3["p"] = r4["p"] = pdrop
-            rows += [r3, r4]
+            rows.append(table_row("bias_dropout_add_ln_bwd", cfg, 4 * T, timed(fbwd, ns), graphed(fbwd, ns), note=tag))
             del extra
         del bufs
         torch.cuda.empty_cache()
@@ -384,28 +531,46 @@ def kernel_table(L, dev, iters):
             L.ok(lib.oslo_multi_tensor_adam(tables[0], tables[1], tables[2], tables[3], sizes, n, 1e-3, 0.9, 0.999,
                                             1e-8, step_no[0], 1, 1, 0.01, code, L.stream()))
 
-        row = table_row("multi_tensor_adam", "-", [n, nel], str(tdt).split(".")[-1], 7 * nel * esz, timed(adam, 1))
-        row["tensors"] = n
-        rows.append(row)
+        rows.append(table_row("multi_tensor_adam", str(tdt).split(".")[-1], 7 * nel * esz,
+                              time_launches(torch, adam, max(10, iters // 4), 1), note="%d tensors" % n))
         del lists, tables
         torch.cuda.empty_cache()
 
-    # ---- plain copy with the same load/store path: the practical ceiling ----
-    nbytes = 1 << 30
-    src = [torch.empty(nbytes, dtype=torch.uint8, device=dev) for _ in range(2)]
-    dst = [torch.empty(nbytes, dtype=torch.uint8, device=dev) for _ in range(2)]
-    for s_ in src:
-        s_.fill_(1)
+    # ---- plain copies with the same load/store path, at the traffic of the
+    # short kernels above and at 2 GiB: the practical ceiling at each size ----
+    for total_mb in (75.5, 100.8, 201.3, 268.4, 402.7, 830.0, 2147.5):
+        nbytes = int(total_mb * 1e6 / 2) // 16 * 16
+        ns = nsets_for(2 * nbytes)
+        src = [torch.empty(nbytes, dtype=torch.uint8, device=dev) for _ in range(ns)]
+        dst = [torch.empty(nbytes, dtype=torch.uint8, device=dev) for _ in range(ns)]
+        for s_ in src:
+            s_.fill_(1)
 
-    def cp(i):
-        L.ok(lib.oslo_copy_probe(p(src[i]), p(dst[i]), nbytes, L.stream()))
+        def cp(i):
+            L.ok(lib.oslo_copy_probe(p(src[i]), p(dst[i]), nbytes, L.stream()))
 
-    rows.append(table_row("copy_probe", "-", [nbytes], "u8", 2 * nbytes, timed(cp, 2)))
+        rows.append(table_row("copy_probe", "-", 2 * nbytes, timed(cp, ns), note="plain copy, read + write"))
+        del src, dst
+        torch.cuda.empty_cache()
     return rows
 
 
-def cpu_baseline(n1, n2, reps):
-    """The reference's unfused torch path on the host cores, same workload."""
+def cpu_model():
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("model name"):
+                return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
+def cpu_baseline(budget_s=4.0):
+    """The reference's unfused torch path for the chain of the headline step on
+    the host cores.  Each stage runs on a bounded sample of its rows (the CPU
+    rate does not depend on the row count at these sizes) and its time is
+    scaled to the full stage; `value` = the step's algorithmic bytes / the sum
+    of the scaled stage times."""
     import torch
 
     from oracle import torch_path as tp
@@ -413,36 +578,72 @@ def cpu_baseline(n1, n2, reps):
     threads = min(os.cpu_count() or 1, 16)
     torch.set_num_threads(threads)
     g = torch.Generator().manual_seed(0)
-    x = torch.randn(n1, n2, generator=g).to(torch.bfloat16)
-    dy = torch.randn(n1, n2, generator=g).to(torch.bfloat16)
-    gamma = (1 + 0.02 * torch.randn(n2, generator=g)).to(torch.bfloat16)
-    beta = (0.02 * torch.randn(n2, generator=g)).to(torch.bfloat16)
+    bf = torch.bfloat16
+    c = CHAIN
 
-    def step():
+    def rnd(shape, std=1.0, mean=0.0):
+        return (mean + std * torch.randn(shape, generator=g)).to(bf)
+
+    def timed(fn):
+        fn()
+        times, spent = [], 0.0
+        while len(times) < 3 or (spent < budget_s and len(times) < 7):
+            t0 = time.perf_counter()
+            fn()
+            times.append(time.perf_counter() - t0)
+            spent += times[-1]
+        times.sort()
+        return times[len(times) // 2]
+
+    stages = []
+    # LayerNorm: the whole [8192, 6144] tensor (a smaller sample would stay in the host caches)
+    n1, h = c["tokens"], c["hidden"]
+    x, dy = rnd((n1, h)), rnd((n1, h))
+    gamma, beta = rnd((h,), 0.02, 1.0), rnd((h,), 0.02)
+
+    def ln():
         xr = x.clone().requires_grad_()
         w, b = gamma.clone().requires_grad_(), beta.clone().requires_grad_()
         tp.layer_norm(xr, w, b, 1e-5).backward(dy)
-        xr = x.clone().requires_grad_()
-        w = gamma.clone().requires_grad_()
-        tp.rms_norm(xr, w, 1e-5).backward(dy)
+    stages.append(("layer_norm", "[8192,6144] (all)", timed(ln), 1.0))
+    # causal softmax: 8 of the 256 attention batches
+    s = c["seq"]
+    xs, ds = rnd((8, s, s)), rnd((8, s, s))
 
-    step()
-    times = []
-    for _ in range(reps):
-        t0 = time.perf_counter()
-        step()
-        times.append(time.perf_counter() - t0)
-    times.sort()
-    med = times[len(times) // 2]
-    nbytes = 10 * n1 * n2 * 2
+    def sm():
+        xr = xs.clone().requires_grad_()
+        tp.causal_softmax(xr, c["scale"]).backward(ds)
+    stages.append(("softmax_causal", "[8,2048,2048] of 256 batches", timed(sm), c["attn_batches"] / 8.0))
+    del xs, ds
+    # bias-GeLU: 1024 of the 8192 rows
+    xg, dg, bg = rnd((1024, c["ffn"])), rnd((1024, c["ffn"])), rnd((c["ffn"],), 0.02)
+
+    def ge():
+        xr, br = xg.clone().requires_grad_(), bg.clone().requires_grad_()
+        tp.bias_gelu(xr, br).backward(dg)
+    stages.append(("bias_gelu", "[1024,24576] of 8192 rows", timed(ge), n1 / 1024.0))
+    del xg, dg
+    # bias-dropout-add: 2048 of the 8192 rows
+    xb, rb, db, bb = rnd((2048, h)), rnd((2048, h)), rnd((2048, h)), rnd((h,), 0.02)
+
+    def bd():
+        xr, br = xb.clone().requires_grad_(), bb.clone().requires_grad_()
+        tp.bias_dropout_add(xr, br, rb, c["p"], True).backward(db)
+    stages.append(("bias_dropout_add", "[2048,6144] of 8192 rows", timed(bd), n1 / 2048.0))
+
+    full_s = sum(t * k for _, _, t, k in stages)
+    nbytes = sum(b for _, b in chain_bytes())
     return {
-        "value": round(nbytes / med / 1e9, 3),
+        "value": round(nbytes / full_s / 1e9, 3),
         "unit": "GB/s",
         "cores": threads,
+        "cpu": cpu_model(),
         "kind": "port",
-        "sample": "full workload [%d,%d] bf16, LN+RMS fwd+bwd via torch CPU ops (F.layer_norm, manual_rms_norm, autograd), "
-                  "median of %d reps, %.2f s each" % (n1, n2, reps, med),
-        "ms_per_step": round(med * 1e3, 1),
+        "sample": "forward + backward through torch CPU ops and autograd, bf16, median of 3-7 runs per stage; "
+                  + "; ".join("%s %s %.2f s x %g" % (n, smp, t, k) for n, smp, t, k in stages)
+                  + "; stage times scaled to the full stage and summed",
+        "ms_per_step_scaled": round(full_s * 1e3, 1),
+        "cpu_seconds_measured": round(sum(t for _, _, t, _ in stages), 2),
     }
 
 
@@ -463,12 +664,11 @@ def cpu_path_table(gpu_rows, budget_s=3.0):
     def rnd(shape, dtype, std=1.0):
         return (std * torch.randn(shape, generator=g)).to(dtype)
 
-    def gpu_rate(names, cfg, **match):
-        rows = [r for r in gpu_rows if r["kernel"] in names and r["config"] == cfg
-                and all(r.get(k) == v for k, v in match.items())]
+    def gpu_rate(names, cfg, note=None):
+        rows = [r for r in gpu_rows if r[0] in names and r[1] == cfg and (note is None or r[9] == note)]
         if len(rows) != len(names):
             return None
-        return sum(r["algorithmic_MB"] for r in rows) / sum(r["us"] for r in rows) * 1e3
+        return sum(r[2] for r in rows) / sum(r[3] for r in rows) * 1e3
 
     def timed(fn):
         fn()
@@ -516,6 +716,17 @@ def cpu_path_table(gpu_rows, budget_s=3.0):
         entry("layer_norm fwd+bwd", cfg, "[%d,%d] bf16" % (n1, n2), 5 * n1 * n2 * 2, fn,
               gpu_rate(("ln_fwd", "ln_bwd"), cfg))
 
+    def norm_rms(cfg, n1, n2):
+        x, dy = rnd((n1, n2), BF16), rnd((n1, n2), BF16)
+        gamma = rnd((n2,), BF16, 0.02) + 1
+
+        def fn():
+            xr = x.clone().requires_grad_()
+            w = gamma.clone().requires_grad_()
+            tp.rms_norm(xr, w, 1e-5).backward(dy)
+        entry("rms_norm fwd+bwd", cfg, "[%d,%d] bf16" % (n1, n2), 5 * n1 * n2 * 2, fn,
+              gpu_rate(("rms_fwd", "rms_bwd"), cfg))
+
     def gelu(cfg, n1, n2):
         x, dy, b = rnd((n1, n2), BF16), rnd((n1, n2), BF16), rnd((n2,), BF16, 0.02)
 
@@ -532,9 +743,11 @@ def cpu_path_table(gpu_rows, budget_s=3.0):
             xr, br = x.clone().requires_grad_(), b.clone().requires_grad_()
             tp.bias_dropout_add(xr, br, res, 0.1, True).backward(dy)
         entry("bias_dropout_add fwd+bwd (p=0.1)", cfg, "[%d,%d] bf16" % (n1, n2), 5 * n1 * n2 * 2, fn,
-              gpu_rate(("bias_dropout_add_fwd", "bias_dropout_add_bwd"), cfg, p=0.1))
+              gpu_rate(("bias_dropout_add_fwd", "bias_dropout_add_bwd"), cfg, "p=0.1"))
 
     causal("cfg1", 48, 512, F32, 0.125, 4)
+    norm_ln("cfg2", 16384, 4096)
+    norm_rms("cfg2", 16384, 4096)
     # cfg3: two of the sixteen batch entries
     b_, h, s = 2, 16, 1024
     x, dy = rnd((b_, h, s, s), F16, 2.0), rnd((b_, h, s, s), F16)
@@ -577,40 +790,40 @@ def main():
     torch.cuda.set_device(dev)
     L = Lib(torch, _C)
 
-    n1, n2 = 16384, 4096
-    T = n1 * n2 * 2
-    nsets = 4
-    calls = make_norm_calls(L, dev, n1, n2, nsets, seed=0)
+    # the counter summary must hold the roofline kernel's row: fail before timing anything
+    traffic = traffic_from_profile("softmax_bwd_kernel", 131072, 256)
 
-    def step(i):
-        k = i % nsets
-        calls["ln_fwd"](k)
-        calls["ln_bwd"](k)
-        calls["rms_fwd"](k)
-        calls["rms_bwd"](k)
+    calls, keep = make_chain(L, dev)
+    names_bytes = chain_bytes()
+    step_bytes = sum(b for _, b in names_bytes)
+    roof_idx = 3  # softmax_causal_bwd: the step's largest launch
+    roof_bytes = names_bytes[roof_idx][1]
 
-    for i in range(args.warmup):
-        step(i)
+    def step():
+        for fn in calls:
+            fn()
+
+    for _ in range(args.warmup):
+        step()
     torch.cuda.synchronize()
 
     ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
     t0 = time.perf_counter()
     for i in range(args.steps):
-        k = i % nsets
-        calls["ln_fwd"](k)
-        ev[i][0].record()
-        calls["ln_bwd"](k)
-        ev[i][1].record()
-        calls["rms_fwd"](k)
-        calls["rms_bwd"](k)
+        for k, fn in enumerate(calls):
+            if k == roof_idx:
+                ev[i][0].record()
+                fn()
+                ev[i][1].record()
+            else:
+                fn()
     torch.cuda.synchronize()
     t1 = time.perf_counter()
 
-    ms_per_step = (t1 - t0) * 1e3 / args.steps
-    step_bytes = 10 * T
+    ms_per_step = (t1 - t0) * 1e3 / max(args.steps, 1)
     value = step_bytes / (ms_per_step * 1e-3) / 1e9
-    bwd_ms = sum(a.elapsed_time(b) for a, b in ev) / len(ev)
-    achieved = 3 * T / (bwd_ms * 1e-3) / 1e9
+    roof_ms = sum(a.elapsed_time(b) for a, b in ev) / max(len(ev), 1)
+    achieved = roof_bytes / (roof_ms * 1e-3) / 1e9
 
     out = {
         "metric": METRIC,
@@ -626,37 +839,47 @@ def main():
         "dtype": "f32",
         "data": "synthetic",
         "config": {
-            "workload": "BASELINE.json configs[1]: LayerNorm + RMSNorm fwd+bwd, bf16 [16384,4096], eps 1e-5; "
-                        "step = ln_fwd, ln_bwd, rms_fwd, rms_bwd",
+            "workload": "BASELINE.json configs[4]: GPT-NeoX-20B-layer-shaped non-GEMM chain fwd+bwd, bf16, batch 4, "
+                        "seq 2048, hidden 6144, 64 heads; step = ln_fwd, ln_bwd [8192,6144], softmax_causal_fwd, _bwd "
+                        "[256,2048,2048], bias_gelu_fwd, _bwd [8192,24576], bias_dropout_add_fwd, _bwd [8192,6144] p=0.1",
             "io_dtype": "bf16",
             "algorithmic_MB_per_step": round(step_bytes / 1e6, 1),
-            "rotating_buffer_sets": nsets,
+            "algorithmic_MB_per_launch": {n: round(b / 1e6, 1) for n, b in names_bytes},
         },
         "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBPS, 2),
         "roofline": {
-            "kernel": "oslo_ln_bwd = norm_bwd_reg_kernel + colsum_finalize_kernel",
+            "kernel": "oslo_softmax_causal_bwd = softmax_bwd_kernel<bf16, 4 chunks per lane, 1 row per wave, causal> "
+                      "(131072 x 256)",
             "bound": "hbm",
             "achieved": round(achieved, 1),
             "peak": HBM_PEAK_GBPS,
             "unit": "GB/s",
             "frac": round(achieved / HBM_PEAK_GBPS, 4),
-            "traffic": LN_BWD_TRAFFIC_BYTES,
-            "traffic_unit": "HBM bytes per oslo_ln_bwd call, rocprofv3 FETCH_SIZE + WRITE_SIZE scaled by a 1 GiB copy",
-            "algorithmic_MB_per_launch": round(3 * T / 1e6, 1),
-            "avg_us": round(bwd_ms * 1e3, 2),
+            "traffic": traffic,
+            "traffic_unit": "HBM bytes per launch: rocprofv3 FETCH_SIZE + WRITE_SIZE scaled by a 1 GiB copy, read "
+                            "from profiles/bench_all_kernels_hbm_traffic.txt",
+            "algorithmic_MB_per_launch": round(roof_bytes / 1e6, 1),
+            "avg_us": round(roof_ms * 1e3, 2),
         },
     }
-    del calls
+    del calls, keep
     torch.cuda.empty_cache()
 
     if args.table_iters > 0:
-        out["kernels"] = kernel_table(L, dev, args.table_iters)
+        rows = kernel_table(L, dev, args.table_iters, graph_column=not args.no_graph_column)
+        out["kernels"] = {
+            "cols": TABLE_COLS,
+            "units": "MB = algorithmic bytes per launch / 1e6; us = mean over %d launches (events on the launch "
+                     "stream, %d batches), us_med / us_min = median / smallest batch mean; frac = GBps / 8000; "
+                     "graph_us = per launch inside a captured HIP graph" % (args.table_iters, BATCHES),
+            "rows": rows,
+        }
     if not args.no_cpu_baseline:
-        cb = cpu_baseline(n1, n2, args.cpu_reps)
+        cb = cpu_baseline()
         cb["speedup_gpu_over_cpu"] = round(value / cb["value"], 1) if cb["value"] > 0 else None
         out["cpu_baseline"] = cb
         if "kernels" in out:
-            out["cpu_path"] = cpu_path_table(out["kernels"])
+            out["cpu_path"] = cpu_path_table(out["kernels"]["rows"])
     print(json.dumps(out))
 
 
