@@ -371,7 +371,7 @@ int oslo_wave_reduce_selftest(float *out4, void *stream);
  * "norm_fwd_vpl", "norm_bwd_vpl", "norm_bwd_blocks_per_cu", "norm_bwd_waves",
  * "norm_fwd_waves", "norm_bwd_prefetch", "norm_fwd_iters",
  * "norm_lanes_per_row", "softmax_lanes_per_row" (64 switches the
- * side-by-side short rows off, 1 the two-chunks-per-lane forward), "softmax_rows_per_wave",
+ * side-by-side short rows off, 1 the two-chunks-per-lane forward), "softmax_rows_per_wave", "softmax_rows_per_block" (rows, or sets of side-by-side rows, per workgroup: 1..16),
  * "softmax_fwd_elems", "eltwise_unroll", "eltwise_rowgroups",
  * "eltwise_fwd_steps", "eltwise_tile_max", "eltwise_tile_min" (lanes along
  * the columns of an element-wise tile; 64 as the minimum restores whole-wave

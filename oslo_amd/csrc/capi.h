@@ -33,6 +33,7 @@ struct Tuning {
   int softmax_rows_per_wave;
   int softmax_lanes_per_row;
   int softmax_fwd_elems;
+  int softmax_rows_per_block;
   int norm_lanes_per_row;
   int eltwise_tile_max;
   int eltwise_tile_min;

@@ -99,6 +99,7 @@ int oslo_tune(const char *key, int value) {
       {"softmax_rows_per_wave", &oslo::g_tune.softmax_rows_per_wave, kPow2, 1, 4},
       {"softmax_lanes_per_row", &oslo::g_tune.softmax_lanes_per_row, kLanes, 1, 64},
       {"softmax_fwd_elems", &oslo::g_tune.softmax_fwd_elems, kPow2, 16, 64},
+      {"softmax_rows_per_block", &oslo::g_tune.softmax_rows_per_block, kRange, 1, 16},
       {"norm_lanes_per_row", &oslo::g_tune.norm_lanes_per_row, kLanes, 8, 64},
       {"eltwise_tile_max", &oslo::g_tune.eltwise_tile_max, kPow2, 1, 256},
       {"eltwise_tile_min", &oslo::g_tune.eltwise_tile_min, kPow2, 1, 256},

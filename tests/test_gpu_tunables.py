@@ -20,7 +20,7 @@ pytestmark = pytest.mark.gpu
 F32, F16, BF16 = torch.float32, torch.float16, torch.bfloat16
 
 KEYS = [
-    "softmax_rows_per_wave", "softmax_lanes_per_row", "softmax_fwd_elems",
+    "softmax_rows_per_wave", "softmax_lanes_per_row", "softmax_fwd_elems", "softmax_rows_per_block",
     "eltwise_tile_max", "eltwise_tile_min", "eltwise_unroll", "eltwise_rowgroups", "eltwise_fwd_steps",
     "adam_unroll",
 ]
@@ -37,6 +37,8 @@ SOFTMAX_OVERRIDES = [
     ("softmax_rows_per_wave", 1), ("softmax_rows_per_wave", 2), ("softmax_rows_per_wave", 4),
     ("softmax_lanes_per_row", 1), ("softmax_lanes_per_row", 64),
     ("softmax_fwd_elems", 16), ("softmax_fwd_elems", 32), ("softmax_fwd_elems", 64),
+    ("softmax_rows_per_block", 1), ("softmax_rows_per_block", 3), ("softmax_rows_per_block", 4),
+    ("softmax_rows_per_block", 16),
 ]
 
 # (sq, sk, dtype): one to eight chunks per lane, one or several waves per row
