@@ -1098,7 +1098,8 @@ static SoftmaxPlan plan_softmax(int64_t sk, int E, int max_elems,
       p.vpl = 2;
       p.rpw = want >= 2 && 2 * 2 * E <= max_elems ? 2 : 1;
       p.wpr = 1;
-      p.rpb = g_tune.softmax_rows_per_block > 0 ? g_tune.softmax_rows_per_block : 4;
+      // (one wave per workgroup: 6 % faster at sequence length 128)
+      p.rpb = g_tune.softmax_rows_per_block > 0 ? g_tune.softmax_rows_per_block : 1;
       p.lpr = (int)q;
       p.ok = true;
       return p;
