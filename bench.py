@@ -417,6 +417,34 @@ def kernel_table(L, dev, iters, graph_column=True):
     del bufs
     torch.cuda.empty_cache()
 
+    # ---- causal + key-padding mask in one call, cfg5 shape [4,64,2048,2048]
+    # bf16 with valid lengths ~ U[1024, 2048]: reads stop at the diagonal and
+    # at the valid length, whichever comes first ----
+    b, h, s = 4, 64, 2048
+    T = b * h * s * s * 2
+    g = torch.Generator(device=dev).manual_seed(6)
+    valid = torch.randint(1024, 2049, (b,), generator=torch.Generator().manual_seed(6))
+    qi = torch.arange(1, s + 1, dtype=torch.float64)
+    r = float(torch.minimum(qi[None, :], valid[:, None].double()).mean()) / s
+    mask = (torch.arange(s)[None, :] >= valid[:, None]).view(b, 1, 1, s).to(dev).view(torch.uint8)
+    x = torch.randn(b, h, s, s, generator=g, device=dev).to(torch.bfloat16)
+    dy = torch.randn(b, h, s, s, generator=g, device=dev).to(torch.bfloat16)
+    y, dx = torch.empty_like(x), torch.empty_like(x)
+    sc = 1.0 / math.sqrt(96.0)
+
+    def cmfwd(i):
+        L.ok(lib.oslo_softmax_causal_masked_fwd(p(x), p(mask), p(y), b, h, s, s, b, 1, sc, BF16, L.stream()))
+
+    def cmbwd(i):
+        L.ok(lib.oslo_softmax_causal_masked_bwd(p(dy), p(y), p(mask), p(dx), b, h, s, s, b, 1, sc, BF16, L.stream()))
+
+    rows.append(table_row("softmax_causal_masked_fwd", "cfg5pad", (r + 1) * T, timed(cmfwd, 1),
+                          note="visible %.4f of the square" % r))
+    rows.append(table_row("softmax_causal_masked_bwd", "cfg5pad", (2 * r + 1) * T, timed(cmbwd, 1),
+                          note="visible %.4f of the square" % r))
+    del x, dy, y, dx
+    torch.cuda.empty_cache()
+
     # ---- bias-GeLU: cfg4 and cfg5 ----
     for cfg, n1, n2 in (("cfg4", 16384, 16384), ("cfg5", 8192, 24576)):
         T = n1 * n2 * 2

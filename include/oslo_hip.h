@@ -171,6 +171,27 @@ int oslo_softmax_masked_bwd(const void *dy, const void *y, const uint8_t *mask,
                             int64_t sk, int64_t mask_b, int64_t mask_sq,
                             float scale, int dtype, void *stream);
 
+/* Causal mask and padding mask in one call: the attention of a causal model
+ * that is run on padded batches.  The reference applies both,
+ * torch.where(causal, w, -1e4) followed by "+ attention_mask"
+ * (oslo/transformers/models/gpt2/modeling_gpt2.py:126-136, mask built at
+ * :573-581); its softmax shim has no entry point for the combination.  Same
+ * arguments as oslo_softmax_masked_fwd / _bwd; key j of query i is hidden when
+ * the mask says so OR j > i + (sk - sq).  Loads stop at the diagonal as in
+ * oslo_softmax_causal_fwd, and mask bytes beyond it are not read.  Hidden
+ * keys get probability exactly 0; a row without any visible key (a fully
+ * padded sample, left padding) becomes the uniform 1/sk, as in
+ * oslo_softmax_masked_fwd.  In the backward entry point mask may be NULL.   */
+int oslo_softmax_causal_masked_fwd(const void *x, const uint8_t *mask, void *y,
+                                   int64_t b, int64_t np, int64_t sq,
+                                   int64_t sk, int64_t mask_b, int64_t mask_sq,
+                                   float scale, int dtype, void *stream);
+int oslo_softmax_causal_masked_bwd(const void *dy, const void *y,
+                                   const uint8_t *mask, void *dx, int64_t b,
+                                   int64_t np, int64_t sq, int64_t sk,
+                                   int64_t mask_b, int64_t mask_sq, float scale,
+                                   int dtype, void *stream);
+
 /* Replaces get_batch_per_block (FusedScaleMaskSoftmaxBinder.cpp:66-70,
  * 118-121): softmax rows one workgroup of the masked kernel handles.  The
  * kernels here have no divisibility requirement on it.  Negative on error. */
@@ -217,6 +238,24 @@ int oslo_softmax_masked_dropout_bwd(const void *dout, const void *x,
                                     int64_t sk, int64_t mask_b, int64_t mask_sq,
                                     float scale, float p, uint64_t seed,
                                     uint64_t offset, int dtype, void *stream);
+
+/* The same pair for the causal + padding mask combination
+ * (oslo_softmax_causal_masked_fwd above).                                   */
+int oslo_softmax_causal_masked_dropout_fwd(const void *x, const uint8_t *mask,
+                                           void *out, float *stats, int64_t b,
+                                           int64_t np, int64_t sq, int64_t sk,
+                                           int64_t mask_b, int64_t mask_sq,
+                                           float scale, float p, uint64_t seed,
+                                           uint64_t offset, int dtype,
+                                           void *stream);
+int oslo_softmax_causal_masked_dropout_bwd(const void *dout, const void *x,
+                                           const uint8_t *mask,
+                                           const float *stats, void *dx,
+                                           int64_t b, int64_t np, int64_t sq,
+                                           int64_t sk, int64_t mask_b,
+                                           int64_t mask_sq, float scale, float p,
+                                           uint64_t seed, uint64_t offset,
+                                           int dtype, void *stream);
 
 /* ---- dropout state in device memory ------------------------------------- *
  * No counterpart in the reference.  For callers that capture launches in a

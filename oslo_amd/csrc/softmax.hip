@@ -33,6 +33,7 @@ struct SoftmaxGeom {
   int mask_b_stride_rows;  // mask rows per batch entry: mask_sq, or 0 if mask_b == 1
   int mask_per_query;      // 1 if mask_sq == sq else 0
   int wpr, rpb;     // waves per row, rows per workgroup pass (without RPW)
+  int causal;       // masked mode: key j of query i is also hidden when j > i + (sk - sq)
 };
 
 // Reductions over the wpr (<= 16) consecutive waves of a row: lane 0 of each
@@ -88,6 +89,20 @@ __device__ __forceinline__ uint32_t load_mask_bits(const uint8_t *p) {
   return bits;
 }
 
+// Mask bits of chunk c (E keys) of a row that sees `visible` keys through the
+// diagonal: the keys from `visible` on are hidden as well.  Chunks that lie
+// beyond the diagonal altogether do not read their mask bytes.
+template <int E>
+__device__ __forceinline__ uint32_t masked_chunk_bits(const uint8_t *mrow, int c,
+                                                      int visible) {
+  constexpr uint32_t kAllBits = (1u << E) - 1u;
+  const int left = visible - c * E;  // keys of the chunk below the diagonal
+  if (left <= 0) return kAllBits;
+  uint32_t mb = load_mask_bits<E>(mrow + (int64_t)c * E);
+  if (left < E) mb |= kAllBits & ~((1u << left) - 1u);
+  return mb;
+}
+
 // Row bookkeeping shared by forward and backward.  Rows are numbered so that
 // a workgroup's rows are consecutive; in causal mode the order inside an
 // attention batch is reversed (long rows first) so the tail of the launch
@@ -113,7 +128,13 @@ __device__ __forceinline__ void row_setup(const SoftmaxGeom &g, int64_t r,
   } else if constexpr (MODE == kModeMasked) {
     const int64_t bh =
         small ? (int64_t)((uint32_t)r / (uint32_t)g.sq) : r / g.sq;
-    const int qi = (int)(r - bh * g.sq);
+    int qi = (int)(r - bh * g.sq);
+    if (g.causal) {  // uniform over the launch: long rows first, as in causal mode
+      qi = g.sq - 1 - qi;
+      row = bh * g.sq + qi;
+      const int v = qi + 1 + (g.sk - g.sq);
+      visible = v < 0 ? 0 : (v > g.sk ? g.sk : v);
+    }
     const int64_t bi =
         small ? (int64_t)((uint32_t)bh / (uint32_t)g.np) : bh / g.np;
     const int64_t mr =
@@ -180,7 +201,7 @@ __global__ __launch_bounds__(1024) void softmax_fwd_kernel(
           const int left = visible - c * E;  // visible keys in this chunk
           mb = left >= E ? 0u : (left <= 0 ? mb : (mb & ~((1u << left) - 1u)));
         } else {
-          mb = load_mask_bits<E>(mrow + (int64_t)c * E);
+          mb = masked_chunk_bits<E>(mrow, c, visible);
         }
       }
       mbits[j][k] = mb;
@@ -403,7 +424,7 @@ __global__ __launch_bounds__(1024) void softmax_dropout_bwd_kernel(
           const int left = visible - c * E;
           mb = left >= E ? 0u : (left <= 0 ? mb : (mb & ~((1u << left) - 1u)));
         } else {
-          mb = load_mask_bits<E>(mrow + (int64_t)c * E);
+          mb = masked_chunk_bits<E>(mrow, c, visible);
         }
       }
       mbits[j][k] = mb;
@@ -533,7 +554,7 @@ __global__ __launch_bounds__(1024) void softmax_bwd_kernel(
         if constexpr (MODE == kModeCausal) {
           sk_ = visible - c * E <= 0;
         } else if constexpr (MODE == kModeMasked) {
-          sk_ = load_mask_bits<E>(mrow + (int64_t)c * E) == kAll;
+          sk_ = masked_chunk_bits<E>(mrow, c, visible) == kAll;
         } else {
           sk_ = false;
         }
@@ -652,14 +673,14 @@ __global__ __launch_bounds__(256) void softmax_fwd_generic_kernel(
     T *yr = y + row * g.sk;
     float m = ninf;
     for (int i = threadIdx.x; i < g.sk; i += 256) {
-      const bool hidden = MODE == kModeCausal ? i >= visible : mrow[i] != 0;
+      const bool hidden = MODE == kModeCausal ? i >= visible : (mrow[i] != 0 || i >= visible);
       if (!hidden) m = fmaxf(m, mul_rn(io<T>::from_scalar(xr[i]), c2));
     }
     m = block_reduce_256(m, sh, true);
     const bool empty = m == ninf;
     float s = 0.f;
     for (int i = threadIdx.x; i < g.sk; i += 256) {
-      const bool hidden = MODE == kModeCausal ? i >= visible : mrow[i] != 0;
+      const bool hidden = MODE == kModeCausal ? i >= visible : (mrow[i] != 0 || i >= visible);
       if (!hidden)
         s += __builtin_amdgcn_exp2f(
             sub_rn(mul_rn(io<T>::from_scalar(xr[i]), c2), m));
@@ -668,7 +689,7 @@ __global__ __launch_bounds__(256) void softmax_fwd_generic_kernel(
     const float inv = empty ? 0.f : 1.0f / s;
     const float fill = empty ? 1.0f / (float)g.sk : 0.f;
     for (int i = threadIdx.x; i < g.sk; i += 256) {
-      const bool hidden = MODE == kModeCausal ? i >= visible : mrow[i] != 0;
+      const bool hidden = MODE == kModeCausal ? i >= visible : (mrow[i] != 0 || i >= visible);
       float p = 0.f;
       if (!hidden)
         p = __builtin_amdgcn_exp2f(
@@ -707,7 +728,7 @@ __global__ __launch_bounds__(256) void softmax_dropout_bwd_generic_kernel(
     const bool empty = inv < 0.f;
     auto prob = [&](int i) {
       if (empty) return -inv;
-      const bool hidden = MODE == kModeCausal ? i >= visible : mrow[i] != 0;
+      const bool hidden = MODE == kModeCausal ? i >= visible : (mrow[i] != 0 || i >= visible);
       if (hidden) return 0.f;
       return __builtin_amdgcn_exp2f(
                  sub_rn(mul_rn(io<T>::from_scalar(xr[i]), c2), m)) *
@@ -850,14 +871,15 @@ __global__ __launch_bounds__(256) void softmax_fwd_wave_kernel(
         // mask first measures 30 % slower than the loads it can save)
         uint32_t hid = 0;
         if constexpr (MODE != kModeCausal) hid = ld_mask_small<EW>(mrow + i0);
-        const bool none = MODE == kModeCausal ? i0 >= visible : false;
+        const bool none = i0 >= visible;  // (visible == sk without a diagonal)
         if (!none) {
           float t[EW];
           ld_small<T, EW>(xr + i0, t);
 #pragma unroll
           for (int e = 0; e < EW; ++e) {
             const bool hidden =
-                MODE == kModeCausal ? i0 + e >= visible : ((hid >> e) & 1u) != 0;
+                MODE == kModeCausal ? i0 + e >= visible
+                                    : (((hid >> e) & 1u) != 0 || i0 + e >= visible);
             if (!hidden) v[k][e] = mul_rn(t[e], c2);
             m = fmaxf(m, v[k][e]);
           }
@@ -939,7 +961,7 @@ __global__ __launch_bounds__(256) void softmax_dropout_bwd_wave_kernel(
         if constexpr (MODE != kModeCausal) hid = ld_mask_small<EW>(mrow + i0);
         // keys beyond the diagonal contribute nothing and are not loaded
         // (a row without a visible key is uniform: every key counts)
-        none = !empty && (MODE == kModeCausal ? i0 >= visible : false);
+        none = !empty && i0 >= visible;
       }
       if (!none) {
         float xt[EW], gt[EW];
@@ -949,7 +971,8 @@ __global__ __launch_bounds__(256) void softmax_dropout_bwd_wave_kernel(
 #pragma unroll
         for (int e = 0; e < EW; ++e) {
           const bool hidden =
-              MODE == kModeCausal ? i0 + e >= visible : ((hid >> e) & 1u) != 0;
+              MODE == kModeCausal ? i0 + e >= visible
+                                  : (((hid >> e) & 1u) != 0 || i0 + e >= visible);
           float p = 0.f;
           if (empty)
             p = -inv;
@@ -1442,7 +1465,7 @@ int oslo_softmax_causal_bwd(const void *dy, const void *y, void *dx,
 
 static int masked_geom(const char *what, int64_t b, int64_t np, int64_t sq,
                        int64_t sk, int64_t mask_b, int64_t mask_sq,
-                       SoftmaxGeom *g) {
+                       SoftmaxGeom *g, int causal = 0) {
   if (b < 0 || np < 0 || np > 0x7fffffff)
     return fail(OSLO_ERR_INVALID_ARGUMENT, "%s: bad batch/head count", what);
   if (!(mask_b == 1 || mask_b == b) || !(mask_sq == 1 || mask_sq == sq))
@@ -1458,45 +1481,83 @@ static int masked_geom(const char *what, int64_t b, int64_t np, int64_t sq,
                    (int)(mask_b == 1 ? 0 : mask_sq),
                    (int)(mask_sq == sq && sq != 1 ? 1 : 0),
                    1,
-                   1};
+                   1,
+                   causal};
   return OSLO_OK;
 }
 
-int oslo_softmax_masked_fwd(const void *x, const uint8_t *mask, void *y,
-                            int64_t b, int64_t np, int64_t sq, int64_t sk,
-                            int64_t mask_b, int64_t mask_sq, float scale,
-                            int dtype, void *stream) {
-  int rc = check_softmax_shape("softmax masked fwd", b, sq, sk, dtype);
+static int masked_fwd_entry(const char *what, int causal, const void *x,
+                            const uint8_t *mask, void *y, int64_t b, int64_t np,
+                            int64_t sq, int64_t sk, int64_t mask_b,
+                            int64_t mask_sq, float scale, int dtype,
+                            void *stream) {
+  int rc = check_softmax_shape(what, b, sq, sk, dtype);
   if (rc != OSLO_OK) return rc;
   SoftmaxGeom g;
-  rc = masked_geom("softmax masked fwd", b, np, sq, sk, mask_b, mask_sq, &g);
+  rc = masked_geom(what, b, np, sq, sk, mask_b, mask_sq, &g, causal);
   if (rc != OSLO_OK) return rc;
   if (g.rows == 0) return OSLO_OK;
-  OSLO_REQUIRE(x && y && mask, "softmax masked fwd: null tensor pointer");
+  OSLO_REQUIRE(x && y && mask, "%s: null tensor pointer", what);
   OSLO_SM_DISPATCH(dtype, kModeMasked, launch_softmax_fwd, x, mask, y, nullptr,
                    DropArgs{}, g, scale, (hipStream_t)stream);
 }
 
-int oslo_softmax_masked_bwd(const void *dy, const void *y, const uint8_t *mask,
-                            void *dx, int64_t b, int64_t np, int64_t sq,
-                            int64_t sk, int64_t mask_b, int64_t mask_sq,
-                            float scale, int dtype, void *stream) {
-  int rc = check_softmax_shape("softmax masked bwd", b, sq, sk, dtype);
+static int masked_bwd_entry(const char *what, int causal, const void *dy,
+                            const void *y, const uint8_t *mask, void *dx,
+                            int64_t b, int64_t np, int64_t sq, int64_t sk,
+                            int64_t mask_b, int64_t mask_sq, float scale,
+                            int dtype, void *stream) {
+  int rc = check_softmax_shape(what, b, sq, sk, dtype);
   if (rc != OSLO_OK) return rc;
   SoftmaxGeom g;
   if (mask == nullptr) {
     mask_b = 1;
     mask_sq = 1;
   }
-  rc = masked_geom("softmax masked bwd", b, np, sq, sk, mask_b, mask_sq, &g);
+  rc = masked_geom(what, b, np, sq, sk, mask_b, mask_sq, &g, causal);
   if (rc != OSLO_OK) return rc;
   if (g.rows == 0) return OSLO_OK;
-  OSLO_REQUIRE(dy && y && dx, "softmax masked bwd: null tensor pointer");
+  OSLO_REQUIRE(dy && y && dx, "%s: null tensor pointer", what);
+  // without the mask every key is read: a row that had no visible key holds
+  // the uniform distribution, beyond the diagonal too
   if (mask == nullptr)
     OSLO_SM_DISPATCH(dtype, kModeDense, launch_softmax_bwd, dy, y, nullptr, dx,
                      g, scale, (hipStream_t)stream);
   OSLO_SM_DISPATCH(dtype, kModeMasked, launch_softmax_bwd, dy, y, mask, dx, g,
                    scale, (hipStream_t)stream);
+}
+
+int oslo_softmax_masked_fwd(const void *x, const uint8_t *mask, void *y,
+                            int64_t b, int64_t np, int64_t sq, int64_t sk,
+                            int64_t mask_b, int64_t mask_sq, float scale,
+                            int dtype, void *stream) {
+  return masked_fwd_entry("softmax masked fwd", 0, x, mask, y, b, np, sq, sk,
+                          mask_b, mask_sq, scale, dtype, stream);
+}
+
+int oslo_softmax_masked_bwd(const void *dy, const void *y, const uint8_t *mask,
+                            void *dx, int64_t b, int64_t np, int64_t sq,
+                            int64_t sk, int64_t mask_b, int64_t mask_sq,
+                            float scale, int dtype, void *stream) {
+  return masked_bwd_entry("softmax masked bwd", 0, dy, y, mask, dx, b, np, sq,
+                          sk, mask_b, mask_sq, scale, dtype, stream);
+}
+
+int oslo_softmax_causal_masked_fwd(const void *x, const uint8_t *mask, void *y,
+                                   int64_t b, int64_t np, int64_t sq,
+                                   int64_t sk, int64_t mask_b, int64_t mask_sq,
+                                   float scale, int dtype, void *stream) {
+  return masked_fwd_entry("softmax causal masked fwd", 1, x, mask, y, b, np, sq,
+                          sk, mask_b, mask_sq, scale, dtype, stream);
+}
+
+int oslo_softmax_causal_masked_bwd(const void *dy, const void *y,
+                                   const uint8_t *mask, void *dx, int64_t b,
+                                   int64_t np, int64_t sq, int64_t sk,
+                                   int64_t mask_b, int64_t mask_sq, float scale,
+                                   int dtype, void *stream) {
+  return masked_bwd_entry("softmax causal masked bwd", 1, dy, y, mask, dx, b,
+                          np, sq, sk, mask_b, mask_sq, scale, dtype, stream);
 }
 
 int oslo_softmax_batch_per_block(int64_t sq, int64_t sk, int64_t b,
@@ -1556,24 +1617,53 @@ int oslo_softmax_causal_dropout_bwd(const void *dout, const void *x,
                    (hipStream_t)stream);
 }
 
+static int masked_dropout_fwd_entry(const char *what, int causal, const void *x,
+                                    const uint8_t *mask, void *out, float *stats,
+                                    int64_t b, int64_t np, int64_t sq,
+                                    int64_t sk, int64_t mask_b, int64_t mask_sq,
+                                    float scale, float p, uint64_t seed,
+                                    uint64_t offset, int dtype, void *stream) {
+  int rc = check_softmax_shape(what, b, sq, sk, dtype);
+  if (rc == OSLO_OK) rc = check_dropout_p(what, p);
+  if (rc != OSLO_OK) return rc;
+  SoftmaxGeom g;
+  rc = masked_geom(what, b, np, sq, sk, mask_b, mask_sq, &g, causal);
+  if (rc != OSLO_OK) return rc;
+  if (g.rows == 0) return OSLO_OK;
+  OSLO_REQUIRE(x && out && mask && stats, "%s: null pointer", what);
+  OSLO_SM_DISPATCH(dtype, kModeMasked, launch_softmax_fwd, x, mask, out, stats,
+                   make_drop(p, seed, offset), g, scale, (hipStream_t)stream);
+}
+
+static int masked_dropout_bwd_entry(const char *what, int causal,
+                                    const void *dout, const void *x,
+                                    const uint8_t *mask, const float *stats,
+                                    void *dx, int64_t b, int64_t np, int64_t sq,
+                                    int64_t sk, int64_t mask_b, int64_t mask_sq,
+                                    float scale, float p, uint64_t seed,
+                                    uint64_t offset, int dtype, void *stream) {
+  int rc = check_softmax_shape(what, b, sq, sk, dtype);
+  if (rc == OSLO_OK) rc = check_dropout_p(what, p);
+  if (rc != OSLO_OK) return rc;
+  SoftmaxGeom g;
+  rc = masked_geom(what, b, np, sq, sk, mask_b, mask_sq, &g, causal);
+  if (rc != OSLO_OK) return rc;
+  if (g.rows == 0) return OSLO_OK;
+  OSLO_REQUIRE(dout && x && mask && stats && dx, "%s: null pointer", what);
+  OSLO_SM_DISPATCH(dtype, kModeMasked, launch_softmax_dropout_bwd, dout, x,
+                   stats, mask, dx, make_drop(p, seed, offset), g, scale,
+                   (hipStream_t)stream);
+}
+
 int oslo_softmax_masked_dropout_fwd(const void *x, const uint8_t *mask,
                                     void *out, float *stats, int64_t b,
                                     int64_t np, int64_t sq, int64_t sk,
                                     int64_t mask_b, int64_t mask_sq,
                                     float scale, float p, uint64_t seed,
                                     uint64_t offset, int dtype, void *stream) {
-  const char *what = "softmax masked dropout fwd";
-  int rc = check_softmax_shape(what, b, sq, sk, dtype);
-  if (rc == OSLO_OK) rc = check_dropout_p(what, p);
-  if (rc != OSLO_OK) return rc;
-  SoftmaxGeom g;
-  rc = masked_geom(what, b, np, sq, sk, mask_b, mask_sq, &g);
-  if (rc != OSLO_OK) return rc;
-  if (g.rows == 0) return OSLO_OK;
-  OSLO_REQUIRE(x && out && mask && stats,
-               "softmax masked dropout fwd: null pointer");
-  OSLO_SM_DISPATCH(dtype, kModeMasked, launch_softmax_fwd, x, mask, out, stats,
-                   make_drop(p, seed, offset), g, scale, (hipStream_t)stream);
+  return masked_dropout_fwd_entry("softmax masked dropout fwd", 0, x, mask, out,
+                                  stats, b, np, sq, sk, mask_b, mask_sq, scale,
+                                  p, seed, offset, dtype, stream);
 }
 
 int oslo_softmax_masked_dropout_bwd(const void *dout, const void *x,
@@ -1582,19 +1672,37 @@ int oslo_softmax_masked_dropout_bwd(const void *dout, const void *x,
                                     int64_t sk, int64_t mask_b, int64_t mask_sq,
                                     float scale, float p, uint64_t seed,
                                     uint64_t offset, int dtype, void *stream) {
-  const char *what = "softmax masked dropout bwd";
-  int rc = check_softmax_shape(what, b, sq, sk, dtype);
-  if (rc == OSLO_OK) rc = check_dropout_p(what, p);
-  if (rc != OSLO_OK) return rc;
-  SoftmaxGeom g;
-  rc = masked_geom(what, b, np, sq, sk, mask_b, mask_sq, &g);
-  if (rc != OSLO_OK) return rc;
-  if (g.rows == 0) return OSLO_OK;
-  OSLO_REQUIRE(dout && x && mask && stats && dx,
-               "softmax masked dropout bwd: null pointer");
-  OSLO_SM_DISPATCH(dtype, kModeMasked, launch_softmax_dropout_bwd, dout, x,
-                   stats, mask, dx, make_drop(p, seed, offset), g, scale,
-                   (hipStream_t)stream);
+  return masked_dropout_bwd_entry("softmax masked dropout bwd", 0, dout, x,
+                                  mask, stats, dx, b, np, sq, sk, mask_b,
+                                  mask_sq, scale, p, seed, offset, dtype,
+                                  stream);
+}
+
+int oslo_softmax_causal_masked_dropout_fwd(const void *x, const uint8_t *mask,
+                                           void *out, float *stats, int64_t b,
+                                           int64_t np, int64_t sq, int64_t sk,
+                                           int64_t mask_b, int64_t mask_sq,
+                                           float scale, float p, uint64_t seed,
+                                           uint64_t offset, int dtype,
+                                           void *stream) {
+  return masked_dropout_fwd_entry("softmax causal masked dropout fwd", 1, x,
+                                  mask, out, stats, b, np, sq, sk, mask_b,
+                                  mask_sq, scale, p, seed, offset, dtype,
+                                  stream);
+}
+
+int oslo_softmax_causal_masked_dropout_bwd(const void *dout, const void *x,
+                                           const uint8_t *mask,
+                                           const float *stats, void *dx,
+                                           int64_t b, int64_t np, int64_t sq,
+                                           int64_t sk, int64_t mask_b,
+                                           int64_t mask_sq, float scale, float p,
+                                           uint64_t seed, uint64_t offset,
+                                           int dtype, void *stream) {
+  return masked_dropout_bwd_entry("softmax causal masked dropout bwd", 1, dout,
+                                  x, mask, stats, dx, b, np, sq, sk, mask_b,
+                                  mask_sq, scale, p, seed, offset, dtype,
+                                  stream);
 }
 
 }

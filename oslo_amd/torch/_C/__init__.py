@@ -77,6 +77,24 @@ _SIGNATURES = {
         _int,
         [_p, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _i64, _f32, _int, _p],
     ),
+    "oslo_softmax_causal_masked_fwd": (
+        _int,
+        [_p, _p, _p, _i64, _i64, _i64, _i64, _i64, _i64, _f32, _int, _p],
+    ),
+    "oslo_softmax_causal_masked_bwd": (
+        _int,
+        [_p, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _i64, _f32, _int, _p],
+    ),
+    "oslo_softmax_causal_masked_dropout_fwd": (
+        _int,
+        [_p, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _i64, _f32, _f32, _u64, _u64,
+         _int, _p],
+    ),
+    "oslo_softmax_causal_masked_dropout_bwd": (
+        _int,
+        [_p, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _i64, _f32, _f32, _u64,
+         _u64, _int, _p],
+    ),
     "oslo_softmax_batch_per_block": (_int, [_i64, _i64, _i64, _i64]),
     "oslo_softmax_causal_dropout_fwd": (
         _int,
@@ -564,7 +582,9 @@ class _SoftmaxKernel:
             return mask.contiguous()
         return (mask != 0).contiguous().view(torch.uint8)
 
-    def fused_scaled_masked_softmax_forward(self, input, mask, scale_factor):
+    def fused_scaled_masked_softmax_forward(self, input, mask, scale_factor, causal=False):
+        """``causal=True`` (not in the reference's shim) hides the keys beyond
+        the diagonal as well: causal attention on a padded batch."""
         lib = self._lib
         if input.dim() != 4:
             raise RuntimeError("expected 4D tensor")
@@ -581,7 +601,8 @@ class _SoftmaxKernel:
         m8 = self._mask_u8(mask)
         out = torch.empty_like(input)
         with _device_of(input):
-            rc = lib.oslo_softmax_masked_fwd(
+            fn = lib.oslo_softmax_causal_masked_fwd if causal else lib.oslo_softmax_masked_fwd
+            rc = fn(
                 _ptr(input), _ptr(m8), _ptr(out), b, np_, sq, sk, mb, msq,
                 float(scale_factor), _dtype_code(input, "input"), _stream(input),
             )
@@ -589,7 +610,8 @@ class _SoftmaxKernel:
         return out
 
     def fused_scaled_masked_softmax_backward(
-        self, output_grads, softmax_results, scale_factor, mask=None, inplace=False
+        self, output_grads, softmax_results, scale_factor, mask=None, inplace=False,
+        causal=False,
     ):
         lib = self._lib
         if output_grads.dim() != 4 or softmax_results.dim() != 4:
@@ -608,7 +630,8 @@ class _SoftmaxKernel:
         # written for does
         grad_input = output_grads if inplace else torch.empty_like(output_grads)
         with _device_of(output_grads):
-            rc = lib.oslo_softmax_masked_bwd(
+            fn = lib.oslo_softmax_causal_masked_bwd if causal else lib.oslo_softmax_masked_bwd
+            rc = fn(
                 _ptr(output_grads), _ptr(softmax_results), _ptr(m8), _ptr(grad_input),
                 b, np_, sq, sk, mb, msq, float(scale_factor),
                 _dtype_code(output_grads, "output_grads"), _stream(output_grads),
@@ -676,13 +699,14 @@ class _SoftmaxKernel:
             )
         return b, np_, sq, sk, mb, msq
 
-    def softmax_dropout_forward(self, input, mask, scale_factor, p, seed, offset):
+    def softmax_dropout_forward(self, input, mask, scale_factor, p, seed, offset, causal=False):
         """``dropout(softmax(mask(scale * input)), p)`` -> ``[out, stats]``.
 
         ``mask=None`` selects the causal form on a 3-D ``[attn_batches, sq, sk]``
         input, otherwise ``input`` is ``[b, np, sq, sk]`` and ``mask`` a 4-D
-        padding mask.  ``stats`` (float32 ``[rows, 2]``) and ``input`` are what
-        the backward pass needs.
+        padding mask (with ``causal=True`` the keys beyond the diagonal are
+        hidden as well).  ``stats`` (float32 ``[rows, 2]``) and ``input`` are
+        what the backward pass needs.
         """
         lib = self._lib
         _check_input(input, "input")
@@ -702,7 +726,9 @@ class _SoftmaxKernel:
             else:
                 b, np_, sq, sk, mb, msq = self._masked_dims(input, mask)
                 m8 = self._mask_u8(mask)
-                rc = lib.oslo_softmax_masked_dropout_fwd(
+                fn = (lib.oslo_softmax_causal_masked_dropout_fwd if causal
+                      else lib.oslo_softmax_masked_dropout_fwd)
+                rc = fn(
                     _ptr(input), _ptr(m8), _ptr(out), _ptr(stats), b, np_, sq, sk,
                     mb, msq, float(scale_factor), float(p), int(seed), int(offset),
                     _dtype_code(input, "input"), _stream(input),
@@ -712,7 +738,7 @@ class _SoftmaxKernel:
 
     def softmax_dropout_backward(
         self, output_grads, input, stats, mask, scale_factor, p, seed, offset,
-        inplace=False,
+        inplace=False, causal=False,
     ):
         lib = self._lib
         _check_input(output_grads, "output_grads")
@@ -737,7 +763,9 @@ class _SoftmaxKernel:
             else:
                 b, np_, sq, sk, mb, msq = self._masked_dims(input, mask)
                 m8 = self._mask_u8(mask)
-                rc = lib.oslo_softmax_masked_dropout_bwd(
+                fn = (lib.oslo_softmax_causal_masked_dropout_bwd if causal
+                      else lib.oslo_softmax_masked_dropout_bwd)
+                rc = fn(
                     _ptr(output_grads), _ptr(input), _ptr(m8), _ptr(stats),
                     _ptr(grad_input), b, np_, sq, sk, mb, msq, float(scale_factor),
                     float(p), int(seed), int(offset), _dtype_code(input, "input"),

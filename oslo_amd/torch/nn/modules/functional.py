@@ -433,16 +433,18 @@ class _ScaledMaskedSoftmax(torch.autograd.Function):
     """
     Fused: scale -> padding mask -> softmax, on [b, np, sq, sk] with a
     [b or 1, 1, sq or 1, sk] mask, True = masked out
-    (FusedScaleMaskSoftmaxBinder.cpp:39-70).
+    (FusedScaleMaskSoftmaxBinder.cpp:39-70).  ``causal=True`` hides the keys
+    beyond the diagonal as well, the combination a causal model applies to a
+    padded batch (oslo/transformers/models/gpt2/modeling_gpt2.py:126-136).
     """
 
     @staticmethod
-    def forward(ctx, inputs, mask, scale):
+    def forward(ctx, inputs, mask, scale, causal=False):
         scale = float(scale)
         softmax_results = get_softmax_kernel().fused_scaled_masked_softmax_forward(
-            inputs.contiguous(), mask, scale
+            inputs.contiguous(), mask, scale, causal=causal
         )
-        ctx.scale = scale
+        ctx.scale, ctx.causal = scale, bool(causal)
         ctx.save_for_backward(softmax_results, mask)
         return softmax_results
 
@@ -450,9 +452,9 @@ class _ScaledMaskedSoftmax(torch.autograd.Function):
     def backward(ctx, output_grads):
         softmax_results, mask = ctx.saved_tensors
         input_grads = get_softmax_kernel().fused_scaled_masked_softmax_backward(
-            output_grads.contiguous(), softmax_results, ctx.scale, mask=mask
+            output_grads.contiguous(), softmax_results, ctx.scale, mask=mask, causal=ctx.causal
         )
-        return input_grads, None, None
+        return input_grads, None, None, None
 
 
 class _ScaledMaskedSoftmaxDropout(torch.autograd.Function):
@@ -469,14 +471,15 @@ class _ScaledMaskedSoftmaxDropout(torch.autograd.Function):
     """
 
     @staticmethod
-    def forward(ctx, inputs, mask, scale, p, seed, offset):
+    def forward(ctx, inputs, mask, scale, p, seed, offset, causal=False):
         scale = float(scale)
         inputs = inputs.contiguous()
         with _rng(seed):
             out, stats = get_softmax_kernel().softmax_dropout_forward(
-                inputs, mask, scale, p, _seed_arg(seed), offset
+                inputs, mask, scale, p, _seed_arg(seed), offset, causal=causal
             )
         ctx.scale, ctx.p, ctx.seed, ctx.offset = scale, p, seed, offset
+        ctx.causal = bool(causal)
         ctx.has_mask = mask is not None
         if mask is not None:
             ctx.save_for_backward(inputs, stats, mask)
@@ -493,9 +496,9 @@ class _ScaledMaskedSoftmaxDropout(torch.autograd.Function):
         with _rng(ctx.seed):
             input_grads = get_softmax_kernel().softmax_dropout_backward(
                 output_grads.contiguous(), inputs, stats, mask, ctx.scale, ctx.p,
-                _seed_arg(ctx.seed), ctx.offset,
+                _seed_arg(ctx.seed), ctx.offset, causal=ctx.causal,
             )
-        return input_grads, None, None, None, None, None
+        return input_grads, None, None, None, None, None, None
 
 
 """
@@ -624,9 +627,10 @@ def scaled_upper_triang_masked_softmax(input, scale=1.0):
     return _ScaledUpperTriangMaskedSoftmax.apply(input, scale)
 
 
-def scaled_masked_softmax(input, mask, scale=1.0):
-    """softmax(scale * input) with `mask` (True = masked out); input is [b, np, sq, sk]."""
-    return _ScaledMaskedSoftmax.apply(input, mask, scale)
+def scaled_masked_softmax(input, mask, scale=1.0, causal=False):
+    """softmax(scale * input) with `mask` (True = masked out); input is [b, np, sq, sk].
+    With ``causal=True`` key j of query i is hidden when j > i + (sk - sq) as well."""
+    return _ScaledMaskedSoftmax.apply(input, mask, scale, causal)
 
 
 def _check_dropout_p(p):
@@ -646,11 +650,12 @@ def scaled_upper_triang_masked_softmax_dropout(input, scale=1.0, p=0.0, training
     return _ScaledMaskedSoftmaxDropout.apply(input, None, scale, p_eff, seed, offset)
 
 
-def scaled_masked_softmax_dropout(input, mask, scale=1.0, p=0.0, training=True):
-    """dropout(softmax(scale * input) with `mask`, p); input is [b, np, sq, sk]."""
+def scaled_masked_softmax_dropout(input, mask, scale=1.0, p=0.0, training=True, causal=False):
+    """dropout(softmax(scale * input) with `mask`, p); input is [b, np, sq, sk];
+    ``causal`` as in ``scaled_masked_softmax``."""
     _check_dropout_p(p)
     p_eff = float(p) if training else 0.0
     if p_eff == 0.0:
-        return _ScaledMaskedSoftmax.apply(input, mask, scale)
+        return _ScaledMaskedSoftmax.apply(input, mask, scale, causal)
     seed, offset = _next_philox_state(input.device)
-    return _ScaledMaskedSoftmaxDropout.apply(input, mask, scale, p_eff, seed, offset)
+    return _ScaledMaskedSoftmaxDropout.apply(input, mask, scale, p_eff, seed, offset, causal)

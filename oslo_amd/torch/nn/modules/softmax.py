@@ -47,8 +47,11 @@ class FusedScaleMaskSoftmax(nn.Module):
 
     ``forward(input, mask)``: ``input`` is ``[b, np, sq, sk]``; ``mask`` is a
     boolean ``[b or 1, 1, sq or 1, sk]`` tensor with True = masked out, or None.
-    With the causal type and no mask, key ``j`` of query ``i`` is visible when
-    ``j <= i + (sk - sq)``.
+    With the causal type key ``j`` of query ``i`` is hidden when
+    ``j > i + (sk - sq)``, whether or not a mask is given: a key-padding mask
+    then combines with the diagonal in one kernel (the loads still stop at the
+    diagonal), which is what a causal model applies to a padded batch
+    (``modeling_gpt2.py:126-136``).
     """
 
     def __init__(
@@ -116,7 +119,8 @@ class FusedScaleMaskSoftmax(nn.Module):
             return probs.view(b, np, sq, sk)
         if mask is None:
             mask = torch.zeros(1, 1, 1, sk, dtype=torch.bool, device=input.device)
-        return onn_f.scaled_masked_softmax_dropout(input, mask, scale, p, training)
+        causal = self.attn_mask_type == AttnMaskType.causal
+        return onn_f.scaled_masked_softmax_dropout(input, mask, scale, p, training, causal=causal)
 
     def forward_torch_softmax(self, input, mask):
         orig_dtype = input.dtype
@@ -124,12 +128,13 @@ class FusedScaleMaskSoftmax(nn.Module):
             input = input.float()
         if self.scale is not None:
             input = input * self.scale
-        if self.attn_mask_type == AttnMaskType.causal and mask is None:
+        if self.attn_mask_type == AttnMaskType.causal:
             sq, sk = input.size(2), input.size(3)
             causal = torch.ones(sq, sk, dtype=torch.bool, device=input.device).triu(
                 diagonal=1 + sk - sq
             )
-            mask = causal.view(1, 1, sq, sk)
+            causal = causal.view(1, 1, sq, sk)
+            mask = causal if mask is None else (mask.bool() | causal)
         mask_output = self.mask_func(input, mask) if mask is not None else input
         probs = torch.nn.Softmax(dim=-1)(mask_output)
         if self.input_in_float16 and self.softmax_in_fp32:

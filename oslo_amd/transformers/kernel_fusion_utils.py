@@ -356,6 +356,23 @@ def _repeat_kv(hidden_states, n_rep):
     return hidden_states.reshape(b, kv_heads * n_rep, s, d)
 
 
+def _unfused_probs(scores, scaling, attention_mask, causal, p, training, out_dtype):
+    """The reference's unfused chain: scale, mask (boolean True = attend, or an
+    additive float term), softmax, dropout."""
+    sq, sk = scores.shape[-2], scores.shape[-1]
+    t = scores * scaling
+    if attention_mask is not None:
+        if attention_mask.dtype == torch.bool:
+            t = t.masked_fill(~attention_mask, -10000.0)
+        else:
+            t = t + attention_mask
+    elif causal:
+        hidden = torch.ones(sq, sk, dtype=torch.bool, device=t.device).triu(1 + sk - sq)
+        t = t.masked_fill(hidden, -10000.0)
+    probs = torch.softmax(t, dim=-1).to(out_dtype)
+    return torch.nn.functional.dropout(probs, p=p, training=training)
+
+
 def fused_attention_forward(module, query, key, value, attention_mask, scaling=None,
                             dropout=0.0, **kwargs):
     """Attention with the scale -> mask -> softmax -> dropout chain in one kernel.
@@ -363,9 +380,15 @@ def fused_attention_forward(module, query, key, value, attention_mask, scaling=N
     Signature and return value of the attention functions of Hugging Face
     transformers (``(module, query, key, value, attention_mask, scaling,
     dropout, **kwargs) -> (attn_output [b, sq, heads, d], attn_weights)``).
-    ``attention_mask`` is None (causal when the module is), a boolean
-    ``[b or 1, 1, sq or 1, sk]`` tensor with True = attend, or an additive float
-    mask of that shape.
+    ``attention_mask`` is None (causal when the module is) or a boolean
+    ``[b or 1, 1, sq or 1, sk]`` tensor with True = attend.  A mask built by
+    ``fused_attention_mask`` for a causal model on a padded batch carries the
+    key-padding part by itself; the kernel then applies the diagonal and reads
+    ``[b, sk]`` mask bytes instead of ``[b, sq, sk]``.  A floating-point mask is
+    an additive term (a relative-position bias as in
+    oslo/transformers/models/t5/modeling_t5.py:508-514, ALiBi, or -10000
+    fills): the fused kernels know no additive term, so such a call takes the
+    reference's unfused chain, on the GPU as on the CPU.
     """
     if scaling is None:
         scaling = query.size(-1) ** -0.5
@@ -381,31 +404,27 @@ def fused_attention_forward(module, query, key, value, attention_mask, scaling=N
             causal = getattr(module, "is_causal", True)
     else:
         causal = False
-    if not scores.is_cuda:
-        # CPU tensors: the unfused chain
-        t = scores * scaling
-        if attention_mask is not None:
-            if attention_mask.dtype == torch.bool:
-                t = t.masked_fill(~attention_mask, -10000.0)
-            else:
-                t = t + attention_mask
-        elif causal:
-            hidden = torch.ones(sq, sk, dtype=torch.bool, device=t.device).triu(1 + sk - sq)
-            t = t.masked_fill(hidden, -10000.0)
-        probs = torch.softmax(t, dim=-1).to(value.dtype)
-        probs = torch.nn.functional.dropout(probs, p=p, training=module.training)
+        if attention_mask.dim() == 4 and attention_mask.size(-1) > sk:
+            attention_mask = attention_mask[..., :sk]
+    key_visible = getattr(attention_mask, "_oslo_key_visible", None)
+    if not scores.is_cuda or (attention_mask is not None and attention_mask.dtype != torch.bool):
+        probs = _unfused_probs(scores, scaling, attention_mask, causal, p, module.training, value.dtype)
     elif attention_mask is None and causal:
         probs = onn_f.scaled_upper_triang_masked_softmax_dropout(
             scores.reshape(b * heads, sq, sk), scaling, p, module.training
         ).view(b, heads, sq, sk)
+    elif (key_visible is not None and key_visible.dim() == 2 and key_visible.size(-1) == sk
+          and key_visible.size(0) in (1, b) and key_visible.device == scores.device):
+        # causal pattern x key padding: the diagonal is applied by the kernel
+        hidden = (~key_visible).view(key_visible.size(0), 1, 1, sk)
+        probs = onn_f.scaled_masked_softmax_dropout(
+            scores, hidden, scaling, p, module.training, causal=True
+        )
     else:
         if attention_mask is None:
             hidden = torch.zeros(1, 1, 1, sk, dtype=torch.bool, device=scores.device)
-        elif attention_mask.dtype == torch.bool:
-            hidden = ~attention_mask
         else:
-            hidden = attention_mask < -1.0
-        hidden = hidden[..., :sk]
+            hidden = ~attention_mask
         probs = onn_f.scaled_masked_softmax_dropout(
             scores, hidden, scaling, p, module.training
         )
@@ -413,19 +432,50 @@ def fused_attention_forward(module, query, key, value, attention_mask, scaling=N
     return attn_output, probs
 
 
+def fused_attention_mask(batch_size, q_length, kv_length, q_offset=0, kv_offset=0,
+                         mask_function=None, attention_mask=None, **kwargs):
+    """Mask builder registered with transformers' mask interface next to
+    ``fused_attention_forward``: the boolean mask of ``sdpa_mask`` (True =
+    attend), which is correct by itself.  When the pattern is the plain causal
+    one whose diagonal is the kernel's (key j of query i visible when
+    j <= i + (sk - sq)) and a 2-D padding mask is given, the key-padding part
+    ``[b, sk]`` rides along as the attribute ``_oslo_key_visible`` and the
+    attention function lets the kernel apply the diagonal."""
+    from transformers import masking_utils as mu
+
+    if mask_function is None:
+        mask_function = mu.causal_mask_function
+    if attention_mask is not None and attention_mask.dtype != torch.bool:
+        attention_mask = attention_mask != 0
+    full = mu.sdpa_mask(batch_size, q_length, kv_length, q_offset=q_offset, kv_offset=kv_offset,
+                        mask_function=mask_function, attention_mask=attention_mask, **kwargs)
+    if (full is not None and full.dtype == torch.bool and attention_mask is not None
+            and mask_function is mu.causal_mask_function
+            and isinstance(q_offset, int) and isinstance(kv_offset, int)
+            and q_offset - kv_offset == kv_length - q_length):
+        try:
+            kv = mu.prepare_padding_mask(attention_mask, kv_length, kv_offset)
+            kv = kv[:, kv_offset:kv_offset + kv_length]
+        except Exception:  # noqa: BLE001 - an internal helper: without it the full mask is used
+            kv = None
+        if kv is not None and kv.dim() == 2 and kv.size(-1) == kv_length and kv.size(0) in (1, batch_size):
+            full._oslo_key_visible = kv.to(device=full.device, dtype=torch.bool)
+    return full
+
+
 def register_fused_attention(name=ATTENTION_NAME):
-    """Registers ``fused_attention_forward`` (and a boolean mask builder) with
+    """Registers ``fused_attention_forward`` (and its boolean mask builder) with
     transformers' attention interface under ``name``."""
     try:
         from transformers import AttentionInterface
-        from transformers.masking_utils import AttentionMaskInterface, sdpa_mask
+        from transformers.masking_utils import AttentionMaskInterface, sdpa_mask  # noqa: F401
     except ImportError as e:  # older transformers: no pluggable attention
         raise ImportError(
             "fused_scale_mask_softmax needs a transformers version with "
             "AttentionInterface (%s)" % e
         ) from None
     AttentionInterface.register(name, fused_attention_forward)
-    AttentionMaskInterface.register(name, sdpa_mask)
+    AttentionMaskInterface.register(name, fused_attention_mask)
     return name
 
 

@@ -187,3 +187,31 @@ def test_mask_dtypes_and_argument_checks(device):
     with pytest.raises(RuntimeError, match="broadcast"):
         k.fused_scaled_masked_softmax_forward(x, m_bool[:, :, :, :32], 1.0)
     assert k.get_batch_per_block(1024, 1024, 16, 16) >= 1
+
+
+def test_row_without_a_visible_key_follows_the_masked_fill_form(device):
+    """The two mask forms of the reference differ for a row whose keys are all
+    masked: masked_fill(mask, -10000) followed by softmax gives the uniform
+    1/sk, the additive form scores * scale + mask
+    (oslo/transformers/models/bert/modeling_bert.py:298-306) gives
+    softmax(scale * x) because the constant cancels.  The kernel follows the
+    masked_fill form; rows that see at least one key are the same in both."""
+    b, np_, sq, sk = 2, 2, 8, 64
+    x = randn((b, np_, sq, sk), F32, seed=4, std=2.0)
+    mask = torch.zeros(b, 1, sq, sk, dtype=torch.bool)
+    mask[0, 0, 2, :] = True            # one row without a visible key
+    mask[1, 0, :, 40:] = True          # ordinary key padding elsewhere
+    scale = 0.25
+    filled = torch.softmax((x * scale).masked_fill(mask, -10000.0), dim=-1)
+    additive = torch.softmax(x * scale + mask.to(F32) * -10000.0, dim=-1)
+    k = _C.get_softmax_kernel()
+    y = k.fused_scaled_masked_softmax_forward(x.to(device), mask.to(device), scale).cpu()
+    assert torch.allclose(y, filled, rtol=1e-5, atol=1e-7)
+    assert torch.equal(y[0, :, 2, :], torch.full((np_, sk), 1.0 / sk))
+    # the additive form agrees on every other row and differs on that one
+    others = torch.ones(b, np_, sq, dtype=torch.bool)
+    others[0, :, 2] = False
+    assert torch.allclose(y[others], additive[others], rtol=1e-5, atol=1e-7)
+    # (the sum with -10000 is rounded to fp32: the constant cancels up to 1e-3)
+    assert torch.allclose(additive[0, :, 2, :], torch.softmax(x[0, :, 2, :] * scale, dim=-1), rtol=5e-3, atol=1e-6)
+    assert not torch.allclose(y[0, :, 2, :], additive[0, :, 2, :], rtol=1e-2, atol=1e-4)

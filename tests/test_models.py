@@ -502,3 +502,115 @@ def test_t5_through_the_fused_rms_norm(device, dtype):
             continue
         scale = pr.grad.float().abs().max().item() + floor
         assert (pr.grad.float() - pf.grad.float()).abs().max().item() <= gtol * scale + 1e-6, n
+
+
+# ---------------------------------------------------------------------------
+# the attention function registered with transformers: masks it may be handed
+# ---------------------------------------------------------------------------
+class _AttnStub(torch.nn.Module):
+    def __init__(self, is_causal):
+        super().__init__()
+        self.is_causal = is_causal
+
+
+def _eager_attention(q, k, v, scaling, additive):
+    t = torch.matmul(q, k.transpose(-1, -2)) * scaling
+    if additive is not None:
+        t = t + additive
+    return torch.matmul(torch.softmax(t, dim=-1), v).transpose(1, 2)
+
+
+def _t5_style_bias(heads, sq, sk, seed):
+    """A finite relative-position bias per head plus a -10000 key-padding fill,
+    the sum T5 hands to its attention
+    (oslo/transformers/models/t5/modeling_t5.py:508-514)."""
+    g = torch.Generator().manual_seed(seed)
+    rel = torch.randn(heads, 2 * max(sq, sk) - 1, generator=g)
+    idx = torch.arange(sk)[None, :] - torch.arange(sq)[:, None] + max(sq, sk) - 1
+    bias = rel[:, idx].unsqueeze(0)                      # [1, heads, sq, sk]
+    pad = torch.zeros(2, 1, 1, sk)
+    pad[1, ..., sk - 5:] = -10000.0
+    return bias + pad                                    # [2, heads, sq, sk]
+
+
+def test_additive_float_mask_is_applied_not_dropped_cpu():
+    from oslo_amd.transformers.kernel_fusion_utils import fused_attention_forward
+
+    g = torch.Generator().manual_seed(0)
+    q, k, v = (torch.randn(2, 4, 24, 16, generator=g) for _ in range(3))
+    bias = _t5_style_bias(4, 24, 24, seed=1)
+    out, _ = fused_attention_forward(_AttnStub(False).eval(), q, k, v, bias, scaling=1.0)
+    assert torch.allclose(out, _eager_attention(q, k, v, 1.0, bias), rtol=1e-5, atol=1e-6)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_additive_float_mask_is_applied_not_dropped(device, dtype):
+    """A relative-position bias is a finite additive term: the fused kernels
+    know none, so the call must take the unfused chain and give the eager
+    result (it used to be turned into `mask < -1` and lost)."""
+    from oslo_amd.transformers.kernel_fusion_utils import fused_attention_forward
+
+    g = torch.Generator().manual_seed(0)
+    q, k, v = (torch.randn(2, 4, 24, 16, generator=g).to(device, dtype) for _ in range(3))
+    bias = _t5_style_bias(4, 24, 24, seed=1).to(device, dtype)
+    out, _ = fused_attention_forward(_AttnStub(False).eval(), q, k, v, bias, scaling=1.0)
+    ref = _eager_attention(q.float(), k.float(), v.float(), 1.0, bias.float())
+    tol = 1e-5 if dtype == torch.float32 else 3e-2
+    assert (out.float() - ref).abs().max().item() <= tol * (ref.abs().max().item() + 1.0)
+    # and it is not what dropping the finite part would give
+    dropped = _eager_attention(q.float(), k.float(), v.float(), 1.0,
+                               torch.where(bias.float() < -1.0, -10000.0, 0.0))
+    assert (out.float() - dropped).abs().max().item() > 10 * tol
+
+
+def test_mask_builder_returns_the_full_mask_and_the_key_part():
+    from transformers import masking_utils as mu
+
+    from oslo_amd.transformers.kernel_fusion_utils import fused_attention_mask
+
+    am = torch.ones(3, 20, dtype=torch.long)
+    am[1, 15:] = 0
+    am[2, :4] = 0
+    full = fused_attention_mask(3, 20, 20, attention_mask=am)
+    ref = mu.sdpa_mask(3, 20, 20, attention_mask=am.bool())
+    assert full.dtype == torch.bool and torch.equal(full, ref)
+    assert torch.equal(full._oslo_key_visible, am.bool())
+    # causal & key padding is exactly the full mask: the factorisation the kernel relies on
+    causal = torch.tril(torch.ones(20, 20, dtype=torch.bool))
+    assert torch.equal(full, causal[None, None] & am.bool()[:, None, None, :])
+    # cached decoding: one query against 20 keys (the diagonal offset is sk - sq)
+    step = fused_attention_mask(3, 1, 20, q_offset=19, attention_mask=am)
+    assert step is None or torch.equal(step._oslo_key_visible, am.bool())
+    # another pattern (sliding window) carries no key part
+    sw = fused_attention_mask(3, 20, 20, mask_function=mu.sliding_window_causal_mask_function(4), attention_mask=am)
+    assert getattr(sw, "_oslo_key_visible", None) is None
+    # a diagonal that is not the kernel's (queries offset against the keys) carries none either
+    off = fused_attention_mask(3, 10, 20, q_offset=5, attention_mask=am)
+    assert off is None or getattr(off, "_oslo_key_visible", None) is None
+
+
+@pytest.mark.gpu
+def test_causal_model_on_a_padded_batch_takes_the_causal_masked_kernel(device, monkeypatch):
+    from oslo_amd.torch.nn.modules import functional as onn_f
+
+    calls = []
+    real = onn_f.scaled_masked_softmax_dropout
+
+    def spy(input, mask, scale=1.0, p=0.0, training=True, causal=False):
+        calls.append((tuple(mask.shape), causal))
+        return real(input, mask, scale, p, training, causal=causal)
+
+    monkeypatch.setattr(onn_f, "scaled_masked_softmax_dropout", spy)
+    m = tiny_gpt2().to(device).eval()
+    ids, am = inputs()
+    ids, am = ids.to(device), am.to(device)
+    with torch.no_grad():
+        ref = m(ids, attention_mask=am).logits
+    fused_scale_mask_softmax(m)
+    with torch.no_grad():
+        out = m(ids, attention_mask=am).logits
+    valid = am.bool()
+    assert (out[valid] - ref[valid]).abs().max().item() <= 2e-4
+    b, s = ids.shape
+    assert calls and all(shape == (b, 1, 1, s) and causal for shape, causal in calls), calls
