@@ -160,9 +160,9 @@ class _FusedBiasDropoutAddFunction(torch.autograd.Function):
 
 # Dropout state in device memory, one per device, for launches captured in a
 # graph: {seed, offset} as two int64.  Created by the first eager dropout call
-# on the device (a host-to-device copy cannot be captured) and re-seeded when
-# torch's seed changes; its offsets start 2^40 above the generator's so that the
-# two sequences stay apart.
+# on the device (a host-to-device copy cannot be captured) and re-seeded in
+# place when torch's seed changes; its offsets start 2^40 above the generator's
+# so that the two sequences stay apart.
 _graph_rng = {}
 
 
@@ -172,12 +172,18 @@ def _as_i64(v):
 
 
 def _graph_rng_state(index, seed, offset):
+    """The state tensor of device `index`, created on first use and never
+    replaced: captured graphs hold its address, so a new seed is written into
+    the same memory (eager calls only; nothing is captured here)."""
     entry = _graph_rng.get(index)
-    if entry is None or entry[0] != seed:
+    if entry is None:
         state = torch.tensor([_as_i64(seed), _as_i64(offset + (1 << 40))], dtype=torch.int64,
                              device=torch.device("cuda", index))
-        _graph_rng[index] = (seed, state)
+        _graph_rng[index] = [seed, state]
         return state
+    if entry[0] != seed:
+        entry[1].copy_(torch.tensor([_as_i64(seed), _as_i64(offset + (1 << 40))], dtype=torch.int64))
+        entry[0] = seed
     return entry[1]
 
 
@@ -349,6 +355,9 @@ class _FusedBiasDropoutAddNormFunction(torch.autograd.Function):
     def forward(ctx, input, bias, residual, weight, norm_bias, normalized_shape, eps,
                 p, seed, offset, rms):
         kernel = get_layernorm_kernel()
+        # an output nobody consumes (h of a post-LN block) gets no zero-filled
+        # gradient: backward sees None and the kernel skips that operand
+        ctx.set_materialize_grads(False)
         with _rng(seed):
             y, h, mean, invvar = kernel.bias_dropout_add_norm_forward(
                 rms,
@@ -380,6 +389,17 @@ class _FusedBiasDropoutAddNormFunction(torch.autograd.Function):
         has_bias, has_res, has_weight, has_nbias = ctx.has
         weight = saved[-1] if has_weight else None
         need_b = has_bias and ctx.needs_input_grad[1]
+        if grad_y is None:
+            if grad_h is None:
+                return (None,) * 11
+            # only h was used: the backward of dropout(input + bias) + residual
+            with _rng(ctx.seed):
+                g_in, g_bias = get_fused_elementwise_kernel().bias_dropout_add_backward(
+                    grad_h.contiguous(), ctx.p, _seed_arg(ctx.seed), ctx.offset,
+                    need_input_grad=ctx.needs_input_grad[0], need_bias_grad=need_b,
+                )
+            return (g_in, g_bias if need_b else None, grad_h if has_res else None,
+                    None, None, None, None, None, None, None, None)
         with _rng(ctx.seed):
             g_res, g_in, g_gamma, g_beta, g_bias = (
                 get_layernorm_kernel().bias_dropout_add_norm_backward(
@@ -532,12 +552,69 @@ def mixed_dtype_fused_rms_norm_affine(input, weight, normalized_shape, eps=1e-6)
     return _apply_outside_autocast(_FusedRMSNormAffineMixedDtypesFunction, input, weight, normalized_shape, eps)
 
 
+_KERNEL_DTYPES = (torch.float32, torch.float16, torch.bfloat16)
+
+
+def _elementwise_operands(x, bias, residual=None):
+    """Operands of the element-wise kernels, which take one dtype and a bias
+    of shape ``[x.shape[-1]]``.  The reference evaluates ``x + bias`` with
+    torch's promotion and broadcasting (functional.py:36-50, 295-298), so it
+    accepts whatever the model holds; here, inside an autocast region every
+    floating-point operand is cast to the autocast dtype (what the norm
+    wrappers do, functional.py:16-20 there), outside of one ``bias`` and
+    ``residual`` follow ``x``.  Returns ``(x, bias, residual, fits)``; with
+    ``fits`` False (a bias that is not such a vector, a residual of another
+    shape, a dtype without a kernel) the caller evaluates the torch formula."""
+    autocast = x.is_cuda and torch.is_autocast_enabled("cuda")
+    if autocast:
+        x, bias, residual = _cast_if_autocast_enabled(x, bias, residual)
+    else:
+        if bias is not None and bias.dtype != x.dtype:
+            bias = bias.to(x.dtype)
+        if residual is not None and residual.dtype != x.dtype:
+            residual = residual.to(x.dtype)
+    fits = (
+        x.dim() >= 1
+        and x.dtype in _KERNEL_DTYPES
+        and (bias is None or (bias.dim() == 1 and bias.shape[0] == x.shape[-1] and bias.device == x.device))
+        and (residual is None or (residual.shape == x.shape and residual.device == x.device))
+    )
+    return x, bias, residual, fits
+
+
+def _outside_autocast(x):
+    """Context in which a Function runs on operands that were cast already."""
+    if x.is_cuda and torch.is_autocast_enabled("cuda"):
+        return torch.amp.autocast("cuda", enabled=False)
+    return _NullContext()
+
+
+class _NullContext:
+    def __enter__(self):
+        return None
+
+    def __exit__(self, *exc):
+        return False
+
+
 def fused_gelu(x):
-    return _FusedGeLUFunction.apply(x)
+    if not x.is_cuda:
+        return _FusedGeLUFunction.apply(x)
+    x, _, _, fits = _elementwise_operands(x, None)
+    with _outside_autocast(x):
+        if not fits:
+            return _gelu_fwd_torch(x)
+        return _FusedGeLUFunction.apply(x)
 
 
 def fused_bias_gelu(x, bias):
-    return _FusedBiasGeLUFunction.apply(x, bias)
+    if not x.is_cuda:
+        return _FusedBiasGeLUFunction.apply(x, bias)
+    x, bias, _, fits = _elementwise_operands(x, bias)
+    with _outside_autocast(x):
+        if not fits:
+            return _gelu_fwd_torch(x + bias)
+        return _FusedBiasGeLUFunction.apply(x, bias)
 
 
 def fused_bias_dropout(x, bias, p, training, inplace):
@@ -563,11 +640,18 @@ def fused_bias_dropout_add(x, bias, residual, p, training, inplace=False):
         y = x if bias is None else x + bias
         y = F.dropout(y, p=p, training=training, inplace=inplace and bias is None)
         return y if residual is None else y + residual
-    p_eff = float(p) if training else 0.0
-    seed, offset = _next_philox_state(x.device) if p_eff > 0.0 else (0, 0)
-    return _FusedBiasDropoutAddFunction.apply(
-        x, bias, residual, p_eff, seed, offset, bool(inplace)
-    )
+    x_in = x
+    x, bias, residual, fits = _elementwise_operands(x, bias, residual)
+    with _outside_autocast(x):
+        if not fits:
+            y = x if bias is None else x + bias
+            y = F.dropout(y, p=p, training=training)
+            return y if residual is None else y + residual
+        p_eff = float(p) if training else 0.0
+        seed, offset = _next_philox_state(x.device) if p_eff > 0.0 else (0, 0)
+        return _FusedBiasDropoutAddFunction.apply(
+            x, bias, residual, p_eff, seed, offset, bool(inplace) and x is x_in
+        )
 
 
 def _bias_dropout_add_norm(rms, x, bias, residual, weight, norm_bias, normalized_shape,

@@ -159,3 +159,41 @@ def test_captured_dropout_draws_a_new_mask_on_every_replay(device):
     graph.replay()
     torch.cuda.synchronize()
     assert torch.equal(same, x)
+
+
+def test_reseeding_keeps_the_state_tensor_that_captured_graphs_hold(device):
+    """torch.manual_seed followed by an eager dropout call re-seeds the dropout
+    state of the device.  A captured graph holds the address of that state, so
+    the new seed must land in the same memory: a replay afterwards draws the
+    mask of the new (seed, offset) pair, and the tensor is the one the graph
+    was captured with."""
+    import numpy as np
+
+    from oracle import philox
+    from oslo_amd.torch.nn.modules import functional as F_
+
+    n1, n2, p = 64, 512, 0.25
+    x = torch.ones(n1, n2, dtype=BF16, device=device)
+    b = torch.zeros(n2, dtype=BF16, device=device)
+    torch.manual_seed(11)
+    F_.fused_bias_dropout_add(x, b, None, p, True)  # eager: creates (or re-seeds) the state
+    index = device.index if device.index is not None else torch.cuda.current_device()
+    state = F_._graph_rng[index][1]
+    ptr = state.data_ptr()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        out = F_.fused_bias_dropout_add(x, b, None, p, True)
+    graph.replay()
+    torch.cuda.synchronize()
+    torch.manual_seed(2024)
+    F_.fused_bias_dropout_add(x, b, None, p, True)  # eager call after the seed change
+    junk = [torch.full((2,), -1, dtype=torch.int64, device=device) for _ in range(64)]  # reuses freed blocks
+    assert F_._graph_rng[index][1] is state and state.data_ptr() == ptr
+    seed, offset = (int(v) for v in state.cpu())
+    assert seed == 2024
+    graph.replay()
+    torch.cuda.synchronize()
+    keep = philox.keep_mask(n1 * n2, p, seed % 2 ** 64, offset % 2 ** 64).reshape(n1, n2).astype(bool)
+    assert np.array_equal((out != 0).cpu().numpy(), keep), "replay after re-seeding: mask differs from the oracle"
+    assert int(state.cpu()[1]) == offset + 4
+    assert all(int(j.cpu()[0]) == -1 for j in junk), "a replay wrote outside the state tensor"

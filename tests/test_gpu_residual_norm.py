@@ -217,3 +217,54 @@ def test_module_and_autograd(device, rms):
     else:
         oy0, _, _ = cf.layer_norm_fwd(f64(h_eval), f64(gamma), f64(beta), 1e-5, "bf16")
     check(y_eval, oy0, "module eval y", atol=1e-6, max_ulp=2 if rms else 1)
+
+
+def test_unused_outputs_get_no_materialised_gradient(device, monkeypatch):
+    """A post-LN block uses y only: backward must hand the kernel no dh_extra
+    (not a zero-filled tensor, which costs a fill and a full read).  A caller
+    that uses h only gets the backward of dropout(x + bias) + residual."""
+    import oslo_amd.torch.nn as onn
+    from oslo_amd.torch import _C
+
+    n1, n2, p = 64, 512, 0.1
+    x, res, bias, gamma, beta, dy, dh = make_inputs(n1, n2, BF16, 5)
+    seen = []
+    kernel = _C.get_layernorm_kernel()
+    real = kernel.bias_dropout_add_norm_backward
+
+    def spy(rms, grad_y, grad_h, *a, **k):
+        seen.append(grad_h)
+        return real(rms, grad_y, grad_h, *a, **k)
+
+    monkeypatch.setattr(kernel, "bias_dropout_add_norm_backward", spy)
+    leaves = [t.to(device).requires_grad_(True) for t in (x, bias, res)]
+    w, b = gamma.to(device).requires_grad_(True), beta.to(device).requires_grad_(True)
+    torch.manual_seed(3)
+    y = onn.fused_bias_dropout_add_layer_norm(*leaves, w, b, (n2,), 1e-5, p, True)
+    (y * dy.to(device)).sum().backward()
+    assert seen == [None], "the unused h must not produce a gradient tensor"
+    both = [t.grad.clone() for t in leaves]
+    # the same call with return_sum, h consumed with a zero weight: same gradients
+    for t in leaves + [w, b]:
+        t.grad = None
+    torch.manual_seed(3)
+    y2, h2 = onn.fused_bias_dropout_add_layer_norm(*leaves, w, b, (n2,), 1e-5, p, True, return_sum=True)
+    ((y2 * dy.to(device)).sum() + (h2 * 0).sum()).backward()
+    for a, t in zip(both, leaves):
+        assert torch.equal(a, t.grad)
+    # h only: equals bias-dropout-add's own backward on the same Philox state
+    for t in leaves + [w, b]:
+        t.grad = None
+    torch.manual_seed(3)
+    _, h3 = onn.fused_bias_dropout_add_layer_norm(*leaves, w, b, (n2,), 1e-5, p, True, return_sum=True)
+    (h3 * dh.to(device)).sum().backward()
+    got = [t.grad.clone() for t in leaves]
+    assert w.grad is None or float(w.grad.abs().max()) == 0.0
+    for t in leaves:
+        t.grad = None
+    torch.manual_seed(3)
+    h4 = onn.fused_bias_dropout_add(*leaves, p, True)
+    (h4 * dh.to(device)).sum().backward()
+    assert torch.equal(h3, h4)
+    for a, t in zip(got, leaves):
+        assert torch.equal(a, t.grad)

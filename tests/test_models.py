@@ -614,3 +614,78 @@ def test_causal_model_on_a_padded_batch_takes_the_causal_masked_kernel(device, m
     assert (out[valid] - ref[valid]).abs().max().item() <= 2e-4
     b, s = ids.shape
     assert calls and all(shape == (b, 1, 1, s) and causal for shape, causal in calls), calls
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("family", ["gpt2", "bert"])
+def test_fully_swapped_model_under_autocast_with_fp32_parameters(device, family):
+    """torch.autocast with fp32 parameters: the GEMM outputs arrive in bf16, the
+    biases and norm parameters are fp32.  The reference's TorchScript bodies
+    take that through torch's promotion; the fused functions cast their
+    operands to the autocast dtype, as the norm wrappers do.  Forward and
+    backward of the fully swapped model against the unfused model under the
+    same autocast."""
+    from oslo_amd.transformers import fuse_all
+
+    ids, am = inputs(b=3, s=32)
+    ids, am = ids.to(device), am.to(device)
+    if family == "gpt2":
+        kw = dict(attn_pdrop=0.0, resid_pdrop=0.0, embd_pdrop=0.0)
+        ref, fused = tiny_gpt2(seed=5, **kw).to(device).train(), tiny_gpt2(seed=5, **kw).to(device).train()
+    else:
+        # (the tanh form of GeLU, so that the intermediate blocks take the bias-GeLU kernel)
+        kw = dict(hidden_dropout_prob=0.0, attention_probs_dropout_prob=0.0, hidden_act="gelu_new")
+        ref, fused = tiny_bert(seed=5, **kw).to(device).train(), tiny_bert(seed=5, **kw).to(device).train()
+    changed = fuse_all(fused)
+    assert changed["fused_bias_gelu"] > 0 and changed["fused_layer_norm"] + changed["fused_pre_ln_block"] > 0
+
+    wproj = torch.randn(3, 32, 128, generator=torch.Generator().manual_seed(9)).to(device)
+
+    def loss_of(m):
+        with torch.autocast("cuda", dtype=torch.bfloat16):
+            if family == "gpt2":
+                return m(ids, attention_mask=am, labels=ids).loss
+            h = m(ids, attention_mask=am).last_hidden_state
+            return (h.float() * wproj)[am.bool()].sum() / 64.0
+
+    lr, lf = loss_of(ref), loss_of(fused)
+    assert torch.isfinite(lf) and abs(lr.item() - lf.item()) <= 3e-2 * (abs(lr.item()) + 1.0)
+    lr.backward()
+    lf.backward()
+    for (n, pr), (_, pf) in zip(ref.named_parameters(), fused.named_parameters()):
+        if pr.grad is None:
+            continue
+        assert pf.grad is not None and pf.grad.dtype == pr.grad.dtype == torch.float32, n
+        # bf16 activations on both sides, rounded at different points (and the
+        # unfused norms run in fp32 under autocast): compare in the L2 sense
+        err = (pr.grad - pf.grad).norm().item()
+        # (the absolute floor covers gradients that are zero in exact arithmetic,
+        #  such as the key bias of an attention layer)
+        assert err <= 0.1 * pr.grad.norm().item() + 1e-4, (n, err, pr.grad.norm().item())
+
+
+@pytest.mark.gpu
+def test_elementwise_functions_accept_what_torch_promotion_accepts(device):
+    """bias / residual of another dtype follow x; a bias that is not a vector
+    over the last dimension takes the torch formula."""
+    x = torch.randn(6, 32, device=device, dtype=torch.bfloat16)
+    b32 = torch.randn(32, device=device) * 0.1
+    y = onn.fused_bias_gelu(x, b32)
+    ref = onn.fused_bias_gelu(x, b32.to(torch.bfloat16))
+    assert y.dtype == torch.bfloat16 and torch.equal(y, ref)
+    r32 = torch.randn(6, 32, device=device)
+    z = onn.fused_bias_dropout_add(x, b32, r32, 0.0, True)
+    assert z.dtype == torch.bfloat16
+    assert torch.equal(z, onn.fused_bias_dropout_add(x, b32.to(torch.bfloat16), r32.to(torch.bfloat16), 0.0, True))
+    bcol = torch.randn(6, 1, device=device, dtype=torch.bfloat16)   # broadcasts over the columns
+    w = onn.fused_bias_gelu(x, bcol)
+    u = (x + bcol).float()
+    want = u * 0.5 * (1.0 + torch.tanh(0.79788456 * u * (1 + 0.044715 * u * u)))
+    assert (w.float() - want).abs().max().item() <= 3e-2
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        x32 = torch.randn(6, 32, device=device, requires_grad=True)
+        b = torch.nn.Parameter(b32.clone())
+        out = onn.fused_bias_gelu(x32, b)
+        assert out.dtype == torch.bfloat16
+        out.float().sum().backward()
+    assert x32.grad.dtype == torch.float32 and b.grad.dtype == torch.float32 and b.grad.shape == (32,)
