@@ -295,7 +295,11 @@ int oslo_bias_gelu_bwd(const void *g, const void *x, const void *bias,
  * group's four 32-bit words are Philox4x32-10 with key = seed and counter =
  * (offset_lo, offset_hi, group_lo, group_hi); element i takes the 16-bit half
  * ((i % 8) & 1) of word (i % 8) / 2 (low half first) and is KEPT when that
- * value >= round(p * 65536).  Kept values are scaled by 1 / (1 - p).       */
+ * value >= round(p * 65536).  Kept values are scaled by 1 / (1 - p).
+ * The keep probability is therefore 1 - round(p * 65536) / 65536, p rounded
+ * to a multiple of 2^-16, while the scale uses p itself: for p = 0.1 an
+ * element is kept with probability 0.899994 and the expectation of the
+ * output is 7e-6 (relative) below the input's.                              */
 
 /* Replaces fused_bias_dropout (functional.py:295-298:
  * F.dropout(x + bias, p, training)) plus the residual add its callers do
@@ -406,7 +410,8 @@ int oslo_copy_probe(const void *src, void *dst, int64_t bytes, void *stream);
  * 2016, 63, 2016, 4032.                                                    */
 int oslo_wave_reduce_selftest(float *out4, void *stream);
 
-/* Overrides a launch heuristic (for tuning sweeps): key is one of
+/* FOR TESTS AND TUNING SWEEPS ONLY, not for production callers: overrides a
+ * launch heuristic; key is one of
  * "norm_fwd_vpl", "norm_bwd_vpl", "norm_bwd_blocks_per_cu", "norm_bwd_waves",
  * "norm_fwd_waves", "norm_bwd_prefetch", "norm_fwd_iters",
  * "norm_lanes_per_row", "softmax_lanes_per_row" (64 switches the
@@ -425,7 +430,10 @@ int oslo_wave_reduce_selftest(float *out4, void *stream);
  * element-wise kernels then keep their default),
  * softmax_fwd_elems 16, 32 or 64, eltwise tile widths powers of two up to
  * 256, eltwise_rowgroups 1..4096, eltwise_fwd_steps 1..64.
- * Process-wide, not thread-safe.                                           */
+ * The table is process-wide and written under a lock; every entry point
+ * copies it once when it is called, so a launch never sees a half-changed
+ * table, but calls that are already planned keep the old values.  No
+ * accepted value changes a result beyond the order of summation.           */
 int oslo_tune(const char *key, int value);
 
 #ifdef __cplusplus

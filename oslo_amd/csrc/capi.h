@@ -46,7 +46,13 @@ struct Tuning {
   int norm_fwd_iters;
   int adam_unroll;
 };
-extern Tuning g_tune;
+// oslo_tune() writes a process-wide table under a lock; every entry point
+// copies that table into a per-thread snapshot before it plans a launch
+// (tune_snapshot()), and the launch code reads only the snapshot: a sweep
+// that changes a knob on another thread cannot change a launch half way.
+extern thread_local Tuning t_tune;
+void tune_snapshot();
+#define g_tune (::oslo::t_tune)
 
 inline bool aligned16(const void *p) {
   return (reinterpret_cast<uintptr_t>(p) & 15u) == 0;

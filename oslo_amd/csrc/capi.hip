@@ -4,6 +4,8 @@
 
 #include <string.h>
 
+#include <mutex>
+
 namespace oslo {
 
 static thread_local char t_err[512] = "";
@@ -41,7 +43,14 @@ int device_cu_count() {
   return cached[dev];
 }
 
-Tuning g_tune = {};  // all zero: every heuristic at its built-in choice
+static Tuning s_tune_shared = {};  // all zero: every heuristic at its built-in choice
+static std::mutex s_tune_lock;
+thread_local Tuning t_tune = {};
+
+void tune_snapshot() {
+  std::lock_guard<std::mutex> guard(s_tune_lock);
+  t_tune = s_tune_shared;
+}
 
 }  // namespace oslo
 
@@ -59,6 +68,7 @@ const char *oslo_hip_arch(void) { return "gfx950"; }
 int oslo_hip_abi_version(void) { return OSLO_HIP_ABI_VERSION; }
 
 int64_t oslo_workspace_bytes(int op, int64_t n1, int64_t n2) {
+  oslo::tune_snapshot();
   if (n1 < 0 || n2 < 1) {
     oslo::fail(OSLO_ERR_INVALID_ARGUMENT, "workspace_bytes: bad shape");
     return OSLO_ERR_INVALID_ARGUMENT;
@@ -92,25 +102,27 @@ int oslo_tune(const char *key, int value) {
     Kind kind;
     int lo, hi;  // kPow2: powers of two in [lo, hi]; kRange: lo..hi
   };
+  std::lock_guard<std::mutex> guard(oslo::s_tune_lock);
+  oslo::Tuning &shared = oslo::s_tune_shared;
   const Entry table[] = {
-      {"norm_fwd_vpl", &oslo::g_tune.norm_fwd_vpl, kPow2, 1, 8},
-      {"norm_bwd_vpl", &oslo::g_tune.norm_bwd_vpl, kPow2, 1, 4},
-      {"norm_bwd_blocks_per_cu", &oslo::g_tune.norm_bwd_blocks_per_cu, kRange, 1, 8},
-      {"softmax_rows_per_wave", &oslo::g_tune.softmax_rows_per_wave, kPow2, 1, 4},
-      {"softmax_lanes_per_row", &oslo::g_tune.softmax_lanes_per_row, kLanes, 1, 64},
-      {"softmax_fwd_elems", &oslo::g_tune.softmax_fwd_elems, kPow2, 16, 64},
-      {"softmax_rows_per_block", &oslo::g_tune.softmax_rows_per_block, kRange, 1, 16},
-      {"norm_lanes_per_row", &oslo::g_tune.norm_lanes_per_row, kLanes, 8, 64},
-      {"eltwise_tile_max", &oslo::g_tune.eltwise_tile_max, kPow2, 1, 256},
-      {"eltwise_tile_min", &oslo::g_tune.eltwise_tile_min, kPow2, 1, 256},
-      {"eltwise_unroll", &oslo::g_tune.eltwise_unroll, kPow2, 1, 8},
-      {"eltwise_rowgroups", &oslo::g_tune.eltwise_rowgroups, kRange, 1, 4096},
-      {"eltwise_fwd_steps", &oslo::g_tune.eltwise_fwd_steps, kRange, 1, 64},
-      {"norm_bwd_waves", &oslo::g_tune.norm_bwd_waves, kRange, 1, 16},
-      {"norm_fwd_waves", &oslo::g_tune.norm_fwd_waves, kRange, 1, 16},
-      {"norm_bwd_prefetch", &oslo::g_tune.norm_bwd_prefetch, kRange, 1, 2},
-      {"norm_fwd_iters", &oslo::g_tune.norm_fwd_iters, kRange, 1, 16},
-      {"adam_unroll", &oslo::g_tune.adam_unroll, kPow2, 1, 4},
+      {"norm_fwd_vpl", &shared.norm_fwd_vpl, kPow2, 1, 8},
+      {"norm_bwd_vpl", &shared.norm_bwd_vpl, kPow2, 1, 4},
+      {"norm_bwd_blocks_per_cu", &shared.norm_bwd_blocks_per_cu, kRange, 1, 8},
+      {"softmax_rows_per_wave", &shared.softmax_rows_per_wave, kPow2, 1, 4},
+      {"softmax_lanes_per_row", &shared.softmax_lanes_per_row, kLanes, 1, 64},
+      {"softmax_fwd_elems", &shared.softmax_fwd_elems, kPow2, 16, 64},
+      {"softmax_rows_per_block", &shared.softmax_rows_per_block, kRange, 1, 16},
+      {"norm_lanes_per_row", &shared.norm_lanes_per_row, kLanes, 8, 64},
+      {"eltwise_tile_max", &shared.eltwise_tile_max, kPow2, 1, 256},
+      {"eltwise_tile_min", &shared.eltwise_tile_min, kPow2, 1, 256},
+      {"eltwise_unroll", &shared.eltwise_unroll, kPow2, 1, 8},
+      {"eltwise_rowgroups", &shared.eltwise_rowgroups, kRange, 1, 4096},
+      {"eltwise_fwd_steps", &shared.eltwise_fwd_steps, kRange, 1, 64},
+      {"norm_bwd_waves", &shared.norm_bwd_waves, kRange, 1, 16},
+      {"norm_fwd_waves", &shared.norm_fwd_waves, kRange, 1, 16},
+      {"norm_bwd_prefetch", &shared.norm_bwd_prefetch, kRange, 1, 2},
+      {"norm_fwd_iters", &shared.norm_fwd_iters, kRange, 1, 16},
+      {"adam_unroll", &shared.adam_unroll, kPow2, 1, 4},
   };
   for (const Entry &e : table) {
     if (strcmp(e.name, key) == 0) {

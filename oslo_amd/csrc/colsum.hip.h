@@ -3,7 +3,7 @@
 #pragma once
 
 #include "capi.h"
-#include "common.cuh"
+#include "common.hip.h"
 
 namespace oslo {
 

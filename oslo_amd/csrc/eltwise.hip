@@ -18,8 +18,8 @@
 // derivative with the constants 0.79788456, 0.044715, 0.1070322243),
 // :295-298 (dropout(x + bias)).
 #include "capi.h"
-#include "colsum.cuh"
-#include "common.cuh"
+#include "colsum.hip.h"
+#include "common.hip.h"
 
 namespace oslo {
 
@@ -810,6 +810,7 @@ using namespace oslo;
 
 int oslo_bias_gelu_fwd(const void *x, const void *bias, void *y, int64_t rows,
                        int64_t cols, int dtype, void *stream) {
+  oslo::tune_snapshot();
   int rc = check_elt("bias_gelu fwd", rows, cols, dtype);
   if (rc != OSLO_OK) return rc;
   if (rows == 0) return OSLO_OK;
@@ -822,6 +823,7 @@ int oslo_bias_gelu_bwd(const void *g, const void *x, const void *bias,
                        void *dx, void *dbias, void *workspace,
                        int64_t workspace_bytes, int64_t rows, int64_t cols,
                        int dtype, void *stream) {
+  oslo::tune_snapshot();
   int rc = check_elt("bias_gelu bwd", rows, cols, dtype);
   if (rc != OSLO_OK) return rc;
   if (rows == 0) {
@@ -838,6 +840,7 @@ int oslo_bias_dropout_add_fwd(const void *x, const void *bias,
                               uint8_t *mask_out, int64_t rows, int64_t cols,
                               float p, uint64_t seed, uint64_t offset,
                               int dtype, void *stream) {
+  oslo::tune_snapshot();
   int rc = check_elt("bias_dropout_add fwd", rows, cols, dtype);
   if (rc != OSLO_OK) return rc;
   OSLO_REQUIRE(p >= 0.f && p <= 1.f, "bias_dropout_add fwd: p = %f not in [0, 1]",
@@ -853,6 +856,7 @@ int oslo_bias_dropout_add_bwd(const void *g, void *dx, void *dbias,
                               int64_t rows, int64_t cols, float p,
                               uint64_t seed, uint64_t offset, int dtype,
                               void *stream) {
+  oslo::tune_snapshot();
   int rc = check_elt("bias_dropout_add bwd", rows, cols, dtype);
   if (rc != OSLO_OK) return rc;
   OSLO_REQUIRE(p >= 0.f && p <= 1.f, "bias_dropout_add bwd: p = %f not in [0, 1]",
@@ -871,6 +875,7 @@ int oslo_bias_dropout_add_bwd(const void *g, void *dx, void *dbias,
 
 int oslo_philox_mask(uint8_t *mask_out, int64_t n, float p, uint64_t seed,
                      uint64_t offset, void *stream) {
+  oslo::tune_snapshot();
   OSLO_REQUIRE(n >= 0 && p >= 0.f && p <= 1.f, "philox_mask: bad arguments");
   if (n == 0) return OSLO_OK;
   OSLO_REQUIRE(mask_out != nullptr, "philox_mask: null output");
@@ -882,6 +887,7 @@ int oslo_philox_mask(uint8_t *mask_out, int64_t n, float p, uint64_t seed,
 
 int oslo_philox_words(uint32_t *out, int64_t ngroups, int64_t first_group,
                       uint64_t seed, uint64_t offset, void *stream) {
+  oslo::tune_snapshot();
   OSLO_REQUIRE(ngroups >= 0, "philox_words: bad arguments");
   if (ngroups == 0) return OSLO_OK;
   OSLO_REQUIRE(out != nullptr, "philox_words: null output");
@@ -892,6 +898,7 @@ int oslo_philox_words(uint32_t *out, int64_t ngroups, int64_t first_group,
 }
 
 int oslo_copy_probe(const void *src, void *dst, int64_t bytes, void *stream) {
+  oslo::tune_snapshot();
   OSLO_REQUIRE(bytes >= 0 && bytes % 16 == 0 && aligned16(src) && aligned16(dst),
                "copy_probe: bytes must be a multiple of 16 and pointers "
                "16-byte aligned");
@@ -905,6 +912,7 @@ int oslo_copy_probe(const void *src, void *dst, int64_t bytes, void *stream) {
 }
 
 int oslo_wave_reduce_selftest(float *out4, void *stream) {
+  oslo::tune_snapshot();
   OSLO_REQUIRE(out4 != nullptr, "wave_reduce_selftest: null output");
   wave_reduce_selftest_kernel<<<1, 64, 0, (hipStream_t)stream>>>(out4);
   return check_launch("wave_reduce_selftest_kernel");

@@ -20,8 +20,8 @@
 #include <type_traits>
 
 #include "capi.h"
-#include "common.cuh"
-#include "colsum.cuh"
+#include "common.hip.h"
+#include "colsum.hip.h"
 
 namespace oslo {
 
@@ -1591,6 +1591,7 @@ extern "C" {
 int oslo_ln_fwd(const void *x, const void *gamma, const void *beta, void *y,
                 void *mean, void *invvar, int64_t n1, int64_t n2, double eps,
                 int dtype_in, int dtype_out, void *stream) {
+  oslo::tune_snapshot();
   return oslo::norm_fwd_entry(false, x, gamma, beta, y, mean, invvar, n1, n2,
                               eps, dtype_in, dtype_out, stream);
 }
@@ -1598,6 +1599,7 @@ int oslo_ln_fwd(const void *x, const void *gamma, const void *beta, void *y,
 int oslo_rms_fwd(const void *x, const void *gamma, void *y, void *invvar,
                  int64_t n1, int64_t n2, double eps, int dtype_in,
                  int dtype_out, void *stream) {
+  oslo::tune_snapshot();
   return oslo::norm_fwd_entry(true, x, gamma, nullptr, y, nullptr, invvar, n1,
                               n2, eps, dtype_in, dtype_out, stream);
 }
@@ -1607,6 +1609,7 @@ int oslo_ln_bwd(const void *dy, const void *x, const void *mean,
                 void *dbeta, void *workspace, int64_t workspace_bytes,
                 int64_t n1, int64_t n2, int dtype_in, int dtype_out,
                 void *stream) {
+  oslo::tune_snapshot();
   return oslo::norm_bwd_entry(false, dy, x, mean, invvar, gamma, dx, dgamma,
                               dbeta, workspace, workspace_bytes, n1, n2,
                               dtype_in, dtype_out, stream);
@@ -1616,6 +1619,7 @@ int oslo_rms_bwd(const void *dy, const void *x, const void *invvar,
                  const void *gamma, void *dx, void *dgamma, void *workspace,
                  int64_t workspace_bytes, int64_t n1, int64_t n2, int dtype_in,
                  int dtype_out, void *stream) {
+  oslo::tune_snapshot();
   return oslo::norm_bwd_entry(true, dy, x, nullptr, invvar, gamma, dx, dgamma,
                               nullptr, workspace, workspace_bytes, n1, n2,
                               dtype_in, dtype_out, stream);
@@ -1625,6 +1629,7 @@ int oslo_ln_bwd_static(const void *dy, const void *x, const void *mean,
                        const void *invvar, const void *gamma, void *dx,
                        void *dgamma, void *dbeta, int64_t n1, int64_t n2,
                        int dtype_in, int dtype_out, void *stream) {
+  oslo::tune_snapshot();
   using namespace oslo;
   OSLO_REQUIRE(n1 >= 0 && n2 >= 1, "ln bwd static: bad shape [%lld, %lld]",
                (long long)n1, (long long)n2);
@@ -1656,6 +1661,7 @@ int oslo_bias_dropout_add_norm_fwd(const void *x, const void *bias,
                                    int64_t n2, double eps, float p,
                                    uint64_t seed, uint64_t offset, int rms,
                                    int dtype, void *stream) {
+  oslo::tune_snapshot();
   using namespace oslo;
   int rc = check_norm_dtypes(dtype, dtype);
   if (rc != OSLO_OK) return rc;
@@ -1703,6 +1709,7 @@ int oslo_bias_dropout_add_norm_bwd(const void *dy, const void *dh_extra,
                                    int64_t n2, float p, uint64_t seed,
                                    uint64_t offset, int rms, int dtype,
                                    void *stream) {
+  oslo::tune_snapshot();
   using namespace oslo;
   int rc = check_norm_dtypes(dtype, dtype);
   if (rc != OSLO_OK) return rc;

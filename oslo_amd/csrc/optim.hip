@@ -13,7 +13,7 @@
 #include <math.h>
 
 #include "capi.h"
-#include "common.cuh"
+#include "common.hip.h"
 
 namespace oslo {
 
@@ -165,6 +165,7 @@ int oslo_multi_tensor_adam(const void *const *g, void *const *p, void *const *m,
                            int64_t ntensors, float lr, float beta1, float beta2,
                            float eps, int step, int mode, int bias_correction,
                            float weight_decay, int dtype, void *stream) {
+  oslo::tune_snapshot();
   using namespace oslo;
   if (!valid_dtype(dtype))
     return fail(OSLO_ERR_INVALID_ARGUMENT, "multi_tensor_adam: unknown dtype %d", dtype);

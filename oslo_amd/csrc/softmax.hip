@@ -16,7 +16,7 @@
 // mask); entry-point shapes follow
 // oslo/torch/_C/csrc/FusedScaleMaskSoftmaxBinder.cpp:39-105.
 #include "capi.h"
-#include "common.cuh"
+#include "common.hip.h"
 
 namespace oslo {
 
@@ -1442,6 +1442,7 @@ using namespace oslo;
 int oslo_softmax_causal_fwd(const void *x, void *y, int64_t attn_batches,
                             int64_t sq, int64_t sk, float scale, int dtype,
                             void *stream) {
+  oslo::tune_snapshot();
   int rc = check_softmax_shape("softmax causal fwd", attn_batches, sq, sk, dtype);
   if (rc != OSLO_OK) return rc;
   if (attn_batches * sq == 0) return OSLO_OK;
@@ -1454,6 +1455,7 @@ int oslo_softmax_causal_fwd(const void *x, void *y, int64_t attn_batches,
 int oslo_softmax_causal_bwd(const void *dy, const void *y, void *dx,
                             int64_t attn_batches, int64_t sq, int64_t sk,
                             float scale, int dtype, void *stream) {
+  oslo::tune_snapshot();
   int rc = check_softmax_shape("softmax causal bwd", attn_batches, sq, sk, dtype);
   if (rc != OSLO_OK) return rc;
   if (attn_batches * sq == 0) return OSLO_OK;
@@ -1531,6 +1533,7 @@ int oslo_softmax_masked_fwd(const void *x, const uint8_t *mask, void *y,
                             int64_t b, int64_t np, int64_t sq, int64_t sk,
                             int64_t mask_b, int64_t mask_sq, float scale,
                             int dtype, void *stream) {
+  oslo::tune_snapshot();
   return masked_fwd_entry("softmax masked fwd", 0, x, mask, y, b, np, sq, sk,
                           mask_b, mask_sq, scale, dtype, stream);
 }
@@ -1539,6 +1542,7 @@ int oslo_softmax_masked_bwd(const void *dy, const void *y, const uint8_t *mask,
                             void *dx, int64_t b, int64_t np, int64_t sq,
                             int64_t sk, int64_t mask_b, int64_t mask_sq,
                             float scale, int dtype, void *stream) {
+  oslo::tune_snapshot();
   return masked_bwd_entry("softmax masked bwd", 0, dy, y, mask, dx, b, np, sq,
                           sk, mask_b, mask_sq, scale, dtype, stream);
 }
@@ -1547,6 +1551,7 @@ int oslo_softmax_causal_masked_fwd(const void *x, const uint8_t *mask, void *y,
                                    int64_t b, int64_t np, int64_t sq,
                                    int64_t sk, int64_t mask_b, int64_t mask_sq,
                                    float scale, int dtype, void *stream) {
+  oslo::tune_snapshot();
   return masked_fwd_entry("softmax causal masked fwd", 1, x, mask, y, b, np, sq,
                           sk, mask_b, mask_sq, scale, dtype, stream);
 }
@@ -1556,12 +1561,14 @@ int oslo_softmax_causal_masked_bwd(const void *dy, const void *y,
                                    int64_t np, int64_t sq, int64_t sk,
                                    int64_t mask_b, int64_t mask_sq, float scale,
                                    int dtype, void *stream) {
+  oslo::tune_snapshot();
   return masked_bwd_entry("softmax causal masked bwd", 1, dy, y, mask, dx, b,
                           np, sq, sk, mask_b, mask_sq, scale, dtype, stream);
 }
 
 int oslo_softmax_batch_per_block(int64_t sq, int64_t sk, int64_t b,
                                  int64_t np) {
+  oslo::tune_snapshot();
   if (sq < 1 || sk < 1 || b < 1 || np < 1)
     return fail(OSLO_ERR_INVALID_ARGUMENT,
                 "softmax_batch_per_block: bad shape");
@@ -1586,6 +1593,7 @@ int oslo_softmax_causal_dropout_fwd(const void *x, void *out, float *stats,
                                     int64_t sk, float scale, float p,
                                     uint64_t seed, uint64_t offset, int dtype,
                                     void *stream) {
+  oslo::tune_snapshot();
   const char *what = "softmax causal dropout fwd";
   int rc = check_softmax_shape(what, attn_batches, sq, sk, dtype);
   if (rc == OSLO_OK) rc = check_dropout_p(what, p);
@@ -1604,6 +1612,7 @@ int oslo_softmax_causal_dropout_bwd(const void *dout, const void *x,
                                     int64_t sk, float scale, float p,
                                     uint64_t seed, uint64_t offset, int dtype,
                                     void *stream) {
+  oslo::tune_snapshot();
   const char *what = "softmax causal dropout bwd";
   int rc = check_softmax_shape(what, attn_batches, sq, sk, dtype);
   if (rc == OSLO_OK) rc = check_dropout_p(what, p);
@@ -1661,6 +1670,7 @@ int oslo_softmax_masked_dropout_fwd(const void *x, const uint8_t *mask,
                                     int64_t mask_b, int64_t mask_sq,
                                     float scale, float p, uint64_t seed,
                                     uint64_t offset, int dtype, void *stream) {
+  oslo::tune_snapshot();
   return masked_dropout_fwd_entry("softmax masked dropout fwd", 0, x, mask, out,
                                   stats, b, np, sq, sk, mask_b, mask_sq, scale,
                                   p, seed, offset, dtype, stream);
@@ -1672,6 +1682,7 @@ int oslo_softmax_masked_dropout_bwd(const void *dout, const void *x,
                                     int64_t sk, int64_t mask_b, int64_t mask_sq,
                                     float scale, float p, uint64_t seed,
                                     uint64_t offset, int dtype, void *stream) {
+  oslo::tune_snapshot();
   return masked_dropout_bwd_entry("softmax masked dropout bwd", 0, dout, x,
                                   mask, stats, dx, b, np, sq, sk, mask_b,
                                   mask_sq, scale, p, seed, offset, dtype,
@@ -1685,6 +1696,7 @@ int oslo_softmax_causal_masked_dropout_fwd(const void *x, const uint8_t *mask,
                                            float scale, float p, uint64_t seed,
                                            uint64_t offset, int dtype,
                                            void *stream) {
+  oslo::tune_snapshot();
   return masked_dropout_fwd_entry("softmax causal masked dropout fwd", 1, x,
                                   mask, out, stats, b, np, sq, sk, mask_b,
                                   mask_sq, scale, p, seed, offset, dtype,
@@ -1699,6 +1711,7 @@ int oslo_softmax_causal_masked_dropout_bwd(const void *dout, const void *x,
                                            int64_t mask_sq, float scale, float p,
                                            uint64_t seed, uint64_t offset,
                                            int dtype, void *stream) {
+  oslo::tune_snapshot();
   return masked_dropout_bwd_entry("softmax causal masked dropout bwd", 1, dout,
                                   x, mask, stats, dx, b, np, sq, sk, mask_b,
                                   mask_sq, scale, p, seed, offset, dtype,

@@ -259,11 +259,35 @@ def _check_input(t, name):
         raise RuntimeError("%s must be contiguous" % name)
 
 
+# Backward workspaces (fp32 partial rows of the parameter gradients), kept per
+# (device, stream, op) and grown on demand instead of allocated per call.  Calls
+# that share a stream are ordered, so the finalize launch of one call has read
+# the partial rows before the next call overwrites them; calls on different
+# streams or devices never share a workspace.  The memory stays torch's.
+_ws_cache = {}
+_ws_bytes_cache = {}
+
+
 def _workspace(lib, op, n1, n2, device):
-    nbytes = lib.oslo_workspace_bytes(op, n1, n2)
-    if nbytes < 0:
-        _check(int(nbytes), lib)
-    return torch.empty(max(int(nbytes), 16), dtype=torch.uint8, device=device), int(nbytes)
+    key = (op, n1, n2)
+    nbytes = _ws_bytes_cache.get(key)
+    if nbytes is None:
+        nbytes = int(lib.oslo_workspace_bytes(op, n1, n2))
+        if nbytes < 0:
+            _check(nbytes, lib)
+        if len(_ws_bytes_cache) < 4096:
+            _ws_bytes_cache[key] = nbytes
+    index = device.index if device.index is not None else torch.cuda.current_device()
+    stream = _raw_stream(index) if _raw_stream is not None else torch.cuda.current_stream(device).cuda_stream
+    slot = (index, stream, op)
+    ws = _ws_cache.get(slot)
+    if ws is None or ws.numel() < nbytes:
+        # (round up so that a sweep over growing shapes settles quickly)
+        size = max(nbytes, 16)
+        size = (size + (1 << 20) - 1) & ~((1 << 20) - 1) if size > (1 << 16) else size
+        ws = torch.empty(size, dtype=torch.uint8, device=device)
+        _ws_cache[slot] = ws
+    return ws, nbytes
 
 
 class device_rng:
@@ -297,6 +321,7 @@ def tune(key, value):
     """Overrides a launch heuristic of the library (0 restores the default)."""
     lib = load_library()
     _check(lib.oslo_tune(key.encode(), int(value)), lib)
+    _ws_bytes_cache.clear()  # workspace sizes depend on the launch shapes
 
 
 # ---------------------------------------------------------------------------
