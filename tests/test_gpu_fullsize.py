@@ -152,6 +152,68 @@ def test_padding_softmax_full_size(device):
     check(dxb, cf.softmax_bwd(f64(gb), f64(yb), scale), "cfg3 bwd rows", atol=1e-7)
 
 
+# --------------------------------------------------------------------------- cfg5 shape, causal + key padding
+def test_causal_padding_softmax_full_size(device):
+    """The attention of a causal model on a padded batch
+    (oslo/transformers/models/gpt2/modeling_gpt2.py:126-136, 573-581) at the
+    cfg5 shape: diagonal and key-padding mask in one call, with and without the
+    fused dropout."""
+    b, h, s = 4, 64, 2048
+    scale = 1.0 / math.sqrt(96.0)
+    x = gpu_randn((b, h, s, s), BF16, 11, device)
+    g = gpu_randn((b, h, s, s), BF16, 12, device)
+    valid = torch.randint(1024, 2049, (b,), generator=torch.Generator().manual_seed(5))
+    pad = torch.arange(s)[None, :] >= valid[:, None]
+    mask = pad.view(b, 1, 1, s).to(device)
+    k = _C.get_softmax_kernel()
+    y = k.fused_scaled_masked_softmax_forward(x, mask, scale, causal=True)
+    dx = k.fused_scaled_masked_softmax_backward(g, y, scale, mask=mask, causal=True)
+    assert torch.equal(dx, k.fused_scaled_masked_softmax_backward(g, y, scale, causal=True))
+    ar = torch.arange(1, s + 1, device=device)
+    for bi in range(b):
+        v = int(valid[bi])
+        for h0 in range(0, h, 16):
+            yb = y[bi, h0:h0 + 16].float()
+            assert (yb.sum(-1) - 1).abs().max().item() <= 2e-3
+            assert torch.triu(yb, diagonal=1).count_nonzero().item() == 0
+            assert yb[..., v:].count_nonzero().item() == 0
+            assert ((yb > 0).sum(-1) <= torch.clamp(ar, max=v)).all()
+            dxb = dx[bi, h0:h0 + 16].float()
+            assert torch.triu(dxb, diagonal=1).count_nonzero().item() == 0
+            assert dxb[..., v:].count_nonzero().item() == 0
+            gscale = g[bi, h0:h0 + 16].float().abs().amax(-1) * scale
+            assert (dxb.sum(-1).abs() <= 8e-3 * gscale + 1e-6).all()
+    rows = sample_rows(b * h * s)
+    sel = rows.to(device)
+    xb, yb = x.view(-1, s)[sel].cpu(), y.view(-1, s)[sel].cpu()
+    gb, dxb = g.view(-1, s)[sel].cpu(), dx.view(-1, s)[sel].cpu()
+    bi = (rows // (h * s)).numpy()
+    qi = (rows % s).numpy()
+    hidden = pad.numpy()[bi] | (np.arange(s)[None, :] > qi[:, None])
+    check(yb, cf.softmax_masked_fwd(f64(xb), hidden, scale), "causal+padding fwd rows", atol=1e-9)
+    check(dxb, cf.softmax_bwd(f64(gb), f64(yb), scale), "causal+padding bwd rows", atol=1e-7)
+    del dx
+    # with the dropout of the probabilities fused in
+    p, seed, offset = 0.1, 777, 8
+    out, stats = k.softmax_dropout_forward(x, mask, scale, p, seed, offset, causal=True)
+    keep = _C.get_fused_elementwise_kernel().philox_mask(x.numel(), p, seed, offset, device).view(b, h, s, s)
+    for bi in range(b):
+        for h0 in range(0, h, 16):
+            ob, yb, kb = out[bi, h0:h0 + 16].float(), y[bi, h0:h0 + 16].float(), keep[bi, h0:h0 + 16].bool()
+            assert ob[~kb].count_nonzero().item() == 0
+            want = yb / (1.0 - p)
+            assert ((ob - want)[kb].abs() <= 2.0 ** -7 * want[kb] + 1e-30).all()
+    del keep, y
+    dxd = k.softmax_dropout_backward(g, x, stats, mask, scale, p, seed, offset, causal=True)
+    ob, dxb = out.view(-1, s)[sel].cpu(), dxd.view(-1, s)[sel].cpu()
+    keep_rows = np.stack(
+        [philox.keep_mask(s, p, seed, offset, first_element=int(r) * s) for r in rows]
+    ).astype(bool)
+    check(ob, cf.softmax_dropout_fwd(f64(xb), hidden, scale, keep_rows, p), "causal+padding dropout fwd rows", atol=1e-9)
+    check(dxb, cf.softmax_dropout_bwd(f64(gb), f64(xb), hidden, scale, keep_rows, p), "causal+padding dropout bwd rows",
+          atol=2e-7)
+
+
 # --------------------------------------------------------------------------- cfg2 / cfg5 norms
 @pytest.mark.parametrize("n1,n2", [(16384, 4096), (8192, 6144)])
 @pytest.mark.parametrize("rms", [False, True])
