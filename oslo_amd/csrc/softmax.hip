@@ -34,7 +34,36 @@ struct SoftmaxGeom {
   int mask_per_query;      // 1 if mask_sq == sq else 0
   int wpr, rpb;     // waves per row, rows per workgroup pass (without RPW)
   int causal;       // masked mode: key j of query i is also hidden when j > i + (sk - sq)
+  // n / sq and n / np for n < 2^31 as mulhi(n, mul) >> shift (shift == 32: divisor 1),
+  // filled in by set_fast_div on the host
+  uint32_t sq_mul = 0, sq_shift = 32, np_mul = 0, np_shift = 32;
 };
+
+// Division of n < 2^31 by a divisor 1 <= d < 2^31 fixed for the launch: with
+// l = ceil(log2 d) and mul = ceil(2^(31 + l) / d) < 2^32, floor(n / d) equals
+// mulhi(n, mul) >> (l - 1) exactly (the error term n * e / (d * 2^(31 + l)) with
+// e < d stays below 2^-l <= 1 / d).  A run-time division costs about as many
+// vector instructions as the softmax of a short row.
+static inline void fast_div_make(uint32_t d, uint32_t *mul, uint32_t *shift) {
+  if (d <= 1) {
+    *mul = 0;
+    *shift = 32;
+    return;
+  }
+  uint32_t l = 0;
+  while ((1ull << l) < d) ++l;
+  *mul = (uint32_t)(((1ull << (31 + l)) + d - 1) / d);
+  *shift = l - 1;
+}
+
+static inline void set_fast_div(SoftmaxGeom &g) {
+  fast_div_make((uint32_t)g.sq, &g.sq_mul, &g.sq_shift);
+  fast_div_make((uint32_t)g.np, &g.np_mul, &g.np_shift);
+}
+
+__device__ __forceinline__ uint32_t fast_div(uint32_t n, uint32_t mul, uint32_t shift) {
+  return shift == 32 ? n : __umulhi(n, mul) >> shift;
+}
 
 // Reductions over the wpr (<= 16) consecutive waves of a row: lane 0 of each
 // wave publishes its wave's value in LDS, lane l < wpr then reads the value of
@@ -115,19 +144,18 @@ __device__ __forceinline__ void row_setup(const SoftmaxGeom &g, int64_t r,
   mrow = nullptr;
   visible = g.sk;
   row = r;
-  // 32-bit division where the row count allows it: a 64-bit division costs
-  // about as many instructions as the softmax of a short row itself
+  // multiplication by a precomputed reciprocal where the row count allows it
   const bool small = g.rows <= 0x7fffffff;
   if constexpr (MODE == kModeCausal) {
     const int64_t batch =
-        small ? (int64_t)((uint32_t)r / (uint32_t)g.sq) : r / g.sq;
+        small ? (int64_t)fast_div((uint32_t)r, g.sq_mul, g.sq_shift) : r / g.sq;
     const int qi = g.sq - 1 - (int)(r - batch * g.sq);
     row = batch * g.sq + qi;
     int v = qi + 1 + (g.sk - g.sq);
     visible = v < 0 ? 0 : (v > g.sk ? g.sk : v);
   } else if constexpr (MODE == kModeMasked) {
     const int64_t bh =
-        small ? (int64_t)((uint32_t)r / (uint32_t)g.sq) : r / g.sq;
+        small ? (int64_t)fast_div((uint32_t)r, g.sq_mul, g.sq_shift) : r / g.sq;
     int qi = (int)(r - bh * g.sq);
     if (g.causal) {  // uniform over the launch: long rows first, as in causal mode
       qi = g.sq - 1 - qi;
@@ -136,7 +164,7 @@ __device__ __forceinline__ void row_setup(const SoftmaxGeom &g, int64_t r,
       visible = v < 0 ? 0 : (v > g.sk ? g.sk : v);
     }
     const int64_t bi =
-        small ? (int64_t)((uint32_t)bh / (uint32_t)g.np) : bh / g.np;
+        small ? (int64_t)fast_div((uint32_t)bh, g.np_mul, g.np_shift) : bh / g.np;
     const int64_t mr =
         bi * g.mask_b_stride_rows + (g.mask_per_query ? qi : 0);
     mrow = mask + mr * g.sk;
@@ -183,6 +211,7 @@ __global__ __launch_bounds__(1024) void softmax_fwd_kernel(
   uint32_t mbits[RPW][VPL];  // bit e set: key masked out
   int64_t row[RPW];
   bool rvalid[RPW];
+  const uint8_t *mrow0 = nullptr;
 
 #pragma unroll
   for (int j = 0; j < RPW; ++j) {
@@ -192,11 +221,20 @@ __global__ __launch_bounds__(1024) void softmax_fwd_kernel(
     const uint8_t *mrow = nullptr;
     row[j] = 0;
     if (rvalid[j]) row_setup<MODE>(g, r, mask, row[j], visible, mrow);
+    // consecutive rows of a wave normally share their mask row (a key-padding
+    // mask [b, 1, 1, sk]): its bits are then read and unpacked once
+    bool shared = false;
+    if constexpr (MODE == kModeMasked && RPW > 1) {
+      if (j == 0) mrow0 = mrow;
+      shared = j > 0 && rvalid[j] && rvalid[0] && mrow == mrow0 && !g.causal;
+    }
 #pragma unroll
     for (int k = 0; k < VPL; ++k) {
       const int c = c0 + k * cstride;
       uint32_t mb = (1u << E) - 1u;
-      if (rvalid[j] && c < nchunks) {
+      if (shared) {
+        mb = mbits[0][k];
+      } else if (rvalid[j] && c < nchunks) {
         if constexpr (MODE == kModeCausal) {
           const int left = visible - c * E;  // visible keys in this chunk
           mb = left >= E ? 0u : (left <= 0 ? mb : (mb & ~((1u << left) - 1u)));
@@ -1216,6 +1254,7 @@ static int launch_softmax_fwd(const void *x, const uint8_t *mask, void *y,
                               float *stats, DropArgs d, SoftmaxGeom g,
                               float scale, hipStream_t st) {
   constexpr int E = io<T>::EPV;
+  set_fast_div(g);
   const bool drop = stats != nullptr;
   // 64 bytes of the operand per lane (32 16-bit or 16 fp32 elements) measure
   // 10-25 % faster than twice that (rows of 4096 and more 16-bit keys then
@@ -1298,6 +1337,7 @@ static int launch_softmax_bwd(const void *dy, const void *y,
                               const uint8_t *mask, void *dx, SoftmaxGeom g,
                               float scale, hipStream_t st) {
   constexpr int E = io<T>::EPV;
+  set_fast_div(g);
   // (fp32: 16 elements of each operand per lane, as in the forward)
   SoftmaxPlan pl = plan_softmax(g.sk, E, sizeof(T) == 4 ? 16 : kBwdMaxElems, 1, 1);
   if (!pl.ok && sizeof(T) == 4) pl = plan_softmax(g.sk, E, kBwdMaxElems, 1, 1);
@@ -1359,6 +1399,7 @@ static int launch_softmax_dropout_bwd(const void *dy, const void *x,
                                       void *dx, DropArgs d, SoftmaxGeom g,
                                       float scale, hipStream_t st) {
   constexpr int E = io<T>::EPV;
+  set_fast_div(g);
   // (fp32: 16 elements of each operand per lane, as in the forward)
   SoftmaxPlan pl = plan_softmax(g.sk, E, sizeof(T) == 4 ? 16 : kBwdMaxElems, 1, 1);
   if (!pl.ok && sizeof(T) == 4) pl = plan_softmax(g.sk, E, kBwdMaxElems, 1, 1);
