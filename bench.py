@@ -29,7 +29,8 @@ Prints ONE JSON line.  Beside the contract's keys it carries
                 copies of matching sizes,
   cpu_path      the reference's unfused torch path, forward + backward, per
                 configuration on bounded samples, with the GPU rate of the
-                same pair and their ratio.
+                same fused forward + backward pair (the metric's own unit:
+                gpu_GBps and gpu_frac of the peak) and their ratio.
 """
 import argparse
 import json
@@ -729,6 +730,7 @@ def cpu_path_table(gpu_rows, budget_s=3.0):
             "kernel": name, "config": cfg, "sample": sample, "cores": threads,
             "cpu_ms": round(t * 1e3, 1), "cpu_GBps": round(cpu, 2),
             "gpu_GBps": None if gpu is None else round(gpu, 1),
+            "gpu_frac": None if gpu is None else round(gpu / HBM_PEAK_GBPS, 4),
             "speedup": None if gpu is None else round(gpu / cpu, 1),
         })
 
