@@ -215,3 +215,48 @@ def test_row_without_a_visible_key_follows_the_masked_fill_form(device):
     # (the sum with -10000 is rounded to fp32: the constant cancels up to 1e-3)
     assert torch.allclose(additive[0, :, 2, :], torch.softmax(x[0, :, 2, :] * scale, dim=-1), rtol=5e-3, atol=1e-6)
     assert not torch.allclose(y[0, :, 2, :], additive[0, :, 2, :], rtol=1e-2, atol=1e-4)
+
+
+@pytest.mark.parametrize("b,np_,sq,sk,dtype", [
+    (37, 5, 13, 64, BF16),      # nothing a power of two: batch, heads and queries are recovered by division
+    (11, 7, 33, 128, F16),
+    (64, 3, 1, 256, BF16),      # one query per head
+    (9, 1, 47, 512, F32),       # one head
+    (3, 96, 31, 40, BF16),
+    (250, 2, 3, 24, F16),
+])
+def test_row_to_batch_head_query_mapping(device, b, np_, sq, sk, dtype):
+    """A kernel row r stands for (batch, head, query) = (r / (np sq), (r / sq) % np,
+    r % sq).  Per-batch masks with a different valid length in every batch, and
+    the diagonal in causal mode, make any slip in that mapping visible: the
+    zeros of a row would sit in the wrong places."""
+    x = randn((b, np_, sq, sk), dtype, seed=b + sq, std=2.0)
+    r = np.random.default_rng(b * 131 + sk)
+    valid = r.integers(1, sk + 1, size=b)
+    mask = torch.from_numpy(np.arange(sk)[None, :] >= valid[:, None]).view(b, 1, 1, sk)
+    k = _C.get_softmax_kernel()
+    y = k.fused_scaled_masked_softmax_forward(x.to(device), mask.to(device), 0.25)
+    hidden = np.broadcast_to(mask.numpy(), (b, np_, sq, sk))
+    check(y, cf.softmax_masked_fwd(f64(x), hidden, 0.25), "masked fwd", atol=1e-9)
+    yc = y.cpu()
+    for bi in range(b):
+        assert yc[bi, :, :, valid[bi]:].count_nonzero().item() == 0
+        assert (yc[bi, :, :, :valid[bi]] > 0).all()
+    # per-query masks: the query index matters as well
+    pq = torch.from_numpy(r.random((b, 1, sq, sk)) < 0.4)
+    pq[..., 0] = False
+    y2 = k.fused_scaled_masked_softmax_forward(x.to(device), pq.to(device), 0.25)
+    check(y2, cf.softmax_masked_fwd(f64(x), np.broadcast_to(pq.numpy(), (b, np_, sq, sk)), 0.25),
+          "per-query mask fwd", atol=1e-9)
+    assert (y2.cpu()[pq.expand(b, np_, sq, sk)] == 0).all()
+    # causal on [b * np, sq, sk]: the query index of every row
+    x3 = x.view(b * np_, sq, sk)
+    yc3 = k.fused_scaled_upper_triang_masked_softmax_forward(x3.to(device), 0.25)
+    hid = cf.causal_hidden(sq, sk)[None]
+    check(yc3, cf.softmax_masked_fwd(f64(x3), np.broadcast_to(hid, (b * np_, sq, sk)), 0.25), "causal fwd", atol=1e-9)
+    dy = randn((b * np_, sq, sk), dtype, seed=7)
+    dx = k.fused_scaled_upper_triang_masked_softmax_backward(dy.to(device), yc3, 0.25)
+    check(dx, cf.softmax_bwd(f64(dy), f64(yc3), 0.25), "causal bwd", atol=1e-7)
+    # both at once
+    ycm = k.fused_scaled_masked_softmax_forward(x.to(device), mask.to(device), 0.25, causal=True)
+    check(ycm, cf.softmax_masked_fwd(f64(x), hidden | hid[None], 0.25), "causal + padding fwd", atol=1e-9)
