@@ -37,6 +37,7 @@ struct SoftmaxGeom {
   // n / sq and n / np for n < 2^31 as mulhi(n, mul) >> shift (shift == 32: divisor 1),
   // filled in by set_fast_div on the host
   uint32_t sq_mul = 0, sq_shift = 32, np_mul = 0, np_shift = 32;
+  float inv_sk = 0.f;  // 1 / sk, the value of a row without a visible key
 };
 
 // Division of n < 2^31 by a divisor 1 <= d < 2^31 fixed for the launch: with
@@ -59,10 +60,19 @@ static inline void fast_div_make(uint32_t d, uint32_t *mul, uint32_t *shift) {
 static inline void set_fast_div(SoftmaxGeom &g) {
   fast_div_make((uint32_t)g.sq, &g.sq_mul, &g.sq_shift);
   fast_div_make((uint32_t)g.np, &g.np_mul, &g.np_shift);
+  g.inv_sk = 1.0f / (float)g.sk;
 }
 
 __device__ __forceinline__ uint32_t fast_div(uint32_t n, uint32_t mul, uint32_t shift) {
   return shift == 32 ? n : __umulhi(n, mul) >> shift;
+}
+
+// 1 / s for the row sum s >= 1 of a softmax: the hardware reciprocal refined by
+// one Newton step (within an ulp of the quotient; an IEEE division costs ten
+// instructions).  Every softmax kernel forms its normaliser with this function.
+__device__ __forceinline__ float row_recip(float s) {
+  const float r = __builtin_amdgcn_rcpf(s);
+  return __builtin_fmaf(r, __builtin_fmaf(-s, r, 1.0f), r);
 }
 
 // Reductions over the wpr (<= 16) consecutive waves of a row: lane 0 of each
@@ -193,7 +203,7 @@ __global__ __launch_bounds__(1024) void softmax_fwd_kernel(
   const int lane = threadIdx.x & 63;
   // the wave index is uniform: keep it (and the row arithmetic) in scalar registers
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int rslot = wave / g.wpr;
+  const int rslot = g.wpr == 1 ? wave : wave / g.wpr;  // (uniform: the division is skipped)
   const int first = rslot * g.wpr;
   const int nchunks = g.sk / E;
   const int cstride = LPR == kWave ? kWave * g.wpr : LPR;
@@ -251,12 +261,9 @@ __global__ __launch_bounds__(1024) void softmax_fwd_kernel(
 #pragma unroll
     for (int k = 0; k < VPL; ++k) {
       const int c = c0 + k * cstride;
-      if (mbits[j][k] != (1u << E) - 1u) {
-        load_chunk<T, E>(xr + (int64_t)c * E, v[j][k]);
-      } else {
-#pragma unroll
-        for (int e = 0; e < E; ++e) v[j][k][e] = 0.f;
-      }
+      // (a chunk without a visible key is not loaded; its registers are never
+      //  used: every select below takes the masked branch for it)
+      if (mbits[j][k] != (1u << E) - 1u) load_chunk<T, E>(xr + (int64_t)c * E, v[j][k]);
     }
   }
 
@@ -334,8 +341,8 @@ __global__ __launch_bounds__(1024) void softmax_fwd_kernel(
     // a row without any visible key: uniform distribution, as softmax of a
     // constant fill value gives
     const bool empty = mx[j] == ninf;
-    const float inv = empty ? 0.f : 1.0f / sm[j];
-    const float fill = empty ? 1.0f / (float)g.sk : 0.f;
+    const float inv = empty ? 0.f : row_recip(sm[j]);
+    const float fill = empty ? g.inv_sk : 0.f;
     T *yr = y + row[j] * g.sk;
     if constexpr (DROP) {
       if (c0 == 0) {
@@ -419,7 +426,7 @@ __global__ __launch_bounds__(1024) void softmax_dropout_bwd_kernel(
   __shared__ float red[16];
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int rslot = wave / g.wpr;
+  const int rslot = g.wpr == 1 ? wave : wave / g.wpr;  // (uniform: the division is skipped)
   const int first = rslot * g.wpr;
   const int nchunks = g.sk / E;
   const int cstride = LPR == kWave ? kWave * g.wpr : LPR;
@@ -559,7 +566,7 @@ __global__ __launch_bounds__(1024) void softmax_bwd_kernel(
   const int lane = threadIdx.x & 63;
   // the wave index is uniform: keep it (and the row arithmetic) in scalar registers
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int rslot = wave / g.wpr;
+  const int rslot = g.wpr == 1 ? wave : wave / g.wpr;  // (uniform: the division is skipped)
   const int first = rslot * g.wpr;
   const int nchunks = g.sk / E;
   const int cstride = LPR == kWave ? kWave * g.wpr : LPR;
@@ -724,8 +731,8 @@ __global__ __launch_bounds__(256) void softmax_fwd_generic_kernel(
             sub_rn(mul_rn(io<T>::from_scalar(xr[i]), c2), m));
     }
     s = block_reduce_256(s, sh, false);
-    const float inv = empty ? 0.f : 1.0f / s;
-    const float fill = empty ? 1.0f / (float)g.sk : 0.f;
+    const float inv = empty ? 0.f : row_recip(s);
+    const float fill = empty ? g.inv_sk : 0.f;
     for (int i = threadIdx.x; i < g.sk; i += 256) {
       const bool hidden = MODE == kModeCausal ? i >= visible : (mrow[i] != 0 || i >= visible);
       float p = 0.f;
@@ -937,8 +944,8 @@ __global__ __launch_bounds__(256) void softmax_fwd_wave_kernel(
         s += p;
       }
     s = wave_sum(s);
-    const float inv = empty ? 0.f : 1.0f / s;
-    const float fill = empty ? 1.0f / (float)g.sk : 0.f;
+    const float inv = empty ? 0.f : row_recip(s);
+    const float fill = empty ? g.inv_sk : 0.f;
 #pragma unroll
     for (int k = 0; k < K; ++k) {
       const int i0 = (lane + kWave * k) * EW;
