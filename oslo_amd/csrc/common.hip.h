@@ -500,4 +500,50 @@ __device__ __forceinline__ uint32_t chunk_keep_bits(int64_t row, int row_length,
   return keep;
 }
 
+// The same keep decisions straight from the generator's words, for kernels
+// that use every decision once: element e of the chunk is kept when 16-bit
+// field (e & 1) of word w[e >> 1] reaches the threshold.  Comparing a field
+// where it is used (one sub-word compare and one select) takes fewer
+// instructions than packing the decisions into bits and testing the bits again.
+template <int E>
+struct KeepWords {
+  uint32_t w[E / 2];
+  uint32_t threshold;
+  __device__ __host__ __forceinline__ bool kept(int e) const {
+    const uint32_t f = (e & 1) ? (w[e >> 1] >> 16) : (w[e >> 1] & 0xffffu);
+    return f >= threshold;
+  }
+};
+
+template <int E>
+__device__ __host__ __forceinline__ KeepWords<E>
+group_keep_words(uint64_t flat, uint64_t seed, uint64_t offset, uint32_t threshold) {
+  static_assert(E == 4 || E == 8, "a chunk is a dropout group or half of one");
+  const uint64_t group = flat >> 3;
+  const Philox4 r =
+      philox4x32_10((uint32_t)offset, (uint32_t)(offset >> 32),
+                    (uint32_t)group, (uint32_t)(group >> 32), (uint32_t)seed,
+                    (uint32_t)(seed >> 32));
+  KeepWords<E> k;
+  k.threshold = threshold;
+  if constexpr (E == 8) {
+    k.w[0] = r.x;
+    k.w[1] = r.y;
+    k.w[2] = r.z;
+    k.w[3] = r.w;
+  } else {
+    const bool hi = (flat & 4u) != 0u;  // which half of the group the chunk is
+    k.w[0] = hi ? r.z : r.x;
+    k.w[1] = hi ? r.w : r.y;
+  }
+  return k;
+}
+
+template <int E>
+__device__ __forceinline__ KeepWords<E> chunk_keep_words(int64_t row, int row_length, int c,
+                                                         const DropArgs &d) {
+  const uint64_t flat = (uint64_t)row * (uint64_t)row_length + (uint64_t)c * E;
+  return group_keep_words<E>(flat, d.seed, d.offset, d.threshold);
+}
+
 }  // namespace oslo

@@ -394,15 +394,18 @@ __global__ __launch_bounds__(1024) void softmax_fwd_kernel(
         if constexpr (DROP) {
           // exact zeros need no draw (wave-uniform test)
           if (!none_visible[j][k] || empty) {
-            uint32_t keep;
             if constexpr (kPairDraw) {
-              keep = paired ? keepk[k] : chunk_keep_bits<E>(row[j], g.sk, c, d);
-            } else {
-              keep = chunk_keep_bits<E>(row[j], g.sk, c, d);
-            }
+              const uint32_t keep =
+                  paired ? keepk[k] : chunk_keep_bits<E>(row[j], g.sk, c, d);
 #pragma unroll
-            for (int e = 0; e < E; ++e)
-              o[e] = (keep >> e) & 1u ? o[e] * d.scale : 0.f;
+              for (int e = 0; e < E; ++e)
+                o[e] = (keep >> e) & 1u ? o[e] * d.scale : 0.f;
+            } else {
+              const KeepWords<E> keep = chunk_keep_words<E>(row[j], g.sk, c, d);
+#pragma unroll
+              for (int e = 0; e < E; ++e)
+                o[e] = keep.kept(e) ? o[e] * d.scale : 0.f;
+            }
           }
         }
         store_chunk<T, E>(yr + (int64_t)c * E, o);
@@ -510,8 +513,9 @@ __global__ __launch_bounds__(1024) void softmax_dropout_bwd_kernel(
     for (int k = 0; k < VPL; ++k) {
       if (none_loaded[j][k]) continue;
       const int c = c0 + k * cstride;
-      const uint32_t keep =
-          mbits[j][k] != kAll ? chunk_keep_bits<E>(row[j], g.sk, c, d) : 0u;
+      // (a chunk without a visible key was not loaded: its gradients are zeros
+      //  whatever the draw says)
+      const KeepWords<E> keep = chunk_keep_words<E>(row[j], g.sk, c, d);
 #pragma unroll
       for (int e = 0; e < E; ++e) {
         // the product is rounded before the subtraction, exactly as the
@@ -520,7 +524,7 @@ __global__ __launch_bounds__(1024) void softmax_dropout_bwd_kernel(
             __builtin_amdgcn_exp2f(sub_rn(mul_rn(yv[j][k][e], c2), rmax[j])) * rinv[j];
         if (empty) p = -rinv[j];
         if ((mbits[j][k] >> e) & 1u) p = 0.f;
-        const float dp = (keep >> e) & 1u ? mul_rn(gv[j][k][e], d.scale) : 0.f;
+        const float dp = keep.kept(e) ? mul_rn(gv[j][k][e], d.scale) : 0.f;
         yv[j][k][e] = p;
         gv[j][k][e] = dp;
         a += p * dp;
