@@ -41,11 +41,18 @@ __device__ __forceinline__ float gelu_fwd(float u) {
 // d gelu / du = 0.5 u (1 - t^2)(0.79788456 + 0.1070322243 u^2) + 0.5 (1 + t)
 // with t = tanh z; in terms of s = sigmoid(2 z), e = exp(-2 z):
 // 1 + t = 2 s and 1 - t^2 = 4 e s^2.
+// Evaluated as s + w s (1 - s) with w = u (2 * 0.79788456 + 2 * 0.1070322243 u^2)
+// and e s^2 = s (1 - s) formed by one fused multiply-add: nine instructions and
+// two transcendentals.  (Where s rounds to 1 the product term, of relative size
+// below 1e-6, is dropped; elsewhere the form is good to a few 1e-6.)
 __device__ __forceinline__ float gelu_bwd(float u) {
-  const float arg = fminf(u * (kGeluK1 + kGeluK2 * u * u), 80.0f);
+  const float u2 = u * u;
+  const float arg = fminf(u * __builtin_fmaf(kGeluK2, u2, kGeluK1), 80.0f);
   const float e = __builtin_amdgcn_exp2f(arg);
   const float s = __builtin_amdgcn_rcpf(1.0f + e);
-  return 2.0f * u * (e * s * s) * (0.79788456f + 0.1070322243f * u * u) + s;
+  const float t = __builtin_fmaf(-s, s, s);
+  const float w = u * __builtin_fmaf(2.0f * 0.1070322243f, u2, 2.0f * 0.79788456f);
+  return __builtin_fmaf(w, t, s);
 }
 
 struct EltGeom {
