@@ -152,10 +152,12 @@ def _project_gelu(layer, x):
 
 
 # (up projection, down projection or None, activation): GPT-2 / GPT-Neo MLP,
-# GPT-J MLP, BERT-style intermediate block
+# GPT-J MLP, GPT-NeoX / Falcon MLP (no dropout of its own), BERT-style
+# intermediate block.  A ``dropout`` child after the down projection is optional.
 _MLP_SHAPES = (
     ("c_fc", "c_proj", "act"),
     ("fc_in", "fc_out", "act"),
+    ("dense_h_to_4h", "dense_4h_to_h", "act"),
     ("dense", None, "intermediate_act_fn"),
 )
 
@@ -165,17 +167,17 @@ def _mlp_shape(module):
         names = list(inspect.signature(type(module).forward).parameters)
     except (TypeError, ValueError):
         return None
-    if names != ["self", "hidden_states"]:
+    if len(names) != 2 or names[0] != "self":  # forward(self, hidden_states) under any name
         return None
     children = dict(module.named_children())
     for up, down, act in _MLP_SHAPES:
-        expected = {up} | ({down, "dropout"} if down else set())
-        others = set(children) - expected - {act}
-        if others or not expected <= set(children):
+        expected = {up} | ({down} if down else set())
+        optional = {act} | ({"dropout"} if down else set())
+        if not expected <= set(children) or set(children) - expected - optional:
             continue
         if not _is_projection(children[up]) or (down and not _is_projection(children[down])):
             continue
-        if down and not isinstance(children["dropout"], nn.Dropout):
+        if "dropout" in children and not isinstance(children["dropout"], nn.Dropout):
             continue
         fn = getattr(module, act, None)
         if callable(fn) and _is_tanh_gelu(fn):
@@ -188,7 +190,9 @@ def _mlp_forward(self, hidden_states):
     h = _project_gelu(getattr(self, up), hidden_states)
     if down is None:
         return h
-    return self.dropout(getattr(self, down)(h))
+    h = getattr(self, down)(h)
+    dropout = getattr(self, "dropout", None)
+    return h if dropout is None else dropout(h)
 
 
 _MLP_CLASSES = {}
@@ -505,7 +509,10 @@ def fuse_all(model, attention=True):
     if attention and hasattr(model, "config"):
         try:
             fused_scale_mask_softmax(model)
-            changed["fused_scale_mask_softmax"] = True
+            # (a model without pluggable attention keeps its own implementation)
+            changed["fused_scale_mask_softmax"] = (
+                getattr(model.config, "_attn_implementation", None) == ATTENTION_NAME
+            )
         except (ImportError, ValueError):
             pass  # no pluggable attention in this model / library version
     return changed

@@ -458,6 +458,76 @@ def test_fuse_all_on_cpu():
     assert torch.allclose(b(ids, attention_mask=am).last_hidden_state[valid], ref[valid], atol=1e-5, rtol=1e-5)
 
 
+def tiny_neox(seed=0, **kw):
+    from transformers import GPTNeoXConfig, GPTNeoXForCausalLM
+
+    torch.manual_seed(seed)
+    cfg = GPTNeoXConfig(vocab_size=211, hidden_size=64, num_hidden_layers=2, num_attention_heads=4,
+                        intermediate_size=256, hidden_act="gelu_fast", max_position_embeddings=64,
+                        use_parallel_residual=True, attention_dropout=0.0, hidden_dropout=0.0, **kw)
+    return GPTNeoXForCausalLM(cfg)
+
+
+def test_gpt_neox_swaps_on_cpu_keep_the_model_output():
+    """The GPT-NeoX block (the shape of BASELINE configuration 5): its MLP has
+    no dropout of its own and names its projections dense_h_to_4h /
+    dense_4h_to_h; norms, bias-GeLU and the attention function are swapped."""
+    from oslo_amd.transformers import fuse_all
+
+    ids, am = inputs()
+    m = tiny_neox().eval()
+    ref = m(ids, attention_mask=am).logits
+    changed = fuse_all(m)
+    assert changed["fused_bias_gelu"] == 2 and changed["fused_layer_norm"] == 5
+    assert changed["fused_scale_mask_softmax"] is True
+    valid = am.bool()
+    assert torch.allclose(m(ids, attention_mask=am).logits[valid], ref[valid], atol=1e-5, rtol=1e-5)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_gpt_neox_with_every_swap_outputs_and_gradients(device, dtype, monkeypatch):
+    from oslo_amd.torch import _C
+    from oslo_amd.transformers import fuse_all
+
+    ids, am = inputs(b=3, s=32)
+    ids, am = ids.to(device), am.to(device)
+    ref = tiny_neox(seed=5).to(device).to(dtype).train()
+    fused = tiny_neox(seed=5).to(device).to(dtype).train()
+    changed = fuse_all(fused)
+    assert changed["fused_bias_gelu"] == 2 and changed["fused_layer_norm"] == 5
+    kernel = _C.get_fused_elementwise_kernel()
+    sm = _C.get_softmax_kernel()
+    calls = {"gelu": 0, "softmax": 0}
+    gelu_fwd, sm_fwd = kernel.bias_gelu_forward, sm.fused_scaled_masked_softmax_forward
+
+    def counted_gelu(*a, **k):
+        calls["gelu"] += 1
+        return gelu_fwd(*a, **k)
+
+    def counted_softmax(*a, **k):
+        calls["softmax"] += 1
+        return sm_fwd(*a, **k)
+
+    monkeypatch.setattr(kernel, "bias_gelu_forward", counted_gelu)
+    monkeypatch.setattr(sm, "fused_scaled_masked_softmax_forward", counted_softmax)
+    lr = ref(ids, attention_mask=am, labels=ids).loss
+    lf = fused(ids, attention_mask=am, labels=ids).loss
+    assert calls["gelu"] == 2      # one bias-GeLU kernel per block
+    assert calls["softmax"] == 2   # a padded causal batch: the masked softmax kernel, once per block
+    assert abs(lr.item() - lf.item()) <= (1e-4 if dtype == torch.float32 else 3e-2)
+    lr.backward()
+    lf.backward()
+    gtol = 2e-3 if dtype == torch.float32 else 8e-2
+    gmax = max(p.grad.float().abs().max().item() for p in ref.parameters() if p.grad is not None)
+    floor = 1e-8 if dtype == torch.float32 else 1e-3 * gmax
+    for (n, pr), (_, pf) in zip(ref.named_parameters(), fused.named_parameters()):
+        if pr.grad is None:
+            continue
+        scale = pr.grad.float().abs().max().item() + floor
+        assert (pr.grad.float() - pf.grad.float()).abs().max().item() <= gtol * scale + 1e-6, n
+
+
 def tiny_t5(seed=0):
     from transformers import T5Config, T5ForConditionalGeneration
 
