@@ -528,6 +528,83 @@ def test_gpt_neox_with_every_swap_outputs_and_gradients(device, dtype, monkeypat
         assert (pr.grad.float() - pf.grad.float()).abs().max().item() <= gtol * scale + 1e-6, n
 
 
+def _family(name):
+    import transformers as tf
+
+    kw = dict(vocab_size=211, max_position_embeddings=64)
+    if name == "llama":
+        return tf.LlamaForCausalLM(tf.LlamaConfig(hidden_size=64, intermediate_size=128, num_hidden_layers=2,
+                                                  num_attention_heads=4, num_key_value_heads=2, **kw))
+    if name == "mistral":
+        return tf.MistralForCausalLM(tf.MistralConfig(hidden_size=64, intermediate_size=128, num_hidden_layers=2,
+                                                      num_attention_heads=4, num_key_value_heads=2,
+                                                      sliding_window=16, **kw))
+    if name == "gptj":
+        return tf.GPTJForCausalLM(tf.GPTJConfig(vocab_size=211, n_embd=64, n_layer=2, n_head=4, rotary_dim=8,
+                                                n_positions=64))
+    if name == "opt":
+        return tf.OPTForCausalLM(tf.OPTConfig(hidden_size=64, ffn_dim=128, num_hidden_layers=2,
+                                              num_attention_heads=4, word_embed_proj_dim=64, dropout=0.0, **kw))
+    if name == "bloom":
+        return tf.BloomForCausalLM(tf.BloomConfig(vocab_size=211, hidden_size=64, n_layer=2, n_head=4))
+    raise ValueError(name)
+
+
+# what fuse_all finds in each architecture: (layer norms, rms norms, bias-GeLU blocks, attention swapped)
+FAMILIES = {
+    "llama": (0, 5, 0, True),      # RMSNorm, grouped-query attention
+    "mistral": (0, 5, 0, True),    # sliding-window mask: the general masked kernel
+    "gptj": (3, 0, 2, False),      # fc_in / fc_out MLP with gelu_new
+    "opt": (5, 0, 0, True),
+    "bloom": (6, 0, 0, False),
+}
+
+
+@pytest.mark.parametrize("name", sorted(FAMILIES))
+def test_fuse_all_across_architectures_on_cpu(name):
+    from oslo_amd.transformers import fuse_all
+
+    torch.manual_seed(0)
+    m = _family(name).eval()
+    ids, am = inputs()
+    with torch.no_grad():
+        ref = m(ids, attention_mask=am).logits
+    changed = fuse_all(m)
+    ln, rms, gelu, attn = FAMILIES[name]
+    assert (changed["fused_layer_norm"], changed["fused_rms_norm"], changed["fused_bias_gelu"],
+            changed["fused_scale_mask_softmax"]) == (ln, rms, gelu, attn), changed
+    with torch.no_grad():
+        out = m(ids, attention_mask=am).logits
+    valid = am.bool()
+    assert torch.allclose(out[valid], ref[valid], atol=2e-5, rtol=1e-5)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", ["llama", "mistral", "gptj", "opt"])
+def test_fuse_all_across_architectures_on_gpu(device, name):
+    """Logits and every parameter gradient of the swapped model against the
+    model as Hugging Face builds it, fp32, on a right-padded batch."""
+    from oslo_amd.transformers import fuse_all
+
+    ids, am = inputs(b=3, s=32)
+    ids, am = ids.to(device), am.to(device)
+    torch.manual_seed(0)
+    ref = _family(name).to(device).train()
+    torch.manual_seed(0)
+    fused = _family(name).to(device).train()
+    fuse_all(fused)
+    lr = ref(ids, attention_mask=am, labels=ids).loss
+    lf = fused(ids, attention_mask=am, labels=ids).loss
+    assert abs(lr.item() - lf.item()) <= 1e-4
+    lr.backward()
+    lf.backward()
+    for (n, pr), (_, pf) in zip(ref.named_parameters(), fused.named_parameters()):
+        if pr.grad is None:
+            continue
+        scale = pr.grad.abs().max().item() + 1e-8
+        assert (pr.grad - pf.grad).abs().max().item() <= 2e-3 * scale + 1e-6, n
+
+
 def tiny_t5(seed=0):
     from transformers import T5Config, T5ForConditionalGeneration
 
