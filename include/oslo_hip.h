@@ -12,7 +12,10 @@
  *   - Return value: OSLO_OK (0) or a negative OSLO_ERR_* code; the message
  *     for the calling thread's last failure is oslo_hip_last_error().
  *   - dtype arguments take OSLO_DTYPE_* values.  Accumulation is fp32.
- *   - Element counts are 64-bit; a tensor may exceed 2^31 elements.
+ *   - Element counts are 64-bit; a tensor may exceed 2^31 elements, and a
+ *     softmax may have more than 2^31 rows.  A GPU dispatch holds fewer than
+ *     2^32 work-items: an entry point whose problem needs more issues several
+ *     launches on the stream (still without synchronising).
  *
  * Each declaration cites the interface of the reference (EleutherAI/oslo) it
  * replaces; paths are relative to the reference's repository root.

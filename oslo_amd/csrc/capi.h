@@ -68,6 +68,13 @@ inline int dtype_size(int d) {
 
 inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 
+// A dispatch carries its size as a 32-bit count of work-items, so workgroups x
+// workgroup size must stay below 2^32.  The runtime does not report an excess:
+// the count wraps and only part of the grid runs.  Launchers therefore cap the
+// grid of a kernel that strides over its work, and split the work of a kernel
+// that does one unit per workgroup into several launches.
+inline int64_t max_workgroups(int threads) { return (int64_t)0xffffffffll / threads; }
+
 // Double-precision LayerNorm / RMSNorm (norm_f64.hip); every pointer is to
 // double data.
 int launch_norm_f64_fwd(bool rms, const void *x, const void *gamma,

@@ -64,6 +64,9 @@ struct EltGeom {
   int tiles;    // column tiles = ceil(nchunks / tx)
   int64_t slots;  // workgroups per column tile; slot s visits row steps
                   // s, s + slots, s + 2 slots, ... of ty * U rows each
+  // index of the launch's first workgroup among those of the whole problem (a
+  // forward problem beyond 2^32 work-items takes several launches)
+  int64_t blk0 = 0;
 };
 
 // Position of this thread: column chunk cc (may be >= nchunks), its row
@@ -75,7 +78,7 @@ struct EltPos {
   int64_t slot;
 };
 __device__ __forceinline__ EltPos elt_pos(const EltGeom &g) {
-  const int64_t b = blockIdx.x;
+  const int64_t b = (int64_t)blockIdx.x + g.blk0;
   EltPos p;
   p.slot = b / g.tiles;
   p.cc = (int)(b - p.slot * g.tiles) * g.tx + (int)(threadIdx.x % g.tx);
@@ -623,19 +626,23 @@ static int run_bias_gelu_fwd(const void *x, const void *bias, void *y,
     return check_launch("bias_gelu_fwd_generic_kernel");
   }
   const int unroll = eltwise_unroll(2);
-  const EltGeom g = eltwise_geom_fwd(rows, cols, unroll, kE);
+  EltGeom g = eltwise_geom_fwd(rows, cols, unroll, kE);
   const int64_t nblocks = g.slots * g.tiles;
-  OSLO_REQUIRE(nblocks <= 0x7fffffff, "bias_gelu fwd: too many workgroups");
-  const dim3 grid((unsigned)nblocks);
-  OSLO_ELT_U(unroll, {
-    if (bias)
-      bias_gelu_fwd_kernel<T, U, true><<<grid, 256, 0, st>>>(
-          (const T *)x, (const T *)bias, (T *)y, g);
-    else
-      bias_gelu_fwd_kernel<T, U, false><<<grid, 256, 0, st>>>(
-          (const T *)x, nullptr, (T *)y, g);
-  });
-  return check_launch("bias_gelu_fwd_kernel");
+  const int64_t per_launch = max_workgroups(256);
+  for (g.blk0 = 0; g.blk0 < nblocks; g.blk0 += per_launch) {
+    const dim3 grid((unsigned)(nblocks - g.blk0 < per_launch ? nblocks - g.blk0 : per_launch));
+    OSLO_ELT_U(unroll, {
+      if (bias)
+        bias_gelu_fwd_kernel<T, U, true><<<grid, 256, 0, st>>>(
+            (const T *)x, (const T *)bias, (T *)y, g);
+      else
+        bias_gelu_fwd_kernel<T, U, false><<<grid, 256, 0, st>>>(
+            (const T *)x, nullptr, (T *)y, g);
+    });
+    const int rc = check_launch("bias_gelu_fwd_kernel");
+    if (rc != OSLO_OK) return rc;
+  }
+  return OSLO_OK;
 }
 
 template <typename T>
@@ -660,7 +667,7 @@ static int run_bias_gelu_bwd(const void *gr, const void *x, const void *bias,
   const EltGeom g = eltwise_geom_bwd(rows, cols, unroll, kE);
   const int64_t parts = g.slots;
   const int64_t nblocks = parts * g.tiles;
-  OSLO_REQUIRE(nblocks <= 0x7fffffff, "bias_gelu bwd: too many workgroups");
+  OSLO_REQUIRE(nblocks <= max_workgroups(256), "bias_gelu bwd: too many workgroups");
   const dim3 grid((unsigned)nblocks);
   float *part = nullptr;
   if (dbias != nullptr) {
@@ -705,28 +712,32 @@ static int run_bda_fwd(const void *x, const void *bias, const void *res,
     return check_launch("bias_dropout_add_fwd_generic_kernel");
   }
   const int unroll = eltwise_unroll(2) > 2 ? 2 : eltwise_unroll(2);
-  const EltGeom g = eltwise_geom_fwd(rows, cols, unroll, kE);
+  EltGeom g = eltwise_geom_fwd(rows, cols, unroll, kE);
   const int64_t nblocks = g.slots * g.tiles;
-  OSLO_REQUIRE(nblocks <= 0x7fffffff, "bias_dropout_add fwd: too many workgroups");
-  const dim3 grid((unsigned)nblocks);
+  const int64_t per_launch = max_workgroups(256);
 #define OSLO_BDA_FWD(HB, HR, DR)                                            \
   bias_dropout_add_fwd_kernel<T, U, HB, HR, DR><<<grid, 256, 0, st>>>(      \
       (const T *)x, (const T *)bias, (const T *)res, (T *)out, mask_out, g, d)
-  OSLO_ELT_U(unroll, {
-    const int key = (bias ? 4 : 0) | (res ? 2 : 0) | (drop ? 1 : 0);
-    switch (key) {
-      case 0: OSLO_BDA_FWD(false, false, false); break;
-      case 1: OSLO_BDA_FWD(false, false, true); break;
-      case 2: OSLO_BDA_FWD(false, true, false); break;
-      case 3: OSLO_BDA_FWD(false, true, true); break;
-      case 4: OSLO_BDA_FWD(true, false, false); break;
-      case 5: OSLO_BDA_FWD(true, false, true); break;
-      case 6: OSLO_BDA_FWD(true, true, false); break;
-      default: OSLO_BDA_FWD(true, true, true); break;
-    }
-  });
+  for (g.blk0 = 0; g.blk0 < nblocks; g.blk0 += per_launch) {
+    const dim3 grid((unsigned)(nblocks - g.blk0 < per_launch ? nblocks - g.blk0 : per_launch));
+    OSLO_ELT_U(unroll, {
+      const int key = (bias ? 4 : 0) | (res ? 2 : 0) | (drop ? 1 : 0);
+      switch (key) {
+        case 0: OSLO_BDA_FWD(false, false, false); break;
+        case 1: OSLO_BDA_FWD(false, false, true); break;
+        case 2: OSLO_BDA_FWD(false, true, false); break;
+        case 3: OSLO_BDA_FWD(false, true, true); break;
+        case 4: OSLO_BDA_FWD(true, false, false); break;
+        case 5: OSLO_BDA_FWD(true, false, true); break;
+        case 6: OSLO_BDA_FWD(true, true, false); break;
+        default: OSLO_BDA_FWD(true, true, true); break;
+      }
+    });
+    const int rc = check_launch("bias_dropout_add_fwd_kernel");
+    if (rc != OSLO_OK) return rc;
+  }
 #undef OSLO_BDA_FWD
-  return check_launch("bias_dropout_add_fwd_kernel");
+  return OSLO_OK;
 }
 
 template <typename T>
@@ -762,7 +773,7 @@ static int run_bda_bwd(const void *gr, void *dx, void *dbias, void *ws,
   const EltGeom g = eltwise_geom_bwd(rows, cols, unroll, kE);
   const int64_t parts = g.slots;
   const int64_t nblocks = parts * g.tiles;
-  OSLO_REQUIRE(nblocks <= 0x7fffffff, "bias_dropout_add bwd: too many workgroups");
+  OSLO_REQUIRE(nblocks <= max_workgroups(256), "bias_dropout_add bwd: too many workgroups");
   const dim3 grid((unsigned)nblocks);
   float *part = nullptr;
   if (dbias != nullptr) {
@@ -912,7 +923,7 @@ int oslo_copy_probe(const void *src, void *dst, int64_t bytes, void *stream) {
   if (bytes == 0) return OSLO_OK;
   const int64_t nvec = bytes / 16;
   int64_t grid = ceil_div(nvec, 256);
-  if (grid > 0x7fffffff) grid = 0x7fffffff;
+  if (grid > max_workgroups(256)) grid = max_workgroups(256);  // (the kernel strides over the vectors)
   copy_probe_kernel<<<dim3((unsigned)grid), 256, 0, (hipStream_t)stream>>>(
       (const u32x4 *)src, (u32x4 *)dst, nvec);
   return check_launch("copy_probe_kernel");

@@ -116,8 +116,8 @@ static int launch_adam(const void *const *g, void *const *p, void *const *m,
     if (tab.ntensors == 0) return OSLO_OK;
     const int64_t blocks = tab.first_block[tab.ntensors];
     if (blocks > 0) {
-      if (blocks > 0x7fffffff)
-        return fail(OSLO_ERR_UNSUPPORTED, "multi_tensor_adam: too many workgroups");
+      if (blocks > max_workgroups(kAdamThreads))
+        return fail(OSLO_ERR_UNSUPPORTED, "multi_tensor_adam: a tensor too large for one launch");
       multi_tensor_adam_kernel<T, kAdamUnroll>
           <<<dim3((unsigned)blocks), kAdamThreads, 0, st>>>(tab, a);
       const int rc = check_launch("multi_tensor_adam_kernel");
@@ -134,9 +134,9 @@ static int launch_adam(const void *const *g, void *const *p, void *const *m,
     if (!g[i] || !p[i] || !m[i] || !v[i])
       return fail(OSLO_ERR_INVALID_ARGUMENT, "multi_tensor_adam: tensor %lld has a null pointer",
                   (long long)i);
-    // one launch stays below 2^31 workgroups
+    // one launch stays below 2^32 work-items
     if (tab.ntensors > 0 &&
-        tab.first_block[tab.ntensors] + ceil_div(sizes[i], kPiece) > 0x7fffffff) {
+        tab.first_block[tab.ntensors] + ceil_div(sizes[i], kPiece) > max_workgroups(kAdamThreads)) {
       const int rc = flush();
       if (rc != OSLO_OK) return rc;
     }

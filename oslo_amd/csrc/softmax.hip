@@ -38,6 +38,9 @@ struct SoftmaxGeom {
   // filled in by set_fast_div on the host
   uint32_t sq_mul = 0, sq_shift = 32, np_mul = 0, np_shift = 32;
   float inv_sk = 0.f;  // 1 / sk, the value of a row without a visible key
+  // index of the launch's first workgroup among those of the whole problem (a
+  // problem beyond 2^32 work-items takes several launches)
+  int64_t blk0 = 0;
 };
 
 // Division of n < 2^31 by a divisor 1 <= d < 2^31 fixed for the launch: with
@@ -214,7 +217,7 @@ __global__ __launch_bounds__(1024) void softmax_fwd_kernel(
 
   // first row of this lane: the wave's first row plus the lane group's index
   const int64_t rbase =
-      ((int64_t)blockIdx.x * g.rpb + rslot) * (RPW * SUB) +
+      (((int64_t)blockIdx.x + g.blk0) * g.rpb + rslot) * (RPW * SUB) +
       (LPR == kWave ? 0 : lane / LPR);
 
   float v[RPW][VPL][E];
@@ -436,7 +439,7 @@ __global__ __launch_bounds__(1024) void softmax_dropout_bwd_kernel(
   constexpr int SUB = kWave / LPR;
   const int sl = LPR == kWave ? lane : (lane & (LPR - 1));
   const int c0 = (wave - first) * kWave + sl;
-  const int64_t rbase = ((int64_t)blockIdx.x * g.rpb + rslot) * (RPW * SUB) +
+  const int64_t rbase = (((int64_t)blockIdx.x + g.blk0) * g.rpb + rslot) * (RPW * SUB) +
                         (LPR == kWave ? 0 : lane / LPR);
   const float c2 = scale * kLog2e;
 
@@ -578,7 +581,7 @@ __global__ __launch_bounds__(1024) void softmax_bwd_kernel(
   const int sl = LPR == kWave ? lane : (lane & (LPR - 1));
   const int c0 = (wave - first) * kWave + sl;
 
-  const int64_t rbase = ((int64_t)blockIdx.x * g.rpb + rslot) * (RPW * SUB) +
+  const int64_t rbase = (((int64_t)blockIdx.x + g.blk0) * g.rpb + rslot) * (RPW * SUB) +
                         (LPR == kWave ? 0 : lane / LPR);
 
   float yv[RPW][VPL][E], gv[RPW][VPL][E];
@@ -1323,9 +1326,9 @@ static int launch_softmax_fwd(const void *x, const uint8_t *mask, void *y,
   g.wpr = pl.wpr;
   g.rpb = pl.rpb;
   const int threads = kWave * pl.wpr * pl.rpb;
-  const int64_t grid =
+  const int64_t nblocks =
       ceil_div(g.rows, (int64_t)pl.rpb * pl.rpw * (kWave / pl.lpr));
-  OSLO_REQUIRE(grid <= 0x7fffffff, "softmax fwd: too many rows");
+  const int64_t per_launch = max_workgroups(threads);
 #define OSLO_SM_FWD(VPL, RPW, LPR_)                                  \
   if constexpr (VPL * RPW * E <= kFwdMaxElems) {                     \
     if (drop)                                                        \
@@ -1338,9 +1341,14 @@ static int launch_softmax_fwd(const void *x, const uint8_t *mask, void *y,
               (const T *)x, mask, (T *)y, nullptr, g, scale, d);     \
   } else                                                             \
     return fail(OSLO_ERR_UNSUPPORTED, "softmax fwd: no kernel for %d x %d chunks per lane", VPL, RPW)
-  OSLO_SM_CASES(OSLO_SM_FWD)
+  for (g.blk0 = 0; g.blk0 < nblocks; g.blk0 += per_launch) {
+    const int64_t grid = nblocks - g.blk0 < per_launch ? nblocks - g.blk0 : per_launch;
+    OSLO_SM_CASES(OSLO_SM_FWD)
+    const int rc = check_launch("softmax_fwd_kernel");
+    if (rc != OSLO_OK) return rc;
+  }
 #undef OSLO_SM_FWD
-  return check_launch("softmax_fwd_kernel");
+  return OSLO_OK;
 }
 
 template <typename T, int MODE>
@@ -1389,9 +1397,9 @@ static int launch_softmax_bwd(const void *dy, const void *y,
   g.wpr = pl.wpr;
   g.rpb = pl.rpb;
   const int threads = kWave * pl.wpr * pl.rpb;
-  const int64_t grid =
+  const int64_t nblocks =
       ceil_div(g.rows, (int64_t)pl.rpb * pl.rpw * (kWave / pl.lpr));
-  OSLO_REQUIRE(grid <= 0x7fffffff, "softmax bwd: too many rows");
+  const int64_t per_launch = max_workgroups(threads);
 #define OSLO_SM_BWD(VPL, RPW, LPR_)                        \
   if constexpr (VPL * RPW * E <= kBwdMaxElems)             \
     softmax_bwd_kernel<T, VPL, RPW, MODE, LPR_>            \
@@ -1399,9 +1407,14 @@ static int launch_softmax_bwd(const void *dy, const void *y,
             (const T *)dy, (const T *)y, mask, (T *)dx, g, scale); \
   else                                                     \
     return fail(OSLO_ERR_UNSUPPORTED, "softmax bwd: no kernel for %d x %d chunks per lane", VPL, RPW)
-  OSLO_SM_CASES(OSLO_SM_BWD)
+  for (g.blk0 = 0; g.blk0 < nblocks; g.blk0 += per_launch) {
+    const int64_t grid = nblocks - g.blk0 < per_launch ? nblocks - g.blk0 : per_launch;
+    OSLO_SM_CASES(OSLO_SM_BWD)
+    const int rc = check_launch("softmax_bwd_kernel");
+    if (rc != OSLO_OK) return rc;
+  }
 #undef OSLO_SM_BWD
-  return check_launch("softmax_bwd_kernel");
+  return OSLO_OK;
 }
 
 template <typename T, int MODE>
@@ -1452,9 +1465,9 @@ static int launch_softmax_dropout_bwd(const void *dy, const void *x,
   g.wpr = pl.wpr;
   g.rpb = pl.rpb;
   const int threads = kWave * pl.wpr * pl.rpb;
-  const int64_t grid =
+  const int64_t nblocks =
       ceil_div(g.rows, (int64_t)pl.rpb * pl.rpw * (kWave / pl.lpr));
-  OSLO_REQUIRE(grid <= 0x7fffffff, "softmax dropout bwd: too many rows");
+  const int64_t per_launch = max_workgroups(threads);
 #define OSLO_SM_DBWD(VPL, RPW, LPR_)                                \
   if constexpr (VPL * RPW * E <= kBwdMaxElems)                      \
     softmax_dropout_bwd_kernel<T, VPL, RPW, MODE, LPR_>             \
@@ -1463,9 +1476,14 @@ static int launch_softmax_dropout_bwd(const void *dy, const void *x,
             scale, d);                                              \
   else                                                              \
     return fail(OSLO_ERR_UNSUPPORTED, "softmax dropout bwd: no kernel for %d x %d chunks per lane", VPL, RPW)
-  OSLO_SM_CASES(OSLO_SM_DBWD)
+  for (g.blk0 = 0; g.blk0 < nblocks; g.blk0 += per_launch) {
+    const int64_t grid = nblocks - g.blk0 < per_launch ? nblocks - g.blk0 : per_launch;
+    OSLO_SM_CASES(OSLO_SM_DBWD)
+    const int rc = check_launch("softmax_dropout_bwd_kernel");
+    if (rc != OSLO_OK) return rc;
+  }
 #undef OSLO_SM_DBWD
-  return check_launch("softmax_dropout_bwd_kernel");
+  return OSLO_OK;
 }
 
 #define OSLO_SM_DISPATCH(dtype, MODE, FN, ...)                       \

@@ -87,6 +87,90 @@ def test_softmax_beyond_2_31_elements(device):
           "huge softmax dropout bwd", atol=3e-7)
 
 
+def test_softmax_with_more_than_2_31_rows(device):
+    """Beyond 2^31 rows the kernels recover (batch, head, query) from the row
+    index with 64-bit divisions instead of the 32-bit reciprocal multiply:
+    short rows (8 keys), 2.15e9 of them, rows on both sides of 2^31 checked."""
+    sk = 8
+    sm = _C.get_softmax_kernel()
+    # causal [attn_batches, sq, sk], sq = sk
+    ab = 4097 * 65536  # = 4097 * 64 * 8192 / 8: the same tensor serves the [b, heads, sq, sk] case below
+    rows_total = ab * sk
+    assert rows_total > 2 ** 31
+    x = gpu_randn((ab, sk, sk), BF16, 9, device, std=2.0)
+    y = sm.fused_scaled_upper_triang_masked_softmax_forward(x, 0.5)
+    rows = torch.tensor(sorted({0, 1, 7, 8, 2 ** 31 - 9, 2 ** 31 - 1, 2 ** 31, 2 ** 31 + 1, 2 ** 31 + 11,
+                                rows_total - 9, rows_total - 2, rows_total - 1}))
+    sel = rows.to(device)
+    qi = (rows % sk).numpy()
+    hidden = np.arange(sk)[None, :] > qi[:, None]
+    check(y.view(-1, sk)[sel], cf.softmax_masked_fwd(f64(x.view(-1, sk)[sel]), hidden, 0.5), "causal fwd", atol=1e-9)
+    # whole-tensor property on a slab around 2^31: the zeros sit above the diagonal, rows sum to 1
+    b0 = 2 ** 28 - 4096
+    slab = y[b0:b0 + 8192].float()
+    assert torch.triu(slab, diagonal=1).count_nonzero().item() == 0
+    assert (slab.sum(-1) - 1).abs().max().item() <= 1e-2
+    assert (slab[:, 0, 0] == 1).all()
+    del y, slab
+    # key padding [b, np, sq, sk] with one mask row per batch entry: b and np both matter
+    b, heads, sq = 4097, 64, 8192
+    assert b * heads * sq == x.numel() // sk
+    x4 = x.view(b, heads, sq, sk)
+    valid = torch.randint(1, sk + 1, (b,), generator=torch.Generator().manual_seed(3))
+    pad = torch.arange(sk)[None, :] >= valid[:, None]
+    y4 = sm.fused_scaled_masked_softmax_forward(x4, pad.view(b, 1, 1, sk).to(device), 0.5)
+    bi = (rows // (heads * sq)).numpy()
+    hidden = pad.numpy()[bi]
+    check(y4.view(-1, sk)[sel], cf.softmax_masked_fwd(f64(x.view(-1, sk)[sel]), hidden, 0.5), "padding fwd", atol=1e-9)
+    # every batch entry: exactly its padded keys are zero (a wrong batch index would show at some entry)
+    for e in (0, 1, 2047, 2048, 2049, 4095, 4096):
+        ye = y4[e, ::16, ::512].float()
+        v = int(valid[e])
+        assert ye[..., v:].count_nonzero().item() == 0
+        assert (ye[..., :v] > 0).all()
+    # the backward and the dropout pair at this row count (x doubles as the incoming gradient)
+    hidden = np.arange(sk)[None, :] > qi[:, None]
+    y = y4.view(ab, sk, sk)
+    del y4
+    y = sm.fused_scaled_upper_triang_masked_softmax_forward(x, 0.5)
+    dx = sm.fused_scaled_upper_triang_masked_softmax_backward(x, y, 0.5)
+    check(dx.view(-1, sk)[sel], cf.softmax_bwd(f64(x.view(-1, sk)[sel]), f64(y.view(-1, sk)[sel]), 0.5),
+          "causal bwd", atol=2e-7)
+    del dx, y
+    p, seed, offset = 0.2, 5, 16
+    out, stats = sm.softmax_dropout_forward(x, None, 0.5, p, seed, offset)
+    keep = np.stack([philox.keep_mask(sk, p, seed, offset, first_element=int(r) * sk) for r in rows]).astype(bool)
+    check(out.view(-1, sk)[sel], cf.softmax_dropout_fwd(f64(x.view(-1, sk)[sel]), hidden, 0.5, keep, p),
+          "causal dropout fwd", atol=1e-9)
+    ddx = sm.softmax_dropout_backward(out, x, stats, None, 0.5, p, seed, offset)
+    check(ddx.view(-1, sk)[sel],
+          cf.softmax_dropout_bwd(f64(out.view(-1, sk)[sel]), f64(x.view(-1, sk)[sel]), hidden, 0.5, keep, p),
+          "causal dropout bwd", atol=3e-7, min_exact=0.98)
+
+
+def test_elementwise_forward_beyond_2_32_work_items(device):
+    """A dispatch holds fewer than 2^32 work-items: a forward with one 128-bit
+    vector per lane over 1.72e10 fp32 elements takes two launches.  Rows on both
+    sides of the split, and the last ones, against the oracle."""
+    n2 = 1024
+    n1 = (2 ** 32 // 256) * 256 * 4 // n2 + 4096  # just beyond 2^32 lanes of 4 elements
+    assert n1 * n2 // 4 > 2 ** 32
+    F32 = torch.float32
+    x = gpu_randn((n1, n2), F32, 13, device)
+    bias = gpu_randn((n2,), F32, 14, device, std=0.1)
+    k = _C.get_fused_elementwise_kernel()
+    _C.tune("eltwise_unroll", 1)
+    try:
+        y = k.bias_gelu_forward(x, bias)
+    finally:
+        _C.tune("eltwise_unroll", 0)
+    split = 2 ** 32 * 4 // n2  # first row of the second launch
+    rows = torch.tensor(sorted({0, 1, split - 2, split - 1, split, split + 1, n1 - 2, n1 - 1}))
+    sel = rows.to(device)
+    check(y[sel], cf.bias_gelu_fwd(f64(x[sel]), f64(bias)), "huge bias-GeLU fwd", atol=1e-7)
+    assert torch.isfinite(y[-8192:]).all() and y[-8192:].abs().sum().item() > 0
+
+
 def test_adam_on_a_tensor_beyond_2_31_elements(device):
     n = 2 ** 31 + 4099
     g = torch.empty(n, device=device, dtype=BF16).normal_()
