@@ -171,6 +171,69 @@ def test_elementwise_forward_beyond_2_32_work_items(device):
     assert torch.isfinite(y[-8192:]).all() and y[-8192:].abs().sum().item() > 0
 
 
+def test_norm_with_more_than_2_31_rows(device):
+    """LayerNorm and RMSNorm over 2.15e9 rows of 8 elements: row indices beyond 32 bits in the
+    side-by-side short-row kernels, forward and backward, rows on both sides of 2^31."""
+    n2 = 8
+    n1 = 2 ** 31 + 4104
+    x = gpu_randn((n1, n2), BF16, 21, device, std=1.5, mean=0.25)
+    gamma = gpu_randn((n2,), BF16, 22, device, std=0.1, mean=1.0)
+    beta = gpu_randn((n2,), BF16, 23, device, std=0.1)
+    k = _C.get_layernorm_kernel()
+    rows = torch.tensor(sorted({0, 1, 63, 64, 2 ** 31 - 65, 2 ** 31 - 1, 2 ** 31, 2 ** 31 + 1, 2 ** 31 + 77,
+                                n1 - 65, n1 - 2, n1 - 1}))
+    sel = rows.to(device)
+    y, mean, invvar = k.layer_norm_forward_affine(x, (n2,), gamma, beta, 1e-5)
+    oy, omean, oinv = cf.layer_norm_fwd(f64(x[sel]), f64(gamma), f64(beta), 1e-5, "bf16")
+    check(y[sel], oy, "huge-n1 ln fwd", atol=2e-5, max_ulp=2, min_exact=0.97)
+    assert np.allclose(f64(mean[sel]), omean, rtol=1e-5, atol=1e-6)
+    assert np.allclose(f64(invvar[sel]), oinv, rtol=1e-5)
+    # x doubles as the incoming gradient
+    dx, dg, db = k.layer_norm_backward_affine(x, mean, invvar, x, (n2,), gamma, beta, 1e-5)
+    odx, _, _ = cf.layer_norm_bwd(f64(x[sel]), f64(x[sel]), f64(mean[sel]), f64(invvar[sel]), f64(gamma))
+    amp = float(np.abs(f64(invvar[sel])).max()) * 8.0
+    check(dx[sel], odx, "huge-n1 ln dx", atol=2e-5 + 2.5e-7 * amp)
+    # dbeta = column sums of dy over all 2.15e9 rows (float64 on the GPU, in slabs)
+    want_db = torch.zeros(n2, dtype=torch.float64, device=device)
+    for r0 in range(0, n1, 2 ** 27):
+        want_db += x[r0:r0 + 2 ** 27].double().sum(0)
+    assert torch.allclose(db.double(), want_db, rtol=2e-2, atol=50.0), (db, want_db)
+    del y, dx
+    y, invvar = k.rms_norm_forward_affine(x, (n2,), gamma, 1e-5)
+    oy, _ = cf.rms_norm_fwd(f64(x[sel]), f64(gamma), 1e-5, "bf16")
+    check(y[sel], oy, "huge-n1 rms fwd", atol=2e-5, max_ulp=2, min_exact=0.97)
+
+
+def test_elementwise_with_more_than_2_31_rows(device):
+    """bias-GeLU and bias-dropout-add over 2.15e9 rows of 8 columns, forward and backward."""
+    n2 = 8
+    n1 = 2 ** 31 + 4104
+    x = gpu_randn((n1, n2), BF16, 31, device)
+    bias = gpu_randn((n2,), BF16, 32, device, std=0.1)
+    ek = _C.get_fused_elementwise_kernel()
+    rows = torch.tensor(sorted({0, 1, 255, 256, 2 ** 31 - 257, 2 ** 31 - 1, 2 ** 31, 2 ** 31 + 1, 2 ** 31 + 300,
+                                n1 - 257, n1 - 2, n1 - 1}))
+    sel = rows.to(device)
+    act = ek.bias_gelu_forward(x, bias)
+    check(act[sel], cf.bias_gelu_fwd(f64(x[sel]), f64(bias)), "huge-n1 gelu fwd", atol=1e-6)
+    dact, dbias = ek.bias_gelu_backward(act, x, bias)
+    check(dact[sel], cf.bias_gelu_bwd(f64(act[sel]), f64(x[sel]), f64(bias))[0], "huge-n1 gelu bwd", atol=1e-6)
+    want = torch.zeros(n2, dtype=torch.float64, device=device)
+    for r0 in range(0, n1, 2 ** 27):
+        want += dact[r0:r0 + 2 ** 27].double().sum(0)
+    assert torch.allclose(dbias.double(), want, rtol=2e-2, atol=50.0), (dbias, want)
+    del dact
+    p, seed, offset = 0.1, 11, 4
+    out = ek.bias_dropout_add_forward(x, bias, act, p, seed, offset)
+    keep = np.stack([philox.keep_mask(n2, p, seed, offset, first_element=int(r) * n2) for r in rows]).astype(bool)
+    check(out[sel], cf.bias_dropout_add_fwd(f64(x[sel]), f64(bias), f64(act[sel]), keep, p), "huge-n1 bda fwd",
+          atol=1e-6, min_exact=0.97)
+    del out, act
+    dx, db = ek.bias_dropout_add_backward(x, p, seed, offset)
+    want_dx = np.where(keep, f64(x[sel]) / (1.0 - p), 0.0)
+    check(dx[sel], want_dx, "huge-n1 bda bwd", atol=1e-6, min_exact=0.97)
+
+
 def test_adam_on_a_tensor_beyond_2_31_elements(device):
     n = 2 ** 31 + 4099
     g = torch.empty(n, device=device, dtype=BF16).normal_()
