@@ -41,18 +41,20 @@ __device__ __forceinline__ float gelu_fwd(float u) {
 // d gelu / du = 0.5 u (1 - t^2)(0.79788456 + 0.1070322243 u^2) + 0.5 (1 + t)
 // with t = tanh z; in terms of s = sigmoid(2 z), e = exp(-2 z):
 // 1 + t = 2 s and 1 - t^2 = 4 e s^2.
-// Evaluated as s + w s (1 - s) with w = u (2 * 0.79788456 + 2 * 0.1070322243 u^2)
-// and e s^2 = s (1 - s) formed by one fused multiply-add: nine instructions and
-// two transcendentals.  (Where s rounds to 1 the product term, of relative size
-// below 1e-6, is dropped; elsewhere the form is good to a few 1e-6.)
+// Evaluated as s + (u s (1 - s)) q with q = 2 * 0.79788456 + 2 * 0.1070322243 u^2
+// and e s^2 = s (1 - s) formed by one fused multiply-add: eight instructions
+// and two transcendentals.  e itself is never multiplied, so it may overflow:
+// for u << 0 it becomes inf, s and the product term exact zeros, as tanh = -1
+// makes them in the reference's form; the result is finite as long as u^2 is.
+// (Where s rounds to 1 the product term, of relative size below 1e-6, is
+// dropped; elsewhere the form is good to a few 1e-6.)
 __device__ __forceinline__ float gelu_bwd(float u) {
   const float u2 = u * u;
-  const float arg = fminf(u * __builtin_fmaf(kGeluK2, u2, kGeluK1), 80.0f);
-  const float e = __builtin_amdgcn_exp2f(arg);
+  const float e = __builtin_amdgcn_exp2f(u * __builtin_fmaf(kGeluK2, u2, kGeluK1));
   const float s = __builtin_amdgcn_rcpf(1.0f + e);
   const float t = __builtin_fmaf(-s, s, s);
-  const float w = u * __builtin_fmaf(2.0f * 0.1070322243f, u2, 2.0f * 0.79788456f);
-  return __builtin_fmaf(w, t, s);
+  const float q = __builtin_fmaf(2.0f * 0.1070322243f, u2, 2.0f * 0.79788456f);
+  return __builtin_fmaf(u * t, q, s);
 }
 
 struct EltGeom {

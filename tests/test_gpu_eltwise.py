@@ -206,3 +206,34 @@ def test_dbias_is_the_sum_of_dx_as_stored(device, dtype):
         g_res, g_in, _, _, g_bias = ln.bias_dropout_add_norm_backward(
             False, dy.to(device), None, h.to(device), mean, invvar, (n2,), gamma.to(device), p, 5, 0)
         assert torch.equal(g_in[0], g_bias)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_bias_gelu_far_from_the_origin(device, dtype):
+    """Saturated inputs: gelu(u) = u and gelu'(u) = 1 for u >> 0, both 0 for
+    u << 0, exactly, for every magnitude whose square is finite in fp32 (the
+    range of the reference's own formula, functional.py:43-50); around the
+    point where exp(-2 z) leaves the fp32 range the values follow the oracle."""
+    mags = [7.5, 8.0, 8.5, 9.0, 9.5, 10.0, 12.0, 13.0, 30.0, 1e3, 1e6, 1e9, 1e12, 1e15, 1e18]
+    vals = torch.tensor([m for m in mags] + [-m for m in mags], dtype=torch.float32)
+    n2 = 64
+    x = vals.repeat_interleave(n2).view(-1, n2).to(dtype)
+    g = randn(tuple(x.shape), dtype, seed=9)
+    bias = torch.zeros(n2, dtype=dtype)
+    k = _C.get_fused_elementwise_kernel()
+    y = k.bias_gelu_forward(x.to(device), bias.to(device)).cpu()
+    dx, _ = k.bias_gelu_backward(g.to(device), x.to(device), bias.to(device))
+    dx = dx.cpu()
+    assert torch.isfinite(y).all() and torch.isfinite(dx).all()
+    xf = x.float()
+    far = xf.abs() >= 12.0
+    assert torch.equal(y[far & (xf > 0)], x[far & (xf > 0)])
+    assert (y[far & (xf < 0)] == 0).all()
+    assert torch.equal(dx[far & (xf > 0)], g[far & (xf > 0)])
+    assert (dx[far & (xf < 0)] == 0).all()
+    near = ~far
+    oy = cf.bias_gelu_fwd(f64(x), f64(bias))
+    odx = cf.bias_gelu_bwd(f64(g), f64(x), f64(bias))[0]
+    m = near.numpy()
+    assert np.allclose(f64(y)[m], oy[m], rtol=1e-2 if dtype == torch.bfloat16 else 2e-5, atol=1e-12)
+    assert np.allclose(f64(dx)[m], odx[m], rtol=1e-2 if dtype == torch.bfloat16 else 2e-5, atol=1e-12)
