@@ -11,7 +11,10 @@ the non-GEMM chain of one GPT-NeoX-20B-shaped layer, bf16, batch 4, sequence
     bias_gelu_fwd, _bwd             [8192, 24576]
     bias_dropout_add_fwd, _bwd      [8192, 6144], p = 0.1
 every buffer resident in HBM and pre-allocated; each stage has its own
-synthetic input (the GEMMs between the stages are not part of the path).
+synthetic input (the GEMMs between the stages are not part of the path).  The
+four 2 GB tensors of the softmax stage are carved from one allocation at
+staggered offsets (see `staggered`): that kernel is sensitive to operands that
+alias in the memory channels, and a plain allocation leaves it to luck.
 `value` = algorithmic bytes of a step (10 537.7 MB) / wall time per step.
 
 Prints ONE JSON line.  Beside the contract's keys it carries
@@ -220,6 +223,23 @@ CHAIN = {
 }
 
 
+def staggered(torch, dev, shape, dtype, count, step=(1 << 20) + 4096):
+    """`count` tensors of `shape` carved from one allocation: tensor k starts
+    k * step bytes into its own 2 MiB-aligned slot.  The causal softmax backward
+    streams three 2 GB tensors at identical offsets; when all of them start on
+    the same 2 MiB phase their requests meet in the same memory channels and the
+    kernel runs 1.5-4 % slower (measured: 687-699 us staggered against 701-736 us
+    aligned, depending on the box), which of the two a plain allocation gives is
+    luck.  The other kernels show no such sensitivity."""
+    n = 1
+    for d in shape:
+        n *= d
+    nbytes = n * torch.empty(0, dtype=dtype).element_size()
+    slot = (nbytes + count * step + (2 << 20) - 1) // (2 << 20) * (2 << 20)
+    base = torch.empty(slot * count, dtype=torch.uint8, device=dev)
+    return [base[k * slot + k * step:k * slot + k * step + nbytes].view(dtype).view(*shape) for k in range(count)]
+
+
 def chain_bytes():
     """Algorithmic bytes of each launch of the step (bf16: 2 bytes per element)."""
     c = CHAIN
@@ -254,8 +274,9 @@ def make_chain(L, dev):
           "invvar": torch.empty(n1, device=dev), "gamma": rnd(h, std=0.02, mean=1.0), "beta": rnd(h, std=0.02)}
     ln["dgamma"], ln["dbeta"] = torch.empty_like(ln["gamma"]), torch.empty_like(ln["beta"])
     ws_ln, ws_ln_b = L.ws(L._C.OSLO_OP_LN_BWD, n1, h, dev)
-    sm = {"x": rnd(ab, s, s), "dy": rnd(ab, s, s)}
-    sm["y"], sm["dx"] = torch.empty_like(sm["x"]), torch.empty_like(sm["x"])
+    sm = dict(zip(("x", "y", "dy", "dx"), staggered(torch, dev, (ab, s, s), bf, 4)))
+    sm["x"].normal_(generator=g)
+    sm["dy"].normal_(generator=g)
     ge = {"x": rnd(n1, ff), "g": rnd(n1, ff), "bias": rnd(ff, std=0.02)}
     ge["y"], ge["dx"], ge["dbias"] = torch.empty_like(ge["x"]), torch.empty_like(ge["x"]), torch.empty_like(ge["bias"])
     ws_ge, ws_ge_b = L.ws(L._C.OSLO_OP_BIAS_GELU_BWD, n1, ff, dev)
@@ -361,9 +382,10 @@ def kernel_table(L, dev, iters, graph_column=True):
         g = torch.Generator(device=dev).manual_seed(2)
         bufs = []
         for _ in range(ns):
-            x = torch.randn(ab, s, s, generator=g, device=dev).to(tdt)
-            dy = torch.randn(ab, s, s, generator=g, device=dev).to(tdt)
-            bufs.append((x, torch.empty_like(x), dy, torch.empty_like(x)))
+            x, y, dy, dx = staggered(torch, dev, (ab, s, s), tdt, 4)
+            x.normal_(generator=g)
+            dy.normal_(generator=g)
+            bufs.append((x, y, dy, dx))
 
         def fwd(i):
             x, y, dy, dx = bufs[i]
@@ -435,9 +457,9 @@ def kernel_table(L, dev, iters, graph_column=True):
     qi = torch.arange(1, s + 1, dtype=torch.float64)
     r = float(torch.minimum(qi[None, :], valid[:, None].double()).mean()) / s
     mask = (torch.arange(s)[None, :] >= valid[:, None]).view(b, 1, 1, s).to(dev).view(torch.uint8)
-    x = torch.randn(b, h, s, s, generator=g, device=dev).to(torch.bfloat16)
-    dy = torch.randn(b, h, s, s, generator=g, device=dev).to(torch.bfloat16)
-    y, dx = torch.empty_like(x), torch.empty_like(x)
+    x, y, dy, dx = staggered(torch, dev, (b, h, s, s), torch.bfloat16, 4)
+    x.normal_(generator=g)
+    dy.normal_(generator=g)
     sc = 1.0 / math.sqrt(96.0)
 
     def cmfwd(i):
