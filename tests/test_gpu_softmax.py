@@ -153,6 +153,12 @@ def test_masked(device, b, np_, sq, sk, dtype, scale, kind):
     check(dx_m, odx, "masked bwd (mask given)", atol=1e-7)
     check(dx_d, odx, "masked bwd (dense)", atol=1e-7)
     assert torch.equal(dx_m, dx_d)
+    # dx may alias dy: the gradient is overwritten in place, with and without the mask
+    g1, g2 = dy.to(device).clone(), dy.to(device).clone()
+    r1 = k.fused_scaled_masked_softmax_backward(g1, y, scale, mask=mask.to(device), inplace=True)
+    r2 = k.fused_scaled_masked_softmax_backward(g2, y, scale, inplace=True)
+    assert r1.data_ptr() == g1.data_ptr() and r2.data_ptr() == g2.data_ptr()
+    assert torch.equal(r1, dx_m) and torch.equal(r2, dx_m)
 
 
 def test_padding_fp16_matches_reference_chain(device):

@@ -93,6 +93,9 @@ def test_causal_masked(device, b, np_, sq, sk, dtype, scale, kind):
     check(dx_m, odx, "causal+padding bwd (mask given)", atol=1e-7)
     check(dx_d, odx, "causal+padding bwd (no mask)", atol=1e-7)
     assert torch.equal(dx_m, dx_d)
+    gi = dy.to(device).clone()
+    ri = k.fused_scaled_masked_softmax_backward(gi, y, scale, mask=mask.to(device), inplace=True, causal=True)
+    assert ri.data_ptr() == gi.data_ptr() and torch.equal(ri, dx_m)  # dx may alias dy
 
 
 def test_matches_the_reference_chain_where_every_row_sees_a_key(device):
