@@ -445,6 +445,10 @@ class _LayerNormKernel:
                 raise RuntimeError(
                     "%s has dtype %s, expected %s" % (name, t.dtype, _stat_dtype(input))
                 )
+            if t is not None and t.numel() != n1:
+                raise RuntimeError(
+                    "%s has %d elements for %d rows of input" % (name, t.numel(), n1)
+                )
         grad_input = torch.empty_like(input)
         grad_gamma = grad_beta = None
         ws, ws_bytes = None, 0
@@ -551,6 +555,11 @@ class _LayerNormKernel:
         n1, n2 = _compute_n1_n2(h, normalized_shape)
         if dout.shape != h.shape or dout.dtype != h.dtype:
             raise RuntimeError("dout and h differ in shape or dtype")
+        if not rms:
+            _check_input(mean, "mean")
+        for name, t in (("invvar", invvar), ("mean", None if rms else mean)):
+            if t is not None and (t.dtype != torch.float32 or t.numel() != n1):
+                raise RuntimeError("%s must be float32 with one element per row of h" % name)
         if dh_extra is not None:
             _check_input(dh_extra, "dh_extra")
             if dh_extra.shape != h.shape or dh_extra.dtype != h.dtype:
@@ -561,6 +570,11 @@ class _LayerNormKernel:
         grad_gamma = grad_beta = grad_bias = None
         if gamma is not None:
             _check_input(gamma, "gamma")
+            _check_param(gamma, normalized_shape, "gamma")
+            if gamma.dtype != h.dtype:
+                raise RuntimeError(
+                    "gamma has dtype %s but h has dtype %s" % (gamma.dtype, h.dtype)
+                )
             grad_gamma = torch.empty_like(gamma)
             if not rms:
                 grad_beta = torch.empty_like(gamma)
@@ -600,7 +614,13 @@ class _SoftmaxKernel:
         self._lib = lib
 
     @staticmethod
-    def _mask_u8(mask):
+    def _mask_u8(mask, like):
+        """The mask as contiguous bytes (non-zero = masked out); it has to live
+        on the device of ``like``, since the kernel reads it through a raw pointer."""
+        if mask.device != like.device:
+            raise RuntimeError(
+                "mask is on %s but the softmax operand is on %s" % (mask.device, like.device)
+            )
         if mask.dtype == torch.bool:
             return mask.contiguous().view(torch.uint8)
         if mask.dtype == torch.uint8:
@@ -611,19 +631,9 @@ class _SoftmaxKernel:
         """``causal=True`` (not in the reference's shim) hides the keys beyond
         the diagonal as well: causal attention on a padded batch."""
         lib = self._lib
-        if input.dim() != 4:
-            raise RuntimeError("expected 4D tensor")
-        if mask.dim() != 4:
-            raise RuntimeError("expected 4D tensor")
+        b, np_, sq, sk, mb, msq = self._masked_dims(input, mask)
         _check_input(input, "input")
-        b, np_, sq, sk = input.shape
-        mb, mh, msq, msk = mask.shape
-        if mh != 1 or msk != sk or mb not in (1, b) or msq not in (1, sq):
-            raise RuntimeError(
-                "mask of size %s does not broadcast to [%d, 1, %d, %d]"
-                % (list(mask.shape), b, sq, sk)
-            )
-        m8 = self._mask_u8(mask)
+        m8 = self._mask_u8(mask, input)
         out = torch.empty_like(input)
         with _device_of(input):
             fn = lib.oslo_softmax_causal_masked_fwd if causal else lib.oslo_softmax_masked_fwd
@@ -645,12 +655,14 @@ class _SoftmaxKernel:
         _check_input(softmax_results, "softmax_results")
         if output_grads.dtype != softmax_results.dtype:
             raise RuntimeError("output_grads and softmax_results differ in dtype")
+        if output_grads.shape != softmax_results.shape:
+            raise RuntimeError("output_grads and softmax_results differ in shape")
         b, np_, sq, sk = softmax_results.shape
         mb = msq = 1
         m8 = None
         if mask is not None:
-            mb, _, msq, _ = mask.shape
-            m8 = self._mask_u8(mask)
+            _, _, _, _, mb, msq = self._masked_dims(softmax_results, mask)
+            m8 = self._mask_u8(mask, softmax_results)
         # inplace=True overwrites output_grads, as the kernel this shim was
         # written for does
         grad_input = output_grads if inplace else torch.empty_like(output_grads)
@@ -698,6 +710,8 @@ class _SoftmaxKernel:
         _check_input(softmax_results, "softmax_results")
         if output_grads.dtype != softmax_results.dtype:
             raise RuntimeError("output_grads and softmax_results differ in dtype")
+        if output_grads.shape != softmax_results.shape:
+            raise RuntimeError("output_grads and softmax_results differ in shape")
         ab, sq, sk = softmax_results.shape
         grad_input = output_grads if inplace else torch.empty_like(output_grads)
         with _device_of(output_grads):
@@ -750,7 +764,7 @@ class _SoftmaxKernel:
                 )
             else:
                 b, np_, sq, sk, mb, msq = self._masked_dims(input, mask)
-                m8 = self._mask_u8(mask)
+                m8 = self._mask_u8(mask, input)
                 fn = (lib.oslo_softmax_causal_masked_dropout_fwd if causal
                       else lib.oslo_softmax_masked_dropout_fwd)
                 rc = fn(
@@ -787,7 +801,7 @@ class _SoftmaxKernel:
                 )
             else:
                 b, np_, sq, sk, mb, msq = self._masked_dims(input, mask)
-                m8 = self._mask_u8(mask)
+                m8 = self._mask_u8(mask, input)
                 fn = (lib.oslo_softmax_causal_masked_dropout_bwd if causal
                       else lib.oslo_softmax_masked_dropout_bwd)
                 rc = fn(
@@ -843,6 +857,10 @@ class _FusedElementwiseKernel:
         _check_input(input, "input")
         if grad_output.dtype != input.dtype or grad_output.shape != input.shape:
             raise RuntimeError("grad_output does not match input")
+        if bias is not None:
+            _check_input(bias, "bias")
+            if bias.dtype != input.dtype:
+                raise RuntimeError("bias and input differ in dtype")
         rows, cols = _rows_cols(input, bias)
         grad_input = torch.empty_like(input)
         grad_bias = None

@@ -597,6 +597,13 @@ class _NullContext:
         return False
 
 
+def _check_dropout_p(p):
+    if p < 0.0 or p > 1.0:
+        raise ValueError(
+            "dropout probability has to be between 0 and 1, but got {}".format(p)
+        )
+
+
 def fused_gelu(x):
     if not x.is_cuda:
         return _FusedGeLUFunction.apply(x)
@@ -632,10 +639,7 @@ def fused_bias_dropout_add(x, bias, residual, p, training, inplace=False):
     residual here folds that add into the same pass.  ``bias`` and ``residual``
     may be None.
     """
-    if p < 0.0 or p > 1.0:
-        raise ValueError(
-            "dropout probability has to be between 0 and 1, but got {}".format(p)
-        )
+    _check_dropout_p(p)
     if not x.is_cuda:
         y = x if bias is None else x + bias
         y = F.dropout(y, p=p, training=training, inplace=inplace and bias is None)
@@ -715,13 +719,6 @@ def scaled_masked_softmax(input, mask, scale=1.0, causal=False):
     """softmax(scale * input) with `mask` (True = masked out); input is [b, np, sq, sk].
     With ``causal=True`` key j of query i is hidden when j > i + (sk - sq) as well."""
     return _ScaledMaskedSoftmax.apply(input, mask, scale, causal)
-
-
-def _check_dropout_p(p):
-    if p < 0.0 or p > 1.0:
-        raise ValueError(
-            "dropout probability has to be between 0 and 1, but got {}".format(p)
-        )
 
 
 def scaled_upper_triang_masked_softmax_dropout(input, scale=1.0, p=0.0, training=True):

@@ -102,6 +102,12 @@ class FusedScaleMaskSoftmax(nn.Module):
             if input.dtype not in (torch.float16, torch.bfloat16, torch.float32):
                 return False
         if mask is not None:
+            # the kernels take "masked out or not" per key; an additive float
+            # mask (which may carry finite biases) is left to mask_func
+            if mask.is_floating_point():
+                return False
+            if input is not None and mask.device != input.device:
+                return False
             if mask.dim() != 4 or mask.size(1) != 1 or mask.size(3) != sk:
                 return False
             if mask.size(0) not in (1, b) or mask.size(2) not in (1, sq):

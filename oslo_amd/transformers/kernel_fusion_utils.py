@@ -377,6 +377,23 @@ def _unfused_probs(scores, scaling, attention_mask, causal, p, training, out_dty
     return torch.nn.functional.dropout(probs, p=p, training=training)
 
 
+def _kernel_takes_mask(attention_mask, scores):
+    """None, or a boolean ``[b or 1, 1, sq or 1, sk]`` tensor on the scores' device;
+    anything else (an additive float mask, one mask per head) is for the unfused chain."""
+    if attention_mask is None:
+        return True
+    b, _, sq, sk = scores.shape
+    return (
+        attention_mask.dtype == torch.bool
+        and attention_mask.device == scores.device
+        and attention_mask.dim() == 4
+        and attention_mask.size(1) == 1
+        and attention_mask.size(3) == sk
+        and attention_mask.size(0) in (1, b)
+        and attention_mask.size(2) in (1, sq)
+    )
+
+
 def fused_attention_forward(module, query, key, value, attention_mask, scaling=None,
                             dropout=0.0, **kwargs):
     """Attention with the scale -> mask -> softmax -> dropout chain in one kernel.
@@ -392,7 +409,8 @@ def fused_attention_forward(module, query, key, value, attention_mask, scaling=N
     an additive term (a relative-position bias as in
     oslo/transformers/models/t5/modeling_t5.py:508-514, ALiBi, or -10000
     fills): the fused kernels know no additive term, so such a call takes the
-    reference's unfused chain, on the GPU as on the CPU.
+    reference's unfused chain, on the GPU as on the CPU, and so does a boolean
+    mask of another shape (one mask per head).
     """
     if scaling is None:
         scaling = query.size(-1) ** -0.5
@@ -411,7 +429,7 @@ def fused_attention_forward(module, query, key, value, attention_mask, scaling=N
         if attention_mask.dim() == 4 and attention_mask.size(-1) > sk:
             attention_mask = attention_mask[..., :sk]
     key_visible = getattr(attention_mask, "_oslo_key_visible", None)
-    if not scores.is_cuda or (attention_mask is not None and attention_mask.dtype != torch.bool):
+    if not scores.is_cuda or not _kernel_takes_mask(attention_mask, scores):
         probs = _unfused_probs(scores, scaling, attention_mask, causal, p, module.training, value.dtype)
     elif attention_mask is None and causal:
         probs = onn_f.scaled_upper_triang_masked_softmax_dropout(

@@ -52,3 +52,38 @@ def test_copy_probe(device):
     out = torch.zeros_like(small)
     _C.get_fused_elementwise_kernel().copy_probe(small, out)
     assert torch.equal(small, out)
+
+
+def test_binding_refuses_operands_that_do_not_fit(device):
+    """The kernels read through raw pointers, so the binding has to turn away
+    what would make them read outside a buffer: a mask in host memory, gradients
+    of another shape, statistics of the wrong length."""
+    from oslo_amd.torch._C import get_fused_elementwise_kernel, get_layernorm_kernel, get_softmax_kernel
+
+    sm, ln, el = get_softmax_kernel(), get_layernorm_kernel(), get_fused_elementwise_kernel()
+    x = torch.randn(2, 3, 8, 16, device=device)
+    y = torch.softmax(x, -1)
+    mask = torch.zeros(2, 1, 1, 16, dtype=torch.bool)
+    with pytest.raises(RuntimeError, match="mask is on"):
+        sm.fused_scaled_masked_softmax_forward(x, mask, 1.0)
+    with pytest.raises(RuntimeError, match="mask is on"):
+        sm.fused_scaled_masked_softmax_backward(y, y, 1.0, mask=mask)
+    with pytest.raises(RuntimeError, match="does not broadcast"):
+        sm.fused_scaled_masked_softmax_backward(y, y, 1.0, mask=torch.zeros(2, 1, 1, 8, dtype=torch.bool, device=device))
+    with pytest.raises(RuntimeError, match="differ in shape"):
+        sm.fused_scaled_masked_softmax_backward(y[:, :, :4].contiguous(), y, 1.0)
+    y3 = y.view(6, 8, 16)
+    with pytest.raises(RuntimeError, match="differ in shape"):
+        sm.fused_scaled_upper_triang_masked_softmax_backward(y3[:3].contiguous(), y3, 1.0)
+
+    h = torch.randn(12, 64, device=device)
+    out, mean, invvar = ln.layer_norm_forward(h, (64,), 1e-5)
+    with pytest.raises(RuntimeError, match="elements for 12 rows"):
+        ln.layer_norm_backward(out, mean[:6].contiguous(), invvar, h, (64,), 1e-5)
+    with pytest.raises(RuntimeError, match="one element per row"):
+        ln.bias_dropout_add_norm_backward(False, out, None, h, mean, invvar[:6].contiguous(), (64,), None, 0.0, 0, 0)
+    with pytest.raises(RuntimeError, match="gamma has dtype"):
+        ln.bias_dropout_add_norm_backward(False, out, None, h, mean, invvar, (64,),
+                                          torch.ones(64, device=device, dtype=torch.float16), 0.0, 0, 0)
+    with pytest.raises(RuntimeError, match="differ in dtype"):
+        el.bias_gelu_backward(out, h, torch.zeros(64, device=device, dtype=torch.float16))

@@ -711,6 +711,22 @@ def test_additive_float_mask_is_applied_not_dropped(device, dtype):
     assert (out.float() - dropped).abs().max().item() > 10 * tol
 
 
+@pytest.mark.gpu
+def test_boolean_mask_per_head_takes_the_unfused_chain(device):
+    """The kernels broadcast one mask over the heads; a boolean mask that differs
+    from head to head is applied by the unfused chain instead of being refused."""
+    from oslo_amd.transformers.kernel_fusion_utils import fused_attention_forward
+
+    g = torch.Generator().manual_seed(3)
+    q, k, v = (torch.randn(2, 4, 24, 16, generator=g).to(device) for _ in range(3))
+    attend = torch.rand(2, 4, 24, 24, generator=g) > 0.3
+    attend[..., 0] = True  # every query sees a key
+    out, _ = fused_attention_forward(_AttnStub(False).eval(), q, k, v, attend.to(device), scaling=0.25)
+    additive = torch.where(attend, 0.0, -10000.0).to(device)
+    ref = _eager_attention(q, k, v, 0.25, additive)
+    assert torch.allclose(out, ref, rtol=1e-5, atol=1e-6)
+
+
 def test_mask_builder_returns_the_full_mask_and_the_key_part():
     from transformers import masking_utils as mu
 
