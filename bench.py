@@ -589,9 +589,60 @@ def kernel_table(L, dev, iters, graph_column=True):
             L.ok(lib.oslo_multi_tensor_adam(tables[0], tables[1], tables[2], tables[3], sizes, n, 1e-3, 0.9, 0.999,
                                             1e-8, step_no[0], 1, 1, 0.01, code, L.stream()))
 
-        rows.append(table_row("multi_tensor_adam", str(tdt).split(".")[-1], 7 * nel * esz,
-                              time_launches(torch, adam, max(10, iters // 4), 1), note="%d tensors" % n))
-        del lists, tables
+        dname = str(tdt).split(".")[-1]
+        opt_iters = max(10, iters // 4)
+        rows.append(table_row("multi_tensor_adam", dname, 7 * nel * esz,
+                              time_launches(torch, adam, opt_iters, 1), note="%d tensors" % n))
+
+        # the other optimizer steps on the same tensors (values moved per element:
+        # SGD with momentum and Adagrad read 3 and write 2; NovoGrad reads the
+        # gradients once more for their norms; LAMB = parameter norms 1 + stage 1
+        # (reads 4, writes 3) + update norms 1 + stage 2 (reads 2, writes 1))
+        need = int(lib.oslo_multi_tensor_norm_partials(sizes, n, code))
+        partials = torch.empty(need, dtype=torch.float32, device=dev)
+        norms = torch.ones(n, dtype=torch.float32, device=dev)
+        norms2 = torch.ones(n, dtype=torch.float32, device=dev)
+        gnorm = torch.ones(1, dtype=torch.float32, device=dev)
+
+        def sgd(i):
+            L.ok(lib.oslo_multi_tensor_sgd(tables[0], tables[1], tables[2], None, sizes, n, 0.01, 0.9, 0.0, 1e-3,
+                                           0, 0, 0, 1.0, code, code, 0, None, L.stream()))
+
+        def adagrad(i):
+            L.ok(lib.oslo_multi_tensor_adagrad(tables[0], tables[1], tables[3], sizes, n, 1e-3, 1e-10, 0, 0.01,
+                                               code, L.stream()))
+
+        def l2norm(i):
+            L.ok(lib.oslo_multi_tensor_norm(tables[0], sizes, n, code, p(partials), need, p(gnorm), p(norms), 2, 0,
+                                            0.0, 0.0, None, L.stream()))
+
+        def novograd(i):
+            step_no[0] += 1
+            L.ok(lib.oslo_multi_tensor_norm(tables[0], sizes, n, code, p(partials), need, None, p(norms), 2, 1,
+                                            0.98, 0.02, None, L.stream()))
+            L.ok(lib.oslo_multi_tensor_novograd(tables[0], tables[1], tables[2], sizes, n, p(norms), 1e-3, 0.95, 0.98,
+                                                1e-8, step_no[0], 1, 0.01, 1, 1, code, L.stream()))
+
+        def lamb(i):
+            step_no[0] += 1
+            L.ok(lib.oslo_multi_tensor_norm(tables[1], sizes, n, code, p(partials), need, None, p(norms), 2, 0,
+                                            0.0, 0.0, None, L.stream()))
+            L.ok(lib.oslo_multi_tensor_lamb_stage1(tables[0], tables[1], tables[2], tables[3], sizes, n, 0.9, 0.999,
+                                                   1e-6, step_no[0], 1, 0.01, 1, 1, p(gnorm), 1.0, code, L.stream()))
+            L.ok(lib.oslo_multi_tensor_norm(tables[0], sizes, n, code, p(partials), need, None, p(norms2), 2, 0,
+                                            0.0, 0.0, None, L.stream()))
+            L.ok(lib.oslo_multi_tensor_lamb_stage2(tables[0], tables[1], sizes, n, p(norms), p(norms2), 1e-3, 0.01,
+                                                   0, code, L.stream()))
+
+        for name, fn, values in (("multi_tensor_sgd", sgd, 5), ("multi_tensor_adagrad", adagrad, 5),
+                                 ("multi_tensor_l2norm", l2norm, 1), ("multi_tensor_novograd", novograd, 6),
+                                 ("multi_tensor_lamb", lamb, 12)):
+            if fn is lamb:  # stage 1 overwrites the gradients: start every timing from fresh ones
+                for t in lists[0]:
+                    t.normal_()
+            rows.append(table_row(name, dname, values * nel * esz, time_launches(torch, fn, opt_iters, 1),
+                                  note="%d tensors" % n))
+        del lists, tables, partials
         torch.cuda.empty_cache()
 
     # ---- plain copies with the same load/store path, at the traffic of the

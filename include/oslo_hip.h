@@ -393,6 +393,101 @@ int oslo_multi_tensor_adam(const void *const *g, void *const *p, void *const *m,
                            float eps, int step, int mode, int bias_correction,
                            float weight_decay, int dtype, void *stream);
 
+/* ---- the other multi-tensor optimizer steps and their norms ------------- *
+ * Same conventions as oslo_multi_tensor_adam: the list arguments are HOST
+ * arrays of ntensors device pointers, sizes the element counts, the math is
+ * fp32, nothing is allocated or copied, the tensor table travels in kernel
+ * arguments (48 tensors per launch).  Tensors without elements are allowed.  */
+
+/* Replaces multi_tensor_sgd (oslo/torch/_C/csrc/multi_tensor_sgd.cu:124-208,
+ * functor :29-122), called by FusedSGD.step (oslo/torch/optim/fused_sgd.py:
+ * 268-282).  g, w, mom: gradient, weight, momentum buffer; w_copy (or null): a
+ * 16-bit copy of the updated float32 weight (dtype_copy f16 or bf16).
+ *   g *= scale;  [g += wd w]  (before the momentum unless wd_after_momentum)
+ *   momentum != 0:  mom = first_run ? g : momentum mom + (1 - dampening) g
+ *                   g = nesterov ? g + momentum mom : mom
+ *   w += -lr g
+ * Type combinations: gradients and weights of one type (f32, f16, bf16), or
+ * 16-bit gradients with f32 weights (the reference: the four cases of :139-201).
+ * mom has the weights' type and is written only when momentum != 0.  When
+ * noop_flag (device int, or null) is non-zero the launch changes nothing (:35).  */
+int oslo_multi_tensor_sgd(const void *const *g, void *const *w, void *const *mom,
+                          void *const *w_copy, const int64_t *sizes, int64_t ntensors,
+                          float weight_decay, float momentum, float dampening, float lr,
+                          int nesterov, int first_run, int wd_after_momentum, float scale,
+                          int dtype_grad, int dtype_weight, int dtype_copy,
+                          const int *noop_flag, void *stream);
+
+/* Replaces multi_tensor_adagrad (oslo/torch/_C/csrc/multi_tensor_adagrad.cu:
+ * 86-101, functor :24-84), called by FusedAdagrad.step
+ * (oslo/torch/optim/fused_adagrad.py:112-131).  g, p, h: gradient, parameter,
+ * sum of squares, one dtype.
+ *   mode 0 (L2):  g += decay p;  h += g g;  p -= lr g / (sqrt(h) + eps)
+ *   mode 1:       h += g g;  p -= lr (g / (sqrt(h) + eps) + decay p)        */
+int oslo_multi_tensor_adagrad(const void *const *g, void *const *p, void *const *h,
+                              const int64_t *sizes, int64_t ntensors, float lr, float eps,
+                              int mode, float weight_decay, int dtype, void *stream);
+
+/* The element-wise part of multi_tensor_novograd (oslo/torch/_C/csrc/
+ * multi_tensor_novograd.cu:111-148, functor :30-109), called by
+ * FusedNovograd.step (oslo/torch/optim/fused_novograd.py:228-262).
+ * grad_norms: device float[ntensors], the blended per-tensor gradient norms
+ * (the reference's host function updates them first through
+ * multi_tensor_norm_out: call oslo_multi_tensor_norm with blend = 1,
+ * alpha = beta2, beta = 1 - beta2 before this).  With
+ * denom = grad_norms[t] / bc2 + eps, bc1 = 1 - beta1^step,
+ * bc2 = sqrt(1 - beta2^step) (both 1 without bias_correction) and
+ * beta3 = grad_averaging ? 1 - beta1 : 1:
+ *   moment_mode 0:  g = g / denom + decay p;  m = beta1 m + beta3 g;  p -= lr m / bc1
+ *   moment_mode 1:  m = beta1 m + beta3 g;  p -= lr ((m / bc1) / denom + decay p)  */
+int oslo_multi_tensor_novograd(const void *const *g, void *const *p, void *const *m,
+                               const int64_t *sizes, int64_t ntensors, const float *grad_norms,
+                               float lr, float beta1, float beta2, float eps, int step,
+                               int bias_correction, float weight_decay, int grad_averaging,
+                               int moment_mode, int dtype, void *stream);
+
+/* The two element-wise stages of multi_tensor_lamb (oslo/torch/_C/csrc/
+ * multi_tensor_lamb.cu:285-352; stage 1 :41-204, stage 2 :208-283).  The
+ * reference's host function runs: per-tensor L2 norms of the parameters,
+ * stage 1, per-tensor L2 norms of the updates, stage 2; the norms are
+ * oslo_multi_tensor_norm calls.
+ * Stage 1 (g, p, m, v; the update direction overwrites g):
+ *   g /= clip, clip = *global_grad_norm > max_grad_norm ? ratio of the two : 1
+ *   mode 0: g += decay p
+ *   m = beta1 m + beta3 g;  v = beta2 v + (1 - beta2) g g
+ *   update = (m / bc1) / (sqrt(v / bc2) + eps)  [+ decay p in mode 1]
+ * Stage 2 (update, p):  p -= ratio update, ratio = lr * param_norm / update_norm
+ * for tensors under weight decay (all tensors with use_nvlamb) when both norms
+ * are non-zero, else lr.  global_grad_norm, param_norms, update_norms: device
+ * floats.                                                                   */
+int oslo_multi_tensor_lamb_stage1(void *const *g, const void *const *p, void *const *m,
+                                  void *const *v, const int64_t *sizes, int64_t ntensors,
+                                  float beta1, float beta2, float eps, int step,
+                                  int bias_correction, float weight_decay, int grad_averaging,
+                                  int mode, const float *global_grad_norm, float max_grad_norm,
+                                  int dtype, void *stream);
+int oslo_multi_tensor_lamb_stage2(const void *const *update, void *const *p,
+                                  const int64_t *sizes, int64_t ntensors,
+                                  const float *param_norms, const float *update_norms, float lr,
+                                  float weight_decay, int use_nvlamb, int dtype, void *stream);
+
+/* Replaces multi_tensor_l2norm (oslo/torch/_C/csrc/multi_tensor_l2norm.cu:
+ * 257-317; kernels :29-98, clean-up :174-198) and multi_tensor_norm_out
+ * (:323-385; max norm :102-172, clean-up :200-255).  norm_type 2: L2 norm,
+ * 0: largest magnitude.  out_global (device float, or null): the norm over all
+ * tensors.  out_per_tensor (device float[ntensors], or null): one norm per
+ * tensor, written (blend = 0) or blended into the stored value (blend = 1):
+ *   L2:  out = sqrt(alpha out^2 + beta sum of squares);  max:  out = alpha out + beta max.
+ * partials: workspace of partials_len floats, at least
+ * oslo_multi_tensor_norm_partials(sizes, ntensors, dtype); the sums are folded
+ * in a fixed order (no atomics).  A partial result that is not finite sets
+ * *noop_flag (device int, or null) to 1 (:87-89).                            */
+int64_t oslo_multi_tensor_norm_partials(const int64_t *sizes, int64_t ntensors, int dtype);
+int oslo_multi_tensor_norm(const void *const *x, const int64_t *sizes, int64_t ntensors,
+                           int dtype, float *partials, int64_t partials_len, float *out_global,
+                           float *out_per_tensor, int norm_type, int blend, float alpha,
+                           float beta, int *noop_flag, void *stream);
+
 /* ---- test and measurement hooks (no counterpart in the reference) ------ */
 
 /* Writes the keep mask (1 = kept) of n elements as uint8. */

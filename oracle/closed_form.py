@@ -9,8 +9,9 @@ File:line citations are into the reference repository (EleutherAI/oslo).
 Pinning: the reference holds no numeric vectors, known answers or fixtures for
 these ops (its tests compare two of its own paths on unseeded data), so none of
 the functions here is pinned by reference-held data.  Each one is pinned
-instead by tests/test_oracle_closed_form.py, test_oracle_philox.py and
-test_oracle_adam.py: torch library routines and torch autograd in float64,
+instead by tests/test_oracle_closed_form.py, test_oracle_philox.py,
+test_oracle_adam.py and test_oracle_optimizers.py: torch library routines
+(torch.optim among them) and torch autograd in float64,
 finite differences, invariants (row sums, shift invariance, exact zeros,
 orthogonality of the norm gradients), brute force on tiny inputs and the
 Random123 known-answer vectors.
@@ -39,7 +40,9 @@ def round_bf16(a):
 
 
 def round_f16(a):
-    return np.asarray(a, dtype=np.float64).astype(np.float16).astype(np.float32)
+    """Round-to-nearest-even to float16 by way of float32 (see round_to),
+    returned as float32 values."""
+    return np.asarray(a, dtype=np.float64).astype(np.float32).astype(np.float16).astype(np.float32)
 
 
 def round_to(a, out):
@@ -369,3 +372,155 @@ def adam_step(g, p, m, v, lr, beta1, beta2, eps, step, mode, bias_correction, we
         update = update + f(weight_decay) * p
     p = p - f(lr) * update
     return round_to(p, out), round_to(m, out), round_to(v, out)
+
+
+# ---------------------------------------------------------------------------
+# SGD, Adagrad, NovoGrad, LAMB steps and the tensor norms they use
+# ---------------------------------------------------------------------------
+def _f32(x, acc):
+    """A scalar argument as the kernel receives it: a float32 value."""
+    return acc(np.float32(x))
+
+
+def sgd_step(g, w, mom, lr, weight_decay, momentum, dampening, nesterov, first_run,
+             wd_after_momentum=False, scale=1.0, out="f64", copy=None, acc=np.float64):
+    """One SGD update of one tensor; returns the new ``(w, mom, w_copy)``.
+
+    oslo/torch/_C/csrc/multi_tensor_sgd.cu:87-117: the gradient is multiplied
+    by ``scale``; weight decay joins it before (default) or after the momentum
+    step; on the first run the momentum buffer becomes the gradient, afterwards
+    ``momentum * mom + (1 - dampening) * g``; Nesterov adds ``momentum * mom``
+    to the gradient, plain momentum replaces the gradient by the buffer; the
+    weight moves by ``-lr * g`` and is rounded to its storage type; ``w_copy``
+    is that stored weight converted to the 16-bit type ``copy`` (:112-113).
+    ``mom`` is returned unchanged when ``momentum == 0`` (never written, :116)."""
+    g = np.asarray(g, dtype=acc) * _f32(scale, acc)
+    w = np.asarray(w, dtype=acc)
+    mom = np.asarray(mom, dtype=acc)
+    wd, mu = _f32(weight_decay, acc), _f32(momentum, acc)
+    if weight_decay != 0 and not wd_after_momentum:
+        g = g + wd * w
+    new_mom = mom
+    if momentum != 0:
+        # 1 - dampening is formed in float32 (:97), which is not exact for 0.1
+        keep = acc(np.float32(1.0) - np.float32(dampening))
+        new_mom = g if first_run else mom * mu + keep * g
+        g = g + mu * new_mom if nesterov else new_mom
+    if weight_decay != 0 and wd_after_momentum:
+        g = g + wd * w
+    w_new = round_to(w + (-_f32(lr, acc) * g), out)
+    w_copy = None if copy is None else round_to(w_new, copy)
+    return w_new, (round_to(new_mom, out) if momentum != 0 else mom), w_copy
+
+
+def adagrad_step(g, p, h, lr, eps, mode, weight_decay, out="f64", acc=np.float64):
+    """One Adagrad update; returns the new ``(p, h)``.
+
+    oslo/torch/_C/csrc/multi_tensor_adagrad.cu:63-73: mode 0 adds ``decay * p``
+    to the gradient (L2), mode 1 adds ``decay * p`` to the step; ``h`` is the
+    running sum of squared gradients."""
+    g = np.asarray(g, dtype=acc)
+    p = np.asarray(p, dtype=acc)
+    h = np.asarray(h, dtype=acc)
+    lr_, eps_, wd = _f32(lr, acc), _f32(eps, acc), _f32(weight_decay, acc)
+    if mode == 0:
+        g = g + wd * p
+        h = h + g * g
+        p = p - lr_ * (g / (np.sqrt(h) + eps_))
+    else:
+        h = h + g * g
+        p = p - lr_ * (g / (np.sqrt(h) + eps_) + wd * p)
+    return round_to(p, out), round_to(h, out)
+
+
+def tensor_norm(x, norm_type=2, acc=np.float64):
+    """L2 norm (``norm_type`` 2) or largest magnitude (0) of one tensor
+    (oslo/torch/_C/csrc/multi_tensor_l2norm.cu:62-98, 135-172)."""
+    x = np.asarray(x, dtype=acc).reshape(-1)
+    if x.size == 0:
+        return acc(0.0)
+    return np.sqrt(np.sum(x * x)) if norm_type == 2 else np.max(np.abs(x))
+
+
+def blend_norm(old, x, alpha, beta, norm_type=2, acc=np.float64):
+    """The stored per-tensor norm after a step (multi_tensor_l2norm.cu:319-322,
+    226-253): L2 ``sqrt(alpha * old**2 + beta * |x|_2**2)``, max
+    ``alpha * old + beta * max|x|``."""
+    a, b = _f32(alpha, acc), _f32(beta, acc)
+    n = tensor_norm(x, norm_type, acc)
+    if norm_type == 2:
+        return np.sqrt(a * acc(old) * acc(old) + b * n * n)
+    return a * acc(old) + b * n
+
+
+def novograd_step(g, p, m, grad_norm, lr, beta1, beta2, eps, step, bias_correction,
+                  weight_decay, grad_averaging, moment_mode, out="f64", acc=np.float64):
+    """The element-wise part of one NovoGrad update; ``grad_norm`` is the
+    tensor's blended gradient norm (``blend_norm``).  Returns the new ``(p, m)``.
+
+    oslo/torch/_C/csrc/multi_tensor_novograd.cu:80-96 and host code :118-129:
+    ``bc1 = 1 - beta1**step``, ``bc2 = sqrt(1 - beta2**step)`` (float32),
+    ``beta3 = 1 - beta1`` with gradient averaging, else 1."""
+    g = np.asarray(g, dtype=acc)
+    p = np.asarray(p, dtype=acc)
+    m = np.asarray(m, dtype=acc)
+    b1 = _f32(beta1, acc)
+    bc1 = bc2 = acc(1.0)
+    if bias_correction:
+        bc1 = acc(np.float32(1.0 - float(np.float32(beta1)) ** step))
+        bc2 = acc(np.float32(np.sqrt(1.0 - float(np.float32(beta2)) ** step)))
+    b3 = acc(1.0) - b1 if grad_averaging else acc(1.0)
+    denom = acc(grad_norm) / bc2 + _f32(eps, acc)
+    wd, lr_ = _f32(weight_decay, acc), _f32(lr, acc)
+    if moment_mode == 0:
+        g = g / denom + wd * p
+        m = b1 * m + b3 * g
+        p = p - lr_ * (m / bc1)
+    else:
+        m = b1 * m + b3 * g
+        p = p - lr_ * ((m / bc1) / denom + wd * p)
+    return round_to(p, out), round_to(m, out)
+
+
+def lamb_stage1(g, p, m, v, beta1, beta2, eps, step, bias_correction, weight_decay,
+                grad_averaging, mode, global_grad_norm, max_grad_norm, out="f64",
+                acc=np.float64):
+    """LAMB stage 1 for one tensor: returns ``(update, m, v)``
+    (oslo/torch/_C/csrc/multi_tensor_lamb.cu:111-130; bias corrections and
+    beta3 from the host code :300-311)."""
+    g = np.asarray(g, dtype=acc)
+    p = np.asarray(p, dtype=acc)
+    m = np.asarray(m, dtype=acc)
+    v = np.asarray(v, dtype=acc)
+    b1, b2 = _f32(beta1, acc), _f32(beta2, acc)
+    bc1 = bc2 = acc(1.0)
+    if bias_correction:
+        bc1 = acc(np.float32(1.0 - float(np.float32(beta1)) ** step))
+        bc2 = acc(np.float32(1.0 - float(np.float32(beta2)) ** step))
+    b3 = acc(1.0) - b1 if grad_averaging else acc(1.0)
+    gn, mx = acc(global_grad_norm), _f32(max_grad_norm, acc)
+    clip = gn / mx if gn > mx else acc(1.0)
+    wd = _f32(weight_decay, acc)
+    g = g / clip
+    if mode == 0:
+        g = g + wd * p
+    m = m * b1 + b3 * g
+    v = v * b2 + (acc(1.0) - b2) * g * g
+    update = (m / bc1) / (np.sqrt(v / bc2) + _f32(eps, acc))
+    if mode != 0:
+        update = update + wd * p
+    return round_to(update, out), round_to(m, out), round_to(v, out)
+
+
+def lamb_stage2(update, p, param_norm, update_norm, lr, weight_decay, use_nvlamb, out="f64",
+                acc=np.float64):
+    """LAMB stage 2 for one tensor: ``p - ratio * update`` with the trust ratio
+    ``lr * param_norm / update_norm`` for tensors under weight decay (every
+    tensor with ``use_nvlamb``) when both norms are non-zero, else ``lr``
+    (multi_tensor_lamb.cu:224-233, 262-264)."""
+    ratio = _f32(lr, acc)
+    if use_nvlamb or weight_decay != 0:
+        if update_norm != 0 and param_norm != 0:
+            ratio = _f32(lr, acc) * (acc(param_norm) / acc(update_norm))
+    p = np.asarray(p, dtype=acc) - ratio * np.asarray(update, dtype=acc)
+    return round_to(p, out)

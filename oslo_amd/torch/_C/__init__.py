@@ -138,6 +138,28 @@ _SIGNATURES = {
         _int,
         [_p, _p, _p, _p, _p, _i64, _f32, _f32, _f32, _f32, _int, _int, _int, _f32, _int, _p],
     ),
+    "oslo_multi_tensor_sgd": (
+        _int,
+        [_p, _p, _p, _p, _p, _i64, _f32, _f32, _f32, _f32, _int, _int, _int, _f32, _int, _int,
+         _int, _p, _p],
+    ),
+    "oslo_multi_tensor_adagrad": (_int, [_p, _p, _p, _p, _i64, _f32, _f32, _int, _f32, _int, _p]),
+    "oslo_multi_tensor_novograd": (
+        _int,
+        [_p, _p, _p, _p, _i64, _p, _f32, _f32, _f32, _f32, _int, _int, _f32, _int, _int, _int, _p],
+    ),
+    "oslo_multi_tensor_lamb_stage1": (
+        _int,
+        [_p, _p, _p, _p, _p, _i64, _f32, _f32, _f32, _int, _int, _f32, _int, _int, _p, _f32,
+         _int, _p],
+    ),
+    "oslo_multi_tensor_lamb_stage2": (
+        _int, [_p, _p, _p, _i64, _p, _p, _f32, _f32, _int, _int, _p],
+    ),
+    "oslo_multi_tensor_norm_partials": (_i64, [_p, _i64, _int]),
+    "oslo_multi_tensor_norm": (
+        _int, [_p, _p, _i64, _int, _p, _i64, _p, _p, _int, _int, _f32, _f32, _p, _p],
+    ),
     "oslo_rng_from_device": (_int, [_p]),
     "oslo_philox_mask": (_int, [_p, _i64, _f32, _u64, _u64, _p]),
     "oslo_philox_words": (_int, [_p, _i64, _i64, _u64, _u64, _p]),
@@ -988,8 +1010,36 @@ def get_softmax_kernel():
 
 
 # ---------------------------------------------------------------------------
-# multi-tensor Adam
+# multi-tensor optimizer steps
 # ---------------------------------------------------------------------------
+def _tensor_tables(tensor_lists, names, dtypes=None):
+    """Checks lists of equally long, pairwise equally sized contiguous GPU
+    tensors (the checks of the reference's multi_tensor_apply.cuh:44-72) and
+    returns ``(pointer tables, sizes, n, first tensor)``; ``dtypes[k]`` None
+    means list k follows the dtype of its first tensor."""
+    n = len(tensor_lists[0])
+    for lst in tensor_lists:
+        if len(lst) != n:
+            raise RuntimeError("Size mismatch among tensor lists")
+    if n == 0:
+        return None, None, 0, None
+    ref = tensor_lists[0][0]
+    for k, lst in enumerate(tensor_lists):
+        want = lst[0].dtype if dtypes is None or dtypes[k] is None else dtypes[k]
+        for i, t in enumerate(lst):
+            _check_input(t, "%s %d" % (names[k], i))
+            if t.dtype != want or t.device != ref.device:
+                raise RuntimeError(
+                    "A tensor was not the same dtype / on the same device as the first tensor"
+                )
+            if t.numel() != tensor_lists[0][i].numel():
+                raise RuntimeError("Size mismatch among tensor lists")
+    arr = ctypes.c_void_p * n
+    sizes = (ctypes.c_int64 * n)(*[t.numel() for t in tensor_lists[0]])
+    tables = [arr(*[t.data_ptr() for t in lst]) for lst in tensor_lists]
+    return tables, sizes, n, ref
+
+
 class _AdamKernel:
     """``multi_tensor_adam`` of the reference's ``oslo_fused_adam`` module
     (``oslo/torch/_C/csrc/FusedAdamBinder.cpp:12-15``), same argument list."""
@@ -1008,27 +1058,12 @@ class _AdamKernel:
         lib = self._lib
         if len(tensor_lists) != 4:
             raise RuntimeError("tensor_lists must hold [grads, params, exp_avgs, exp_avg_sqs]")
-        gs, ps, ms, vs = tensor_lists
-        n = len(ps)
-        if not (len(gs) == len(ms) == len(vs) == n):
-            raise RuntimeError("Size mismatch among tensor lists")
+        names = ("grad", "param", "exp_avg", "exp_avg_sq")
+        ref_dtype = tensor_lists[1][0].dtype if len(tensor_lists[1]) else None
+        tables, sizes, n, ref = _tensor_tables(tensor_lists, names, [ref_dtype] * 4)
         if n == 0:
             return
-        ref = ps[0]
         code = _dtype_code(ref, "params[0]")
-        for i in range(n):
-            sz = ps[i].numel()
-            for name, t in (("grad", gs[i]), ("param", ps[i]), ("exp_avg", ms[i]), ("exp_avg_sq", vs[i])):
-                _check_input(t, "%s %d" % (name, i))
-                if t.dtype != ref.dtype or t.device != ref.device:
-                    raise RuntimeError(
-                        "A tensor was not the same dtype / on the same device as the first tensor"
-                    )
-                if t.numel() != sz:
-                    raise RuntimeError("Size mismatch among tensor lists")
-        arr = ctypes.c_void_p * n
-        sizes = (ctypes.c_int64 * n)(*[t.numel() for t in ps])
-        tables = [arr(*[t.data_ptr() for t in lst]) for lst in (gs, ps, ms, vs)]
         with _device_of(ref):
             rc = lib.oslo_multi_tensor_adam(
                 tables[0], tables[1], tables[2], tables[3], sizes, n, float(lr), float(beta1),
@@ -1038,14 +1073,247 @@ class _AdamKernel:
             _check(rc, lib)
 
 
-_adam_kernel = None
+def _flag_ptr(noop_flag, ref):
+    """Device pointer of the overflow flag (an int32 tensor), or None."""
+    if noop_flag is None:
+        return None
+    if not (noop_flag.is_cuda and noop_flag.dtype == torch.int32 and noop_flag.numel() >= 1):
+        raise RuntimeError("noop_flag must be an int32 tensor on the GPU")
+    if ref is not None and noop_flag.device != ref.device:
+        raise RuntimeError("expected noop flag to be on the same device as tensors")
+    return noop_flag.data_ptr()
+
+
+class _SGDKernel:
+    """``multi_tensor_sgd`` of ``oslo/torch/_C/csrc/FusedSGDBinder.cpp``."""
+
+    def __init__(self, lib):
+        self._lib = lib
+
+    def multi_tensor_sgd(
+        self, chunk_size, noop_flag, tensor_lists, wd, momentum, dampening, lr, nesterov,
+        first_run, wd_after_momentum, scale,
+    ):
+        """``tensor_lists`` = ``[grads, weights, momentum buffers]`` or, with a
+        fourth list, additionally 16-bit copies of the updated float32 weights
+        (``multi_tensor_sgd.cu:139-201``).  Nothing happens while ``noop_flag``
+        is non-zero."""
+        lib = self._lib
+        if len(tensor_lists) not in (3, 4):
+            raise RuntimeError("tensor_lists must hold [grads, weights, momentums(, weight copies)]")
+        names = ("grad", "weight", "momentum", "weight copy")
+        wdtype = tensor_lists[1][0].dtype if len(tensor_lists[1]) else None
+        dts = [None, wdtype, wdtype, None][: len(tensor_lists)]
+        tables, sizes, n, ref = _tensor_tables(tensor_lists, names, dts)
+        if n == 0:
+            return
+        copy = len(tensor_lists) == 4
+        if copy and tensor_lists[3][0].dtype not in (torch.float16, torch.bfloat16):
+            raise RuntimeError("Additional output tensors should always be fp16 (or bf16).")
+        with _device_of(ref):
+            rc = lib.oslo_multi_tensor_sgd(
+                tables[0], tables[1], tables[2], tables[3] if copy else None, sizes, n,
+                float(wd), float(momentum), float(dampening), float(lr), int(bool(nesterov)),
+                int(bool(first_run)), int(bool(wd_after_momentum)), float(scale),
+                _dtype_code(tensor_lists[0][0], "grads[0]"),
+                _dtype_code(tensor_lists[1][0], "weights[0]"),
+                _dtype_code(tensor_lists[3][0], "copies[0]") if copy else 0,
+                _flag_ptr(noop_flag, ref), _stream(ref),
+            )
+            _check(rc, lib)
+
+
+class _AdagradKernel:
+    """``multi_tensor_adagrad`` of ``oslo/torch/_C/csrc/FusedAdagradBinder.cpp``."""
+
+    def __init__(self, lib):
+        self._lib = lib
+
+    def multi_tensor_adagrad(self, chunk_size, noop_flag, tensor_lists, lr, epsilon, mode,
+                             weight_decay):
+        """``tensor_lists`` = ``[grads, params, sums of squares]``, one dtype."""
+        lib = self._lib
+        if len(tensor_lists) != 3:
+            raise RuntimeError("tensor_lists must hold [grads, params, sums]")
+        d = tensor_lists[0][0].dtype if len(tensor_lists[0]) else None
+        tables, sizes, n, ref = _tensor_tables(tensor_lists, ("grad", "param", "sum"), [d] * 3)
+        if n == 0:
+            return
+        with _device_of(ref):
+            rc = lib.oslo_multi_tensor_adagrad(
+                tables[0], tables[1], tables[2], sizes, n, float(lr), float(epsilon), int(mode),
+                float(weight_decay), _dtype_code(ref, "grads[0]"), _stream(ref),
+            )
+            _check(rc, lib)
+
+
+class _L2NormKernel:
+    """``multi_tensor_l2norm`` of ``oslo/torch/_C/csrc/FusedL2NormBinder.cpp``,
+    and ``norm_out``, the blend into stored per-tensor norms that the
+    reference's NovoGrad step calls internally
+    (``multi_tensor_l2norm.cu:323-385``)."""
+
+    def __init__(self, lib):
+        self._lib = lib
+
+    def _run(self, tensors, out_global, out_per_tensor, norm_type, blend, alpha, beta, noop_flag):
+        lib = self._lib
+        tables, sizes, n, ref = _tensor_tables([tensors], ("tensor",))
+        code = _dtype_code(ref, "tensors[0]")
+        need = int(lib.oslo_multi_tensor_norm_partials(sizes, n, code))
+        if need < 0:
+            _check(need, lib)
+        partials = torch.empty(need, dtype=torch.float32, device=ref.device)
+        with _device_of(ref):
+            rc = lib.oslo_multi_tensor_norm(
+                tables[0], sizes, n, code, _ptr(partials), need, _ptr(out_global),
+                _ptr(out_per_tensor), int(norm_type), int(blend), float(alpha), float(beta),
+                _flag_ptr(noop_flag, ref), _stream(ref),
+            )
+            _check(rc, lib)
+
+    def multi_tensor_l2norm(self, chunk_size, noop_flag, tensor_lists, per_tensor=False):
+        """Returns ``(norm over all tensors [1], norm of each tensor [n] or an
+        empty tensor)``, float32.  A sum that is not finite sets ``noop_flag``."""
+        if len(tensor_lists) != 1:
+            raise RuntimeError("tensor_lists must hold one list")
+        tensors = tensor_lists[0]
+        if len(tensors) == 0:
+            raise RuntimeError("multi_tensor_l2norm: no tensors")
+        dev = tensors[0].device
+        ret = torch.empty(1, dtype=torch.float32, device=dev)
+        ret_per_tensor = torch.empty(len(tensors) if per_tensor else 0, dtype=torch.float32,
+                                     device=dev)
+        self._run(tensors, ret, ret_per_tensor if per_tensor else None, 2, 0, 0.0, 0.0, noop_flag)
+        return ret, ret_per_tensor
+
+    def multi_tensor_norm_out(self, chunk_size, noop_flag, tensor_lists, out, alpha, beta,
+                              norm_type):
+        """``out[t] = sqrt(alpha * out[t]**2 + beta * |x_t|_2**2)`` (``norm_type``
+        2) or ``alpha * out[t] + beta * max|x_t|`` (``norm_type`` 0), in place."""
+        tensors = tensor_lists[0]
+        if len(tensors) == 0:
+            return
+        _check_input(out, "out")
+        if out.dtype != torch.float32 or out.numel() != len(tensors):
+            raise RuntimeError("out must be float32 with one element per tensor")
+        if norm_type not in (0, 2):
+            raise RuntimeError("only the L2 norm (2) and the max norm (0) are supported")
+        self._run(tensors, None, out, norm_type, 1, alpha, beta, noop_flag)
+
+
+class _NovogradKernel:
+    """``multi_tensor_novograd`` of ``oslo/torch/_C/csrc/FusedNovogradBinder.cpp``."""
+
+    def __init__(self, lib):
+        self._lib = lib
+
+    def multi_tensor_novograd(
+        self, chunk_size, noop_flag, tensor_lists, grad_norms, lr, beta1, beta2, epsilon, step,
+        bias_correction, weight_decay, grad_averaging, moment_mode, norm_type,
+    ):
+        """``tensor_lists`` = ``[grads, params, exp_avgs]``; ``grad_norms`` holds
+        one float32 per tensor and is blended with this step's gradient norms
+        first, as in the reference's host function
+        (``multi_tensor_novograd.cu:131-136``)."""
+        lib = self._lib
+        if len(tensor_lists) != 3:
+            raise RuntimeError("tensor_lists must hold [grads, params, exp_avgs]")
+        d = tensor_lists[0][0].dtype if len(tensor_lists[0]) else None
+        tables, sizes, n, ref = _tensor_tables(tensor_lists, ("grad", "param", "exp_avg"), [d] * 3)
+        if n == 0:
+            return
+        get_l2norm_kernel().multi_tensor_norm_out(
+            chunk_size, noop_flag, [tensor_lists[0]], grad_norms, beta2, 1.0 - beta2, norm_type
+        )
+        with _device_of(ref):
+            rc = lib.oslo_multi_tensor_novograd(
+                tables[0], tables[1], tables[2], sizes, n, _ptr(grad_norms), float(lr),
+                float(beta1), float(beta2), float(epsilon), int(step), int(bias_correction),
+                float(weight_decay), int(grad_averaging), int(moment_mode),
+                _dtype_code(ref, "grads[0]"), _stream(ref),
+            )
+            _check(rc, lib)
+
+
+class _LambKernel:
+    """``multi_tensor_lamb`` of ``oslo/torch/_C/csrc/FusedLambBinder.cpp``."""
+
+    def __init__(self, lib):
+        self._lib = lib
+
+    def multi_tensor_lamb(
+        self, chunk_size, noop_flag, tensor_lists, lr, beta1, beta2, epsilon, step,
+        bias_correction, weight_decay, grad_averaging, mode, global_grad_norm, max_grad_norm,
+        use_nvlamb=False,
+    ):
+        """``tensor_lists`` = ``[grads, params, exp_avgs, exp_avg_sqs]``, one
+        dtype; the gradients are overwritten with the update direction
+        (``multi_tensor_lamb.cu:313-317``).  ``global_grad_norm`` is a float32
+        tensor with the norm of all gradients."""
+        lib = self._lib
+        if len(tensor_lists) != 4:
+            raise RuntimeError("tensor_lists must hold [grads, params, exp_avgs, exp_avg_sqs]")
+        names = ("grad", "param", "exp_avg", "exp_avg_sq")
+        d = tensor_lists[0][0].dtype if len(tensor_lists[0]) else None
+        tables, sizes, n, ref = _tensor_tables(tensor_lists, names, [d] * 4)
+        if n == 0:
+            return
+        _check_input(global_grad_norm, "global_grad_norm")
+        if global_grad_norm.dtype != torch.float32 or global_grad_norm.numel() < 1:
+            raise RuntimeError("global_grad_norm must be a float32 tensor")
+        code = _dtype_code(ref, "grads[0]")
+        norms = get_l2norm_kernel()
+        _, param_norms = norms.multi_tensor_l2norm(chunk_size, noop_flag, [tensor_lists[1]], True)
+        with _device_of(ref):
+            rc = lib.oslo_multi_tensor_lamb_stage1(
+                tables[0], tables[1], tables[2], tables[3], sizes, n, float(beta1), float(beta2),
+                float(epsilon), int(step), int(bias_correction), float(weight_decay),
+                int(grad_averaging), int(mode), _ptr(global_grad_norm), float(max_grad_norm),
+                code, _stream(ref),
+            )
+            _check(rc, lib)
+        _, update_norms = norms.multi_tensor_l2norm(chunk_size, noop_flag, [tensor_lists[0]], True)
+        with _device_of(ref):
+            rc = lib.oslo_multi_tensor_lamb_stage2(
+                tables[0], tables[1], sizes, n, _ptr(param_norms), _ptr(update_norms), float(lr),
+                float(weight_decay), int(bool(use_nvlamb)), code, _stream(ref),
+            )
+            _check(rc, lib)
+
+
+_optimizer_kernels = {}
+
+
+def _optimizer_kernel(cls):
+    kernel = _optimizer_kernels.get(cls)
+    if kernel is None:
+        kernel = _optimizer_kernels[cls] = cls(load_library())
+    return kernel
 
 
 def get_adam_kernel():
-    global _adam_kernel
-    if _adam_kernel is None:
-        _adam_kernel = _AdamKernel(load_library())
-    return _adam_kernel
+    return _optimizer_kernel(_AdamKernel)
+
+
+def get_sgd_kernel():
+    return _optimizer_kernel(_SGDKernel)
+
+
+def get_adagrad_kernel():
+    return _optimizer_kernel(_AdagradKernel)
+
+
+def get_novograd_kernel():
+    return _optimizer_kernel(_NovogradKernel)
+
+
+def get_l2norm_kernel():
+    return _optimizer_kernel(_L2NormKernel)
+
+
+def get_lamb_kernel():
+    return _optimizer_kernel(_LambKernel)
 
 
 def get_fused_elementwise_kernel():

@@ -53,17 +53,29 @@ def rel_l2(actual64, truth64):
     return float(num / den) if den > 0 else float(num)
 
 
-def check_lowp(actual, truth64, what, min_exact=0.998, max_ulp=1, l2_tol=2e-3, atol=0.0):
+def check_lowp(actual, truth64, what, min_exact=0.998, max_ulp=1, l2_tol=2e-3, atol=0.0,
+               single_rounding_too=False):
     """16-bit parity (see module docstring).  `actual` is a torch tensor of the
     storage dtype, `truth64` the float64 oracle (unrounded).  An element whose
     absolute error is within `atol` counts as exact: results that cancel to
     almost nothing carry the absolute error of the fp32 arithmetic, which can be
-    many ulps of a tiny value."""
+    many ulps of a tiny value.
+
+    The expected value is the oracle rounded to float32 and then to the storage
+    type, the two roundings of an fp32 evaluation.  `single_rounding_too` also
+    accepts the oracle rounded to float16 directly: where the last operation is
+    a multiply-add the hardware can form it and round it to float16 in one
+    instruction, which differs from the two roundings exactly when the fp32
+    value falls on a float16 tie -- common for 16-bit operands times short
+    constants (0.9 m + 0.1 g)."""
     actual = actual.detach().cpu()
     truth64 = np.asarray(truth64, dtype=np.float64).reshape(actual.shape)
     expect = torch.from_numpy(truth64).to(torch.float32).to(actual.dtype)
     assert torch.isfinite(actual.float()).all(), what + ": non-finite output"
     d = ulp_distance(actual, expect)
+    if single_rounding_too and actual.dtype == torch.float16:
+        direct = torch.from_numpy(truth64.astype(np.float16))
+        d = torch.minimum(d, ulp_distance(actual, direct))
     if atol > 0:
         within = torch.from_numpy(np.abs(f64(actual) - truth64) <= atol)
         d = torch.where(within, torch.zeros_like(d), d)

@@ -1,0 +1,386 @@
+"""Multi-tensor SGD, Adagrad, NovoGrad, LAMB and the tensor norms on the GPU,
+through the C ABI, against the float64 oracle (oracle/closed_form.py, pinned by
+test_oracle_optimizers.py): fp32 to 1e-5 relative, 16-bit results against the
+oracle rounded once to the storage type."""
+import numpy as np
+import pytest
+import torch
+
+from helpers import NP_NAME, check, f64, randn
+from oracle import closed_form as cf
+from oslo_amd.torch import _C
+
+pytestmark = pytest.mark.gpu
+
+F32, F16, BF16 = torch.float32, torch.float16, torch.bfloat16
+
+# lengths around the vector and piece boundaries of every dtype, an empty tensor,
+# and more tensors than one launch carries (48)
+SIZES = [1, 7, 4096, 4097, 8191, 8192, 100003, 3, 1 << 19, 0, 12345] + [257 + i for i in range(45)]
+CHECKED = [0, 1, 2, 3, 4, 5, 6, 7, 8, 10, 11, 47, 48, 49, 55]
+
+
+def make_lists(dtypes, seed, device, positive=()):
+    host = []
+    for k, dt in enumerate(dtypes):
+        lst = []
+        for i, n in enumerate(SIZES):
+            t = randn((n,), dt, seed + 1000 * k + i, std=0.1 if k in positive else 1.0)
+            lst.append(t.abs() if k in positive else t)
+        host.append(lst)
+    return host, [[t.to(device) for t in lst] for lst in host]
+
+
+# 16-bit: the fp32 evaluation (several roundings before the store) lands on the
+# other side of a rounding tie slightly more often than 0.2 % of the time; and a
+# final multiply-add may be rounded to float16 once instead of twice
+def kw(dtype):
+    return {} if dtype == F32 else {"min_exact": 0.99, "single_rounding_too": True}
+
+
+def unrounded(dtype):
+    """The oracle's `out` for a check: 16-bit results are compared from the
+    unrounded float64 value, so that either rounding can be recognised."""
+    return "f64" if dtype != F32 else "f32"
+
+
+@pytest.mark.parametrize("gdtype,wdtype,copy", [(F32, F32, None), (F16, F16, None), (BF16, BF16, None),
+                                                (F16, F32, F16), (BF16, F32, BF16), (F32, F32, BF16),
+                                                (BF16, F32, None)])
+@pytest.mark.parametrize("momentum,dampening,nesterov,wd,after", [
+    (0.0, 0.0, False, 0.0, False), (0.9, 0.0, False, 0.01, False), (0.9, 0.1, False, 0.01, True),
+    (0.9, 0.0, True, 0.01, False)])
+def test_multi_tensor_sgd_vs_oracle(device, gdtype, wdtype, copy, momentum, dampening, nesterov, wd, after):
+    dts = [gdtype, wdtype, wdtype] + ([copy] if copy else [])
+    host, devl = make_lists(dts, 20, device)
+    k = _C.get_sgd_kernel()
+    flag = torch.zeros(1, dtype=torch.int32, device=device)
+    lr, scale = 0.05, 0.5
+    want_w = [f64(t) for t in host[1]]
+    want_m = [f64(t) for t in host[2]]
+    for step in range(3):
+        k.multi_tensor_sgd(2048 * 32, flag, devl, wd, momentum, dampening, lr, nesterov, step == 0, after, scale)
+        for i in CHECKED:
+            w, m, c = cf.sgd_step(f64(host[0][i]), want_w[i], want_m[i], lr, wd, momentum, dampening,
+                                  nesterov, step == 0, after, scale, out=unrounded(wdtype),
+                                  copy=NP_NAME[copy] if copy else None)
+            what = "tensor %d step %d" % (i, step)
+            if SIZES[i]:
+                check(devl[1][i], w, "w " + what, atol=1e-6, **kw(wdtype))
+                if momentum:
+                    # 0.9 mom + 0.9 g of two 16-bit values lies within 3e-8 (relative) of
+                    # a rounding tie for about one value in ten -- float32(0.9) is that
+                    # far from 0.9 -- which is the resolution of the float32 evaluation
+                    # itself: which neighbour is stored then depends on the order of the
+                    # float32 operations (never more than 1 ulp apart)
+                    loose = dict(kw(wdtype), min_exact=0.95) if wdtype != F32 else {}
+                    check(devl[2][i], m, "mom " + what, atol=1e-6, **loose)
+                else:
+                    assert torch.equal(devl[2][i].cpu(), host[2][i]), "momentum buffer written"
+                if copy:
+                    # the copy is a conversion of the weight the kernel stored
+                    assert torch.equal(devl[3][i], devl[1][i].to(copy)), "copy " + what
+            want_w[i], want_m[i] = f64(devl[1][i]), f64(devl[2][i])
+    for i in CHECKED:
+        assert torch.equal(devl[0][i].cpu(), host[0][i]), "gradients must not change"
+    # a raised flag switches the whole launch off
+    before = [t.clone() for t in devl[1]]
+    flag.fill_(1)
+    k.multi_tensor_sgd(2048 * 32, flag, devl, wd, momentum, dampening, lr, nesterov, False, after, scale)
+    assert all(torch.equal(a, b) for a, b in zip(before, devl[1]))
+
+
+@pytest.mark.parametrize("dtype", [F32, F16, BF16])
+@pytest.mark.parametrize("mode,wd", [(0, 0.0), (0, 0.01), (1, 0.01)])
+def test_multi_tensor_adagrad_vs_oracle(device, dtype, mode, wd):
+    host, devl = make_lists([dtype] * 3, 30, device, positive=(2,))
+    k = _C.get_adagrad_kernel()
+    lr, eps = 0.05, 1e-10
+    want_p = [f64(t) for t in host[1]]
+    want_h = [f64(t) for t in host[2]]
+    for step in range(3):
+        k.multi_tensor_adagrad(2048 * 32, None, devl, lr, eps, mode, wd)
+        for i in CHECKED:
+            p, h = cf.adagrad_step(f64(host[0][i]), want_p[i], want_h[i], lr, eps, mode, wd, out=unrounded(dtype))
+            if SIZES[i]:
+                check(devl[1][i], p, "p[%d] step %d" % (i, step), atol=1e-6, **kw(dtype))
+                check(devl[2][i], h, "h[%d] step %d" % (i, step), atol=1e-7, **kw(dtype))
+            want_p[i], want_h[i] = f64(devl[1][i]), f64(devl[2][i])
+
+
+@pytest.mark.parametrize("dtype", [F32, F16, BF16])
+def test_multi_tensor_l2norm(device, dtype):
+    host, devl = make_lists([dtype], 40, device)
+    k = _C.get_l2norm_kernel()
+    flag = torch.zeros(1, dtype=torch.int32, device=device)
+    total, per = k.multi_tensor_l2norm(2048 * 32, flag, devl, True)
+    want = np.array([cf.tensor_norm(f64(t)) for t in host[0]])
+    assert per.dtype == torch.float32 and per.shape == (len(SIZES),)
+    assert np.allclose(f64(per), want, rtol=2e-6, atol=0.0)
+    assert np.isclose(f64(total)[0], np.sqrt((want ** 2).sum()), rtol=2e-6)
+    assert per[SIZES.index(0)].item() == 0.0
+    assert flag.item() == 0
+    total2, per2 = k.multi_tensor_l2norm(2048 * 32, flag, devl, False)
+    assert per2.numel() == 0 and torch.equal(total2, total)  # a fixed summation order
+    # unaligned views take the scalar path
+    base = randn((5000,), dtype, 41).to(device)
+    views = [base[1:1001], base[1003:4000]]
+    _, pv = k.multi_tensor_l2norm(0, None, [views], True)
+    assert np.allclose(f64(pv), [cf.tensor_norm(f64(v)) for v in views], rtol=2e-6)
+    # a value that is not finite reaches the result and raises the flag
+    devl[0][4][17] = float("inf")
+    total3, _ = k.multi_tensor_l2norm(2048 * 32, flag, devl, False)
+    assert torch.isinf(total3).all() and flag.item() == 1
+
+
+@pytest.mark.parametrize("norm_type", [2, 0])
+def test_multi_tensor_norm_out_blends(device, norm_type):
+    host, devl = make_lists([BF16], 50, device)
+    k = _C.get_l2norm_kernel()
+    g = torch.Generator().manual_seed(5)
+    old = torch.rand(len(SIZES), generator=g) + 0.5
+    out = old.to(device)
+    k.multi_tensor_norm_out(2048 * 32, None, devl, out, 0.75, 0.25, norm_type)
+    want = [cf.blend_norm(old[i].item(), f64(t), 0.75, 0.25, norm_type) for i, t in enumerate(host[0])]
+    assert np.allclose(f64(out), want, rtol=2e-6)
+
+
+@pytest.mark.parametrize("dtype", [F32, F16, BF16])
+@pytest.mark.parametrize("moment_mode,wd,averaging,norm_type", [(1, 0.0, 1, 2), (0, 0.01, 1, 2), (1, 0.01, 0, 0)])
+def test_multi_tensor_novograd_vs_oracle(device, dtype, moment_mode, wd, averaging, norm_type):
+    host, devl = make_lists([dtype] * 3, 60, device)
+    k = _C.get_novograd_kernel()
+    lr, b1, b2, eps = 0.01, 0.95, 0.98, 1e-8
+    norms0 = torch.tensor([float(cf.tensor_norm(f64(t), norm_type)) for t in host[0]], dtype=torch.float32)
+    norms = norms0.to(device)
+    want_p = [f64(t) for t in host[1]]
+    want_m = [f64(t) for t in host[2]]
+    want_n = [float(v) for v in norms0]
+    for step in (1, 2, 5):
+        k.multi_tensor_novograd(2048 * 32, None, devl, norms, lr, b1, b2, eps, step, 1, wd, averaging,
+                                moment_mode, norm_type)
+        got_n = f64(norms)
+        for i in CHECKED:
+            n = cf.blend_norm(want_n[i], f64(host[0][i]), b2, 1.0 - b2, norm_type)
+            assert np.isclose(got_n[i], n, rtol=2e-6), "norm %d step %d" % (i, step)
+            # the element-wise step from the norm the kernel stored
+            p, m = cf.novograd_step(f64(host[0][i]), want_p[i], want_m[i], got_n[i], lr, b1, b2, eps, step,
+                                    True, wd, averaging, moment_mode, out=unrounded(dtype))
+            if SIZES[i]:
+                check(devl[1][i], p, "p[%d] step %d" % (i, step), atol=1e-6, **kw(dtype))
+                check(devl[2][i], m, "m[%d] step %d" % (i, step), atol=1e-6, **kw(dtype))
+            want_p[i], want_m[i], want_n[i] = f64(devl[1][i]), f64(devl[2][i]), got_n[i]
+
+
+@pytest.mark.parametrize("dtype", [F32, F16, BF16])
+@pytest.mark.parametrize("mode,wd,nvlamb,clip", [(1, 0.01, False, 1e9), (0, 0.01, False, 1e9),
+                                                 (1, 0.0, False, 1e9), (1, 0.0, True, 1.0)])
+def test_multi_tensor_lamb_vs_oracle(device, dtype, mode, wd, nvlamb, clip):
+    host, devl = make_lists([dtype] * 4, 70, device, positive=(3,))
+    k = _C.get_lamb_kernel()
+    lr, b1, b2, eps, step = 0.01, 0.9, 0.999, 1e-6, 3
+    gn = float(np.sqrt(sum(cf.tensor_norm(f64(t)) ** 2 for t in host[0])))
+    gnorm = torch.tensor([gn], dtype=torch.float32, device=device)
+    k.multi_tensor_lamb(2048 * 32, None, devl, lr, b1, b2, eps, step, 1, wd, 1, mode, gnorm, clip, nvlamb)
+    for i in CHECKED:
+        if not SIZES[i]:
+            continue
+        u, m, v = cf.lamb_stage1(f64(host[0][i]), f64(host[1][i]), f64(host[2][i]), f64(host[3][i]), b1, b2, eps,
+                                 step, True, wd, True, mode, np.float32(gn), clip, out=unrounded(dtype))
+        what = "tensor %d" % i
+        check(devl[0][i], u, "update " + what, atol=1e-6, **kw(dtype))
+        check(devl[2][i], m, "m " + what, atol=1e-7, **kw(dtype))
+        check(devl[3][i], v, "v " + what, atol=1e-8, **kw(dtype))
+        # stage 2 from the update the kernel stored (its norm is what stage 2 saw)
+        ud = f64(devl[0][i])
+        p = cf.lamb_stage2(ud, f64(host[1][i]), np.float32(cf.tensor_norm(f64(host[1][i]))),
+                           np.float32(cf.tensor_norm(ud)), lr, wd, nvlamb, out=unrounded(dtype))
+        check(devl[1][i], p, "p " + what, atol=1e-6, **kw(dtype))
+
+
+def test_argument_checks(device):
+    a = torch.zeros(8, device=device)
+    h = a.half()
+    with pytest.raises(RuntimeError):
+        _C.get_sgd_kernel().multi_tensor_sgd(0, None, [[a], [a]], 0, 0, 0, 0.1, False, True, False, 1.0)
+    with pytest.raises(RuntimeError):  # float32 gradients with 16-bit weights
+        _C.get_sgd_kernel().multi_tensor_sgd(0, None, [[a], [h], [h]], 0, 0, 0, 0.1, False, True, False, 1.0)
+    with pytest.raises(RuntimeError):  # a copy of 16-bit weights
+        _C.get_sgd_kernel().multi_tensor_sgd(0, None, [[h], [h], [h], [h]], 0, 0, 0, 0.1, False, True, False, 1.0)
+    with pytest.raises(RuntimeError):  # momentum of another dtype than the weights
+        _C.get_sgd_kernel().multi_tensor_sgd(0, None, [[h], [a], [h]], 0, 0, 0, 0.1, False, True, False, 1.0)
+    with pytest.raises(RuntimeError):
+        _C.get_adagrad_kernel().multi_tensor_adagrad(0, None, [[a], [a], [a]], 0.1, 1e-10, 2, 0.0)
+    with pytest.raises(RuntimeError):
+        _C.get_adagrad_kernel().multi_tensor_adagrad(0, None, [[a], [a, a], [a]], 0.1, 1e-10, 0, 0.0)
+    with pytest.raises(RuntimeError):
+        _C.get_l2norm_kernel().multi_tensor_norm_out(0, None, [[a]], torch.zeros(2, device=device), 0.5, 0.5, 2)
+    with pytest.raises(RuntimeError):
+        _C.get_l2norm_kernel().multi_tensor_norm_out(0, None, [[a]], torch.zeros(1, device=device), 0.5, 0.5, 1)
+    with pytest.raises(RuntimeError):  # the flag must live on the GPU
+        _C.get_l2norm_kernel().multi_tensor_l2norm(0, torch.zeros(1, dtype=torch.int32), [[a]], False)
+    _C.get_adagrad_kernel().multi_tensor_adagrad(0, None, [[], [], []], 0.1, 1e-10, 0, 0.0)
+
+
+# ---------------------------------------------------------------------------
+# the optimizer classes
+# ---------------------------------------------------------------------------
+def _mlp(device):
+    torch.manual_seed(0)
+    return torch.nn.Sequential(
+        torch.nn.Linear(64, 96), torch.nn.GELU(), torch.nn.Linear(96, 33), torch.nn.LayerNorm(33)
+    ).to(device)
+
+
+def _train(models_and_optimizers, device, steps=8, shared_gradients=False):
+    """`shared_gradients`: every model steps on the gradients of the last one.
+    An optimizer that normalises each element's step (Adagrad) turns a
+    last-place difference in a near-zero gradient into a step of another size,
+    so two trajectories on their own gradients drift apart for reasons that say
+    nothing about the update rule."""
+    g = torch.Generator(device=device).manual_seed(1)
+    for _ in range(steps):
+        x = torch.randn(16, 64, generator=g, device=device)
+        for mdl, opt in models_and_optimizers:
+            opt.zero_grad()
+            mdl(x).square().mean().backward()
+        if shared_gradients:
+            src = list(models_and_optimizers[-1][0].parameters())
+            for mdl, _ in models_and_optimizers[:-1]:
+                for p, q in zip(mdl.parameters(), src):
+                    p.grad = q.grad.clone()
+        for _, opt in models_and_optimizers:
+            opt.step()
+
+
+@pytest.mark.parametrize("kwargs", [dict(), dict(momentum=0.9), dict(momentum=0.9, weight_decay=0.02),
+                                    dict(momentum=0.9, nesterov=True), dict(momentum=0.8, dampening=0.2)])
+def test_fused_sgd_tracks_torch_optim(device, kwargs):
+    from oslo_amd.torch.optim import FusedSGD
+
+    a, b = _mlp(device), _mlp(device)
+    oa = FusedSGD(a.parameters(), lr=0.05, **kwargs)
+    ob = torch.optim.SGD(b.parameters(), lr=0.05, **kwargs)
+    _train([(a, oa), (b, ob)], device)
+    for pa, pb in zip(a.parameters(), b.parameters()):
+        assert torch.allclose(pa, pb, rtol=1e-5, atol=1e-6)
+    if kwargs.get("momentum"):
+        for pa, pb in zip(a.parameters(), b.parameters()):
+            assert torch.allclose(oa.state[pa]["momentum_buffer"], ob.state[pb]["momentum_buffer"],
+                                  rtol=1e-5, atol=1e-7)
+    with pytest.raises(ValueError):
+        FusedSGD(a.parameters(), lr=0.1, nesterov=True)
+    with pytest.raises(ValueError):
+        FusedSGD(a.parameters(), lr=-1.0)
+    oa.zero_grad()
+    assert all(p.grad is not None for p in a.parameters())  # set_grad_none defaults to False here
+
+
+def test_fused_sgd_parameter_added_later_and_bf16(device):
+    """A parameter that joins after the first step starts its momentum buffer on
+    its own first step; bfloat16 and float32 parameters share a group."""
+    from oslo_amd.torch.optim import FusedSGD
+
+    p1 = torch.nn.Parameter(randn((300,), F32, 1).to(device))
+    p2 = torch.nn.Parameter(randn((500,), BF16, 2).to(device))
+    opt = FusedSGD([p1], lr=0.1, momentum=0.9)
+    g1, g2 = randn((300,), F32, 3).to(device), randn((500,), BF16, 4).to(device)
+    p1.grad = g1.clone()
+    opt.step()
+    opt.add_param_group({"params": [p2]})
+    w1, w2 = f64(p1), f64(p2)
+    m1 = f64(opt.state[p1]["momentum_buffer"])
+    p1.grad, p2.grad = g1.clone(), g2.clone()
+    opt.step()
+    want1, wm1, _ = cf.sgd_step(f64(g1), w1, m1, 0.1, 0.0, 0.9, 0.0, False, False, out="f32")
+    want2, wm2, _ = cf.sgd_step(f64(g2), w2, np.zeros(500), 0.1, 0.0, 0.9, 0.0, False, True, out="f64")
+    check(p1.data, want1, "float32 parameter, second step")
+    check(p2.data, want2, "bfloat16 parameter, first step", **kw(BF16))
+    check(opt.state[p2]["momentum_buffer"], wm2, "its momentum buffer", **kw(BF16))
+
+
+@pytest.mark.parametrize("wd", [0.0, 0.02])
+def test_fused_adagrad_tracks_torch_optim(device, wd):
+    from oslo_amd.torch.optim import FusedAdagrad
+
+    a, b = _mlp(device), _mlp(device)
+    oa = FusedAdagrad(a.parameters(), lr=0.05, weight_decay=wd)
+    ob = torch.optim.Adagrad(b.parameters(), lr=0.05, weight_decay=wd, eps=1e-10)
+    _train([(a, oa), (b, ob)], device, shared_gradients=True)
+    for pa, pb in zip(a.parameters(), b.parameters()):
+        assert torch.allclose(pa, pb, rtol=1e-5, atol=1e-6)
+        assert torch.allclose(oa.state[pa]["sum"], ob.state[pb]["sum"], rtol=1e-5, atol=1e-12)
+    oa.zero_grad()
+    assert all(p.grad is None for p in a.parameters())
+
+
+def _param_set(device, dtype):
+    shapes = [(40, 30), (30,), (7, 5, 11)]
+    ps = [torch.nn.Parameter(randn(s, dtype, 80 + i).to(device)) for i, s in enumerate(shapes)]
+    grads = [[randn(s, dtype, 90 + 10 * step + i) for i, s in enumerate(shapes)] for step in range(4)]
+    return ps, grads
+
+
+@pytest.mark.parametrize("dtype", [F32, BF16])
+@pytest.mark.parametrize("init_zero,reg_inside,norm_type", [(False, False, 2), (True, True, 2), (False, False, 0)])
+def test_fused_novograd_follows_the_oracle(device, dtype, init_zero, reg_inside, norm_type):
+    from oslo_amd.torch.optim import FusedNovograd
+
+    ps, grads = _param_set(device, dtype)
+    lr, betas, eps, wd = 0.01, (0.95, 0.98), 1e-8, 0.01
+    opt = FusedNovograd(ps, lr=lr, betas=betas, eps=eps, weight_decay=wd, init_zero=init_zero,
+                        reg_inside_moment=reg_inside, norm_type=norm_type)
+    want_p = [f64(p) for p in ps]
+    want_m = [np.zeros(p.shape) for p in ps]
+    want_n = [None] * len(ps)
+    for step, gs in enumerate(grads, start=1):
+        for p, g in zip(ps, gs):
+            p.grad = g.to(device)
+        opt.step()
+        for i, g in enumerate(gs):
+            if want_n[i] is None:
+                want_n[i] = 0.0 if init_zero else float(cf.tensor_norm(f64(g), norm_type))
+            want_n[i] = float(cf.blend_norm(want_n[i], f64(g), betas[1], 1.0 - betas[1], norm_type))
+            p, m = cf.novograd_step(f64(g), want_p[i], want_m[i], np.float32(want_n[i]), lr, betas[0], betas[1],
+                                    eps, step, True, wd, True, 0 if reg_inside else 1, out=unrounded(dtype))
+            check(ps[i].data, p, "p[%d] step %d" % (i, step), atol=1e-6, **kw(dtype))
+            want_p[i], want_m[i] = f64(ps[i]), f64(opt.state[ps[i]]["exp_avg"])
+    assert opt.param_groups[0]["step"] == len(grads)
+    with pytest.raises(RuntimeError):
+        FusedNovograd(ps, amsgrad=True)
+    with pytest.raises(RuntimeError):
+        FusedNovograd(ps, norm_type=1)
+
+
+@pytest.mark.parametrize("dtype", [F32, BF16])
+@pytest.mark.parametrize("wd,max_grad_norm,nvlamb", [(0.01, 0.0, False), (0.0, 0.5, False), (0.0, 0.0, True)])
+def test_fused_lamb_follows_the_oracle(device, dtype, wd, max_grad_norm, nvlamb):
+    from oslo_amd.torch.optim import FusedLamb
+
+    ps, grads = _param_set(device, dtype)
+    lr, betas, eps = 0.01, (0.9, 0.999), 1e-6
+    opt = FusedLamb(ps, lr=lr, betas=betas, eps=eps, weight_decay=wd, max_grad_norm=max_grad_norm,
+                    use_nvlamb=nvlamb)
+    want_p = [f64(p) for p in ps]
+    want_m = [np.zeros(p.shape) for p in ps]
+    want_v = [np.zeros(p.shape) for p in ps]
+    for step, gs in enumerate(grads, start=1):
+        for p, g in zip(ps, gs):
+            p.grad = g.to(device)
+        opt.step()
+        gn = np.float32(np.sqrt(sum(cf.tensor_norm(f64(g)) ** 2 for g in gs)))
+        clip = max_grad_norm if max_grad_norm > 0 else float("inf")
+        for i, g in enumerate(gs):
+            u, m, v = cf.lamb_stage1(f64(g), want_p[i], want_m[i], want_v[i], betas[0], betas[1], eps, step, True,
+                                     wd, True, 1, gn, clip, out=NP_NAME[dtype])
+            # the update direction is what the step left in the gradient
+            p = cf.lamb_stage2(u, want_p[i], np.float32(cf.tensor_norm(want_p[i])), np.float32(cf.tensor_norm(u)),
+                               lr, wd, nvlamb, out=unrounded(dtype))
+            # (a last-place difference in the stored update moves |update| by far less than the tolerance)
+            check(ps[i].data, p, "p[%d] step %d" % (i, step), atol=2e-6, **kw(dtype))
+            want_p[i] = f64(ps[i])
+            want_m[i], want_v[i] = f64(opt.state[ps[i]]["exp_avg"]), f64(opt.state[ps[i]]["exp_avg_sq"])
+    with pytest.raises(RuntimeError):
+        FusedLamb(ps, amsgrad=True)
+    with pytest.raises(RuntimeError):
+        FusedLamb(ps, max_coeff=5.0)
