@@ -573,15 +573,19 @@ def kernel_table(L, dev, iters, graph_column=True):
     for _ in range(16):
         shapes += [(2048, 6144), (6144,), (2048, 2048), (2048,), (2048, 8192), (8192,), (8192, 2048), (2048,),
                    (2048,), (2048,), (2048,), (2048,)]
-    for tdt, code, esz in ((torch.float32, F32, 4), (torch.bfloat16, BF16, 2)):
+
+    def optimizer_tensors(tdt):
         lists = [[torch.zeros(s, device=dev, dtype=tdt) for s in shapes] for _ in range(4)]
         for t in lists[0]:
             t.normal_()
-        nel = sum(t.numel() for t in lists[0])
         n = len(shapes)
         arr = ctypes.c_void_p * n
         tables = [arr(*[t.data_ptr() for t in lst]) for lst in lists]
         sizes = (ctypes.c_int64 * n)(*[t.numel() for t in lists[0]])
+        return lists, tables, sizes, n, sum(t.numel() for t in lists[0])
+
+    for tdt, code, esz in ((torch.float32, F32, 4), (torch.bfloat16, BF16, 2)):
+        lists, tables, sizes, n, nel = optimizer_tensors(tdt)
         step_no = [0]
 
         def adam(i):
@@ -593,11 +597,36 @@ def kernel_table(L, dev, iters, graph_column=True):
         opt_iters = max(10, iters // 4)
         rows.append(table_row("multi_tensor_adam", dname, 7 * nel * esz,
                               time_launches(torch, adam, opt_iters, 1), note="%d tensors" % n))
+        del lists, tables
+        torch.cuda.empty_cache()
 
-        # the other optimizer steps on the same tensors (values moved per element:
-        # SGD with momentum and Adagrad read 3 and write 2; NovoGrad reads the
-        # gradients once more for their norms; LAMB = parameter norms 1 + stage 1
-        # (reads 4, writes 3) + update norms 1 + stage 2 (reads 2, writes 1))
+    # ---- plain copies with the same load/store path, at the traffic of the
+    # short kernels above and at 2 GiB: the practical ceiling at each size ----
+    for total_mb in (75.5, 100.8, 201.3, 268.4, 402.7, 830.0, 2147.5):
+        nbytes = int(total_mb * 1e6 / 2) // 16 * 16
+        ns = nsets_for(2 * nbytes)
+        src = [torch.empty(nbytes, dtype=torch.uint8, device=dev) for _ in range(ns)]
+        dst = [torch.empty(nbytes, dtype=torch.uint8, device=dev) for _ in range(ns)]
+        for s_ in src:
+            s_.fill_(1)
+
+        def cp(i):
+            L.ok(lib.oslo_copy_probe(p(src[i]), p(dst[i]), nbytes, L.stream()))
+
+        rows.append(table_row("copy_probe", "-", 2 * nbytes, timed(cp, ns), note="plain copy, read + write"))
+        del src, dst
+        torch.cuda.empty_cache()
+
+    # ---- the other multi-tensor optimizer steps on the tensors of the Adam rows
+    # (values moved per element: SGD with momentum and Adagrad read 3 and write 2;
+    # NovoGrad reads the gradients once more for their norms; LAMB = parameter
+    # norms 1 + stage 1 (reads 4, writes 3) + update norms 1 + stage 2 (reads 2,
+    # writes 1)) ----
+    for tdt, code, esz in ((torch.float32, F32, 4), (torch.bfloat16, BF16, 2)):
+        lists, tables, sizes, n, nel = optimizer_tensors(tdt)
+        step_no = [0]
+        dname = str(tdt).split(".")[-1]
+        opt_iters = max(10, iters // 4)
         need = int(lib.oslo_multi_tensor_norm_partials(sizes, n, code))
         partials = torch.empty(need, dtype=torch.float32, device=dev)
         norms = torch.ones(n, dtype=torch.float32, device=dev)
@@ -643,23 +672,6 @@ def kernel_table(L, dev, iters, graph_column=True):
             rows.append(table_row(name, dname, values * nel * esz, time_launches(torch, fn, opt_iters, 1),
                                   note="%d tensors" % n))
         del lists, tables, partials
-        torch.cuda.empty_cache()
-
-    # ---- plain copies with the same load/store path, at the traffic of the
-    # short kernels above and at 2 GiB: the practical ceiling at each size ----
-    for total_mb in (75.5, 100.8, 201.3, 268.4, 402.7, 830.0, 2147.5):
-        nbytes = int(total_mb * 1e6 / 2) // 16 * 16
-        ns = nsets_for(2 * nbytes)
-        src = [torch.empty(nbytes, dtype=torch.uint8, device=dev) for _ in range(ns)]
-        dst = [torch.empty(nbytes, dtype=torch.uint8, device=dev) for _ in range(ns)]
-        for s_ in src:
-            s_.fill_(1)
-
-        def cp(i):
-            L.ok(lib.oslo_copy_probe(p(src[i]), p(dst[i]), nbytes, L.stream()))
-
-        rows.append(table_row("copy_probe", "-", 2 * nbytes, timed(cp, ns), note="plain copy, read + write"))
-        del src, dst
         torch.cuda.empty_cache()
     return rows
 
