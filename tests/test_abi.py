@@ -74,6 +74,43 @@ def test_invalid_arguments_are_rejected_before_any_launch():
     assert lib.oslo_bias_gelu_fwd(None, None, None, 0, 8, 2, None) == 0
 
 
+def test_multi_tensor_entry_points_check_their_arguments():
+    import ctypes
+
+    lib = _C.load_library()
+    one = (ctypes.c_void_p * 1)(None)
+    sizes = (ctypes.c_int64 * 1)(8)
+    neg = (ctypes.c_int64 * 1)(-8)
+    # float32 gradients cannot meet 16-bit weights; a copy needs float32 weights
+    rc = lib.oslo_multi_tensor_sgd(one, one, one, None, sizes, 1, 0, 0, 0, 0.1, 0, 1, 0, 1.0, 0, 1, 0, None, None)
+    assert rc == -1 and b"weights must" in lib.oslo_hip_last_error()
+    rc = lib.oslo_multi_tensor_sgd(one, one, one, one, sizes, 1, 0, 0, 0, 0.1, 0, 1, 0, 1.0, 1, 1, 1, None, None)
+    assert rc == -1 and b"16-bit copy" in lib.oslo_hip_last_error()
+    # a null tensor pointer and a negative length are caught before any launch
+    rc = lib.oslo_multi_tensor_sgd(one, one, one, None, sizes, 1, 0, 0, 0, 0.1, 0, 1, 0, 1.0, 0, 0, 0, None, None)
+    assert rc == -1 and b"null pointer" in lib.oslo_hip_last_error()
+    rc = lib.oslo_multi_tensor_adagrad(one, one, one, neg, 1, 0.1, 1e-10, 0, 0.0, 0, None)
+    assert rc == -1 and b"size -8" in lib.oslo_hip_last_error()
+    assert lib.oslo_multi_tensor_adagrad(one, one, one, sizes, 1, 0.1, 1e-10, 2, 0.0, 0, None) == -1
+    assert lib.oslo_multi_tensor_novograd(one, one, one, sizes, 1, None, 0.1, 0.9, 0.99, 1e-8, 1, 1, 0.0, 1, 1, 0, None) == -1
+    assert lib.oslo_multi_tensor_lamb_stage1(one, one, one, one, sizes, 1, 0.9, 0.99, 1e-6, 1, 1, 0.0, 1, 3,
+                                             None, 1.0, 0, None) == -1
+    assert lib.oslo_multi_tensor_lamb_stage2(one, one, sizes, 1, None, None, 0.1, 0.0, 0, 0, None) == -1
+    assert lib.oslo_multi_tensor_norm(one, sizes, 1, 0, None, 0, None, None, 2, 0, 0.0, 0.0, None, None) == -1
+    assert b"no workspace" in lib.oslo_hip_last_error()
+    assert lib.oslo_multi_tensor_norm(one, sizes, 1, 0, one, 1, None, None, 1, 0, 0.0, 0.0, None, None) == -1
+    assert lib.oslo_multi_tensor_norm(one, sizes, 1, 0, one, 1, None, None, 2, 1, 0.5, 0.5, None, None) == -1
+    assert b"blending needs" in lib.oslo_hip_last_error()
+    # workspace: one value per piece of 16384 float32 / 32768 16-bit elements, at least one
+    three = (ctypes.c_int64 * 3)(16384, 16385, 0)
+    assert lib.oslo_multi_tensor_norm_partials(three, 3, 0) == 3
+    assert lib.oslo_multi_tensor_norm_partials(three, 3, 2) == 2
+    assert lib.oslo_multi_tensor_norm_partials(three, 0, 0) == 1
+    assert lib.oslo_multi_tensor_norm_partials(neg, 1, 0) < 0
+    # no tensors: nothing to do
+    assert lib.oslo_multi_tensor_sgd(None, None, None, None, None, 0, 0, 0, 0, 0.1, 0, 1, 0, 1.0, 0, 0, 0, None, None) == 0
+
+
 def test_batch_per_block():
     lib = _C.load_library()
     assert lib.oslo_softmax_batch_per_block(1024, 1024, 16, 16) >= 1

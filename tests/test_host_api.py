@@ -174,3 +174,38 @@ def test_gpu_entry_points_refuse_cpu_tensors():
     # cast helper is the identity outside autocast
     a = torch.zeros(2)
     assert F_._cast_if_autocast_enabled(a, 3)[0] is a
+
+
+def test_fused_optimizers_mirror_the_reference_constructors():
+    """oslo/torch/optim/__init__.py:1-6: the class names, and the argument checks
+    that need no GPU (fused_sgd.py:98-114, fused_novograd.py:86-87)."""
+    import oslo_amd.torch.optim as optim
+
+    for name in ("FusedAdam", "FusedAdagrad", "FusedLamb", "FusedNovograd", "FusedSGD"):
+        assert issubclass(getattr(optim, name), torch.optim.Optimizer)
+    w = torch.nn.Parameter(torch.zeros(4))
+    sgd = optim.FusedSGD([w], lr=0.1, momentum=0.9, nesterov=True)
+    assert sgd.defaults == dict(lr=0.1, momentum=0.9, dampening=0, weight_decay=0, nesterov=True)
+    assert sgd.wd_after_momentum is False and sgd.most_recent_scale == 1.0
+    for bad in (dict(lr=-0.1), dict(lr=0.1, momentum=-1.0), dict(lr=0.1, weight_decay=-1.0),
+                dict(lr=0.1, nesterov=True), dict(lr=0.1, momentum=0.9, dampening=0.1, nesterov=True)):
+        with pytest.raises(ValueError):
+            optim.FusedSGD([w], **bad)
+    ada = optim.FusedAdagrad([w])
+    assert ada.defaults == dict(lr=1e-3, eps=1e-10, weight_decay=0.0) and ada.adagrad_w_mode == 0
+    novo = optim.FusedNovograd([w], reg_inside_moment=True)
+    assert novo.moment_mode == 0 and novo.defaults["norm_type"] == 2 and novo.defaults["betas"] == (0.9, 0.999)
+    with pytest.raises(RuntimeError):
+        optim.FusedNovograd([w], amsgrad=True)
+    lamb = optim.FusedLamb([w], max_grad_norm=1.0)
+    assert lamb.defaults["max_grad_norm"] == 1.0 and lamb.adam_w_mode == 1
+    with pytest.raises(RuntimeError):
+        optim.FusedLamb([w], eps_inside_sqrt=True)
+    # a step on CPU parameters is refused with a clear message, not attempted
+    w.grad = torch.ones(4)
+    with pytest.raises(RuntimeError, match="GPU-only"):
+        sgd.step()
+    # parameters without gradients: nothing to do, no GPU needed
+    w.grad = None
+    for opt in (sgd, ada, novo, lamb):
+        opt.step()
