@@ -643,23 +643,23 @@ def kernel_table(L, dev, iters, graph_column=True):
 
         def l2norm(i):
             L.ok(lib.oslo_multi_tensor_norm(tables[0], sizes, n, code, p(partials), need, p(gnorm), p(norms), 2, 0,
-                                            0.0, 0.0, None, L.stream()))
+                                            0.0, 0.0, None, 0, L.stream()))
 
         def novograd(i):
             step_no[0] += 1
             L.ok(lib.oslo_multi_tensor_norm(tables[0], sizes, n, code, p(partials), need, None, p(norms), 2, 1,
-                                            0.98, 0.02, None, L.stream()))
+                                            0.98, 0.02, None, 0, L.stream()))
             L.ok(lib.oslo_multi_tensor_novograd(tables[0], tables[1], tables[2], sizes, n, p(norms), 1e-3, 0.95, 0.98,
                                                 1e-8, step_no[0], 1, 0.01, 1, 1, code, L.stream()))
 
         def lamb(i):
             step_no[0] += 1
             L.ok(lib.oslo_multi_tensor_norm(tables[1], sizes, n, code, p(partials), need, None, p(norms), 2, 0,
-                                            0.0, 0.0, None, L.stream()))
+                                            0.0, 0.0, None, 0, L.stream()))
             L.ok(lib.oslo_multi_tensor_lamb_stage1(tables[0], tables[1], tables[2], tables[3], sizes, n, 0.9, 0.999,
                                                    1e-6, step_no[0], 1, 0.01, 1, 1, p(gnorm), 1.0, code, L.stream()))
             L.ok(lib.oslo_multi_tensor_norm(tables[0], sizes, n, code, p(partials), need, None, p(norms2), 2, 0,
-                                            0.0, 0.0, None, L.stream()))
+                                            0.0, 0.0, None, 0, L.stream()))
             L.ok(lib.oslo_multi_tensor_lamb_stage2(tables[0], tables[1], sizes, n, p(norms), p(norms2), 1e-3, 0.01,
                                                    0, code, L.stream()))
 

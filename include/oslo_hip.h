@@ -481,12 +481,45 @@ int oslo_multi_tensor_lamb_stage2(const void *const *update, void *const *p,
  * partials: workspace of partials_len floats, at least
  * oslo_multi_tensor_norm_partials(sizes, ntensors, dtype); the sums are folded
  * in a fixed order (no atomics).  A partial result that is not finite sets
- * *noop_flag (device int, or null) to 1 (:87-89).                            */
+ * *noop_flag (device int, or null) to 1 (:87-89).  With skip_if_flag the
+ * call does nothing (the outputs keep their contents) while *noop_flag is
+ * already raised when its kernels start.                                     */
 int64_t oslo_multi_tensor_norm_partials(const int64_t *sizes, int64_t ntensors, int dtype);
 int oslo_multi_tensor_norm(const void *const *x, const int64_t *sizes, int64_t ntensors,
                            int dtype, float *partials, int64_t partials_len, float *out_global,
                            float *out_per_tensor, int norm_type, int blend, float alpha,
-                           float beta, int *noop_flag, void *stream);
+                           float beta, int *noop_flag, int skip_if_flag, void *stream);
+
+/* The two element-wise stages of multi_tensor_lamb_mp (oslo/torch/_C/csrc/
+ * multi_tensor_lamb_mp.cu:324-426; stage 1 :40-205, stage 2 :209-322), called
+ * by FusedMixedPrecisionLamb.step (oslo/torch/optim/
+ * fused_mixed_precision_lamb.py:268-286).  As the plain stages above, except:
+ * step (int), lr, max_grad_norm and inv_scale (float) are DEVICE scalars, read
+ * when the kernels run, so a training step needs no host synchronisation;
+ * the gradient is multiplied by *inv_scale first; the bias corrections
+ * 1 - beta^step are formed on the device (in double, then rounded to
+ * float, like the host-side ones of the plain stages; the reference forms
+ * them with a float power, :54-59); both stages do nothing while
+ * *noop_flag (device int, or null) is non-zero.  Stage 1: gradients of
+ * dtype_grad, parameters and moments of dtype_param (the same, or f32 master
+ * values).  Stage 2: with p_copy (or null) the new f32 parameter is also
+ * written in the update's type (the model's 16-bit weights).  The norms of
+ * the reference's "mp" host function are oslo_multi_tensor_norm calls with
+ * skip_if_flag = 1 (multi_tensor_l2norm_mp.cu:33-35).                        */
+int oslo_multi_tensor_lamb_mp_stage1(void *const *g, const void *const *p, void *const *m,
+                                     void *const *v, const int64_t *sizes, int64_t ntensors,
+                                     float beta1, float beta2, float eps, const int *step,
+                                     int bias_correction, float weight_decay,
+                                     int grad_averaging, int mode,
+                                     const float *global_grad_norm, const float *max_grad_norm,
+                                     const float *inv_scale, const int *noop_flag,
+                                     int dtype_grad, int dtype_param, void *stream);
+int oslo_multi_tensor_lamb_mp_stage2(const void *const *update, void *const *p,
+                                     void *const *p_copy, const int64_t *sizes,
+                                     int64_t ntensors, const float *param_norms,
+                                     const float *update_norms, const float *lr,
+                                     float weight_decay, int use_nvlamb, const int *noop_flag,
+                                     int dtype_update, int dtype_param, void *stream);
 
 /* ---- test and measurement hooks (no counterpart in the reference) ------ */
 

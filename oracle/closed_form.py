@@ -484,11 +484,14 @@ def novograd_step(g, p, m, grad_norm, lr, beta1, beta2, eps, step, bias_correcti
 
 def lamb_stage1(g, p, m, v, beta1, beta2, eps, step, bias_correction, weight_decay,
                 grad_averaging, mode, global_grad_norm, max_grad_norm, out="f64",
-                acc=np.float64):
+                acc=np.float64, inv_scale=1.0, out_update=None):
     """LAMB stage 1 for one tensor: returns ``(update, m, v)``
     (oslo/torch/_C/csrc/multi_tensor_lamb.cu:111-130; bias corrections and
-    beta3 from the host code :300-311)."""
-    g = np.asarray(g, dtype=acc)
+    beta3 from the host code :300-311).  ``inv_scale`` multiplies the gradient
+    first, as the mixed-precision variant does (multi_tensor_lamb_mp.cu:111),
+    whose update has the gradients' storage type ``out_update`` while the
+    moments have the parameters' (``out``)."""
+    g = np.asarray(g, dtype=acc) * acc(np.float32(inv_scale))
     p = np.asarray(p, dtype=acc)
     m = np.asarray(m, dtype=acc)
     v = np.asarray(v, dtype=acc)
@@ -509,7 +512,7 @@ def lamb_stage1(g, p, m, v, beta1, beta2, eps, step, bias_correction, weight_dec
     update = (m / bc1) / (np.sqrt(v / bc2) + _f32(eps, acc))
     if mode != 0:
         update = update + wd * p
-    return round_to(update, out), round_to(m, out), round_to(v, out)
+    return round_to(update, out_update or out), round_to(m, out), round_to(v, out)
 
 
 def lamb_stage2(update, p, param_norm, update_norm, lr, weight_decay, use_nvlamb, out="f64",

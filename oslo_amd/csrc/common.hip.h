@@ -355,6 +355,17 @@ __device__ __forceinline__ float sub_rn(float a, float b) {
   return a - b;
 }
 
+// The value as it sits in a 32-bit register, hidden from the optimiser.  A
+// second output that must be a conversion of the float32 result *as stored*
+// (the 16-bit copy of a float32 master weight) goes through this: otherwise
+// the conversion may be fused with the multiply-add that produced the value
+// and round the unrounded result once, which differs from converting the
+// stored float32 value whenever that lies on a 16-bit rounding tie.
+__device__ __forceinline__ float pinned(float v) {
+  asm volatile("" : "+v"(v));
+  return v;
+}
+
 // Reduction within each group of LPR (8, 16 or 32) consecutive lanes; every
 // lane of a group receives its group's result (each step is symmetric, so the
 // lanes of a group hold the same bits).

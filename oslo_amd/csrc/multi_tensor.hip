@@ -141,6 +141,16 @@ __global__ __launch_bounds__(kMtThreads) void multi_tensor_apply_kernel(MtTable<
 
 struct NoCtx {};
 
+// base^exponent for a step count, by repeated squaring
+__device__ __forceinline__ double int_power(double base, int exponent) {
+  double r = 1.0;
+  for (int e = exponent > 0 ? exponent : 0; e > 0; e >>= 1) {
+    if (e & 1) r *= base;
+    base *= base;
+  }
+  return r;
+}
+
 // SGD with momentum (oslo/torch/_C/csrc/multi_tensor_sgd.cu:29-122): lists
 // gradient, weight, momentum buffer and, with OUT, a 16-bit copy of the
 // updated weight.  The launch does nothing when *noop is non-zero (:35-36).
@@ -170,7 +180,7 @@ template <typename TG, typename TW, typename TO, bool OUT> struct SgdOp {
     // conversion of the stored weight (:108-113)
     v[1] = io<TW>::round(w + (-lr * g));
     v[2] = mom;
-    if constexpr (OUT) v[3] = v[1];
+    if constexpr (OUT) v[3] = v[1] = pinned(v[1]);
   }
 };
 
@@ -303,6 +313,90 @@ template <typename T> struct LambStage2Op {
   __device__ void update(float (&v)[NL], const Ctx &c) const { v[1] = v[1] - (c.ratio * v[0]); }
 };
 
+// LAMB for mixed precision (oslo/torch/_C/csrc/multi_tensor_lamb_mp.cu): the
+// step count, the learning rate, the clip threshold and the inverse loss scale
+// live in device memory, so that a training step needs no host synchronisation,
+// and both stages do nothing while the overflow flag is raised (:46-48, :246-248).
+// Stage 1 (:40-205): gradients of type TG, parameter and moments of type TP
+// (TG, or float32 master copies); the gradient is unscaled first.
+template <typename TG, typename TP> struct LambMpStage1Op {
+  static constexpr int NL = 4;
+  static constexpr int E = (sizeof(TG) == 2 || sizeof(TP) == 2) ? 8 : 4;
+  using Types = std::tuple<TG, TP, TP, TP>;
+  struct Ctx {
+    float clip, bc1, bc2, inv_scale;
+  };
+  float beta1, beta2, beta3, eps, decay;
+  int mode, bias_correction;
+  const int *step, *noop;
+  const float *global_grad_norm, *max_global_grad_norm, *inv_scale;
+  __device__ bool skip() const { return noop != nullptr && *noop != 0; }
+  __device__ Ctx context(int) const {
+    Ctx c;
+    c.bc1 = 1.0f;
+    c.bc2 = 1.0f;
+    if (bias_correction == 1) {
+      // in double, as the host forms them for the plain stages: 1 - beta^step
+      // cancels, and a float32 power would leave 1 - 0.999^3 good to 2e-5 only
+      const int s = *step;
+      c.bc1 = (float)(1.0 - int_power((double)beta1, s));
+      c.bc2 = (float)(1.0 - int_power((double)beta2, s));
+    }
+    const float gn = *global_grad_norm, mx = *max_global_grad_norm;
+    c.clip = gn > mx ? gn / mx : 1.0f;
+    c.inv_scale = *inv_scale;
+    return c;
+  }
+  __device__ bool reads(int l) const { return l != 1 || decay != 0.f; }
+  __device__ bool writes(int l) const { return l != 1; }
+  __device__ void update(float (&v)[NL], const Ctx &c) const {
+    float g = (v[0] * c.inv_scale) / c.clip;
+    const float p = v[1];
+    float m = v[2], s = v[3];
+    if (mode == 0) g = g + decay * p;
+    m = m * beta1 + beta3 * g;
+    s = s * beta2 + (1.f - beta2) * g * g;
+    float update = (m / c.bc1) / (sqrtf(s / c.bc2) + eps);
+    if (mode != 0) update = update + (decay * p);
+    v[0] = update;
+    v[2] = m;
+    v[3] = s;
+  }
+};
+
+// Stage 2 (:209-328): update of type T, parameter of type TP and, with OUT, a
+// copy of the new parameter in type T (the model's weights next to float32
+// master weights).
+template <typename T, typename TP, bool OUT> struct LambMpStage2Op {
+  static constexpr int NL = OUT ? 3 : 2;
+  static constexpr int E = (sizeof(T) == 2 || sizeof(TP) == 2) ? 8 : 4;
+  using Types = std::tuple<T, TP, T>;
+  struct Ctx {
+    float ratio;
+  };
+  float decay;
+  int use_nvlamb;
+  const float *lr, *param_norms, *update_norms;
+  const int *noop;
+  __device__ bool skip() const { return noop != nullptr && *noop != 0; }
+  __device__ Ctx context(int tensor) const {
+    Ctx c;
+    const float rate = *lr;
+    c.ratio = rate;
+    if (use_nvlamb || decay != 0.f) {
+      const float pn = param_norms[tensor], un = update_norms[tensor];
+      c.ratio = (un != 0.f && pn != 0.f) ? rate * (pn / un) : rate;
+    }
+    return c;
+  }
+  __device__ bool reads(int l) const { return l < 2; }
+  __device__ bool writes(int l) const { return l >= 1; }
+  __device__ void update(float (&v)[NL], const Ctx &c) const {
+    v[1] = io<TP>::round(v[1] - (c.ratio * v[0]));
+    if constexpr (OUT) v[2] = v[1] = pinned(v[1]);
+  }
+};
+
 // ---------------------------------------------------------------------------
 // norms (oslo/torch/_C/csrc/multi_tensor_l2norm.cu:29-98 L2, :102-172 max,
 // clean-up kernels :174-255)
@@ -312,11 +406,16 @@ constexpr int kNormLoops = 4;
 // Workgroup b reduces its piece to one value -- the sum of squares, or the
 // largest magnitude with MAXNORM -- and stores it in partials[block0 + b].
 // A value that is not finite raises *noop (every writer stores the same 1).
+// With skip_if_flag the three norm kernels do nothing while *noop is raised
+// (the "mp" variant, oslo/torch/_C/csrc/multi_tensor_l2norm_mp.cu:33-35, 113-115):
+// the flag is read when a kernel starts, and every workgroup of the first
+// kernel that finds it clear writes its partial value.
 template <typename T, bool MAXNORM>
 __global__ __launch_bounds__(kMtThreads) void multi_tensor_norm_kernel(MtTable<1> tab,
                                                                       float *__restrict__ partials,
-                                                                      int *noop) {
+                                                                      int *noop, int skip_if_flag) {
   constexpr int E = io<T>::EPV, U = kMtUnroll;
+  if (skip_if_flag && *noop != 0) return;
   constexpr int64_t kStep = (int64_t)kMtThreads * U * E;
   constexpr int64_t kPiece = kStep * kNormLoops;
   __shared__ float red[kMtThreads / kWave];
@@ -370,8 +469,9 @@ __global__ __launch_bounds__(kMtThreads) void multi_tensor_norm_kernel(MtTable<1
 template <bool MAXNORM>
 __global__ __launch_bounds__(kMtThreads) void multi_tensor_norm_finalize_kernel(
     MtTable<1> tab, const float *__restrict__ partials, float *__restrict__ out, int blend,
-    float alpha, float beta) {
+    float alpha, float beta, const int *noop, int skip_if_flag) {
   __shared__ float red[kMtThreads / kWave];
+  if (skip_if_flag && *noop != 0) return;
   const int t = blockIdx.x;
   const int64_t lo = tab.block0 + tab.first_block[t], hi = tab.block0 + tab.first_block[t + 1];
   float val = 0.f;
@@ -396,8 +496,10 @@ __global__ __launch_bounds__(kMtThreads) void multi_tensor_norm_finalize_kernel(
 // One workgroup folds all partial values into the norm over every tensor.
 template <bool MAXNORM>
 __global__ __launch_bounds__(1024) void multi_tensor_norm_global_kernel(
-    const float *__restrict__ partials, int64_t total_blocks, float *__restrict__ out) {
+    const float *__restrict__ partials, int64_t total_blocks, float *__restrict__ out,
+    const int *noop, int skip_if_flag) {
   __shared__ float red[1024 / kWave];
+  if (skip_if_flag && *noop != 0) return;
   float val = 0.f;
   for (int64_t i = threadIdx.x; i < total_blocks; i += 1024)
     val = MAXNORM ? fmaxf(val, partials[i]) : val + partials[i];
@@ -487,7 +589,7 @@ static int64_t norm_piece_of(int dtype) {
 template <typename T, bool MAXNORM>
 static int launch_norm(const void *const *x, const int64_t *sizes, int64_t ntensors, float *partials,
                        int64_t partials_len, float *out_global, float *out_per_tensor, int blend,
-                       float alpha, float beta, int *noop, hipStream_t st) {
+                       float alpha, float beta, int *noop, int skip_if_flag, hipStream_t st) {
   void *const *const lists[1] = {const_cast<void *const *>(x)};
   int64_t total = 0;
   const int rc = mt_for_each_table<1>(
@@ -498,14 +600,14 @@ static int launch_norm(const void *const *x, const int64_t *sizes, int64_t ntens
                       (long long)partials_len, (long long)(tab.block0 + blocks));
         if (blocks > 0) {
           multi_tensor_norm_kernel<T, MAXNORM>
-              <<<dim3((unsigned)blocks), kMtThreads, 0, st>>>(tab, partials, noop);
+              <<<dim3((unsigned)blocks), kMtThreads, 0, st>>>(tab, partials, noop, skip_if_flag);
           const int rc1 = check_launch("multi_tensor_norm_kernel");
           if (rc1 != OSLO_OK) return rc1;
         }
         if (out_per_tensor != nullptr) {
           multi_tensor_norm_finalize_kernel<MAXNORM>
               <<<dim3((unsigned)tab.ntensors), kMtThreads, 0, st>>>(tab, partials, out_per_tensor, blend,
-                                                                    alpha, beta);
+                                                                    alpha, beta, noop, skip_if_flag);
           const int rc2 = check_launch("multi_tensor_norm_finalize_kernel");
           if (rc2 != OSLO_OK) return rc2;
         }
@@ -514,7 +616,8 @@ static int launch_norm(const void *const *x, const int64_t *sizes, int64_t ntens
       });
   if (rc != OSLO_OK) return rc;
   if (out_global != nullptr) {
-    multi_tensor_norm_global_kernel<MAXNORM><<<dim3(1), 1024, 0, st>>>(partials, total, out_global);
+    multi_tensor_norm_global_kernel<MAXNORM><<<dim3(1), 1024, 0, st>>>(partials, total, out_global, noop,
+                                                                       skip_if_flag);
     return check_launch("multi_tensor_norm_global_kernel");
   }
   return OSLO_OK;
@@ -713,6 +816,94 @@ int oslo_multi_tensor_lamb_stage2(const void *const *update, void *const *p, con
 #undef OSLO_LAMB2
 }
 
+int oslo_multi_tensor_lamb_mp_stage1(void *const *g, const void *const *p, void *const *m,
+                                     void *const *v, const int64_t *sizes, int64_t ntensors,
+                                     float beta1, float beta2, float eps, const int *step,
+                                     int bias_correction, float weight_decay, int grad_averaging,
+                                     int mode, const float *global_grad_norm,
+                                     const float *max_grad_norm, const float *inv_scale,
+                                     const int *noop_flag, int dtype_grad, int dtype_param,
+                                     void *stream) {
+  using namespace oslo;
+  tune_snapshot();
+  if (!valid_dtype(dtype_grad) || !valid_dtype(dtype_param))
+    return fail(OSLO_ERR_INVALID_ARGUMENT, "multi_tensor_lamb_mp_stage1: unknown dtype %d / %d", dtype_grad,
+                dtype_param);
+  OSLO_REQUIRE(ntensors >= 0, "multi_tensor_lamb_mp_stage1: negative tensor count");
+  OSLO_REQUIRE(mode == 0 || mode == 1, "multi_tensor_lamb_mp_stage1: mode %d is neither 0 (L2) nor 1 (decoupled)",
+               mode);
+  OSLO_REQUIRE(dtype_param == dtype_grad || dtype_param == OSLO_DTYPE_F32,
+               "multi_tensor_lamb_mp_stage1: gradients of dtype %d with parameters of dtype %d (the "
+               "parameters must have the gradients' type or be float32)",
+               dtype_grad, dtype_param);
+  if (ntensors == 0) return OSLO_OK;
+  OSLO_REQUIRE(g && p && m && v && sizes && step && global_grad_norm && max_grad_norm && inv_scale,
+               "multi_tensor_lamb_mp_stage1: null pointer");
+  void *const *const lists[4] = {g, const_cast<void *const *>(p), m, v};
+  hipStream_t st = (hipStream_t)stream;
+#define OSLO_LAMB_MP1(TG_, TP_)                                                            \
+  do {                                                                                     \
+    LambMpStage1Op<TG_, TP_> f;                                                            \
+    f.beta1 = beta1; f.beta2 = beta2; f.beta3 = grad_averaging == 1 ? 1.f - beta1 : 1.f;   \
+    f.eps = eps; f.decay = weight_decay; f.mode = mode; f.bias_correction = bias_correction; \
+    f.step = step; f.noop = noop_flag; f.global_grad_norm = global_grad_norm;              \
+    f.max_global_grad_norm = max_grad_norm; f.inv_scale = inv_scale;                       \
+    return mt_apply("multi_tensor_lamb_mp_stage1", lists, sizes, ntensors, f, st);         \
+  } while (0)
+  if (dtype_param == OSLO_DTYPE_F32) {
+    if (dtype_grad == OSLO_DTYPE_F32) OSLO_LAMB_MP1(float, float);
+    if (dtype_grad == OSLO_DTYPE_F16) OSLO_LAMB_MP1(_Float16, float);
+    OSLO_LAMB_MP1(__bf16, float);
+  }
+  if (dtype_param == OSLO_DTYPE_F16) OSLO_LAMB_MP1(_Float16, _Float16);
+  OSLO_LAMB_MP1(__bf16, __bf16);
+#undef OSLO_LAMB_MP1
+}
+
+int oslo_multi_tensor_lamb_mp_stage2(const void *const *update, void *const *p, void *const *p_copy,
+                                     const int64_t *sizes, int64_t ntensors,
+                                     const float *param_norms, const float *update_norms,
+                                     const float *lr, float weight_decay, int use_nvlamb,
+                                     const int *noop_flag, int dtype_update, int dtype_param,
+                                     void *stream) {
+  using namespace oslo;
+  tune_snapshot();
+  if (!valid_dtype(dtype_update) || !valid_dtype(dtype_param))
+    return fail(OSLO_ERR_INVALID_ARGUMENT, "multi_tensor_lamb_mp_stage2: unknown dtype %d / %d",
+                dtype_update, dtype_param);
+  OSLO_REQUIRE(ntensors >= 0, "multi_tensor_lamb_mp_stage2: negative tensor count");
+  const bool copy = p_copy != nullptr;
+  OSLO_REQUIRE(copy ? dtype_param == OSLO_DTYPE_F32 : dtype_param == dtype_update,
+               "multi_tensor_lamb_mp_stage2: update of dtype %d with parameters of dtype %d (one type, or "
+               "float32 parameters with a copy in the update's type)",
+               dtype_update, dtype_param);
+  if (ntensors == 0) return OSLO_OK;
+  OSLO_REQUIRE(update && p && sizes && param_norms && update_norms && lr,
+               "multi_tensor_lamb_mp_stage2: null pointer");
+  hipStream_t st = (hipStream_t)stream;
+#define OSLO_LAMB_MP2(T_, TP_, OUT_)                                                       \
+  do {                                                                                     \
+    LambMpStage2Op<T_, TP_, OUT_> f;                                                       \
+    f.decay = weight_decay; f.use_nvlamb = use_nvlamb; f.lr = lr;                          \
+    f.param_norms = param_norms; f.update_norms = update_norms; f.noop = noop_flag;        \
+    void *const *const lists[OUT_ ? 3 : 2] = {const_cast<void *const *>(update), p OSLO_LAMB_MP2_COPY_##OUT_}; \
+    return mt_apply("multi_tensor_lamb_mp_stage2", lists, sizes, ntensors, f, st);         \
+  } while (0)
+#define OSLO_LAMB_MP2_COPY_true , p_copy
+#define OSLO_LAMB_MP2_COPY_false
+  if (copy) {
+    if (dtype_update == OSLO_DTYPE_F32) OSLO_LAMB_MP2(float, float, true);
+    if (dtype_update == OSLO_DTYPE_F16) OSLO_LAMB_MP2(_Float16, float, true);
+    OSLO_LAMB_MP2(__bf16, float, true);
+  }
+  if (dtype_update == OSLO_DTYPE_F32) OSLO_LAMB_MP2(float, float, false);
+  if (dtype_update == OSLO_DTYPE_F16) OSLO_LAMB_MP2(_Float16, _Float16, false);
+  OSLO_LAMB_MP2(__bf16, __bf16, false);
+#undef OSLO_LAMB_MP2
+#undef OSLO_LAMB_MP2_COPY_true
+#undef OSLO_LAMB_MP2_COPY_false
+}
+
 int64_t oslo_multi_tensor_norm_partials(const int64_t *sizes, int64_t ntensors, int dtype) {
   using namespace oslo;
   if (!valid_dtype(dtype) || ntensors < 0 || (ntensors > 0 && sizes == nullptr)) {
@@ -734,7 +925,7 @@ int64_t oslo_multi_tensor_norm_partials(const int64_t *sizes, int64_t ntensors, 
 int oslo_multi_tensor_norm(const void *const *x, const int64_t *sizes, int64_t ntensors, int dtype,
                            float *partials, int64_t partials_len, float *out_global,
                            float *out_per_tensor, int norm_type, int blend, float alpha, float beta,
-                           int *noop_flag, void *stream) {
+                           int *noop_flag, int skip_if_flag, void *stream) {
   using namespace oslo;
   tune_snapshot();
   if (!valid_dtype(dtype))
@@ -744,13 +935,16 @@ int oslo_multi_tensor_norm(const void *const *x, const int64_t *sizes, int64_t n
                norm_type);
   OSLO_REQUIRE(blend == 0 || out_per_tensor != nullptr, "multi_tensor_norm: blending needs the per-tensor output");
   OSLO_REQUIRE(partials != nullptr && partials_len >= 1, "multi_tensor_norm: no workspace");
+  OSLO_REQUIRE(!skip_if_flag || noop_flag != nullptr, "multi_tensor_norm: skip_if_flag without a flag");
   OSLO_REQUIRE(ntensors == 0 || (x && sizes), "multi_tensor_norm: null table pointer");
   hipStream_t st = (hipStream_t)stream;
 #define OSLO_NORM(T_)                                                                               \
   (norm_type == 0 ? launch_norm<T_, true>(x, sizes, ntensors, partials, partials_len, out_global,   \
-                                          out_per_tensor, blend, alpha, beta, noop_flag, st)        \
+                                          out_per_tensor, blend, alpha, beta, noop_flag,            \
+                                          skip_if_flag, st)                                         \
                   : launch_norm<T_, false>(x, sizes, ntensors, partials, partials_len, out_global,  \
-                                           out_per_tensor, blend, alpha, beta, noop_flag, st))
+                                           out_per_tensor, blend, alpha, beta, noop_flag,           \
+                                           skip_if_flag, st))
   if (dtype == OSLO_DTYPE_F32) return OSLO_NORM(float);
   if (dtype == OSLO_DTYPE_F16) return OSLO_NORM(_Float16);
   return OSLO_NORM(__bf16);

@@ -158,7 +158,15 @@ _SIGNATURES = {
     ),
     "oslo_multi_tensor_norm_partials": (_i64, [_p, _i64, _int]),
     "oslo_multi_tensor_norm": (
-        _int, [_p, _p, _i64, _int, _p, _i64, _p, _p, _int, _int, _f32, _f32, _p, _p],
+        _int, [_p, _p, _i64, _int, _p, _i64, _p, _p, _int, _int, _f32, _f32, _p, _int, _p],
+    ),
+    "oslo_multi_tensor_lamb_mp_stage1": (
+        _int,
+        [_p, _p, _p, _p, _p, _i64, _f32, _f32, _f32, _p, _int, _f32, _int, _int, _p, _p, _p, _p,
+         _int, _int, _p],
+    ),
+    "oslo_multi_tensor_lamb_mp_stage2": (
+        _int, [_p, _p, _p, _p, _i64, _p, _p, _p, _f32, _int, _p, _int, _int, _p],
     ),
     "oslo_rng_from_device": (_int, [_p]),
     "oslo_philox_mask": (_int, [_p, _i64, _f32, _u64, _u64, _p]),
@@ -1156,7 +1164,8 @@ class _L2NormKernel:
     def __init__(self, lib):
         self._lib = lib
 
-    def _run(self, tensors, out_global, out_per_tensor, norm_type, blend, alpha, beta, noop_flag):
+    def _run(self, tensors, out_global, out_per_tensor, norm_type, blend, alpha, beta, noop_flag,
+             skip_if_flag=False):
         lib = self._lib
         tables, sizes, n, ref = _tensor_tables([tensors], ("tensor",))
         code = _dtype_code(ref, "tensors[0]")
@@ -1168,11 +1177,22 @@ class _L2NormKernel:
             rc = lib.oslo_multi_tensor_norm(
                 tables[0], sizes, n, code, _ptr(partials), need, _ptr(out_global),
                 _ptr(out_per_tensor), int(norm_type), int(blend), float(alpha), float(beta),
-                _flag_ptr(noop_flag, ref), _stream(ref),
+                _flag_ptr(noop_flag, ref), int(bool(skip_if_flag)), _stream(ref),
             )
             _check(rc, lib)
 
-    def multi_tensor_l2norm(self, chunk_size, noop_flag, tensor_lists, per_tensor=False):
+    def multi_tensor_l2norm_mp(self, chunk_size, noop_flag, tensor_lists, per_tensor=False):
+        """``multi_tensor_l2norm`` that does nothing while ``noop_flag`` is
+        raised: the results then hold whatever their memory held
+        (``oslo/torch/_C/csrc/FusedMixedPrecisionL2NormBinder.cpp``,
+        ``multi_tensor_l2norm_mp.cu:33-35, 113-115``)."""
+        if noop_flag is None:
+            raise RuntimeError("multi_tensor_l2norm_mp needs the overflow flag")
+        return self.multi_tensor_l2norm(chunk_size, noop_flag, tensor_lists, per_tensor,
+                                        _skip_if_flag=True)
+
+    def multi_tensor_l2norm(self, chunk_size, noop_flag, tensor_lists, per_tensor=False,
+                            _skip_if_flag=False):
         """Returns ``(norm over all tensors [1], norm of each tensor [n] or an
         empty tensor)``, float32.  A sum that is not finite sets ``noop_flag``."""
         if len(tensor_lists) != 1:
@@ -1184,7 +1204,8 @@ class _L2NormKernel:
         ret = torch.empty(1, dtype=torch.float32, device=dev)
         ret_per_tensor = torch.empty(len(tensors) if per_tensor else 0, dtype=torch.float32,
                                      device=dev)
-        self._run(tensors, ret, ret_per_tensor if per_tensor else None, 2, 0, 0.0, 0.0, noop_flag)
+        self._run(tensors, ret, ret_per_tensor if per_tensor else None, 2, 0, 0.0, 0.0, noop_flag,
+                  _skip_if_flag)
         return ret, ret_per_tensor
 
     def multi_tensor_norm_out(self, chunk_size, noop_flag, tensor_lists, out, alpha, beta,
@@ -1282,6 +1303,76 @@ class _LambKernel:
             _check(rc, lib)
 
 
+def _device_scalar(t, name, dtype, ref):
+    """Pointer of a one-element tensor of ``dtype`` on the device of ``ref``."""
+    if not (isinstance(t, torch.Tensor) and t.is_cuda and t.dtype == dtype and t.numel() >= 1
+            and t.device == ref.device):
+        raise RuntimeError("%s must be a %s tensor on %s" % (name, dtype, ref.device))
+    return t.data_ptr()
+
+
+class _LambMpKernel:
+    """``multi_tensor_lamb_mp`` of
+    ``oslo/torch/_C/csrc/FusedMixedPrecisionLambBinder.cpp``."""
+
+    def __init__(self, lib):
+        self._lib = lib
+
+    def multi_tensor_lamb_mp(
+        self, chunk_size, noop_flag, tensor_lists, lr, beta1, beta2, epsilon, step,
+        bias_correction, weight_decay, grad_averaging, mode, global_grad_norm, max_grad_norm,
+        use_nvlamb, found_inf, inv_scale,
+    ):
+        """``tensor_lists`` = ``[grads, params, exp_avgs, exp_avg_sqs]`` of one
+        dtype, or with a fifth list ``[grads, float32 master params, float32
+        exp_avgs, float32 exp_avg_sqs, model params of the gradients' dtype]``
+        (``multi_tensor_lamb_mp.cu:334-337``).  ``lr``, ``step`` (int32),
+        ``global_grad_norm``, ``max_grad_norm`` and ``inv_scale`` are one-element
+        tensors on the GPU; nothing is updated while ``noop_flag`` is raised.
+        ``found_inf`` is accepted as in the reference, whose kernels do not
+        read it either."""
+        lib = self._lib
+        if len(tensor_lists) not in (4, 5):
+            raise RuntimeError("tensor_lists must hold 4 or 5 lists")
+        names = ("grad", "param", "exp_avg", "exp_avg_sq", "model param")
+        gd = tensor_lists[0][0].dtype if len(tensor_lists[0]) else None
+        pd = tensor_lists[1][0].dtype if len(tensor_lists[1]) else None
+        master = len(tensor_lists) == 5
+        dts = [gd, pd, pd, pd] + ([gd] if master else [])
+        tables, sizes, n, ref = _tensor_tables(tensor_lists, names, dts)
+        if n == 0:
+            return
+        if master and pd != torch.float32:
+            raise RuntimeError("with five lists the parameters and moments are float32 master values")
+        if not master and pd != gd:
+            raise RuntimeError("with four lists all tensors share one dtype")
+        flag = _flag_ptr(noop_flag, ref)
+        if flag is None:
+            raise RuntimeError("multi_tensor_lamb_mp needs the overflow flag")
+        gcode, pcode = _dtype_code(tensor_lists[0][0], "grads[0]"), _dtype_code(tensor_lists[1][0], "params[0]")
+        norms = get_l2norm_kernel()
+        _, param_norms = norms.multi_tensor_l2norm_mp(chunk_size, noop_flag, [tensor_lists[1]], True)
+        with _device_of(ref):
+            rc = lib.oslo_multi_tensor_lamb_mp_stage1(
+                tables[0], tables[1], tables[2], tables[3], sizes, n, float(beta1), float(beta2),
+                float(epsilon), _device_scalar(step, "step", torch.int32, ref), int(bias_correction),
+                float(weight_decay), int(grad_averaging), int(mode),
+                _device_scalar(global_grad_norm, "global_grad_norm", torch.float32, ref),
+                _device_scalar(max_grad_norm, "max_grad_norm", torch.float32, ref),
+                _device_scalar(inv_scale, "inv_scale", torch.float32, ref), flag, gcode, pcode,
+                _stream(ref),
+            )
+            _check(rc, lib)
+        _, update_norms = norms.multi_tensor_l2norm_mp(chunk_size, noop_flag, [tensor_lists[0]], True)
+        with _device_of(ref):
+            rc = lib.oslo_multi_tensor_lamb_mp_stage2(
+                tables[0], tables[1], tables[4] if master else None, sizes, n, _ptr(param_norms),
+                _ptr(update_norms), _device_scalar(lr, "lr", torch.float32, ref),
+                float(weight_decay), int(bool(use_nvlamb)), flag, gcode, pcode, _stream(ref),
+            )
+            _check(rc, lib)
+
+
 _optimizer_kernels = {}
 
 
@@ -1314,6 +1405,14 @@ def get_l2norm_kernel():
 
 def get_lamb_kernel():
     return _optimizer_kernel(_LambKernel)
+
+
+def get_l2norm_mp_kernel():
+    return _optimizer_kernel(_L2NormKernel)
+
+
+def get_lamb_mp_kernel():
+    return _optimizer_kernel(_LambMpKernel)
 
 
 def get_fused_elementwise_kernel():

@@ -96,10 +96,10 @@ def test_multi_tensor_entry_points_check_their_arguments():
     assert lib.oslo_multi_tensor_lamb_stage1(one, one, one, one, sizes, 1, 0.9, 0.99, 1e-6, 1, 1, 0.0, 1, 3,
                                              None, 1.0, 0, None) == -1
     assert lib.oslo_multi_tensor_lamb_stage2(one, one, sizes, 1, None, None, 0.1, 0.0, 0, 0, None) == -1
-    assert lib.oslo_multi_tensor_norm(one, sizes, 1, 0, None, 0, None, None, 2, 0, 0.0, 0.0, None, None) == -1
+    assert lib.oslo_multi_tensor_norm(one, sizes, 1, 0, None, 0, None, None, 2, 0, 0.0, 0.0, None, 0, None) == -1
     assert b"no workspace" in lib.oslo_hip_last_error()
-    assert lib.oslo_multi_tensor_norm(one, sizes, 1, 0, one, 1, None, None, 1, 0, 0.0, 0.0, None, None) == -1
-    assert lib.oslo_multi_tensor_norm(one, sizes, 1, 0, one, 1, None, None, 2, 1, 0.5, 0.5, None, None) == -1
+    assert lib.oslo_multi_tensor_norm(one, sizes, 1, 0, one, 1, None, None, 1, 0, 0.0, 0.0, None, 0, None) == -1
+    assert lib.oslo_multi_tensor_norm(one, sizes, 1, 0, one, 1, None, None, 2, 1, 0.5, 0.5, None, 0, None) == -1
     assert b"blending needs" in lib.oslo_hip_last_error()
     # workspace: one value per piece of 16384 float32 / 32768 16-bit elements, at least one
     three = (ctypes.c_int64 * 3)(16384, 16385, 0)

@@ -372,11 +372,12 @@ def test_fused_lamb_follows_the_oracle(device, dtype, wd, max_grad_norm, nvlamb)
         clip = max_grad_norm if max_grad_norm > 0 else float("inf")
         for i, g in enumerate(gs):
             u, m, v = cf.lamb_stage1(f64(g), want_p[i], want_m[i], want_v[i], betas[0], betas[1], eps, step, True,
-                                     wd, True, 1, gn, clip, out=NP_NAME[dtype])
-            # the update direction is what the step left in the gradient
-            p = cf.lamb_stage2(u, want_p[i], np.float32(cf.tensor_norm(want_p[i])), np.float32(cf.tensor_norm(u)),
+                                     wd, True, 1, gn, clip, out=unrounded(dtype))
+            # the update direction is what the step left in the gradient; stage 2 started from it
+            check(ps[i].grad, u, "update[%d] step %d" % (i, step), atol=1e-6, **kw(dtype))
+            ud = f64(ps[i].grad)
+            p = cf.lamb_stage2(ud, want_p[i], np.float32(cf.tensor_norm(want_p[i])), np.float32(cf.tensor_norm(ud)),
                                lr, wd, nvlamb, out=unrounded(dtype))
-            # (a last-place difference in the stored update moves |update| by far less than the tolerance)
             check(ps[i].data, p, "p[%d] step %d" % (i, step), atol=2e-6, **kw(dtype))
             want_p[i] = f64(ps[i])
             want_m[i], want_v[i] = f64(opt.state[ps[i]]["exp_avg"]), f64(opt.state[ps[i]]["exp_avg_sq"])
@@ -384,3 +385,150 @@ def test_fused_lamb_follows_the_oracle(device, dtype, wd, max_grad_norm, nvlamb)
         FusedLamb(ps, amsgrad=True)
     with pytest.raises(RuntimeError):
         FusedLamb(ps, max_coeff=5.0)
+
+
+# ---------------------------------------------------------------------------
+# LAMB with device-resident scalars, an overflow flag and float32 master weights
+# ---------------------------------------------------------------------------
+def _scalars(device, lr, step, max_norm, inv_scale):
+    f = lambda v, dt=torch.float32: torch.tensor([v], dtype=dt, device=device)
+    return f(lr), f(step, torch.int32), f(max_norm), f(inv_scale)
+
+
+@pytest.mark.parametrize("gdtype,master", [(F32, False), (BF16, False), (F16, True), (BF16, True)])
+@pytest.mark.parametrize("mode,wd,nvlamb", [(1, 0.01, False), (0, 0.01, False), (1, 0.0, True)])
+def test_multi_tensor_lamb_mp_vs_oracle(device, gdtype, master, mode, wd, nvlamb):
+    pdtype = F32 if master else gdtype
+    dts = [gdtype, pdtype, pdtype, pdtype] + ([gdtype] if master else [])
+    host, devl = make_lists(dts, 110, device, positive=(3,))
+    k = _C.get_lamb_mp_kernel()
+    b1, b2, eps, step, scale = 0.9, 0.999, 1e-6, 3, 256.0
+    lr, step_t, max_norm, inv_scale = _scalars(device, 0.01, step, 1.0 * scale, 1.0 / scale)
+    flag = torch.zeros(1, dtype=torch.int32, device=device)
+    # the gradients arrive multiplied by the loss scale; so does their norm
+    gn = np.float32(np.sqrt(sum(cf.tensor_norm(f64(t)) ** 2 for t in host[0])))
+    gnorm = torch.tensor([gn], dtype=torch.float32, device=device)
+    found_inf = torch.zeros(1, device=device)
+    k.multi_tensor_lamb_mp(0, flag, devl, lr, b1, b2, eps, step_t, 1, wd, 1, mode, gnorm, max_norm, nvlamb,
+                           found_inf, inv_scale)
+    assert flag.item() == 0
+    for i in CHECKED:
+        if not SIZES[i]:
+            continue
+        u, m, v = cf.lamb_stage1(f64(host[0][i]), f64(host[1][i]), f64(host[2][i]), f64(host[3][i]), b1, b2, eps,
+                                 step, True, wd, True, mode, gn, 1.0 * scale, out=unrounded(pdtype),
+                                 inv_scale=1.0 / scale, out_update=unrounded(gdtype))
+        what = "tensor %d" % i
+        check(devl[0][i], u, "update " + what, atol=1e-6, **kw(gdtype))
+        check(devl[2][i], m, "m " + what, atol=1e-7, **kw(pdtype))
+        check(devl[3][i], v, "v " + what, atol=1e-8, **kw(pdtype))
+        ud = f64(devl[0][i])
+        p = cf.lamb_stage2(ud, f64(host[1][i]), np.float32(cf.tensor_norm(f64(host[1][i]))),
+                           np.float32(cf.tensor_norm(ud)), 0.01, wd, nvlamb, out=unrounded(pdtype))
+        check(devl[1][i], p, "p " + what, atol=1e-6, **kw(pdtype))
+        if master:
+            assert torch.equal(devl[4][i], devl[1][i].to(gdtype)), "model copy " + what
+    # while the flag is raised nothing is touched, not even the gradients
+    before = [[t.clone() for t in lst] for lst in devl]
+    flag.fill_(1)
+    k.multi_tensor_lamb_mp(0, flag, devl, lr, b1, b2, eps, step_t, 1, wd, 1, mode, gnorm, max_norm, nvlamb,
+                           found_inf, inv_scale)
+    for la, lb in zip(before, devl):
+        assert all(torch.equal(a, b) for a, b in zip(la, lb))
+
+
+def test_l2norm_mp_skips_while_the_flag_is_raised(device):
+    k = _C.get_l2norm_mp_kernel()
+    xs = [randn((5000,), F32, 1).to(device), randn((300,), F32, 2).to(device)]
+    flag = torch.zeros(1, dtype=torch.int32, device=device)
+    total, per = k.multi_tensor_l2norm_mp(0, flag, [xs], True)
+    want = [cf.tensor_norm(f64(x)) for x in xs]
+    assert np.allclose(f64(per), want, rtol=2e-6) and np.isclose(total.item(), np.hypot(*want), rtol=2e-6)
+    # a non-finite value raises the flag; the next call leaves its outputs alone
+    xs[0][7] = float("nan")
+    k.multi_tensor_l2norm_mp(0, flag, [xs], True)
+    assert flag.item() == 1
+    lib = _C.load_library()
+    import ctypes
+    out = torch.full((2,), -7.0, device=device)
+    glob = torch.full((1,), -7.0, device=device)
+    part = torch.zeros(8, device=device)
+    arr = (ctypes.c_void_p * 2)(*[x.data_ptr() for x in xs])
+    sizes = (ctypes.c_int64 * 2)(5000, 300)
+    rc = lib.oslo_multi_tensor_norm(arr, sizes, 2, 0, part.data_ptr(), 8, glob.data_ptr(), out.data_ptr(), 2, 0,
+                                    0.0, 0.0, flag.data_ptr(), 1, torch.cuda.current_stream().cuda_stream)
+    assert rc == 0 and (out == -7.0).all() and glob.item() == -7.0
+    with pytest.raises(RuntimeError):
+        k.multi_tensor_l2norm_mp(0, None, [xs], True)
+
+
+@pytest.mark.parametrize("reduced", [None, BF16])
+def test_fused_mixed_precision_lamb_follows_the_oracle(device, reduced):
+    from oslo_amd.torch.optim import FusedMixedPrecisionLamb
+
+    dtype = reduced or F32
+    ps, grads = _param_set(device, dtype)
+    lr, betas, eps, wd, clip = 0.01, (0.9, 0.999), 1e-6, 0.01, 0.5
+    opt = FusedMixedPrecisionLamb(ps, lr=lr, betas=betas, eps=eps, weight_decay=wd, max_grad_norm=clip,
+                                  reduced_precision_dtype=reduced)
+    want_p = [f64(p) for p in ps]
+    want_m = [np.zeros(p.shape) for p in ps]
+    want_v = [np.zeros(p.shape) for p in ps]
+    for step, gs in enumerate(grads, start=1):
+        for p, g in zip(ps, gs):
+            p.grad = g.to(device)
+        opt.step()
+        gn = np.float32(np.sqrt(sum(cf.tensor_norm(f64(g)) ** 2 for g in gs)))
+        for i, g in enumerate(gs):
+            u, m, v = cf.lamb_stage1(f64(g), want_p[i], want_m[i], want_v[i], betas[0], betas[1], eps, step, True,
+                                     wd, True, 1, gn, clip, out="f32", out_update=unrounded(dtype))
+            # the update direction is what the step left in the gradient; stage 2 started from it
+            check(ps[i].grad, u, "update[%d] step %d" % (i, step), atol=1e-6, **kw(dtype))
+            ud = f64(ps[i].grad)
+            p = cf.lamb_stage2(ud, want_p[i], np.float32(cf.tensor_norm(want_p[i])), np.float32(cf.tensor_norm(ud)),
+                               lr, wd, False, out="f32")
+            full = opt.param_groups_full_precision[0]["params"][i]
+            held = full if reduced else ps[i].data
+            check(held, p, "p[%d] step %d" % (i, step), atol=2e-6)
+            if reduced:
+                assert full.dtype == F32 and torch.equal(ps[i].data, full.to(reduced))
+                assert opt.state[ps[i]]["exp_avg"].dtype == F32
+            want_p[i] = f64(held)
+            want_m[i], want_v[i] = f64(opt.state[ps[i]]["exp_avg"]), f64(opt.state[ps[i]]["exp_avg_sq"])
+    assert opt.param_groups[0]["step"].item() == len(grads) and opt.param_groups[0]["step"].is_cuda
+    # the state survives a round trip without being cast to the parameters' dtype
+    sd = opt.state_dict()
+    opt.load_state_dict(sd)
+    assert opt.state[ps[0]]["exp_avg"].dtype == (F32 if reduced else dtype)
+
+
+def test_fused_mixed_precision_lamb_with_a_grad_scaler(device):
+    """Through torch.amp.GradScaler: scaled gradients give the unscaled step, and
+    a step whose gradients overflow changes nothing and is not counted."""
+    from oslo_amd.torch.optim import FusedMixedPrecisionLamb
+
+    def run(scaled):
+        torch.manual_seed(0)
+        model = torch.nn.Linear(48, 32).to(device)
+        opt = FusedMixedPrecisionLamb(model.parameters(), lr=0.01)
+        scaler = torch.amp.GradScaler("cuda", init_scale=1024.0, enabled=scaled)
+        g = torch.Generator(device=device).manual_seed(1)
+        for _ in range(3):
+            x = torch.randn(8, 48, generator=g, device=device)
+            opt.zero_grad()
+            scaler.scale(model(x).square().mean()).backward()
+            scaler.step(opt)
+            scaler.update()
+        return model, opt, scaler
+
+    plain, _, _ = run(False)
+    model, opt, scaler = run(True)
+    for a, b in zip(plain.parameters(), model.parameters()):
+        assert torch.allclose(a, b, rtol=1e-5, atol=1e-6)
+    before = [p.detach().clone() for p in model.parameters()]
+    opt.zero_grad()
+    scaler.scale(model(torch.full((8, 48), float("inf"), device=device)).square().mean()).backward()
+    scaler.step(opt)
+    scaler.update()
+    assert all(torch.equal(a, b) for a, b in zip(before, model.parameters()))
+    assert opt.param_groups[0]["step"].item() == 3 and scaler.get_scale() == 512.0

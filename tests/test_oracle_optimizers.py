@@ -167,3 +167,19 @@ def test_lamb_trust_ratio_clip_and_modes():
     # no gradient averaging: beta3 = 1
     na = cf.lamb_stage1(g, p, m, v, MU, 0.75, 2.0 ** -20, 2, False, 0.0, False, 1, gn, 1e9)
     assert np.allclose(na[1], MU * m + g, rtol=1e-15)
+
+
+def test_lamb_gradient_scale_and_update_type():
+    """The mixed-precision variant multiplies the gradient by the inverse loss
+    scale first and stores the update in the gradients' type."""
+    r = np.random.default_rng(8)
+    g, p = r.standard_normal(64), r.standard_normal(64)
+    m, v = 0.1 * r.standard_normal(64), np.abs(r.standard_normal(64))
+    a = cf.lamb_stage1(1024.0 * g, p, m, v, MU, 0.75, 2.0 ** -20, 2, True, WD, True, 1, 1.0, 1e9,
+                       inv_scale=2.0 ** -10)
+    b = cf.lamb_stage1(g, p, m, v, MU, 0.75, 2.0 ** -20, 2, True, WD, True, 1, 1.0, 1e9)
+    assert all(np.array_equal(x, y) for x, y in zip(a, b))
+    c = cf.lamb_stage1(g, p, m, v, MU, 0.75, 2.0 ** -20, 2, True, WD, True, 1, 1.0, 1e9, out="f32",
+                       out_update="bf16")
+    assert np.array_equal(c[0], cf.round_bf16(b[0].astype(np.float32)))
+    assert np.array_equal(c[1], b[1].astype(np.float32))
