@@ -181,7 +181,8 @@ def test_fused_optimizers_mirror_the_reference_constructors():
     that need no GPU (fused_sgd.py:98-114, fused_novograd.py:86-87)."""
     import oslo_amd.torch.optim as optim
 
-    for name in ("FusedAdam", "FusedAdagrad", "FusedLamb", "FusedNovograd", "FusedSGD"):
+    for name in ("FusedAdam", "FusedAdagrad", "FusedLamb", "FusedMixedPrecisionLamb", "FusedNovograd",
+                 "FusedSGD"):
         assert issubclass(getattr(optim, name), torch.optim.Optimizer)
     w = torch.nn.Parameter(torch.zeros(4))
     sgd = optim.FusedSGD([w], lr=0.1, momentum=0.9, nesterov=True)
