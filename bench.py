@@ -593,10 +593,9 @@ def kernel_table(L, dev, iters, graph_column=True):
             L.ok(lib.oslo_multi_tensor_adam(tables[0], tables[1], tables[2], tables[3], sizes, n, 1e-3, 0.9, 0.999,
                                             1e-8, step_no[0], 1, 1, 0.01, code, L.stream()))
 
-        dname = str(tdt).split(".")[-1]
+        dname = "f32" if tdt == torch.float32 else "bf16"
         opt_iters = max(10, iters // 4)
-        rows.append(table_row("multi_tensor_adam", dname, 7 * nel * esz,
-                              time_launches(torch, adam, opt_iters, 1), note="%d tensors" % n))
+        rows.append(table_row("mt_adam", dname, 7 * nel * esz, time_launches(torch, adam, opt_iters, 1)))
         del lists, tables
         torch.cuda.empty_cache()
 
@@ -613,7 +612,7 @@ def kernel_table(L, dev, iters, graph_column=True):
         def cp(i):
             L.ok(lib.oslo_copy_probe(p(src[i]), p(dst[i]), nbytes, L.stream()))
 
-        rows.append(table_row("copy_probe", "-", 2 * nbytes, timed(cp, ns), note="plain copy, read + write"))
+        rows.append(table_row("copy_probe", "-", 2 * nbytes, timed(cp, ns)))
         del src, dst
         torch.cuda.empty_cache()
 
@@ -625,7 +624,7 @@ def kernel_table(L, dev, iters, graph_column=True):
     for tdt, code, esz in ((torch.float32, F32, 4), (torch.bfloat16, BF16, 2)):
         lists, tables, sizes, n, nel = optimizer_tensors(tdt)
         step_no = [0]
-        dname = str(tdt).split(".")[-1]
+        dname = "f32" if tdt == torch.float32 else "bf16"
         opt_iters = max(10, iters // 4)
         need = int(lib.oslo_multi_tensor_norm_partials(sizes, n, code))
         partials = torch.empty(need, dtype=torch.float32, device=dev)
@@ -663,14 +662,12 @@ def kernel_table(L, dev, iters, graph_column=True):
             L.ok(lib.oslo_multi_tensor_lamb_stage2(tables[0], tables[1], sizes, n, p(norms), p(norms2), 1e-3, 0.01,
                                                    0, code, L.stream()))
 
-        for name, fn, values in (("multi_tensor_sgd", sgd, 5), ("multi_tensor_adagrad", adagrad, 5),
-                                 ("multi_tensor_l2norm", l2norm, 1), ("multi_tensor_novograd", novograd, 6),
-                                 ("multi_tensor_lamb", lamb, 12)):
+        for name, fn, values in (("mt_sgd", sgd, 5), ("mt_adagrad", adagrad, 5), ("mt_l2norm", l2norm, 1),
+                                 ("mt_novograd", novograd, 6), ("mt_lamb", lamb, 12)):
             if fn is lamb:  # stage 1 overwrites the gradients: start every timing from fresh ones
                 for t in lists[0]:
                     t.normal_()
-            rows.append(table_row(name, dname, values * nel * esz, time_launches(torch, fn, opt_iters, 1),
-                                  note="%d tensors" % n))
+            rows.append(table_row(name, dname, values * nel * esz, time_launches(torch, fn, opt_iters, 1)))
         del lists, tables, partials
         torch.cuda.empty_cache()
     return rows
@@ -1001,7 +998,8 @@ def main():
             "cols": TABLE_COLS,
             "units": "MB = algorithmic bytes per launch / 1e6; us = mean over %d launches (events on the launch "
                      "stream, %d batches), us_med / us_min = median / smallest batch mean; frac = GBps / 8000; "
-                     "graph_us = per launch inside a captured HIP graph" % (args.table_iters, BATCHES),
+                     "graph_us = per launch inside a captured HIP graph; mt_* = multi-tensor optimizer steps over "
+                     "192 tensors; copy_probe = a plain copy" % (args.table_iters, BATCHES),
             "rows": rows,
         }
     if not args.no_cpu_baseline:
