@@ -553,7 +553,8 @@ int oslo_wave_reduce_selftest(float *out4, void *stream);
  * tiles), "adam_unroll";
  * value 0 restores the default.  Other values must be ones the launch code
  * has a kernel build and a valid workgroup shape for, else
- * OSLO_ERR_INVALID_ARGUMENT: chunks per lane (*_vpl: 1, 2, 4, forward also 8),
+ * OSLO_ERR_INVALID_ARGUMENT: chunks per lane (*_vpl: 1, 2, 4, forward also 8,
+ * and 3 for LayerNorm),
  * waves per workgroup 1..16, norm_bwd_prefetch 1 or 2, norm_fwd_iters 1..16,
  * norm_bwd_blocks_per_cu 1..8, lanes per row 8, 16, 32 or 64 (softmax also
  * 1), softmax_rows_per_wave and the unroll factors 1, 2 or 4 (eltwise_unroll

@@ -95,7 +95,7 @@ int oslo_tune(const char *key, int value) {
     return oslo::fail(OSLO_ERR_INVALID_ARGUMENT, "tune: bad arguments");
   // 0 restores the built-in choice; any other value must be one the launch
   // code has a kernel build and a valid workgroup shape for
-  enum Kind { kPow2, kRange, kLanes };
+  enum Kind { kPow2, kRange, kLanes, kPow2or3 };
   struct Entry {
     const char *name;
     int *slot;
@@ -105,7 +105,7 @@ int oslo_tune(const char *key, int value) {
   std::lock_guard<std::mutex> guard(oslo::s_tune_lock);
   oslo::Tuning &shared = oslo::s_tune_shared;
   const Entry table[] = {
-      {"norm_fwd_vpl", &shared.norm_fwd_vpl, kPow2, 1, 8},
+      {"norm_fwd_vpl", &shared.norm_fwd_vpl, kPow2or3, 1, 8},
       {"norm_bwd_vpl", &shared.norm_bwd_vpl, kPow2, 1, 4},
       {"norm_bwd_blocks_per_cu", &shared.norm_bwd_blocks_per_cu, kRange, 1, 8},
       {"softmax_rows_per_wave", &shared.softmax_rows_per_wave, kPow2, 1, 4},
@@ -129,7 +129,7 @@ int oslo_tune(const char *key, int value) {
       bool ok = value == 0;
       if (!ok && value >= e.lo && value <= e.hi) {
         const bool pow2 = (value & (value - 1)) == 0;
-        ok = e.kind == kRange || (e.kind == kPow2 && pow2) ||
+        ok = e.kind == kRange || (e.kind == kPow2 && pow2) || (e.kind == kPow2or3 && (pow2 || value == 3)) ||
              (e.kind == kLanes && (value == 1 || (pow2 && value >= 8)));
       }
       if (!ok)

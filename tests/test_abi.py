@@ -58,7 +58,7 @@ def test_invalid_arguments_are_rejected_before_any_launch():
     assert lib.oslo_tune(b"no_such_knob", 1) == -1
     assert lib.oslo_tune(b"norm_fwd_vpl", 0) == 0
     # values without a kernel build or a valid workgroup shape are refused
-    for key, bad in ((b"norm_fwd_vpl", 3), (b"norm_bwd_vpl", 8), (b"norm_fwd_waves", 17),
+    for key, bad in ((b"norm_fwd_vpl", 5), (b"norm_bwd_vpl", 8), (b"norm_fwd_waves", 17),
                      (b"norm_bwd_prefetch", 3), (b"softmax_rows_per_wave", 3),
                      (b"softmax_lanes_per_row", 4), (b"norm_lanes_per_row", 1),
                      (b"softmax_fwd_elems", 4), (b"eltwise_tile_max", 100),

@@ -21,7 +21,7 @@ KEYS = [
 ]
 
 OVERRIDES = [
-    ("norm_fwd_vpl", 1), ("norm_fwd_vpl", 2), ("norm_fwd_vpl", 4), ("norm_fwd_vpl", 8),
+    ("norm_fwd_vpl", 1), ("norm_fwd_vpl", 2), ("norm_fwd_vpl", 3), ("norm_fwd_vpl", 4), ("norm_fwd_vpl", 8),
     ("norm_fwd_waves", 8), ("norm_fwd_waves", 16),
     ("norm_fwd_iters", 1), ("norm_fwd_iters", 4),
     ("norm_bwd_vpl", 1), ("norm_bwd_vpl", 2),
