@@ -1032,18 +1032,24 @@ def _tensor_tables(tensor_lists, names, dtypes=None):
     if n == 0:
         return None, None, 0, None
     ref = tensor_lists[0][0]
+    device = ref.device
+    counts = [t.numel() for t in tensor_lists[0]]
     for k, lst in enumerate(tensor_lists):
         want = lst[0].dtype if dtypes is None or dtypes[k] is None else dtypes[k]
+        # one pass per list; the slow loop below only runs to name the offender
+        if all(t.is_cuda and t.dtype == want and t.device == device and t.is_contiguous() for t in lst):
+            if k == 0 or [t.numel() for t in lst] == counts:
+                continue
         for i, t in enumerate(lst):
             _check_input(t, "%s %d" % (names[k], i))
-            if t.dtype != want or t.device != ref.device:
+            if t.dtype != want or t.device != device:
                 raise RuntimeError(
                     "A tensor was not the same dtype / on the same device as the first tensor"
                 )
-            if t.numel() != tensor_lists[0][i].numel():
+            if t.numel() != counts[i]:
                 raise RuntimeError("Size mismatch among tensor lists")
     arr = ctypes.c_void_p * n
-    sizes = (ctypes.c_int64 * n)(*[t.numel() for t in tensor_lists[0]])
+    sizes = (ctypes.c_int64 * n)(*counts)
     tables = [arr(*[t.data_ptr() for t in lst]) for lst in tensor_lists]
     return tables, sizes, n, ref
 

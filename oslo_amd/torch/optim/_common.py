@@ -2,9 +2,7 @@
 ``zero_grad`` of the reference's classes."""
 import torch
 
-from oslo_amd.torch.utils.multi_tensor_apply import MultiTensorApply
-
-multi_tensor_applier = MultiTensorApply(2048 * 32)
+from oslo_amd.torch.utils.multi_tensor_apply import multi_tensor_applier  # noqa: F401  (re-exported)
 
 KERNEL_DTYPES = (torch.float16, torch.bfloat16, torch.float32)
 

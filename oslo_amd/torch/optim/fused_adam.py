@@ -11,9 +11,7 @@ dtype bucket, ``:150-182``, which double-counts a group that mixes dtypes).
 import torch
 
 from oslo_amd.torch._C import get_adam_kernel
-from oslo_amd.torch.utils.multi_tensor_apply import MultiTensorApply
-
-multi_tensor_applier = MultiTensorApply(2048 * 32)
+from oslo_amd.torch.utils.multi_tensor_apply import multi_tensor_applier
 
 
 class FusedAdam(torch.optim.Optimizer):
