@@ -24,6 +24,10 @@ from oslo_amd.torch.optim._common import ZeroGradMixin, checked_params, multi_te
 class FusedLamb(ZeroGradMixin, torch.optim.Optimizer):
     """Implements the LAMB algorithm on the GPU.
 
+    ``step()`` leaves the update direction in each parameter's ``.grad`` (the
+    kernel works in place, ``multi_tensor_lamb.cu:313-317``): read the gradients
+    before the step, not after.
+
     Arguments:
         params (iterable): iterable of parameters to optimize or dicts defining
             parameter groups.

@@ -197,3 +197,54 @@ def test_reseeding_keeps_the_state_tensor_that_captured_graphs_hold(device):
     assert np.array_equal((out != 0).cpu().numpy(), keep), "replay after re-seeding: mask differs from the oracle"
     assert int(state.cpu()[1]) == offset + 4
     assert all(int(j.cpu()[0]) == -1 for j in junk), "a replay wrote outside the state tensor"
+
+
+def test_captured_mixed_precision_lamb_step_counts_and_replays(device):
+    """FusedMixedPrecisionLamb keeps its step count, learning rate and loss scale
+    on the device, so a captured step is a whole optimizer step: every replay
+    advances the count and gives what the eager optimizer gives."""
+    from oslo_amd.torch.optim import FusedMixedPrecisionLamb
+
+    shapes = [(64, 48), (48,), (1000,)]
+
+    def make():
+        ps = [torch.nn.Parameter(randn(s, torch.float32, 20 + i).to(device)) for i, s in enumerate(shapes)]
+        for p in ps:
+            p.grad = torch.zeros_like(p)
+        return ps, FusedMixedPrecisionLamb(ps, lr=0.01, weight_decay=0.01, max_grad_norm=1.0)
+
+    grads = [[randn(s, torch.float32, 40 + 10 * k + i).to(device) for i, s in enumerate(shapes)] for k in range(4)]
+
+    def load(ps, k):
+        # the step leaves its update direction in the gradients: refill them every time
+        for p, g in zip(ps, grads[k]):
+            p.grad.copy_(g)
+
+    eager_ps, eager = make()
+    graph_ps, captured = make()
+    # first step eagerly on both (it creates the moments), on a side stream as capture wants
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        load(eager_ps, 0)
+        eager.step()
+        load(graph_ps, 0)
+        captured.step()
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    load(graph_ps, 1)
+    with torch.cuda.graph(graph):
+        captured.step()
+    # (capture does not execute: the step count has not moved yet)
+    assert captured.param_groups[0]["step"].item() == 1
+    for k in (1, 2, 3):
+        load(eager_ps, k)
+        eager.step()
+        load(graph_ps, k)
+        graph.replay()
+        scratch = torch.randn(1 << 16, device=device).sum()  # eager work between the replays
+        torch.cuda.synchronize()
+        assert scratch.isfinite()
+        assert captured.param_groups[0]["step"].item() == k + 1 == eager.param_groups[0]["step"].item()
+        for a, b in zip(eager_ps, graph_ps):
+            assert torch.equal(a, b), "replay %d" % k
