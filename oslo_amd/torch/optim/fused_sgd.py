@@ -93,9 +93,10 @@ class FusedSGD(ZeroGradMixin, torch.optim.Optimizer):
         for group in self.param_groups:
             # one launch set per (dtype, device, first run or not)
             buckets = {}
+            use_momentum = group["momentum"] != 0
             for p in checked_params(group, "FusedSGD"):
                 state = self.state[p]
-                first_run = "momentum_buffer" not in state
+                first_run = use_momentum and "momentum_buffer" not in state
                 if first_run:
                     state["momentum_buffer"] = torch.zeros_like(
                         p.data, memory_format=torch.contiguous_format
@@ -103,7 +104,10 @@ class FusedSGD(ZeroGradMixin, torch.optim.Optimizer):
                 g, w, m = buckets.setdefault((p.dtype, p.device, first_run), ([], [], []))
                 g.append(p.grad.data.contiguous())
                 w.append(p.data)
-                m.append(state["momentum_buffer"])
+                # without momentum the kernel neither reads nor writes the third
+                # list: the weight stands in, and no buffer is allocated (the
+                # reference allocates one per parameter regardless, :133-149)
+                m.append(state["momentum_buffer"] if use_momentum else p.data)
             for (_, _, first_run), lists in buckets.items():
                 multi_tensor_applier(
                     self.multi_tensor_sgd,

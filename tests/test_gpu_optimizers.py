@@ -268,6 +268,8 @@ def test_fused_sgd_tracks_torch_optim(device, kwargs):
         for pa, pb in zip(a.parameters(), b.parameters()):
             assert torch.allclose(oa.state[pa]["momentum_buffer"], ob.state[pb]["momentum_buffer"],
                                   rtol=1e-5, atol=1e-7)
+    if not kwargs.get("momentum"):
+        assert all("momentum_buffer" not in oa.state[p] for p in a.parameters())  # nothing allocated
     with pytest.raises(ValueError):
         FusedSGD(a.parameters(), lr=0.1, nesterov=True)
     with pytest.raises(ValueError):
