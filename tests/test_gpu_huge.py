@@ -250,3 +250,28 @@ def test_adam_on_a_tensor_beyond_2_31_elements(device):
         check(p[sl], want[0], "huge adam p", atol=5e-7, min_exact=0.99)
         check(m[sl], want[1], "huge adam m", atol=1e-7, min_exact=0.99)
         check(v[sl], want[2], "huge adam v", atol=1e-8, min_exact=0.99)
+
+
+def test_optimizer_family_on_a_tensor_beyond_2_31_elements(device):
+    """The generic multi-tensor kernel (here: SGD with momentum, next to a short
+    tensor in the same launch) and the norm kernels index with 64-bit offsets."""
+    n = 2 ** 31 + 4099
+    g = torch.empty(n, device=device, dtype=BF16).normal_()
+    w = torch.empty(n, device=device, dtype=BF16).normal_()
+    mom = torch.empty(n, device=device, dtype=BF16).normal_()
+    small = [torch.ones(100, device=device, dtype=BF16) for _ in range(3)]
+    tail, head = slice(n - 5000, n), slice(0, 5000)
+    before = [(f64(g[s]), f64(w[s]), f64(mom[s])) for s in (head, tail)]
+    # the norm first (it reads the gradients the step leaves alone): against torch in float64 on slices
+    total, per = _C.get_l2norm_kernel().multi_tensor_l2norm(0, None, [[g, small[0]]], True)
+    sumsq = sum(float(g[i:i + (1 << 28)].double().square().sum()) for i in range(0, n, 1 << 28))
+    assert np.isclose(per[0].item(), np.sqrt(sumsq), rtol=1e-5) and np.isclose(per[1].item(), 10.0, rtol=1e-6)
+    assert np.isclose(total.item(), np.sqrt(sumsq + 100.0), rtol=1e-5)
+    _C.get_sgd_kernel().multi_tensor_sgd(0, None, [[g, small[0]], [w, small[1]], [mom, small[2]]],
+                                         0.01, 0.9, 0.0, 0.05, False, False, False, 1.0)
+    for s, (gg, ww, mm) in zip((head, tail), before):
+        want_w, want_m, _ = cf.sgd_step(gg, ww, mm, 0.05, 0.01, 0.9, 0.0, False, False)
+        check(w[s], want_w, "huge sgd w", atol=1e-6, min_exact=0.95, single_rounding_too=True)
+        check(mom[s], want_m, "huge sgd momentum", atol=1e-6, min_exact=0.95, single_rounding_too=True)
+    # g = w = mom = 1: mom' = 0.9 + (1 + 0.01) = 1.91, w' = 1 - 0.05 * 1.91
+    assert torch.equal(small[2], torch.full_like(small[2], 1.91)) and torch.equal(small[1], torch.full_like(small[1], 0.9045))
