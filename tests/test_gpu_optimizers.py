@@ -2,6 +2,8 @@
 through the C ABI, against the float64 oracle (oracle/closed_form.py, pinned by
 test_oracle_optimizers.py): fp32 to 1e-5 relative, 16-bit results against the
 oracle rounded once to the storage type."""
+import os
+
 import numpy as np
 import pytest
 import torch
@@ -534,3 +536,111 @@ def test_fused_mixed_precision_lamb_with_a_grad_scaler(device):
     scaler.update()
     assert all(torch.equal(a, b) for a, b in zip(before, model.parameters()))
     assert opt.param_groups[0]["step"].item() == 3 and scaler.get_scale() == 512.0
+
+
+# ---------------------------------------------------------------------------
+# random lists: tensor counts across the launch boundary, lengths around every
+# piece boundary, views at odd offsets of one buffer, every step and dtype
+# ---------------------------------------------------------------------------
+def _random_cases(count, seed):
+    r = np.random.default_rng(seed)
+    cases = []
+    for i in range(count):
+        nt = int(r.choice([1, 2, 5, 47, 48, 49, 97, 130]))
+        special = [0, 1, 4095, 4096, 4097, 8191, 8192, 8193, 16384, 32768, 32769]
+        sizes = [int(r.choice(special)) if r.random() < 0.3 else int(r.integers(1, 20000)) for _ in range(nt)]
+        cases.append((i, str(r.choice(["sgd", "adagrad", "novograd", "lamb"])), int(r.integers(0, 3)), sizes,
+                      bool(r.integers(0, 2)), int(r.integers(0, 1 << 30))))
+    return cases
+
+
+# OSLO_FUZZ_SEED / OSLO_FUZZ_COUNT draw other and longer sweeps, as in test_gpu_random_shapes.py
+@pytest.mark.parametrize("i,op,dt,sizes,views,seed",
+                         _random_cases(int(os.environ.get("OSLO_FUZZ_COUNT", "48")),
+                                       2024 + int(os.environ.get("OSLO_FUZZ_SEED", "0"))))
+def test_random_tensor_lists(device, i, op, dt, sizes, views, seed):
+    dtype = (F32, F16, BF16)[dt]
+    nlists = {"sgd": 3, "adagrad": 3, "novograd": 3, "lamb": 4}[op]
+    g = torch.Generator().manual_seed(seed)
+    host, devl = [], []
+    for k in range(nlists):
+        positive = (op == "adagrad" and k == 2) or (op == "lamb" and k == 3)
+        if views:
+            # every tensor is a view into one buffer, at an offset that is odd for most of them
+            offs = np.cumsum([3] + [n + 1 + (j % 3) for j, n in enumerate(sizes)])
+            buf = torch.randn(int(offs[-1]) + 8, generator=g)
+            buf = (buf.abs() * 0.1 if positive else buf).to(dtype)
+            dbuf = buf.to(device)
+            host.append([buf[o:o + n] for o, n in zip(offs[:-1], sizes)])
+            devl.append([dbuf[o:o + n] for o, n in zip(offs[:-1], sizes)])
+        else:
+            lst = [torch.randn(n, generator=g) for n in sizes]
+            lst = [(t.abs() * 0.1 if positive else t).to(dtype) for t in lst]
+            host.append(lst)
+            devl.append([t.to(device) for t in lst])
+    r = np.random.default_rng(seed)
+    lr, wd = float(r.choice([0.01, 0.1])), float(r.choice([0.0, 0.01]))
+    picks = sorted(set([0, len(sizes) - 1] + [int(j) for j in r.integers(0, len(sizes), size=6)]))
+    out = unrounded(dtype)
+    k16 = dict(kw(dtype), min_exact=0.95) if dtype != F32 else {}
+    if op == "sgd":
+        mu, nest, first = float(r.choice([0.0, 0.9])), bool(r.integers(0, 2)), bool(r.integers(0, 2))
+        nest = nest and mu > 0
+        _C.get_sgd_kernel().multi_tensor_sgd(0, None, devl, wd, mu, 0.0, lr, nest, first, False, 1.0)
+        for j in picks:
+            w, m, _ = cf.sgd_step(f64(host[0][j]), f64(host[1][j]), f64(host[2][j]), lr, wd, mu, 0.0, nest, first, out=out)
+            if sizes[j]:
+                check(devl[1][j], w, "sgd w %d" % j, atol=1e-6, **k16)
+                if mu:
+                    check(devl[2][j], m, "sgd mom %d" % j, atol=1e-6, **k16)
+    elif op == "adagrad":
+        mode = int(r.integers(0, 2))
+        _C.get_adagrad_kernel().multi_tensor_adagrad(0, None, devl, lr, 1e-10, mode, wd)
+        for j in picks:
+            p, h = cf.adagrad_step(f64(host[0][j]), f64(host[1][j]), f64(host[2][j]), lr, 1e-10, mode, wd, out=out)
+            if sizes[j]:
+                check(devl[1][j], p, "adagrad p %d" % j, atol=1e-6, **k16)
+                check(devl[2][j], h, "adagrad h %d" % j, atol=1e-7, **k16)
+    elif op == "novograd":
+        mode, ntype, step = int(r.integers(0, 2)), int(r.choice([0, 2])), int(r.integers(1, 9))
+        old = torch.rand(len(sizes), generator=g) + 0.5
+        norms = old.to(device)
+        _C.get_novograd_kernel().multi_tensor_novograd(0, None, devl, norms, lr, 0.95, 0.98, 1e-8, step, 1, wd, 1,
+                                                       mode, ntype)
+        got = f64(norms)
+        for j in picks:
+            n = cf.blend_norm(old[j].item(), f64(host[0][j]), 0.98, 1.0 - 0.98, ntype)
+            assert np.isclose(got[j], n, rtol=3e-6), "novograd norm %d" % j
+            p, m = cf.novograd_step(f64(host[0][j]), f64(host[1][j]), f64(host[2][j]), got[j], lr, 0.95, 0.98, 1e-8,
+                                    step, True, wd, True, mode, out=out)
+            if sizes[j]:
+                check(devl[1][j], p, "novograd p %d" % j, atol=1e-6, **k16)
+                check(devl[2][j], m, "novograd m %d" % j, atol=1e-6, **k16)
+    else:
+        mode, nv, step = int(r.integers(0, 2)), bool(r.integers(0, 2)), int(r.integers(1, 9))
+        clip = float(r.choice([1.0, 1e9]))
+        gn = np.float32(np.sqrt(sum(cf.tensor_norm(f64(t)) ** 2 for t in host[0])))
+        gnorm = torch.tensor([gn], dtype=torch.float32, device=device)
+        _C.get_lamb_kernel().multi_tensor_lamb(0, None, devl, lr, 0.9, 0.999, 1e-6, step, 1, wd, 1, mode, gnorm, clip, nv)
+        for j in picks:
+            if not sizes[j]:
+                continue
+            u, m, v = cf.lamb_stage1(f64(host[0][j]), f64(host[1][j]), f64(host[2][j]), f64(host[3][j]), 0.9, 0.999,
+                                     1e-6, step, True, wd, True, mode, gn, clip, out=out)
+            check(devl[0][j], u, "lamb update %d" % j, atol=1e-6, **k16)
+            check(devl[2][j], m, "lamb m %d" % j, atol=1e-7, **k16)
+            check(devl[3][j], v, "lamb v %d" % j, atol=1e-8, **k16)
+            ud = f64(devl[0][j])
+            p = cf.lamb_stage2(ud, f64(host[1][j]), np.float32(cf.tensor_norm(f64(host[1][j]))),
+                               np.float32(cf.tensor_norm(ud)), lr, wd, nv, out=out)
+            check(devl[1][j], p, "lamb p %d" % j, atol=2e-6, **k16)
+    if views:
+        # the gaps between the views are untouched
+        for k in range(1, nlists):
+            full_h = host[k][0]._base if host[k][0]._base is not None else None
+            full_d = devl[k][0]._base
+            if full_h is None or full_d is None:
+                continue
+            offs = np.cumsum([3] + [n + 1 + (j % 3) for j, n in enumerate(sizes)])
+            gaps = torch.tensor([int(o) - 1 for o in offs])
+            assert torch.equal(full_d[gaps.to(device)].cpu(), full_h[gaps]), "gap after list %d" % k
