@@ -260,6 +260,77 @@ int oslo_softmax_causal_masked_dropout_bwd(const void *dout, const void *x,
                                            uint64_t seed, uint64_t offset,
                                            int dtype, void *stream);
 
+/* ---- softmax with an additive floating-point term ------------------------ *
+ * y = softmax(scale * x + M) -- the form in which the reference's models
+ * mask and bias their scores: `attention_scores + attention_mask` with the
+ * [b, 1, 1, sk] term (1 - m) * -10000
+ * (oslo/transformers/models/bert/modeling_bert.py:298-306,
+ * oslo/transformers/models/gpt2/modeling_gpt2.py:136 with the mask built at
+ * :573-581), the finfo.min fill of
+ * oslo/transformers/models/bart/modeling_bart.py:123-136, 262-284, the
+ * relative-position bias [1, np, sq, sk] of
+ * oslo/transformers/models/t5/modeling_t5.py:508-514, and LightSeq's additive
+ * [batch, to_len] mask (oslo/lightseq2/csrc/kernels/cuda/softmax_kernels.cu:
+ * 35-127).  The reference has no fused entry point for it.
+ *
+ * x, y are [b, np, sq, sk].  M ("bias") has the dtype bias_dtype = dtype or
+ * OSLO_DTYPE_F32 and is addressed as
+ *   M[bi * bias_stride_b + hi * bias_stride_h + qi * bias_stride_q + key]
+ * (strides in elements, 0 = that dimension is broadcast; keys contiguous).
+ * The sum is one fused multiply-add in float, so the additive semantics are
+ * those of a float evaluation of the unfused chain: a row whose terms are all
+ * -10000 gives softmax(scale * x), a row whose terms are all the lowest
+ * finite value gives the uniform distribution (the term absorbs the logit),
+ * a row whose terms are all -inf gives NaN, as torch.softmax does.
+ * flags: OSLO_SOFTMAX_CAUSAL hides key j of query i when j > i + (sk - sq)
+ * as well (exact zeros, also in a query row that the diagonal leaves without
+ * any key when sq > sk; neither x nor M is read there);
+ * OSLO_SOFTMAX_SKIP_HIDDEN reads M first and leaves the logits of a 16-byte
+ * chunk unread when every term of it is at or below the lowest finite
+ * bfloat16 (-3.39e38; the lowest float and -inf are), where the float sum is
+ * the term itself whatever the logit (below 1e30 in magnitude): worth it
+ * when M is small (a broadcast mask), not for a dense bias.
+ * The backward pass is that of every softmax,
+ *   dx = scale * y * (dy - sum_j dy_j y_j),
+ * and takes M (may be NULL) only to skip loads under the same flag: y is
+ * exactly 0 where the term absorbs the logit, unless the whole row is like
+ * that (such rows are read in full).  dx may alias dy.  The gradient with
+ * respect to M is dx / scale summed over the broadcast dimensions; it is left
+ * to the caller.                                                            */
+#define OSLO_SOFTMAX_CAUSAL 1
+#define OSLO_SOFTMAX_SKIP_HIDDEN 2
+int oslo_softmax_bias_fwd(const void *x, const void *bias, void *y, int64_t b,
+                          int64_t np, int64_t sq, int64_t sk,
+                          int64_t bias_stride_b, int64_t bias_stride_h,
+                          int64_t bias_stride_q, int bias_dtype, int flags,
+                          float scale, int dtype, void *stream);
+int oslo_softmax_bias_bwd(const void *dy, const void *y, const void *bias,
+                          void *dx, int64_t b, int64_t np, int64_t sq,
+                          int64_t sk, int64_t bias_stride_b,
+                          int64_t bias_stride_h, int64_t bias_stride_q,
+                          int bias_dtype, int flags, float scale, int dtype,
+                          void *stream);
+
+/* The same with the attention-probability dropout fused in (see the dropout
+ * entry points above): stats is float [rows][2] = {max_j (scale * x_j + M_j),
+ * 1 / sum_j exp(scale * x_j + M_j - max)}; the backward pass takes x, M and
+ * stats and recomputes the probabilities.                                   */
+int oslo_softmax_bias_dropout_fwd(const void *x, const void *bias, void *out,
+                                  float *stats, int64_t b, int64_t np,
+                                  int64_t sq, int64_t sk, int64_t bias_stride_b,
+                                  int64_t bias_stride_h, int64_t bias_stride_q,
+                                  int bias_dtype, int flags, float scale,
+                                  float p, uint64_t seed, uint64_t offset,
+                                  int dtype, void *stream);
+int oslo_softmax_bias_dropout_bwd(const void *dout, const void *x,
+                                  const void *bias, const float *stats,
+                                  void *dx, int64_t b, int64_t np, int64_t sq,
+                                  int64_t sk, int64_t bias_stride_b,
+                                  int64_t bias_stride_h, int64_t bias_stride_q,
+                                  int bias_dtype, int flags, float scale,
+                                  float p, uint64_t seed, uint64_t offset,
+                                  int dtype, void *stream);
+
 /* ---- dropout state in device memory ------------------------------------- *
  * No counterpart in the reference.  For callers that capture launches in a
  * HIP graph: a (seed, offset) pair passed by value is frozen into the graph

@@ -153,6 +153,57 @@ def softmax_dropout_bwd(dout, x, hidden, scale, keep, p, out="f64", acc=np.float
     return round_to(acc(scale) * (y * (dp - s)), out)
 
 
+def softmax_bias_fwd(x, bias, scale, causal=False, out="f64", acc=np.float64, sum_f32=True):
+    """y = softmax(scale * x + bias): the scores with an additive term, which
+    is how the reference's models mask and bias them
+    (oslo/transformers/models/bert/modeling_bert.py:298-306: scores / sqrt(d) +
+    attention_mask; modeling_gpt2.py:136 with the (1 - m) * -10000 mask of
+    :573-581; the finfo.min fill of models/bart/modeling_bart.py:123-136,
+    262-284; the position bias of models/t5/modeling_t5.py:508-514).
+
+    `bias` broadcasts against `x`.  With `sum_f32` the sum is rounded to
+    float32 once (the fused kernel forms it by one float multiply-add), so
+    that a term of -10000 costs the logit the same bits here and there and
+    the lowest finite float absorbs the logit altogether; without it the
+    function is the plain float64 softmax of the sum.  `causal` hides key j of
+    query i for j > i + (sk - sq) (probability exactly 0).  A row of -inf
+    sums is NaN, as torch.softmax returns it.
+    """
+    x = np.asarray(x, dtype=acc)
+    with np.errstate(over="ignore", invalid="ignore"):
+        t = x * acc(scale) + np.broadcast_to(np.asarray(bias, dtype=acc), x.shape)
+        if sum_f32:
+            t = t.astype(np.float32).astype(acc)
+    if causal:
+        t = np.where(causal_hidden(x.shape[-2], x.shape[-1]), -np.inf, t)
+    with np.errstate(invalid="ignore"):
+        m = t.max(axis=-1, keepdims=True)
+        e = np.exp(t - m)  # (-inf) - (-inf) = NaN for a row without a finite sum
+        y = e / e.sum(axis=-1, keepdims=True)
+    return round_to(y, out)
+
+
+def softmax_bias_dropout_fwd(x, bias, scale, keep, p, causal=False, out="f64", acc=np.float64):
+    """out = keep * softmax(scale * x + bias) / (1 - p), rounded once."""
+    y = softmax_bias_fwd(x, bias, scale, causal, "f64", acc)
+    if keep is not None:
+        y = np.where(np.asarray(keep, dtype=bool), y * _dropout_scale(p, acc), 0.0)
+    return round_to(y, out)
+
+
+def softmax_bias_dropout_bwd(dout, x, bias, scale, keep, p, causal=False, out="f64",
+                             acc=np.float64):
+    """dx of out = dropout(softmax(scale * x + bias)) given d(out); the
+    gradient of the additive term is dx / scale summed over the dimensions it
+    broadcasts along."""
+    y = softmax_bias_fwd(x, bias, scale, causal, "f64", acc)
+    dp = np.asarray(dout, dtype=acc)
+    if keep is not None:
+        dp = np.where(np.asarray(keep, dtype=bool), dp * _dropout_scale(p, acc), 0.0)
+    s = (dp * y).sum(axis=-1, keepdims=True)
+    return round_to(acc(scale) * (y * (dp - s)), out)
+
+
 # ---------------------------------------------------------------------------
 # LayerNorm / RMSNorm
 # ---------------------------------------------------------------------------

@@ -114,6 +114,24 @@ _SIGNATURES = {
         [_p, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _i64, _f32, _f32, _u64,
          _u64, _int, _p],
     ),
+    "oslo_softmax_bias_fwd": (
+        _int,
+        [_p, _p, _p, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _int, _int, _f32, _int, _p],
+    ),
+    "oslo_softmax_bias_bwd": (
+        _int,
+        [_p, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _int, _int, _f32, _int, _p],
+    ),
+    "oslo_softmax_bias_dropout_fwd": (
+        _int,
+        [_p, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _int, _int, _f32, _f32,
+         _u64, _u64, _int, _p],
+    ),
+    "oslo_softmax_bias_dropout_bwd": (
+        _int,
+        [_p, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _int, _int, _f32, _f32,
+         _u64, _u64, _int, _p],
+    ),
     "oslo_bias_gelu_fwd": (_int, [_p, _p, _p, _i64, _i64, _int, _p]),
     "oslo_bias_gelu_bwd": (_int, [_p, _p, _p, _p, _p, _p, _i64, _i64, _i64, _int, _p]),
     "oslo_bias_dropout_add_fwd": (
@@ -840,6 +858,158 @@ class _SoftmaxKernel:
                     float(p), int(seed), int(offset), _dtype_code(input, "input"),
                     _stream(input),
                 )
+            _check(rc, lib)
+        return grad_input
+
+
+    # -- softmax with an additive floating-point term (no counterpart in the
+    #    reference's shim; its models add the term to the scores with torch,
+    #    oslo/transformers/models/bert/modeling_bert.py:298-306) -------------
+    @staticmethod
+    def _bias_operand(bias, input):
+        """The additive term as the kernel addresses it: ``(tensor, stride_b,
+        stride_h, stride_q, dtype_code)``.  ``bias`` broadcasts against the 4-D
+        ``input``: up to four dimensions, each of the leading three either 1 or
+        the full size (expanded views are fine: their stride is 0), the keys
+        contiguous; its dtype becomes the input's or float32."""
+        if input.dim() != 4:
+            raise RuntimeError("expected 4D tensor")
+        if not bias.is_floating_point():
+            raise RuntimeError("the additive term must be a floating-point tensor")
+        if bias.device != input.device:
+            raise RuntimeError(
+                "the additive term is on %s but the softmax operand is on %s"
+                % (bias.device, input.device)
+            )
+        if bias.dim() > 4:
+            raise RuntimeError("the additive term has more than four dimensions")
+        while bias.dim() < 4:
+            bias = bias.unsqueeze(0)
+        b, np_, sq, sk = input.shape
+        for d, full in enumerate((b, np_, sq)):
+            if bias.size(d) not in (1, full):
+                raise RuntimeError(
+                    "additive term of size %s does not broadcast to %s"
+                    % (list(bias.shape), list(input.shape))
+                )
+        if bias.size(3) != sk:
+            if bias.size(3) != 1:
+                raise RuntimeError(
+                    "additive term of size %s does not broadcast to %s"
+                    % (list(bias.shape), list(input.shape))
+                )
+            bias = bias.expand(-1, -1, -1, sk).contiguous()
+        if bias.dtype != input.dtype and bias.dtype != torch.float32:
+            bias = bias.float()
+        if sk > 1 and bias.stride(3) != 1:
+            bias = bias.contiguous()
+        strides = [0 if bias.size(d) == 1 else bias.stride(d) for d in range(3)]
+        return bias, strides[0], strides[1], strides[2], _DTYPE_CODE[bias.dtype]
+
+    @staticmethod
+    def _bias_flags(causal, skip_hidden, strides):
+        if skip_hidden is None:
+            # reading the term first pays when it is small next to the logits:
+            # a mask shared by the heads or by the queries
+            skip_hidden = strides[1] == 0 or strides[2] == 0
+        return (1 if causal else 0) | (2 if skip_hidden else 0)
+
+    def softmax_bias_forward(self, input, bias, scale_factor, causal=False, skip_hidden=None):
+        """``softmax(scale * input + bias)`` over the last dimension of the
+        ``[b, np, sq, sk]`` input; ``causal`` hides the keys beyond the diagonal
+        as well.  ``skip_hidden`` (default: when the term is shared by heads or
+        queries) lets the kernel leave logits unread whose term is -inf or the
+        lowest finite value."""
+        lib = self._lib
+        _check_input(input, "input")
+        bias, sb, sh, sq_, bcode = self._bias_operand(bias, input)
+        b, np_, sq, sk = input.shape
+        out = torch.empty_like(input)
+        flags = self._bias_flags(causal, skip_hidden, (sb, sh, sq_))
+        with _device_of(input):
+            rc = lib.oslo_softmax_bias_fwd(
+                _ptr(input), _ptr(bias), _ptr(out), b, np_, sq, sk, sb, sh, sq_, bcode,
+                flags, float(scale_factor), _dtype_code(input, "input"), _stream(input),
+            )
+            _check(rc, lib)
+        return out
+
+    def softmax_bias_backward(
+        self, output_grads, softmax_results, scale_factor, bias=None, causal=False,
+        skip_hidden=None, inplace=False,
+    ):
+        """``scale * y * (g - sum(g * y))``; ``bias`` (optional) only lets the
+        kernel skip loads, as in the forward pass."""
+        lib = self._lib
+        if output_grads.dim() != 4 or softmax_results.dim() != 4:
+            raise RuntimeError("expected 4D tensor")
+        _check_input(output_grads, "output_grads")
+        _check_input(softmax_results, "softmax_results")
+        if output_grads.dtype != softmax_results.dtype:
+            raise RuntimeError("output_grads and softmax_results differ in dtype")
+        if output_grads.shape != softmax_results.shape:
+            raise RuntimeError("output_grads and softmax_results differ in shape")
+        b, np_, sq, sk = softmax_results.shape
+        sb = sh = sq_ = 0
+        bcode = _dtype_code(softmax_results, "softmax_results")
+        flags = 1 if causal else 0
+        if bias is not None:
+            bias, sb, sh, sq_, bcode = self._bias_operand(bias, softmax_results)
+            flags = self._bias_flags(causal, skip_hidden, (sb, sh, sq_))
+            if not flags & 2:
+                bias = None
+        grad_input = output_grads if inplace else torch.empty_like(output_grads)
+        with _device_of(output_grads):
+            rc = lib.oslo_softmax_bias_bwd(
+                _ptr(output_grads), _ptr(softmax_results), _ptr(bias), _ptr(grad_input),
+                b, np_, sq, sk, sb, sh, sq_, bcode, flags, float(scale_factor),
+                _dtype_code(output_grads, "output_grads"), _stream(output_grads),
+            )
+            _check(rc, lib)
+        return grad_input
+
+    def softmax_bias_dropout_forward(
+        self, input, bias, scale_factor, p, seed, offset, causal=False, skip_hidden=None
+    ):
+        """``dropout(softmax(scale * input + bias), p)`` -> ``[out, stats]``."""
+        lib = self._lib
+        _check_input(input, "input")
+        bias, sb, sh, sq_, bcode = self._bias_operand(bias, input)
+        b, np_, sq, sk = input.shape
+        out = torch.empty_like(input)
+        stats = torch.empty((b * np_ * sq, 2), dtype=torch.float32, device=input.device)
+        flags = self._bias_flags(causal, skip_hidden, (sb, sh, sq_))
+        with _device_of(input):
+            rc = lib.oslo_softmax_bias_dropout_fwd(
+                _ptr(input), _ptr(bias), _ptr(out), _ptr(stats), b, np_, sq, sk, sb, sh, sq_,
+                bcode, flags, float(scale_factor), float(p), int(seed), int(offset),
+                _dtype_code(input, "input"), _stream(input),
+            )
+            _check(rc, lib)
+        return [out, stats]
+
+    def softmax_bias_dropout_backward(
+        self, output_grads, input, bias, stats, scale_factor, p, seed, offset,
+        causal=False, skip_hidden=None, inplace=False,
+    ):
+        lib = self._lib
+        _check_input(output_grads, "output_grads")
+        _check_input(input, "input")
+        _check_input(stats, "stats")
+        if output_grads.dtype != input.dtype or output_grads.shape != input.shape:
+            raise RuntimeError("output_grads and input differ in dtype or shape")
+        bias, sb, sh, sq_, bcode = self._bias_operand(bias, input)
+        b, np_, sq, sk = input.shape
+        if stats.dtype != torch.float32 or stats.numel() != 2 * b * np_ * sq:
+            raise RuntimeError("stats must be float32 [rows, 2]")
+        flags = self._bias_flags(causal, skip_hidden, (sb, sh, sq_))
+        grad_input = output_grads if inplace else torch.empty_like(output_grads)
+        with _device_of(input):
+            rc = lib.oslo_softmax_bias_dropout_bwd(
+                _ptr(output_grads), _ptr(input), _ptr(bias), _ptr(stats), _ptr(grad_input),
+                b, np_, sq, sk, sb, sh, sq_, bcode, flags, float(scale_factor), float(p),
+                int(seed), int(offset), _dtype_code(input, "input"), _stream(input),
+            )
             _check(rc, lib)
         return grad_input
 

@@ -16,6 +16,8 @@ from oslo_amd.torch.nn.modules.functional import (
     fused_rms_norm_affine,
     mixed_dtype_fused_layer_norm_affine,
     mixed_dtype_fused_rms_norm_affine,
+    scaled_bias_softmax,
+    scaled_bias_softmax_dropout,
     scaled_masked_softmax,
     scaled_masked_softmax_dropout,
     scaled_upper_triang_masked_softmax,
@@ -63,6 +65,8 @@ __all__ = [
     "fused_rms_norm_affine",
     "mixed_dtype_fused_layer_norm_affine",
     "mixed_dtype_fused_rms_norm_affine",
+    "scaled_bias_softmax",
+    "scaled_bias_softmax_dropout",
     "scaled_masked_softmax",
     "scaled_masked_softmax_dropout",
     "scaled_upper_triang_masked_softmax",

@@ -521,6 +521,87 @@ class _ScaledMaskedSoftmaxDropout(torch.autograd.Function):
         return input_grads, None, None, None, None, None, None
 
 
+def _bias_grad(dt, bias):
+    """Gradient of an additive term from the gradient of the sum it was
+    added into: summed over the dimensions the term was broadcast along, as
+    autograd does for ``scores + term``."""
+    g = dt.sum_to_size(bias.shape) if tuple(dt.shape) != tuple(bias.shape) else dt
+    return g.to(bias.dtype)
+
+
+class _ScaledBiasSoftmax(torch.autograd.Function):
+    """
+    Fused: ``softmax(scale * inputs + bias)`` on [b, np, sq, sk], the scores
+    with an additive mask or bias
+    (oslo/transformers/models/bert/modeling_bert.py:298-306,
+    oslo/transformers/models/t5/modeling_t5.py:508-514); ``causal=True`` hides
+    the keys beyond the diagonal as well.  Saves the output; the gradient of
+    the term, when it is asked for, is the gradient of the sum reduced over the
+    broadcast dimensions.
+    """
+
+    @staticmethod
+    def forward(ctx, inputs, bias, scale, causal=False):
+        scale = float(scale)
+        softmax_results = get_softmax_kernel().softmax_bias_forward(
+            inputs.contiguous(), bias, scale, causal=causal
+        )
+        ctx.scale, ctx.causal = scale, bool(causal)
+        ctx.save_for_backward(softmax_results, bias)
+        return softmax_results
+
+    @staticmethod
+    def backward(ctx, output_grads):
+        softmax_results, bias = ctx.saved_tensors
+        kernel = get_softmax_kernel()
+        g = output_grads.contiguous()
+        if not ctx.needs_input_grad[1]:
+            dx = kernel.softmax_bias_backward(g, softmax_results, ctx.scale, bias=bias,
+                                              causal=ctx.causal)
+            return dx, None, None, None
+        # gradient of the sum first (scale 1), then the two operands' shares
+        dt = kernel.softmax_bias_backward(g, softmax_results, 1.0, bias=bias, causal=ctx.causal)
+        dx = None
+        if ctx.needs_input_grad[0]:
+            dx = dt if ctx.scale == 1.0 else dt * ctx.scale
+        return dx, _bias_grad(dt, bias), None, None
+
+
+class _ScaledBiasSoftmaxDropout(torch.autograd.Function):
+    """
+    Fused: ``dropout(softmax(scale * inputs + bias), p)``; saves the inputs
+    and two floats per row (see ``_ScaledMaskedSoftmaxDropout``).
+    """
+
+    @staticmethod
+    def forward(ctx, inputs, bias, scale, p, seed, offset, causal=False):
+        scale = float(scale)
+        inputs = inputs.contiguous()
+        with _rng(seed):
+            out, stats = get_softmax_kernel().softmax_bias_dropout_forward(
+                inputs, bias, scale, p, _seed_arg(seed), offset, causal=causal
+            )
+        ctx.scale, ctx.p, ctx.seed, ctx.offset = scale, p, seed, offset
+        ctx.causal = bool(causal)
+        ctx.save_for_backward(inputs, stats, bias)
+        return out
+
+    @staticmethod
+    def backward(ctx, output_grads):
+        inputs, stats, bias = ctx.saved_tensors
+        want_bias = ctx.needs_input_grad[1]
+        with _rng(ctx.seed):
+            dt = get_softmax_kernel().softmax_bias_dropout_backward(
+                output_grads.contiguous(), inputs, bias, stats, ctx.scale, ctx.p,
+                _seed_arg(ctx.seed), ctx.offset, causal=ctx.causal,
+            )
+        if not want_bias:
+            return dt, None, None, None, None, None, None
+        # (the kernel returns scale * d(sum): the term's share is that without the scale)
+        db = _bias_grad(dt if ctx.scale == 1.0 else dt / ctx.scale, bias)
+        return (dt if ctx.needs_input_grad[0] else None), db, None, None, None, None, None
+
+
 """
 User Functions
 """
@@ -740,3 +821,23 @@ def scaled_masked_softmax_dropout(input, mask, scale=1.0, p=0.0, training=True, 
         return _ScaledMaskedSoftmax.apply(input, mask, scale, causal)
     seed, offset = _next_philox_state(input.device)
     return _ScaledMaskedSoftmaxDropout.apply(input, mask, scale, p_eff, seed, offset, causal)
+
+
+def scaled_bias_softmax(input, bias, scale=1.0, causal=False):
+    """softmax(scale * input + bias) over the last dimension; input is
+    [b, np, sq, sk] and `bias` a floating-point tensor that broadcasts against
+    it (an additive mask such as [b, 1, 1, sk] filled with -10000, the lowest
+    finite value or -inf; a position bias [1, np, sq, sk]).  With
+    ``causal=True`` key j of query i is hidden when j > i + (sk - sq) as well.
+    `bias` may require a gradient."""
+    return _ScaledBiasSoftmax.apply(input, bias, scale, causal)
+
+
+def scaled_bias_softmax_dropout(input, bias, scale=1.0, p=0.0, training=True, causal=False):
+    """dropout(softmax(scale * input + bias), p); see ``scaled_bias_softmax``."""
+    _check_dropout_p(p)
+    p_eff = float(p) if training else 0.0
+    if p_eff == 0.0:
+        return _ScaledBiasSoftmax.apply(input, bias, scale, causal)
+    seed, offset = _next_philox_state(input.device)
+    return _ScaledBiasSoftmaxDropout.apply(input, bias, scale, p_eff, seed, offset, causal)

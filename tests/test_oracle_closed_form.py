@@ -102,6 +102,119 @@ def test_softmax_bwd_vs_autograd_and_row_sum():
     assert not np.allclose(cf.softmax_bwd(g.numpy(), y.detach().numpy(), 1.0), x.grad.numpy())
 
 
+# ------------------------------------------ softmax with an additive term
+@pytest.mark.parametrize("bias_shape", [(3, 1, 1, 12), (1, 4, 5, 12), (3, 4, 5, 12), (1, 1, 5, 12)])
+def test_bias_softmax_vs_torch_additive_chain_and_autograd(bias_shape):
+    """torch.softmax(scale * x + M) in float64 and its autograd: forward, the
+    gradient of x (scale * y * (g - sum g y)) and, through it, the gradient
+    of M (the same without the scale, summed over the broadcast dimensions)."""
+    r = rng(40)
+    x = torch.from_numpy(r.standard_normal((3, 4, 5, 12)) * 2).requires_grad_()
+    m = torch.from_numpy(r.standard_normal(bias_shape) * 3).requires_grad_()
+    g = torch.from_numpy(r.standard_normal((3, 4, 5, 12)))
+    scale = 0.37
+    y = torch.softmax(scale * x + m, dim=-1)
+    y.backward(g)
+    oy = cf.softmax_bias_fwd(x.detach().numpy(), m.detach().numpy(), scale, sum_f32=False)
+    assert np.allclose(oy, y.detach().numpy(), rtol=1e-12, atol=0)
+    dx = cf.softmax_bwd(g.numpy(), oy, scale)
+    assert np.allclose(dx, x.grad.numpy(), rtol=1e-10, atol=1e-14)
+    dm = (dx / scale).reshape(3, 4, 5, 12)
+    for d, size in enumerate(bias_shape[:3]):
+        if size == 1:
+            dm = dm.sum(axis=d, keepdims=True)
+    assert np.allclose(dm, m.grad.numpy(), rtol=1e-10, atol=1e-13)
+    # rounding the sum to float32 moves a probability by a few float32 ulps of the logit
+    assert np.allclose(cf.softmax_bias_fwd(x.detach().numpy(), m.detach().numpy(), scale), oy,
+                       rtol=2e-6, atol=0)
+    # a transposed or dropped term must be visible
+    assert not np.allclose(cf.softmax_bias_fwd(x.detach().numpy(), 0.0, scale), oy, rtol=1e-3)
+
+
+def test_bias_softmax_padding_conventions_of_the_reference():
+    """The -10000 mask of modeling_bert.py / modeling_gpt2.py, the finfo.min
+    mask of modeling_bart.py and a -inf mask against the boolean-mask oracle
+    (pinned above) wherever a row sees a key; and the three conventions on a
+    row that sees none, against torch in float32."""
+    b, h, sq, sk = 3, 2, 4, 16
+    r = rng(41)
+    x = r.standard_normal((b, h, sq, sk)).astype(np.float32) * 2
+    valid = np.array([16, 5, 1])
+    pad = np.arange(sk)[None, :] >= valid[:, None]
+    want = cf.softmax_masked_fwd(x, pad[:, None, None, :], 0.125)
+    for fill in (-10000.0, float(np.finfo(np.float32).min), -np.inf,
+                 float(torch.finfo(torch.bfloat16).min), -65504.0):
+        m = np.where(pad, fill, 0.0)[:, None, None, :]
+        y = cf.softmax_bias_fwd(x, m, 0.125)
+        assert np.allclose(y, want, rtol=1e-6, atol=0), fill
+        assert np.all(y[np.broadcast_to(pad[:, None, None, :], y.shape)] == 0), fill
+    # rows without a visible key
+    xt = torch.from_numpy(x[:1, :1])
+    full = lambda v: torch.full((1, 1, 1, sk), v, dtype=torch.float32)
+    # -10000 everywhere: the softmax of the logits themselves (the float32 sum keeps
+    # the logit to 2^-10, hence the tolerance: torch rounds the product first)
+    y = cf.softmax_bias_fwd(x[:1, :1], full(-10000.0).numpy(), 0.125)
+    assert np.allclose(y, torch.softmax(xt * 0.125 + full(-10000.0), -1).numpy(), rtol=2e-3)
+    assert np.allclose(y, cf.softmax_masked_fwd(x[:1, :1], False, 0.125), rtol=2e-3)
+    assert not np.allclose(y, 1.0 / sk, rtol=0.05)
+    # the lowest float everywhere: it absorbs the logit, the row is uniform
+    lo = float(np.finfo(np.float32).min)
+    y = cf.softmax_bias_fwd(x[:1, :1], full(lo).numpy(), 0.125)
+    assert np.array_equal(y, torch.softmax(xt * 0.125 + full(lo), -1).double().numpy())
+    assert np.all(y == 1.0 / sk)
+    # the lowest float16 does not absorb a float32 logit: the row is the softmax of
+    # the logits, coarsely (the sum keeps them to 2^-8)
+    y = cf.softmax_bias_fwd(x[:1, :1], full(-65504.0).numpy(), 0.125)
+    assert np.allclose(y, cf.softmax_masked_fwd(x[:1, :1], False, 0.125), rtol=5e-3)
+    assert not np.allclose(y, 1.0 / sk, rtol=0.05)
+    # -inf everywhere: NaN, as torch returns
+    y = cf.softmax_bias_fwd(x[:1, :1], full(-np.inf).numpy(), 0.125)
+    assert np.isnan(y).all()
+    assert torch.isnan(torch.softmax(xt * 0.125 + full(-np.inf), -1)).all()
+    # -inf and the lowest float mixed: uniform over the finite ones
+    m = full(lo).numpy().copy()
+    m[..., ::2] = -np.inf
+    y = cf.softmax_bias_fwd(x[:1, :1], m, 0.125)
+    assert np.array_equal(y, torch.softmax(xt * 0.125 + torch.from_numpy(m), -1).double().numpy())
+    assert np.all(y[..., 1::2] == 2.0 / sk) and np.all(y[..., ::2] == 0)
+
+
+def test_bias_softmax_causal_flag_is_a_minus_inf_triangle():
+    r = rng(42)
+    for sq, sk in ((6, 6), (3, 9), (1, 5)):
+        x = r.standard_normal((2, 3, sq, sk))
+        m = r.standard_normal((1, 3, sq, sk))
+        tri = np.where(cf.causal_hidden(sq, sk), -np.inf, 0.0)
+        y = cf.softmax_bias_fwd(x, m, 0.5, causal=True, sum_f32=False)
+        ref = torch.softmax(torch.from_numpy(0.5 * x + m + tri), -1).numpy()
+        assert np.allclose(y, ref, rtol=1e-12, atol=0)
+        assert np.all(y[..., cf.causal_hidden(sq, sk)] == 0)
+        # without a term the causal softmax (pinned above)
+        assert np.allclose(cf.softmax_bias_fwd(x.reshape(6, sq, sk)[None], 0.0, 0.5, causal=True,
+                                               sum_f32=False)[0],
+                           cf.softmax_causal_fwd(x.reshape(6, sq, sk), 0.5), rtol=1e-12, atol=0)
+
+
+def test_bias_softmax_dropout_vs_autograd():
+    r = rng(43)
+    x = torch.from_numpy(r.standard_normal((2, 3, 4, 8))).requires_grad_()
+    m = torch.from_numpy(r.standard_normal((1, 3, 4, 8)))
+    g = torch.from_numpy(r.standard_normal((2, 3, 4, 8)))
+    keep = r.random((2, 3, 4, 8)) >= 0.25
+    p, scale = 0.25, 0.7
+    ps = float(np.float32(1.0) / (np.float32(1.0) - np.float32(p)))
+    out = torch.softmax(scale * x + m, -1) * torch.from_numpy(keep) * ps
+    out.backward(g)
+    o = cf.softmax_bias_dropout_fwd(x.detach().numpy(), m.numpy(), scale, keep, p)
+    # (the float32 sum of the oracle: a few float32 ulps of the logits)
+    assert np.allclose(o, out.detach().numpy(), rtol=2e-6, atol=0)
+    dx = cf.softmax_bias_dropout_bwd(g.numpy(), x.detach().numpy(), m.numpy(), scale, keep, p)
+    assert np.allclose(dx, x.grad.numpy(), rtol=2e-5, atol=1e-7)
+    # p = 0 without a keep mask is the plain pair
+    assert np.array_equal(cf.softmax_bias_dropout_fwd(x.detach().numpy(), m.numpy(), scale, None, 0.0),
+                          cf.softmax_bias_fwd(x.detach().numpy(), m.numpy(), scale))
+
+
 # ---------------------------------------------------------------- norms
 @pytest.mark.parametrize("n2", [1, 7, 64, 513])
 def test_layer_norm_fwd_bwd_vs_torch_fp64(n2):
