@@ -190,7 +190,7 @@ class FusedScaleMaskSoftmax(nn.Module):
             input = input * self.scale
         if mask is not None and mask.is_floating_point():
             # an additive term (modeling_bert.py:298-306)
-            input = input + mask
+            input = input + mask.to(input.dtype)
             mask = None
         if self.attn_mask_type == AttnMaskType.causal:
             sq, sk = input.size(2), input.size(3)

@@ -14,6 +14,7 @@ add and ``nn.LayerNorm`` (``oslo/transformers/models/bert/modeling_bert.py:337-3
 one-kernel op.
 """
 import inspect
+import warnings
 
 import torch
 import torch.nn as nn
@@ -360,11 +361,14 @@ def _repeat_kv(hidden_states, n_rep):
     return hidden_states.reshape(b, kv_heads * n_rep, s, d)
 
 
-def _unfused_probs(scores, scaling, attention_mask, causal, p, training, out_dtype):
-    """The reference's unfused chain: scale, mask (boolean True = attend, or an
-    additive float term), softmax, dropout."""
+def _unfused_probs(scores, scaling, attention_mask, causal, p, training, out_dtype,
+                   position_bias=None):
+    """The reference's unfused chain: scale, position bias, mask (boolean True =
+    attend, or an additive float term), softmax, dropout."""
     sq, sk = scores.shape[-2], scores.shape[-1]
     t = scores * scaling
+    if position_bias is not None:
+        t = t + position_bias
     if attention_mask is not None:
         if attention_mask.dtype == torch.bool:
             t = t.masked_fill(~attention_mask, -10000.0)
@@ -377,40 +381,114 @@ def _unfused_probs(scores, scaling, attention_mask, causal, p, training, out_dty
     return torch.nn.functional.dropout(probs, p=p, training=training)
 
 
-def _kernel_takes_mask(attention_mask, scores):
-    """None, or a boolean ``[b or 1, 1, sq or 1, sk]`` tensor on the scores' device;
-    anything else (an additive float mask, one mask per head) is for the unfused chain."""
-    if attention_mask is None:
-        return True
-    b, _, sq, sk = scores.shape
-    return (
-        attention_mask.dtype == torch.bool
-        and attention_mask.device == scores.device
-        and attention_mask.dim() == 4
-        and attention_mask.size(1) == 1
-        and attention_mask.size(3) == sk
-        and attention_mask.size(0) in (1, b)
-        and attention_mask.size(2) in (1, sq)
-    )
+def _broadcasts_to(t, shape):
+    if t.dim() > len(shape):
+        return False
+    own = (1,) * (len(shape) - t.dim()) + tuple(t.shape)
+    return all(m in (1, full) for m, full in zip(own, shape))
+
+
+def _unfused_reason(attention_mask, position_bias, scores):
+    """None when the fused kernels take the call, else why they cannot."""
+    if not scores.is_cuda:
+        return "the scores are not on the GPU"
+    if scores.dtype not in (torch.float16, torch.bfloat16, torch.float32):
+        return "scores of dtype %s" % scores.dtype
+    for name, t in (("attention mask", attention_mask), ("position bias", position_bias)):
+        if t is None:
+            continue
+        if t.device != scores.device:
+            return "the %s is on %s, the scores on %s" % (name, t.device, scores.device)
+        if not _broadcasts_to(t, scores.shape):
+            return "a %s of size %s does not broadcast to %s" % (
+                name, list(t.shape), list(scores.shape))
+    if position_bias is not None and not position_bias.is_floating_point():
+        return "a position bias of dtype %s" % position_bias.dtype
+    return None
+
+
+_warned = set()
+
+
+def _warn_unfused(reason):
+    """One warning per reason when scores on the GPU take the torch chain."""
+    if reason not in _warned:
+        _warned.add(reason)
+        warnings.warn(
+            "fused_attention_forward runs the unfused torch chain: %s" % reason,
+            RuntimeWarning, stacklevel=3,
+        )
+
+
+class CausalKeyPaddingMask(torch.Tensor):
+    """The boolean ``[b, 1, sq, sk]`` mask ``causal & key_visible`` of a causal
+    model on a padded batch, which remembers its key part ``[b, sk]``: the
+    attention function then lets the kernel apply the diagonal and read
+    ``[b, sk]`` mask bytes instead of ``[b, sq, sk]``.  The pair survives
+    ``.to()`` / ``.cuda()`` / ``.cpu()`` (the key part moves along); any other
+    operation returns a plain tensor, and a mask that was written to in place
+    after it was built no longer counts (its version is checked), so the key
+    part can never describe another mask than the one it travels with."""
+
+    @staticmethod
+    def wrap(full, key_visible):
+        out = full.as_subclass(CausalKeyPaddingMask)
+        out._oslo_key_visible = key_visible
+        out._oslo_version = full._version
+        return out
+
+    @classmethod
+    def __torch_function__(cls, func, types, args=(), kwargs=None):
+        kwargs = kwargs or {}
+        with torch._C.DisableTorchFunctionSubclass():
+            out = func(*args, **kwargs)
+        if func in (torch.Tensor.to, torch.Tensor.cuda, torch.Tensor.cpu):
+            src = args[0]
+            kv = key_visible_of(src)
+            if (kv is not None and isinstance(out, torch.Tensor) and out is not src
+                    and out.dtype == torch.bool and out.shape == src.shape):
+                with torch._C.DisableTorchFunctionSubclass():
+                    out = CausalKeyPaddingMask.wrap(out, kv.to(out.device))
+        return out
+
+
+def key_visible_of(mask):
+    """The key part of a mask built by ``fused_attention_mask`` when it still
+    describes the mask (not written to since), else None."""
+    if type(mask) is not CausalKeyPaddingMask:
+        return None
+    d = mask.__dict__
+    kv = d.get("_oslo_key_visible")
+    with torch._C.DisableTorchFunctionSubclass():
+        if kv is None or d.get("_oslo_version") != mask._version:
+            return None
+    return kv
 
 
 def fused_attention_forward(module, query, key, value, attention_mask, scaling=None,
-                            dropout=0.0, **kwargs):
+                            dropout=0.0, position_bias=None, **kwargs):
     """Attention with the scale -> mask -> softmax -> dropout chain in one kernel.
 
     Signature and return value of the attention functions of Hugging Face
     transformers (``(module, query, key, value, attention_mask, scaling,
     dropout, **kwargs) -> (attn_output [b, sq, heads, d], attn_weights)``).
-    ``attention_mask`` is None (causal when the module is) or a boolean
-    ``[b or 1, 1, sq or 1, sk]`` tensor with True = attend.  A mask built by
-    ``fused_attention_mask`` for a causal model on a padded batch carries the
-    key-padding part by itself; the kernel then applies the diagonal and reads
-    ``[b, sk]`` mask bytes instead of ``[b, sq, sk]``.  A floating-point mask is
-    an additive term (a relative-position bias as in
-    oslo/transformers/models/t5/modeling_t5.py:508-514, ALiBi, or -10000
-    fills): the fused kernels know no additive term, so such a call takes the
-    reference's unfused chain, on the GPU as on the CPU, and so does a boolean
-    mask of another shape (one mask per head).
+    ``attention_mask`` is None (causal when the module is), a boolean tensor
+    with True = attend, or a floating-point tensor, which is an additive term
+    (the ``(1 - m) * -10000`` masks of
+    oslo/transformers/models/bert/modeling_bert.py:298-306 and
+    models/gpt2/modeling_gpt2.py:573-581, the ``finfo.min`` masks of
+    models/bart/modeling_bart.py:123-136, ALiBi); ``position_bias`` is the
+    relative-position bias T5 adds to its scores
+    (models/t5/modeling_t5.py:508-514).  Additive terms go to the kernel that
+    computes ``softmax(scale * scores + term)``; a boolean
+    ``[b or 1, 1, sq or 1, sk]`` mask to the mask kernel; a mask built by
+    ``fused_attention_mask`` for a causal model on a padded batch carries its
+    key-padding part, and the kernel then applies the diagonal itself and reads
+    ``[b, sk]`` mask bytes instead of ``[b, sq, sk]``.  A boolean mask of
+    another shape (one per head) and a boolean mask next to a position bias
+    become one additive term.  Scores that are not on the GPU take the
+    reference's unfused chain; so does a GPU call the kernels cannot take, with
+    a warning that names the reason once.
     """
     if scaling is None:
         scaling = query.size(-1) ** -0.5
@@ -420,17 +498,46 @@ def fused_attention_forward(module, query, key, value, attention_mask, scaling=N
     scores = torch.matmul(query, key.transpose(-1, -2))
     b, heads, sq, sk = scores.shape
     p = float(dropout) if module.training else 0.0
+    key_visible = None
     if attention_mask is None:
         causal = kwargs.get("is_causal")
         if causal is None:
             causal = getattr(module, "is_causal", True)
+        if position_bias is not None and causal and sq == 1:
+            causal = False  # one query against its cache: nothing beyond the diagonal
     else:
         causal = False
+        key_visible = key_visible_of(attention_mask)
         if attention_mask.dim() == 4 and attention_mask.size(-1) > sk:
             attention_mask = attention_mask[..., :sk]
-    key_visible = getattr(attention_mask, "_oslo_key_visible", None)
-    if not scores.is_cuda or not _kernel_takes_mask(attention_mask, scores):
-        probs = _unfused_probs(scores, scaling, attention_mask, causal, p, module.training, value.dtype)
+            key_visible = None
+    reason = _unfused_reason(attention_mask, position_bias, scores)
+    if reason is not None:
+        if scores.is_cuda:
+            _warn_unfused(reason)
+        probs = _unfused_probs(scores, scaling, attention_mask, causal, p, module.training,
+                               value.dtype, position_bias)
+    elif position_bias is not None or (attention_mask is not None
+                                       and attention_mask.is_floating_point()):
+        # additive terms: the position bias, the mask, or their sum (a boolean
+        # mask next to a bias becomes a fill that absorbs the logit)
+        term, use_diagonal = position_bias, bool(causal)
+        if attention_mask is not None:
+            if (key_visible is not None and key_visible.dim() == 2
+                    and key_visible.size(-1) == sk and key_visible.device == scores.device):
+                # causal pattern x key padding: the kernel applies the diagonal
+                attention_mask = key_visible.view(key_visible.size(0), 1, 1, sk)
+                use_diagonal = True
+            if attention_mask.dtype == torch.bool:
+                fill_dtype = term.dtype if term.dtype != torch.float16 else torch.float32
+                term = term.to(fill_dtype).masked_fill(~attention_mask, torch.finfo(fill_dtype).min)
+            elif term is None:
+                term = attention_mask
+            else:
+                term = term + attention_mask
+        probs = onn_f.scaled_bias_softmax_dropout(
+            scores, term, scaling, p, module.training, causal=use_diagonal
+        )
     elif attention_mask is None and causal:
         probs = onn_f.scaled_upper_triang_masked_softmax_dropout(
             scores.reshape(b * heads, sq, sk), scaling, p, module.training
@@ -445,11 +552,25 @@ def fused_attention_forward(module, query, key, value, attention_mask, scaling=N
     else:
         if attention_mask is None:
             hidden = torch.zeros(1, 1, 1, sk, dtype=torch.bool, device=scores.device)
-        else:
+        elif attention_mask.dtype == torch.bool:
             hidden = ~attention_mask
-        probs = onn_f.scaled_masked_softmax_dropout(
-            scores, hidden, scaling, p, module.training
-        )
+        else:
+            hidden = attention_mask == 0
+        while hidden.dim() < 4:
+            hidden = hidden.unsqueeze(0)
+        if hidden.size(1) == 1 and hidden.size(3) == sk:
+            probs = onn_f.scaled_masked_softmax_dropout(
+                scores, hidden, scaling, p, module.training
+            )
+        else:
+            # one mask per head (or per key column only): as an additive term
+            # whose fill absorbs the logit, so that a row without a visible key
+            # is uniform as with the mask kernel
+            fill_dtype = scores.dtype if scores.dtype != torch.float16 else torch.float32
+            term = torch.zeros(hidden.shape, dtype=fill_dtype, device=scores.device).masked_fill_(
+                hidden, torch.finfo(fill_dtype).min
+            )
+            probs = onn_f.scaled_bias_softmax_dropout(scores, term, scaling, p, module.training)
     attn_output = torch.matmul(probs.to(value.dtype), value).transpose(1, 2).contiguous()
     return attn_output, probs
 
@@ -460,9 +581,9 @@ def fused_attention_mask(batch_size, q_length, kv_length, q_offset=0, kv_offset=
     ``fused_attention_forward``: the boolean mask of ``sdpa_mask`` (True =
     attend), which is correct by itself.  When the pattern is the plain causal
     one whose diagonal is the kernel's (key j of query i visible when
-    j <= i + (sk - sq)) and a 2-D padding mask is given, the key-padding part
-    ``[b, sk]`` rides along as the attribute ``_oslo_key_visible`` and the
-    attention function lets the kernel apply the diagonal."""
+    j <= i + (sk - sq)) and a 2-D padding mask is given, the result is a
+    ``CausalKeyPaddingMask`` that carries the key-padding part ``[b, sk]`` and
+    the attention function lets the kernel apply the diagonal."""
     from transformers import masking_utils as mu
 
     if mask_function is None:
@@ -481,7 +602,7 @@ def fused_attention_mask(batch_size, q_length, kv_length, q_offset=0, kv_offset=
         except Exception:  # noqa: BLE001 - an internal helper: without it the full mask is used
             kv = None
         if kv is not None and kv.dim() == 2 and kv.size(-1) == kv_length and kv.size(0) in (1, batch_size):
-            full._oslo_key_visible = kv.to(device=full.device, dtype=torch.bool)
+            full = CausalKeyPaddingMask.wrap(full, kv.to(device=full.device, dtype=torch.bool))
     return full
 
 
@@ -509,6 +630,18 @@ def fused_scale_mask_softmax(model, name=ATTENTION_NAME):
         model.set_attn_implementation(name)
     else:
         model.config._attn_implementation = name
+    # sub-models that hold their own copy of the configuration (the encoder
+    # and decoder stacks of T5) are not reached by the call above
+    seen = {id(getattr(model, "config", None))}
+    for module in model.modules():
+        cfg = getattr(module, "config", None)
+        if cfg is None or id(cfg) in seen or not hasattr(cfg, "_attn_implementation"):
+            continue
+        seen.add(id(cfg))
+        try:
+            cfg._attn_implementation = name
+        except (ValueError, AttributeError):
+            pass  # a configuration that refuses the name keeps its own attention
     return model
 
 

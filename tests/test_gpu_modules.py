@@ -213,16 +213,18 @@ def test_fused_scale_mask_softmax_module(device, dtype, mask_type):
     assert yc.device.type == "cpu"
 
 
-def test_fused_scale_mask_softmax_leaves_additive_masks_to_mask_func(device):
-    """A floating-point mask may carry finite biases; the kernels only know
-    "masked out or not", so the module hands such a mask to mask_func."""
+def test_fused_scale_mask_softmax_adds_a_floating_point_mask(device):
+    """A floating-point mask is an additive term (it may carry finite biases):
+    the fused branch computes softmax(scale * x + mask), never "masked out or
+    not"; a mask on another device leaves the call to the torch chain."""
     b, h, sq, sk = 2, 3, 16, 32
     x = randn((b, h, sq, sk), F32, 5).to(device)
     bias = randn((b, 1, sq, sk), F32, 6).to(device)
-    m = onn.FusedScaleMaskSoftmax(mask_func=lambda scores, add: scores + add, scale=0.5)
-    assert not m.is_kernel_available(bias, b, h, sq, sk, input=x)
-    assert torch.allclose(m(x, bias), torch.softmax(0.5 * x + bias, dim=-1), rtol=1e-6, atol=1e-7)
+    m = onn.FusedScaleMaskSoftmax(scale=0.5)
+    assert m.is_kernel_available(bias, b, h, sq, sk, input=x)
+    assert torch.allclose(m(x, bias), torch.softmax(0.5 * x + bias, dim=-1), rtol=1e-5, atol=1e-7)
     assert not m.is_kernel_available(torch.zeros(b, 1, 1, sk, dtype=torch.bool), b, h, sq, sk, input=x)
+    assert not m.is_kernel_available(torch.zeros(b, 1, 1, sk + 1, device=device), b, h, sq, sk, input=x)
 
 
 def test_skip_bias_add_producers_feed_the_fused_ops(device):

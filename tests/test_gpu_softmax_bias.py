@@ -304,3 +304,78 @@ def test_dropout_row_without_a_visible_key(device):
         dx = k.softmax_bias_dropout_backward(g.to(device), x.to(device), bias.to(device), stats, 0.5, p,
                                              seed, offset, skip_hidden=skip)
         check(dx, cf.softmax_bias_dropout_bwd(f64(g), f64(x), f64(bias), 0.5, keep, p), "bwd", atol=2e-7)
+
+
+@pytest.mark.parametrize("dtype", [F32, BF16])
+@pytest.mark.parametrize("scale", [1.0, 0.25])
+def test_autograd_with_a_learned_term(device, dtype, scale):
+    """scaled_bias_softmax(+ dropout) against torch autograd of the unfused
+    chain in float64: gradient of the scores and of a term that requires one
+    (T5's relative-attention bias: summed over the batch it is broadcast along)."""
+    import oslo_amd.torch.nn as onn
+
+    b, np_, sq, sk = 3, 4, 32, 64
+    x = randn((b, np_, sq, sk), dtype, seed=1, std=2.0)
+    m = randn((1, np_, sq, sk), dtype, seed=2, std=1.5)
+    g = randn((b, np_, sq, sk), dtype, seed=3)
+    xd, md = x.to(device).requires_grad_(), m.to(device).requires_grad_()
+    y = onn.scaled_bias_softmax(xd, md, scale)
+    y.backward(g.to(device))
+    xr, mr = x.double().requires_grad_(), m.double().requires_grad_()
+    ref = torch.softmax(scale * xr + mr, dim=-1)
+    ref.backward(g.double())
+    check(y, ref.detach().numpy(), "fwd", atol=1e-9)
+    tol = dict(rtol=1e-4, atol=1e-6) if dtype == F32 else dict(rtol=3e-2, atol=2e-3)
+    assert torch.allclose(xd.grad.cpu().double(), xr.grad, **tol)
+    assert md.grad.shape == md.shape and md.grad.dtype == dtype
+    assert torch.allclose(md.grad.cpu().double(), mr.grad, **tol)
+    # only the term asks for a gradient
+    x2, m2 = x.to(device), m.to(device).requires_grad_()
+    onn.scaled_bias_softmax(x2, m2, scale).backward(g.to(device))
+    assert torch.equal(m2.grad, md.grad)
+    # with dropout: the keep mask is recovered from the output (kept = non-zero)
+    torch.manual_seed(7)
+    xd2, md2 = x.to(device).requires_grad_(), m.to(device).requires_grad_()
+    out = onn.scaled_bias_softmax_dropout(xd2, md2, scale, p=0.2, training=True)
+    out.backward(g.to(device))
+    keep = (out.detach().cpu() != 0).double()
+    xr2, mr2 = x.double().requires_grad_(), m.double().requires_grad_()
+    ps = float(np.float32(1.0) / (np.float32(1.0) - np.float32(0.2)))
+    (torch.softmax(scale * xr2 + mr2, dim=-1) * keep * ps).backward(g.double())
+    assert 0.7 < keep.mean().item() < 0.9
+    assert torch.allclose(xd2.grad.cpu().double(), xr2.grad, **tol)
+    assert torch.allclose(md2.grad.cpu().double(), mr2.grad, **tol)
+
+
+def test_module_takes_additive_and_per_head_masks(device):
+    """FusedScaleMaskSoftmax with the mask exactly as the reference's BERT and
+    GPT-2 build it ((1 - m) * -10000, [b, 1, 1, sk]), with a T5-style bias,
+    with a boolean mask per head, with and without the causal type: the fused
+    branch against the module's own torch branch."""
+    from oslo_amd.torch.nn.modules.softmax import AttnMaskType, FusedScaleMaskSoftmax
+
+    b, np_, sq, sk = 2, 3, 48, 64
+    x = randn((b, np_, sq, sk), F32, seed=2, std=2.0).to(device)
+    valid = torch.tensor([sk, 40])
+    attn = (torch.arange(sk)[None, :] < valid[:, None]).float()
+    hf_mask = ((1.0 - attn) * -10000.0).view(b, 1, 1, sk).to(device)
+    t5_bias = randn((1, np_, sq, sk), F32, seed=4, std=2.0).to(device)
+    per_head = (torch.rand(b, np_, sq, sk, generator=torch.Generator().manual_seed(1)) < 0.3)
+    per_head[..., 0] = False
+    per_head = per_head.to(device)
+    for mask_type in (AttnMaskType.padding, AttnMaskType.causal):
+        fused = FusedScaleMaskSoftmax(attn_mask_type=mask_type, scale=0.25)
+        unfused = FusedScaleMaskSoftmax(attn_mask_type=mask_type, scale=0.25,
+                                        scaled_masked_softmax_fusion=False)
+        for mask in (hf_mask, t5_bias, per_head, t5_bias[0], hf_mask.double()):
+            assert fused.is_kernel_available(mask, b, np_, sq, sk, input=x)
+            a, c = fused(x, mask), unfused(x, mask)
+            assert torch.allclose(a, c, rtol=1e-5, atol=1e-7), (mask_type, mask.shape, mask.dtype)
+    # the gradient reaches a learned term through the module
+    bias = t5_bias.clone().requires_grad_()
+    xg = x.clone().requires_grad_()
+    FusedScaleMaskSoftmax(scale=0.25)(xg, bias).square().sum().backward()
+    br, xr = t5_bias.clone().requires_grad_(), x.clone().requires_grad_()
+    torch.softmax(0.25 * xr + br, -1).square().sum().backward()
+    assert torch.allclose(bias.grad, br.grad, rtol=1e-4, atol=1e-6)
+    assert torch.allclose(xg.grad, xr.grad, rtol=1e-4, atol=1e-6)

@@ -651,6 +651,78 @@ def test_t5_through_the_fused_rms_norm(device, dtype):
         assert (pr.grad.float() - pf.grad.float()).abs().max().item() <= gtol * scale + 1e-6, n
 
 
+def _eager_everywhere(model):
+    for module in model.modules():
+        if hasattr(module, "config") and hasattr(module.config, "_attn_implementation"):
+            module.config._attn_implementation = "eager"
+    return model
+
+
+def test_t5_attention_reaches_the_registered_function_on_cpu():
+    """T5's stacks hold their own configuration copies: the swap has to reach
+    them, and every attention of the model (encoder with a padding mask,
+    causal decoder, cross attention) then runs through the registered function
+    with its position bias."""
+    m = _eager_everywhere(tiny_t5()).eval()
+    ids, labels = t5_inputs()
+    am = torch.ones_like(ids)
+    am[1, 18:] = 0
+    ref = m(input_ids=ids, attention_mask=am, labels=labels).logits
+    fused_scale_mask_softmax(m)
+    att = m.encoder.block[0].layer[0].SelfAttention
+    assert att.config._attn_implementation == m.decoder.config._attn_implementation == "oslo_fused_softmax"
+    out = m(input_ids=ids, attention_mask=am, labels=labels).logits
+    assert torch.allclose(out, ref, atol=1e-5, rtol=1e-5)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("padded", [False, True])
+def test_t5_through_the_additive_term_softmax(device, dtype, padded, monkeypatch):
+    """The model the reference's kernel_fusion_utils.py:71-87 fuses, with its
+    attention (scores + position bias + mask, modeling_t5.py:508-514) through
+    softmax(scale * x + term) and its norms through the RMS-norm swap: loss
+    and every parameter gradient, the learned relative-attention bias included
+    (its gradient is the gradient of the term summed over the batch)."""
+    calls = _spy(monkeypatch, "scaled_bias_softmax_dropout")
+    ids, labels = t5_inputs()
+    am = torch.ones_like(ids)
+    if padded:
+        am[1, 18:] = 0
+        am[2, 9:] = 0
+    ids, labels, am = ids.to(device), labels.to(device), am.to(device)
+    # the same (rounded) parameters evaluated in float32, eager
+    truth = _eager_everywhere(tiny_t5(seed=2)).to(device).to(dtype).float().train()
+    ref = _eager_everywhere(tiny_t5(seed=2)).to(device).to(dtype).train()   # eager in `dtype`
+    fused = _eager_everywhere(tiny_t5(seed=2)).to(device).to(dtype).train()
+    fused_scale_mask_softmax(fused)
+    assert fused_rms_norm(fused) == 12
+    lt = truth(input_ids=ids, attention_mask=am, labels=labels).loss
+    lr = ref(input_ids=ids, attention_mask=am, labels=labels).loss
+    lf = fused(input_ids=ids, attention_mask=am, labels=labels).loss
+    assert len(calls) == 6  # 2 encoder + 2 decoder self + 2 cross attentions
+    assert abs(lt.item() - lf.item()) <= (1e-4 if dtype == torch.float32 else 5e-2)
+    for loss in (lt, lr, lf):
+        loss.backward()
+    # float32: the fused model against the eager one.  bfloat16: two bfloat16 models differ
+    # by their rounding noise, so each is measured against the float32 model and the fused
+    # one must not be further from it than the eager one (plus a floor).
+    names = []
+    for (n, pt), (_, pr), (_, pf) in zip(truth.named_parameters(), ref.named_parameters(),
+                                         fused.named_parameters()):
+        if pt.grad is None:
+            continue
+        names.append(n)
+        scale = pt.grad.abs().max().item() + 1e-8
+        err_f = (pf.grad.float() - pt.grad).abs().max().item()
+        if dtype == torch.float32:
+            assert err_f <= 2e-3 * scale + 1e-6, n
+        else:
+            err_r = (pr.grad.float() - pt.grad).abs().max().item()
+            assert err_f <= 2.0 * err_r + 2e-2 * scale, (n, err_f, err_r, scale)
+    assert any("relative_attention_bias" in n for n in names)
+
+
 # ---------------------------------------------------------------------------
 # the attention function registered with transformers: masks it may be handed
 # ---------------------------------------------------------------------------
@@ -690,18 +762,36 @@ def test_additive_float_mask_is_applied_not_dropped_cpu():
     assert torch.allclose(out, _eager_attention(q, k, v, 1.0, bias), rtol=1e-5, atol=1e-6)
 
 
+def _spy(monkeypatch, name):
+    """Records the calls of oslo_amd.torch.nn.modules.functional.<name>."""
+    from oslo_amd.torch.nn.modules import functional as onn_f
+
+    calls = []
+    real = getattr(onn_f, name)
+
+    def spy(*args, **kwargs):
+        calls.append((args, kwargs))
+        return real(*args, **kwargs)
+
+    monkeypatch.setattr(onn_f, name, spy)
+    return calls
+
+
 @pytest.mark.gpu
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-def test_additive_float_mask_is_applied_not_dropped(device, dtype):
-    """A relative-position bias is a finite additive term: the fused kernels
-    know none, so the call must take the unfused chain and give the eager
-    result (it used to be turned into `mask < -1` and lost)."""
+def test_additive_float_mask_takes_the_additive_term_kernel(device, dtype, monkeypatch):
+    """A relative-position bias plus a -10000 fill is a finite additive term:
+    it goes to the kernel that computes softmax(scale * x + term) and gives the
+    eager result (a float mask must never be turned into a boolean one: the
+    finite part would be lost)."""
     from oslo_amd.transformers.kernel_fusion_utils import fused_attention_forward
 
+    calls = _spy(monkeypatch, "scaled_bias_softmax_dropout")
     g = torch.Generator().manual_seed(0)
     q, k, v = (torch.randn(2, 4, 24, 16, generator=g).to(device, dtype) for _ in range(3))
     bias = _t5_style_bias(4, 24, 24, seed=1).to(device, dtype)
     out, _ = fused_attention_forward(_AttnStub(False).eval(), q, k, v, bias, scaling=1.0)
+    assert len(calls) == 1
     ref = _eager_attention(q.float(), k.float(), v.float(), 1.0, bias.float())
     tol = 1e-5 if dtype == torch.float32 else 3e-2
     assert (out.float() - ref).abs().max().item() <= tol * (ref.abs().max().item() + 1.0)
@@ -709,14 +799,35 @@ def test_additive_float_mask_is_applied_not_dropped(device, dtype):
     dropped = _eager_attention(q.float(), k.float(), v.float(), 1.0,
                                torch.where(bias.float() < -1.0, -10000.0, 0.0))
     assert (out.float() - dropped).abs().max().item() > 10 * tol
+    # the reference's own mask conventions, [b, 1, 1, sk]: (1 - m) * -10000
+    # (modeling_bert.py:298-306) and finfo.min (modeling_bart.py:123-136)
+    for fill in (-10000.0, torch.finfo(dtype).min):
+        pad = torch.zeros(2, 1, 1, 24, device=device, dtype=dtype)
+        pad[1, ..., 19:] = fill
+        out, _ = fused_attention_forward(_AttnStub(False).eval(), q, k, v, pad, scaling=0.25)
+        ref = _eager_attention(q.float(), k.float(), v.float(), 0.25, pad.float())
+        assert (out.float() - ref).abs().max().item() <= tol * (ref.abs().max().item() + 1.0)
+    assert len(calls) == 3
+    # a separate position bias next to a boolean mask (the arguments T5 passes)
+    rel = _t5_style_bias(4, 24, 24, seed=2)[:1].to(device, dtype)
+    attend = torch.ones(2, 1, 24, 24, dtype=torch.bool, device=device)
+    attend[1, ..., 17:] = False
+    out, _ = fused_attention_forward(_AttnStub(False).eval(), q, k, v, attend, scaling=1.0,
+                                     position_bias=rel)
+    ref = _eager_attention(q.float(), k.float(), v.float(), 1.0,
+                           rel.float() + torch.where(attend, 0.0, -10000.0))
+    assert (out.float() - ref).abs().max().item() <= tol * (ref.abs().max().item() + 1.0)
+    assert len(calls) == 4
 
 
 @pytest.mark.gpu
-def test_boolean_mask_per_head_takes_the_unfused_chain(device):
-    """The kernels broadcast one mask over the heads; a boolean mask that differs
-    from head to head is applied by the unfused chain instead of being refused."""
+def test_boolean_mask_per_head_becomes_an_additive_term(device, monkeypatch):
+    """The mask kernels broadcast one mask over the heads; a boolean mask that
+    differs from head to head goes to the additive-term kernel as a fill that
+    absorbs the logit."""
     from oslo_amd.transformers.kernel_fusion_utils import fused_attention_forward
 
+    calls = _spy(monkeypatch, "scaled_bias_softmax_dropout")
     g = torch.Generator().manual_seed(3)
     q, k, v = (torch.randn(2, 4, 24, 16, generator=g).to(device) for _ in range(3))
     attend = torch.rand(2, 4, 24, 24, generator=g) > 0.3
@@ -725,12 +836,44 @@ def test_boolean_mask_per_head_takes_the_unfused_chain(device):
     additive = torch.where(attend, 0.0, -10000.0).to(device)
     ref = _eager_attention(q, k, v, 0.25, additive)
     assert torch.allclose(out, ref, rtol=1e-5, atol=1e-6)
+    assert len(calls) == 1
+
+
+@pytest.mark.gpu
+def test_unfused_chain_on_the_gpu_warns_once(device):
+    """A call the kernels cannot take (a mask on another device) runs the torch
+    chain and says so, once per reason."""
+    import warnings
+
+    from oslo_amd.transformers import kernel_fusion_utils as kfu
+
+    g = torch.Generator().manual_seed(3)
+    q, k, v = (torch.randn(2, 4, 8, 16, generator=g).to(device).double() for _ in range(3))
+    kfu._warned.clear()
+    with warnings.catch_warnings(record=True) as seen:
+        warnings.simplefilter("always")
+        for _ in range(3):
+            out, _ = kfu.fused_attention_forward(_AttnStub(False).eval(), q, k, v, None, scaling=0.25,
+                                                 is_causal=False)
+    assert len([w for w in seen if "unfused torch chain" in str(w.message)]) == 1
+    assert torch.allclose(out, _eager_attention(q, k, v, 0.25, None))
+    # the module: a mask whose size does not broadcast is a reason, too
+    from oslo_amd.torch.nn.modules.softmax import FusedScaleMaskSoftmax
+
+    FusedScaleMaskSoftmax._warned.clear()
+    m = FusedScaleMaskSoftmax(scale=0.5)
+    x = torch.randn(2, 3, 4, 8, device=device, dtype=torch.float64)
+    with warnings.catch_warnings(record=True) as seen:
+        warnings.simplefilter("always")
+        m(x, None)
+        m(x, None)
+    assert len([w for w in seen if "unfused torch chain" in str(w.message)]) == 1
 
 
 def test_mask_builder_returns_the_full_mask_and_the_key_part():
     from transformers import masking_utils as mu
 
-    from oslo_amd.transformers.kernel_fusion_utils import fused_attention_mask
+    from oslo_amd.transformers.kernel_fusion_utils import fused_attention_mask, key_visible_of
 
     am = torch.ones(3, 20, dtype=torch.long)
     am[1, 15:] = 0
@@ -738,19 +881,28 @@ def test_mask_builder_returns_the_full_mask_and_the_key_part():
     full = fused_attention_mask(3, 20, 20, attention_mask=am)
     ref = mu.sdpa_mask(3, 20, 20, attention_mask=am.bool())
     assert full.dtype == torch.bool and torch.equal(full, ref)
-    assert torch.equal(full._oslo_key_visible, am.bool())
+    assert torch.equal(key_visible_of(full), am.bool())
     # causal & key padding is exactly the full mask: the factorisation the kernel relies on
     causal = torch.tril(torch.ones(20, 20, dtype=torch.bool))
     assert torch.equal(full, causal[None, None] & am.bool()[:, None, None, :])
     # cached decoding: one query against 20 keys (the diagonal offset is sk - sq)
     step = fused_attention_mask(3, 1, 20, q_offset=19, attention_mask=am)
-    assert step is None or torch.equal(step._oslo_key_visible, am.bool())
+    assert step is None or torch.equal(key_visible_of(step), am.bool())
     # another pattern (sliding window) carries no key part
     sw = fused_attention_mask(3, 20, 20, mask_function=mu.sliding_window_causal_mask_function(4), attention_mask=am)
-    assert getattr(sw, "_oslo_key_visible", None) is None
+    assert key_visible_of(sw) is None
     # a diagonal that is not the kernel's (queries offset against the keys) carries none either
     off = fused_attention_mask(3, 10, 20, q_offset=5, attention_mask=am)
-    assert off is None or getattr(off, "_oslo_key_visible", None) is None
+    assert off is None or key_visible_of(off) is None
+    # the pair survives a move or a no-op .to(), but no other operation, and a mask that was
+    # written to in place after it was built no longer counts
+    assert torch.equal(key_visible_of(full.to(full.device)), am.bool())
+    assert torch.equal(key_visible_of(full.to("cpu", copy=True)), am.bool())
+    assert key_visible_of(full[..., :20]) is None and key_visible_of(full.clone()) is None
+    assert key_visible_of(full & full) is None and key_visible_of(full.to(torch.uint8)) is None
+    edited = fused_attention_mask(3, 20, 20, attention_mask=am)
+    edited[0, 0, 5, 2] = False  # e.g. a wrapper that cuts a window into the mask
+    assert key_visible_of(edited) is None and isinstance(edited, torch.Tensor)
 
 
 @pytest.mark.gpu
@@ -777,6 +929,34 @@ def test_causal_model_on_a_padded_batch_takes_the_causal_masked_kernel(device, m
     assert (out[valid] - ref[valid]).abs().max().item() <= 2e-4
     b, s = ids.shape
     assert calls and all(shape == (b, 1, 1, s) and causal for shape, causal in calls), calls
+
+
+@pytest.mark.gpu
+def test_mask_moved_or_edited_between_builder_and_attention(device, monkeypatch):
+    """The mask builder's result moved to the GPU still reaches the
+    causal + key-padding kernel; the same mask written to in place afterwards
+    (a window cut into it) is applied as it then is, by the kernel that reads
+    the whole mask."""
+    from oslo_amd.transformers.kernel_fusion_utils import (
+        fused_attention_forward, fused_attention_mask)
+
+    calls = _spy(monkeypatch, "scaled_masked_softmax_dropout")
+    g = torch.Generator().manual_seed(5)
+    q, k, v = (torch.randn(3, 4, 20, 16, generator=g).to(device) for _ in range(3))
+    am = torch.ones(3, 20, dtype=torch.long)
+    am[1, 15:] = 0
+    mask = fused_attention_mask(3, 20, 20, attention_mask=am)  # built on the CPU
+    moved = mask.to(device)
+    out, _ = fused_attention_forward(_AttnStub(True).eval(), q, k, v, moved, scaling=0.25)
+    assert calls[-1][1].get("causal") is True and tuple(calls[-1][0][1].shape) == (3, 1, 1, 20)
+    ref = _eager_attention(q, k, v, 0.25, torch.where(mask, 0.0, -10000.0).to(device))
+    assert torch.allclose(out, ref, rtol=1e-5, atol=1e-6)
+    moved[:, :, :, 0] = False          # in place: hide key 0 from every query but keep ...
+    moved[:, :, 0, 0] = True           # ... query 0's only key
+    out, _ = fused_attention_forward(_AttnStub(True).eval(), q, k, v, moved, scaling=0.25)
+    assert not calls[-1][1].get("causal") and tuple(calls[-1][0][1].shape) == (3, 1, 20, 20)
+    ref = _eager_attention(q, k, v, 0.25, torch.where(moved, 0.0, -10000.0))
+    assert torch.allclose(out, ref, rtol=1e-5, atol=1e-6)
 
 
 @pytest.mark.gpu
