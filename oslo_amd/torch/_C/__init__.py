@@ -307,16 +307,93 @@ def _check_input(t, name):
         raise RuntimeError("%s must be contiguous" % name)
 
 
-# Backward workspaces (fp32 partial rows of the parameter gradients), kept per
-# (device, stream, op) and grown on demand instead of allocated per call.  Calls
-# that share a stream are ordered, so the finalize launch of one call has read
-# the partial rows before the next call overwrites them; calls on different
-# streams or devices never share a workspace.  The memory stays torch's.
-_ws_cache = {}
+# Backward workspaces (fp32 partial rows of the parameter gradients).  A backward
+# entry point enqueues two launches, the main kernel that writes the partial rows
+# and the finalize kernel that reads them, so a workspace must not be handed to
+# another call before both launches of this one are on the stream:
+#   * eager calls share one workspace per (device, stream, op), grown on demand;
+#     the slot's lock is held from the moment the workspace is picked until the C
+#     call has returned.  Calls that share a stream are then ordered on it as
+#     whole calls (two host threads on one stream cannot interleave their
+#     launches); calls on different streams or devices never share a workspace;
+#   * a call under stream capture neither reads nor writes the cache: it gets a
+#     workspace of its own, which the graph's private pool then owns.  Two graphs
+#     never share partial rows, deleting one graph cannot free memory another one
+#     points at, and the cached tensors are never referenced by a graph, so
+#     replacing one by a larger one is always safe.
+class _WorkspaceSlot:
+    __slots__ = ("lock", "tensor")
+
+    def __init__(self):
+        self.lock = threading.Lock()
+        self.tensor = None
+
+
+class _WorkspaceLease:
+    """``with lease as ws:`` -> ``ws.tensor`` (None when the call needs no
+    workspace) and ``ws.nbytes`` for the duration of one C call."""
+
+    __slots__ = ("tensor", "nbytes", "_cache", "_key", "_slot")
+
+    def __init__(self, cache=None, key=None, nbytes=0):
+        self.tensor, self.nbytes = None, nbytes
+        self._cache, self._key, self._slot = cache, key, None
+
+    def __enter__(self):
+        cache = self._cache
+        if cache is None or self.nbytes <= 0:
+            return self
+        if cache.capturing():
+            self.tensor = cache.allocate(self.nbytes, self._key[0])
+            return self
+        slot = cache.slots.get(self._key)
+        if slot is None:
+            slot = cache.slots.setdefault(self._key, _WorkspaceSlot())
+        slot.lock.acquire()
+        self._slot = slot
+        try:
+            ws = slot.tensor
+            if ws is None or ws.numel() < self.nbytes:
+                # (round up so that a sweep over growing shapes settles quickly)
+                size = max(self.nbytes, 16)
+                if size > (1 << 16):
+                    size = (size + (1 << 20) - 1) & ~((1 << 20) - 1)
+                ws = slot.tensor = cache.allocate(size, self._key[0])
+            self.tensor = ws
+        except BaseException:
+            self._slot = None
+            slot.lock.release()
+            raise
+        return self
+
+    def __exit__(self, *exc):
+        slot, self._slot = self._slot, None
+        if slot is not None:
+            slot.lock.release()
+        return False
+
+
+class _WorkspaceCache:
+    def __init__(self, allocate, capturing):
+        self.slots = {}
+        self.allocate = allocate    # (nbytes, device index) -> uint8 tensor
+        self.capturing = capturing  # () -> bool: the current stream is being captured
+
+    def lease(self, index, stream, op, nbytes):
+        return _WorkspaceLease(self, (index, stream, op), nbytes)
+
+
+def _allocate_workspace(nbytes, index):
+    return torch.empty(nbytes, dtype=torch.uint8, device=torch.device("cuda", index))
+
+
+_ws_cache = _WorkspaceCache(_allocate_workspace, torch.cuda.is_current_stream_capturing)
 _ws_bytes_cache = {}
+_NO_WORKSPACE = _WorkspaceLease()
 
 
 def _workspace(lib, op, n1, n2, device):
+    """Lease of the workspace of backward op `op` on an [n1, n2] problem."""
     key = (op, n1, n2)
     nbytes = _ws_bytes_cache.get(key)
     if nbytes is None:
@@ -327,15 +404,7 @@ def _workspace(lib, op, n1, n2, device):
             _ws_bytes_cache[key] = nbytes
     index = device.index if device.index is not None else torch.cuda.current_device()
     stream = _raw_stream(index) if _raw_stream is not None else torch.cuda.current_stream(device).cuda_stream
-    slot = (index, stream, op)
-    ws = _ws_cache.get(slot)
-    if ws is None or ws.numel() < nbytes:
-        # (round up so that a sweep over growing shapes settles quickly)
-        size = max(nbytes, 16)
-        size = (size + (1 << 20) - 1) & ~((1 << 20) - 1) if size > (1 << 16) else size
-        ws = torch.empty(size, dtype=torch.uint8, device=device)
-        _ws_cache[slot] = ws
-    return ws, nbytes
+    return _ws_cache.lease(index, stream, op, nbytes)
 
 
 class device_rng:
@@ -499,7 +568,7 @@ class _LayerNormKernel:
                 )
         grad_input = torch.empty_like(input)
         grad_gamma = grad_beta = None
-        ws, ws_bytes = None, 0
+        lease = _NO_WORKSPACE
         if gamma is not None:
             _check_input(gamma, "gamma")
             _check_param(gamma, normalized_shape, "gamma")
@@ -510,21 +579,21 @@ class _LayerNormKernel:
             grad_gamma = torch.empty_like(gamma)
             if not rms:
                 grad_beta = torch.empty_like(beta if beta is not None else gamma)
-            ws, ws_bytes = _workspace(
+            lease = _workspace(
                 lib, OSLO_OP_RMS_BWD if rms else OSLO_OP_LN_BWD, n1, n2, input.device
             )
-        with _device_of(input):
+        with _device_of(input), lease as ws:
             if rms:
                 rc = lib.oslo_rms_bwd(
                     _ptr(dout), _ptr(input), _ptr(invvar), _ptr(gamma), _ptr(grad_input),
-                    _ptr(grad_gamma), _ptr(ws), ws_bytes, n1, n2, din, dcode,
+                    _ptr(grad_gamma), _ptr(ws.tensor), ws.nbytes, n1, n2, din, dcode,
                     _stream(input),
                 )
             else:
                 rc = lib.oslo_ln_bwd(
                     _ptr(dout), _ptr(input), _ptr(mean), _ptr(invvar), _ptr(gamma),
-                    _ptr(grad_input), _ptr(grad_gamma), _ptr(grad_beta), _ptr(ws),
-                    ws_bytes, n1, n2, din, dcode, _stream(input),
+                    _ptr(grad_input), _ptr(grad_gamma), _ptr(grad_beta), _ptr(ws.tensor),
+                    ws.nbytes, n1, n2, din, dcode, _stream(input),
                 )
             _check(rc, lib)
         return grad_input, grad_gamma, grad_beta
@@ -628,14 +697,14 @@ class _LayerNormKernel:
                 grad_beta = torch.empty_like(gamma)
         if need_bias_grad:
             grad_bias = torch.empty(n2, dtype=h.dtype, device=h.device)
-        ws, ws_bytes = None, 0
+        lease = _NO_WORKSPACE
         if gamma is not None or need_bias_grad:
-            ws, ws_bytes = _workspace(lib, OSLO_OP_BIAS_DROPOUT_ADD_NORM_BWD, n1, n2, h.device)
-        with _device_of(h):
+            lease = _workspace(lib, OSLO_OP_BIAS_DROPOUT_ADD_NORM_BWD, n1, n2, h.device)
+        with _device_of(h), lease as ws:
             rc = lib.oslo_bias_dropout_add_norm_bwd(
                 _ptr(dout), _ptr(dh_extra), _ptr(h), _ptr(mean), _ptr(invvar), _ptr(gamma),
                 _ptr(grad_res), _ptr(grad_in), _ptr(grad_gamma), _ptr(grad_beta),
-                _ptr(grad_bias), _ptr(ws), ws_bytes, n1, n2, float(p), int(seed),
+                _ptr(grad_bias), _ptr(ws.tensor), ws.nbytes, n1, n2, float(p), int(seed),
                 int(offset), 1 if rms else 0, code, _stream(h),
             )
             _check(rc, lib)
@@ -1064,14 +1133,14 @@ class _FusedElementwiseKernel:
         rows, cols = _rows_cols(input, bias)
         grad_input = torch.empty_like(input)
         grad_bias = None
-        ws, ws_bytes = None, 0
+        lease = _NO_WORKSPACE
         if bias is not None and need_bias_grad:
             grad_bias = torch.empty_like(bias)
-            ws, ws_bytes = _workspace(lib, OSLO_OP_BIAS_GELU_BWD, rows, cols, input.device)
-        with _device_of(input):
+            lease = _workspace(lib, OSLO_OP_BIAS_GELU_BWD, rows, cols, input.device)
+        with _device_of(input), lease as ws:
             rc = lib.oslo_bias_gelu_bwd(
                 _ptr(grad_output), _ptr(input), _ptr(bias), _ptr(grad_input),
-                _ptr(grad_bias), _ptr(ws), ws_bytes, rows, cols,
+                _ptr(grad_bias), _ptr(ws.tensor), ws.nbytes, rows, cols,
                 _dtype_code(input, "input"), _stream(input),
             )
             _check(rc, lib)
@@ -1115,17 +1184,17 @@ class _FusedElementwiseKernel:
         rows = grad_output.numel() // cols if cols > 0 else 0
         grad_input = torch.empty_like(grad_output) if need_input_grad else None
         grad_bias = None
-        ws, ws_bytes = None, 0
+        lease = _NO_WORKSPACE
         if need_bias_grad:
             grad_bias = torch.empty(cols, dtype=grad_output.dtype, device=grad_output.device)
-            ws, ws_bytes = _workspace(
+            lease = _workspace(
                 lib, OSLO_OP_BIAS_DROPOUT_ADD_BWD, rows, cols, grad_output.device
             )
         if grad_input is None and grad_bias is None:
             return None, None
-        with _device_of(grad_output):
+        with _device_of(grad_output), lease as ws:
             rc = lib.oslo_bias_dropout_add_bwd(
-                _ptr(grad_output), _ptr(grad_input), _ptr(grad_bias), _ptr(ws), ws_bytes,
+                _ptr(grad_output), _ptr(grad_input), _ptr(grad_bias), _ptr(ws.tensor), ws.nbytes,
                 rows, cols, float(p), int(seed), int(offset),
                 _dtype_code(grad_output, "grad_output"), _stream(grad_output),
             )

@@ -248,3 +248,73 @@ def test_captured_mixed_precision_lamb_step_counts_and_replays(device):
         assert captured.param_groups[0]["step"].item() == k + 1 == eager.param_groups[0]["step"].item()
         for a, b in zip(eager_ps, graph_ps):
             assert torch.equal(a, b), "replay %d" % k
+
+
+def test_two_graphs_do_not_share_a_backward_workspace(device, monkeypatch):
+    """A backward entry point writes partial rows to a workspace and reads them
+    in a second launch.  A captured call must own its workspace: two graphs
+    that capture the same op at the same shape get different ones, deleting the
+    first graph leaves the second intact, and the two replayed at the same time
+    on two streams give the serial results bit for bit."""
+    n1, n2 = 2048, 1024
+    ln = _C.get_layernorm_kernel()
+    gamma = randn((n2,), BF16, 3, std=0.1, mean=1.0).to(device)
+    beta = randn((n2,), BF16, 4, std=0.1).to(device)
+    xs = [randn((n1, n2), BF16, 10 + i).to(device) for i in range(2)]
+    dys = [randn((n1, n2), BF16, 20 + i).to(device) for i in range(2)]
+    stats = [ln.layer_norm_forward_affine(x, (n2,), gamma, beta, 1e-5)[1:] for x in xs]
+
+    seen = []
+    real = _C._allocate_workspace
+
+    def allocate(nbytes, index):
+        t = real(nbytes, index)
+        seen.append((t.data_ptr(), torch.cuda.is_current_stream_capturing()))
+        return t
+
+    monkeypatch.setattr(_C._ws_cache, "allocate", allocate)
+
+    def bwd(i):
+        mean, invvar = stats[i]
+        return ln.layer_norm_backward_affine(dys[i], mean, invvar, xs[i], (n2,), gamma, beta, 1e-5)
+
+    want = [[t.clone() for t in bwd(i)] for i in range(2)]   # eager (warms the cache up, too)
+    torch.cuda.synchronize()
+    graphs, outs = [], []
+    for i in range(2):
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            outs.append(bwd(i))
+        graphs.append(g)
+    captured = [ptr for ptr, capturing in seen if capturing]
+    assert len(captured) == 2 and captured[0] != captured[1]
+    eager_ptrs = {ptr for ptr, capturing in seen if not capturing}
+    assert not eager_ptrs & set(captured)       # nor the cached one
+    # both at once on two streams, three times, with eager calls of the same op in between
+    streams = [torch.cuda.Stream(device=device) for _ in range(2)]
+    for rep in range(3):
+        for o in outs:
+            for t in o:
+                t.zero_()
+        torch.cuda.synchronize()
+        for g, s in zip(graphs, streams):
+            with torch.cuda.stream(s):
+                g.replay()
+        eager = bwd(rep % 2)                    # shares the device, not the workspace
+        torch.cuda.synchronize()
+        for i in range(2):
+            for k, (a, b) in enumerate(zip(outs[i], want[i])):
+                assert torch.equal(a, b), "graph %d, output %d, replay %d" % (i, k, rep)
+        for a, b in zip(eager, want[rep % 2]):
+            assert torch.equal(a, b)
+    # the second graph does not depend on the first one's memory
+    keep = [t.clone() for t in want[1]]
+    del graphs[0], outs[0]
+    torch.cuda.synchronize()
+    torch.cuda.empty_cache()
+    filler = [torch.full((n1, n2), 7.0, dtype=BF16, device=device) for _ in range(8)]  # reuses freed blocks
+    graphs[0].replay()
+    torch.cuda.synchronize()
+    for a, b in zip(outs[0], keep):
+        assert torch.equal(a, b)
+    del filler

@@ -77,6 +77,64 @@ def test_threads_on_their_own_streams_match_the_serial_results(device):
             assert torch.equal(a, b), "thread %d, output %d differs" % (i, k)
 
 
+def test_threads_that_share_the_default_stream_match_the_serial_results(device):
+    """Two host threads on one stream (autograd's worker thread and the main
+    thread are the everyday case): a backward entry point launches a main
+    kernel and a finalize kernel that share a workspace, and the binding keeps
+    one workspace per stream, so it must hand it out for whole calls only --
+    were the launches of two calls to interleave, one call's finalize would
+    read the other's partial rows."""
+    ln = _C.get_layernorm_kernel()
+    ek = _C.get_fused_elementwise_kernel()
+    n2 = 1024
+    gamma = randn((n2,), BF16, 1, std=0.02, mean=1.0).to(device)
+    beta = randn((n2,), BF16, 2, std=0.02).to(device)
+    nthreads, iters = 2, 40
+    data = []
+    for i in range(nthreads):
+        n1 = 1024 + 512 * i
+        x = randn((n1, n2), BF16, 10 + i).to(device)
+        dy = randn((n1, n2), BF16, 20 + i).to(device)
+        _, mean, invvar = ln.layer_norm_forward_affine(x, (n2,), gamma, beta, 1e-5)
+        data.append((x, dy, mean, invvar))
+
+    def work(i):
+        x, dy, mean, invvar = data[i]
+        outs = []
+        for _ in range(iters):
+            dx, dg, db = ln.layer_norm_backward_affine(dy, mean, invvar, x, (n2,), gamma, beta, 1e-5)
+            dact, dbias = ek.bias_gelu_backward(dy, x, beta)
+            g_in, g_b = ek.bias_dropout_add_backward(dy, 0.1, 5, 8)
+            outs.append((dg, db, dbias, g_b))
+        return outs
+
+    want = [work(i)[0] for i in range(nthreads)]
+    torch.cuda.synchronize()
+    got = [None] * nthreads
+    errors = []
+    start = threading.Barrier(nthreads)
+
+    def run(i):
+        try:
+            start.wait(timeout=60)
+            got[i] = work(i)        # torch's current stream of a new thread is the default stream
+        except Exception as exc:  # reported by the parent thread
+            errors.append((i, repr(exc)))
+
+    threads = [threading.Thread(target=run, args=(i,)) for i in range(nthreads)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join(timeout=110)
+    assert not errors, errors
+    assert all(not t.is_alive() for t in threads)
+    torch.cuda.synchronize()
+    for i in range(nthreads):
+        for it, outs in enumerate(got[i]):
+            for k, (a, b) in enumerate(zip(outs, want[i])):
+                assert torch.equal(a, b), "thread %d, iteration %d, output %d differs" % (i, it, k)
+
+
 def test_the_error_message_belongs_to_the_calling_thread(device):
     lib = _C.load_library()
     seen = {}

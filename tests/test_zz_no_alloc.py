@@ -117,3 +117,70 @@ def test_static_scratch_refuses_problems_beyond_its_size(device):
     assert rc == 0, lib.oslo_hip_last_error()
     torch.cuda.synchronize()
     assert float(dg.float().abs().max()) == 0.0 and float(db.float().abs().max()) == 0.0
+
+
+def test_static_scratch_allocates_nothing_and_can_be_captured(device):
+    """The property the entry point exists for: it can run where device memory
+    cannot be allocated.  Under stream capture an allocation by the library
+    would fail the capture; here the call is captured (the empty-batch form,
+    which clears the parameter gradients with a kernel, included), the graph is
+    replayed with new inputs against oslo_ln_bwd, and the device's free memory
+    is the same before and after the eager calls."""
+    lib = _C.load_library()
+    n1, n2 = 512, 1024
+    x = randn((n1, n2), BF16, 1, std=1.3, mean=0.2).to(device)
+    dy = randn((n1, n2), BF16, 2).to(device)
+    gamma = randn((n2,), BF16, 3, std=0.02, mean=1.0).to(device)
+    beta = randn((n2,), BF16, 4, std=0.02).to(device)
+    y = torch.empty_like(x)
+    mean = torch.empty(n1, dtype=F32, device=device)
+    invvar = torch.empty(n1, dtype=F32, device=device)
+    dx, dg, db = torch.empty_like(x), torch.empty_like(gamma), torch.empty_like(gamma)
+    eg, eb = torch.ones(64, dtype=BF16, device=device), torch.ones(64, dtype=BF16, device=device)
+    nbytes = int(lib.oslo_workspace_bytes(_C.OSLO_OP_LN_BWD, n1, n2))
+    ws = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=device)
+    rdx, rdg, rdb = torch.empty_like(x), torch.empty_like(gamma), torch.empty_like(gamma)
+
+    def fwd(st):
+        assert lib.oslo_ln_fwd(_p(x), _p(gamma), _p(beta), _p(y), _p(mean), _p(invvar), n1, n2, 1e-5,
+                               CODE[BF16], CODE[BF16], st) == 0
+
+    def static(st):
+        rc = lib.oslo_ln_bwd_static(_p(dy), _p(x), _p(mean), _p(invvar), _p(gamma), _p(dx), _p(dg), _p(db),
+                                    n1, n2, CODE[BF16], CODE[BF16], st)
+        assert rc == 0, lib.oslo_hip_last_error()
+        rc = lib.oslo_ln_bwd_static(None, None, None, None, _p(gamma), None, _p(eg), _p(eb), 0, 64,
+                                    CODE[BF16], CODE[BF16], st)
+        assert rc == 0, lib.oslo_hip_last_error()
+
+    # eager: free device memory does not move (the first call has already fetched
+    # the array's address; the array itself is part of the loaded code object)
+    st = torch.cuda.current_stream().cuda_stream
+    fwd(st)
+    static(st)
+    torch.cuda.synchronize()
+    free0, _ = torch.cuda.mem_get_info(device)
+    for _ in range(5):
+        static(st)
+    torch.cuda.synchronize()
+    free1, _ = torch.cuda.mem_get_info(device)
+    assert free1 == free0
+
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        static(torch.cuda.current_stream().cuda_stream)
+    for rep in range(3):
+        x.copy_(randn((n1, n2), BF16, 30 + rep, std=1.3).to(device))
+        dy.copy_(randn((n1, n2), BF16, 40 + rep).to(device))
+        eg.fill_(1.0)
+        st = torch.cuda.current_stream().cuda_stream
+        fwd(st)
+        rc = lib.oslo_ln_bwd(_p(dy), _p(x), _p(mean), _p(invvar), _p(gamma), _p(rdx), _p(rdg), _p(rdb),
+                             _p(ws), nbytes, n1, n2, CODE[BF16], CODE[BF16], st)
+        assert rc == 0, lib.oslo_hip_last_error()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        for a, b, name in ((rdx, dx, "dx"), (rdg, dg, "dgamma"), (rdb, db, "dbeta")):
+            _same_bits(a, b, "replay %d %s" % (rep, name))
+        assert float(eg.float().abs().max()) == 0.0 and float(eb.float().abs().max()) == 0.0
