@@ -12,9 +12,12 @@ the non-GEMM chain of one GPT-NeoX-20B-shaped layer, bf16, batch 4, sequence
     bias_dropout_add_fwd, _bwd      [8192, 6144], p = 0.1
 every buffer resident in HBM and pre-allocated; each stage has its own
 synthetic input (the GEMMs between the stages are not part of the path).  The
-four 2 GB tensors of the softmax stage are carved from one allocation at
-staggered offsets (see `staggered`): that kernel is sensitive to operands that
-alias in the memory channels, and a plain allocation leaves it to luck.
+four 2 GB tensors of the softmax stage are laid out as the Python binding lays
+them out for a user of FusedScaleMaskSoftmax: the scores and the incoming
+gradient are plain torch allocations, the probabilities and the input gradient
+come from the binding's own allocation helper (`_C.empty_staggered`), which
+keeps them off the 2 MiB phase of the operands; the kernel table holds the
+same backward launch on four plain allocations for comparison.
 `value` = algorithmic bytes of a step (10 537.7 MB) / wall time per step.
 
 Prints ONE JSON line.  Beside the contract's keys it carries
@@ -33,7 +36,11 @@ Prints ONE JSON line.  Beside the contract's keys it carries
   cpu_path      the reference's unfused torch path, forward + backward, per
                 configuration on bounded samples, with the GPU rate of the
                 same fused forward + backward pair (the metric's own unit:
-                gpu_GBps and gpu_frac of the peak) and their ratio.
+                gpu_GBps and gpu_frac of the peak) and their ratio,
+  modules       forward + backward through the oslo_amd.torch.nn modules and
+                functions with autograd (output allocation, saved tensors and
+                the binding's checks included), next to the C-ABI pair of the
+                kernel table and their ratio.
 """
 import argparse
 import json
@@ -160,6 +167,34 @@ def time_in_graph(torch, fn, nsets, launches=24, replays=8):
         return None
 
 
+def time_queued(torch, fn, nsets, blocker, calls=16, repeats=6):
+    """ms per call of fn when the host runs ahead of the GPU, the regime of a
+    training step whose GEMMs keep the GPU busy while Python prepares the next
+    launches: `blocker()` first puts a few ms of work on the stream, then
+    `calls` calls of fn are enqueued behind it and timed by events on the
+    stream.  The events bracket GPU time only as long as the host has enqueued
+    every call before the GPU reaches it, which the blocker's length ensures
+    (16 calls x ~0.12 ms of Python against >= 4 ms of blocker)."""
+    e0 = torch.cuda.Event(enable_timing=True)
+    e1 = torch.cuda.Event(enable_timing=True)
+    for i in range(max(3, nsets)):
+        fn(i % nsets)
+    torch.cuda.synchronize()
+    times = []
+    k = 0
+    for _ in range(repeats):
+        blocker()
+        e0.record()
+        for _ in range(calls):
+            fn(k % nsets)
+            k += 1
+        e1.record()
+        torch.cuda.synchronize()
+        times.append(e0.elapsed_time(e1) / calls)
+    times.sort()
+    return times[len(times) // 2]
+
+
 def norm_buffers(torch, dev, n1, n2, nsets, seed):
     g = torch.Generator(device=dev).manual_seed(seed)
     sets = []
@@ -223,21 +258,19 @@ CHAIN = {
 }
 
 
-def staggered(torch, dev, shape, dtype, count, step=(1 << 20) + 4096):
-    """`count` tensors of `shape` carved from one allocation: tensor k starts
-    k * step bytes into its own 2 MiB-aligned slot.  The causal softmax backward
-    streams three 2 GB tensors at identical offsets; when all of them start on
-    the same 2 MiB phase their requests meet in the same memory channels and the
-    kernel runs 1.5-4 % slower (measured: 687-699 us staggered against 701-736 us
-    aligned, depending on the box), which of the two a plain allocation gives is
-    luck.  The other kernels show no such sensitivity."""
-    n = 1
-    for d in shape:
-        n *= d
-    nbytes = n * torch.empty(0, dtype=dtype).element_size()
-    slot = (nbytes + count * step + (2 << 20) - 1) // (2 << 20) * (2 << 20)
-    base = torch.empty(slot * count, dtype=torch.uint8, device=dev)
-    return [base[k * slot + k * step:k * slot + k * step + nbytes].view(dtype).view(*shape) for k in range(count)]
+def softmax_set(L, dev, shape, dtype, policy=True):
+    """The four tensors of a softmax forward + backward pair (x, y, dy, dx) laid
+    out as the product path lays them out: x and dy are what torch hands the
+    binding (plain allocations), y and dx are what the binding allocates, by
+    `_C.empty_staggered` on phases 1 and 2 of a 2 MiB period.  The causal
+    softmax backward streams three 2 GB tensors at identical offsets; when all
+    of them start on the same 2 MiB phase their requests meet in the same
+    memory channels and the kernel runs 1.5-4 % slower (687-699 us against
+    701-736 us, depending on the box).  `policy=False` gives four plain
+    allocations."""
+    torch = L.torch
+    mk = L._C.empty_staggered
+    return [mk(shape, dtype, dev, k if policy else 0) for k in (0, 1, 0, 2)]
 
 
 def chain_bytes():
@@ -274,7 +307,7 @@ def make_chain(L, dev):
           "invvar": torch.empty(n1, device=dev), "gamma": rnd(h, std=0.02, mean=1.0), "beta": rnd(h, std=0.02)}
     ln["dgamma"], ln["dbeta"] = torch.empty_like(ln["gamma"]), torch.empty_like(ln["beta"])
     ws_ln, ws_ln_b = L.ws(L._C.OSLO_OP_LN_BWD, n1, h, dev)
-    sm = dict(zip(("x", "y", "dy", "dx"), staggered(torch, dev, (ab, s, s), bf, 4)))
+    sm = dict(zip(("x", "y", "dy", "dx"), softmax_set(L, dev, (ab, s, s), bf)))
     sm["x"].normal_(generator=g)
     sm["dy"].normal_(generator=g)
     ge = {"x": rnd(n1, ff), "g": rnd(n1, ff), "bias": rnd(ff, std=0.02)}
@@ -382,7 +415,7 @@ def kernel_table(L, dev, iters, graph_column=True):
         g = torch.Generator(device=dev).manual_seed(2)
         bufs = []
         for _ in range(ns):
-            x, y, dy, dx = staggered(torch, dev, (ab, s, s), tdt, 4)
+            x, y, dy, dx = softmax_set(L, dev, (ab, s, s), tdt)
             x.normal_(generator=g)
             dy.normal_(generator=g)
             bufs.append((x, y, dy, dx))
@@ -396,7 +429,25 @@ def kernel_table(L, dev, iters, graph_column=True):
             L.ok(lib.oslo_softmax_causal_bwd(p(dy), p(y), p(dx), ab, s, s, scale, code, L.stream()))
 
         rows.append(table_row("softmax_causal_fwd", cfg, (1 + f) * T, timed(fwd, ns)))
-        rows.append(table_row("softmax_causal_bwd", cfg, (1 + 2 * f) * T, timed(bwd, ns)))
+        rows.append(table_row("softmax_causal_bwd", cfg, (1 + 2 * f) * T, timed(bwd, ns),
+                              note="y, dx placed by the binding's allocation policy" if cfg == "cfg5" else ""))
+        if cfg == "cfg5":
+            # the same launches on four plain torch allocations (all on one 2 MiB phase)
+            plain = softmax_set(L, dev, (ab, s, s), tdt, policy=False)
+            plain[0].copy_(bufs[0][0])
+            plain[2].copy_(bufs[0][2])
+
+            def pfwd(i):
+                L.ok(lib.oslo_softmax_causal_fwd(p(plain[0]), p(plain[1]), ab, s, s, scale, code, L.stream()))
+
+            def pbwd(i):
+                L.ok(lib.oslo_softmax_causal_bwd(p(plain[2]), p(plain[1]), p(plain[3]), ab, s, s, scale, code,
+                                                 L.stream()))
+
+            pfwd(0)
+            rows.append(table_row("softmax_causal_fwd", cfg, (1 + f) * T, timed(pfwd, 1), note="plain allocations"))
+            rows.append(table_row("softmax_causal_bwd", cfg, (1 + 2 * f) * T, timed(pbwd, 1), note="plain allocations"))
+            del plain
 
         # softmax with the attention dropout (p = 0.1) fused in: the same
         # compulsory bytes (backward reads the logits instead of the
@@ -444,7 +495,48 @@ def kernel_table(L, dev, iters, graph_column=True):
     t = timed(mbwd, ns)
     rows.append(table_row("softmax_masked_bwd", "cfg3", (2 * r + 1) * T, t,
                           note="valid %.4f, dense-equivalent %.0f GB/s" % (r, 3 * T / (t[0] * 1e-3) / 1e9)))
-    del bufs
+    # ---- the same configuration with the mask as the reference's models pass it:
+    # an additive fp16 term [16, 1, 1, 1024] (modeling_bert.py:298-306).  A fill
+    # of -10000 obliges the kernel to read every logit (a row whose keys are all
+    # filled is the softmax of the logits): forward 2T, backward 3T.  A fill of
+    # -inf hides the key for good: the loads are skipped as with the boolean
+    # mask.  And a dense fp16 position bias [1, 16, 1024, 1024]
+    # (modeling_t5.py:508-514), read once per batch entry: forward 2T + T/16. ----
+    pad = (torch.arange(s)[None, :] >= valid[:, None]).view(b, 1, 1, s).to(dev)
+    for fill, tag in ((-10000.0, "-10000"), (float("-inf"), "-inf")):
+        term = torch.zeros(b, 1, 1, s, dtype=torch.float16, device=dev).masked_fill_(pad, fill)
+        flags = 2  # OSLO_SOFTMAX_SKIP_HIDDEN, what the binding passes for a term shared by heads and queries
+        dense = fill == -10000.0
+
+        def bfwd(i):
+            x, y, dy, dx = bufs[i]
+            L.ok(lib.oslo_softmax_bias_fwd(p(x), p(term), p(y), b, h, s, s, s, 0, 0, F16, flags, 0.125, F16,
+                                           L.stream()))
+
+        def bbwd(i):
+            x, y, dy, dx = bufs[i]
+            L.ok(lib.oslo_softmax_bias_bwd(p(dy), p(y), p(term), p(dx), b, h, s, s, s, 0, 0, F16, flags, 0.125,
+                                           F16, L.stream()))
+
+        rows.append(table_row("softmax_bias_fwd", "cfg3", (2 if dense else r + 1) * T, timed(bfwd, ns),
+                              note="additive [16,1,1,1024] fp16 mask, fill %s" % tag))
+        rows.append(table_row("softmax_bias_bwd", "cfg3", (3 if dense else 2 * r + 1) * T, timed(bbwd, ns),
+                              note="additive [16,1,1,1024] fp16 mask, fill %s" % tag))
+    term = (2 * torch.randn(1, h, s, s, generator=g, device=dev)).to(torch.float16)
+
+    def tfwd(i):
+        x, y, dy, dx = bufs[i]
+        L.ok(lib.oslo_softmax_bias_fwd(p(x), p(term), p(y), b, h, s, s, 0, s * s, s, F16, 0, 0.125, F16, L.stream()))
+
+    def tbwd(i):
+        x, y, dy, dx = bufs[i]
+        L.ok(lib.oslo_softmax_bias_bwd(p(dy), p(y), None, p(dx), b, h, s, s, 0, 0, 0, F16, 0, 0.125, F16, L.stream()))
+
+    rows.append(table_row("softmax_bias_fwd", "cfg3", 2 * T + T / b, timed(tfwd, ns),
+                          note="position bias [1,16,1024,1024] fp16"))
+    rows.append(table_row("softmax_bias_bwd", "cfg3", 3 * T, timed(tbwd, ns),
+                          note="position bias [1,16,1024,1024] fp16"))
+    del bufs, term
     torch.cuda.empty_cache()
 
     # ---- causal + key-padding mask in one call, cfg5 shape [4,64,2048,2048]
@@ -457,7 +549,7 @@ def kernel_table(L, dev, iters, graph_column=True):
     qi = torch.arange(1, s + 1, dtype=torch.float64)
     r = float(torch.minimum(qi[None, :], valid[:, None].double()).mean()) / s
     mask = (torch.arange(s)[None, :] >= valid[:, None]).view(b, 1, 1, s).to(dev).view(torch.uint8)
-    x, y, dy, dx = staggered(torch, dev, (b, h, s, s), torch.bfloat16, 4)
+    x, y, dy, dx = softmax_set(L, dev, (b, h, s, s), torch.bfloat16)
     x.normal_(generator=g)
     dy.normal_(generator=g)
     sc = 1.0 / math.sqrt(96.0)
@@ -673,14 +765,138 @@ def kernel_table(L, dev, iters, graph_column=True):
     return rows
 
 
+def module_table(L, dev, iters, kernel_rows):
+    """Forward + backward through the public modules and functions of
+    oslo_amd.torch.nn with autograd -- what a user of the drop-in API runs:
+    the binding's checks, the output allocations by torch's caching allocator,
+    the saved tensors and the workspace cache are all inside the timed region
+    (`out = m(x); out.backward(g)` between events, rotating inputs).  Each row
+    carries the rate of the C-ABI pair of the kernel table and the ratio."""
+    torch = L.torch
+    import oslo_amd.torch.nn as onn
+    from oslo_amd.torch.nn.modules.softmax import AttnMaskType
+
+    bf = torch.bfloat16
+    rows = []
+    # ~5 ms of GPU work for time_queued: copies of a 2 GiB buffer
+    blk_src = torch.empty(1 << 31, dtype=torch.uint8, device=dev)
+    blk_dst = torch.empty(1 << 31, dtype=torch.uint8, device=dev)
+
+    def blocker():
+        for _ in range(8):
+            blk_dst.copy_(blk_src, non_blocking=True)
+
+    def abi_rate(names, cfg, note=None, exclude=None):
+        sel = [r for r in kernel_rows if r[0] in names and r[1] == cfg and (note is None or r[9] == note)
+               and (exclude is None or r[9] != exclude)]
+        if len(sel) != len(names):
+            return None
+        return sum(r[2] for r in sel) / sum(r[3] for r in sel) * 1e3  # MB / us -> GB/s
+
+    def run(name, cfg, nbytes, params, make_inputs, call, nsets, abi):
+        g = torch.Generator(device=dev).manual_seed(7)
+        sets = [make_inputs(g) for _ in range(nsets)]
+        leaves = list(params)
+
+        def fn(i):
+            inputs, grad = sets[i]
+            for t in leaves:
+                t.grad = None
+            for t in inputs:
+                if t.requires_grad:
+                    t.grad = None
+            call(*inputs).backward(grad)
+
+        t = time_launches(torch, fn, iters, nsets)
+        gbps = nbytes / (t[0] * 1e-3) / 1e9
+        # the same eager calls enqueued behind a few ms of other GPU work, so that the
+        # host runs ahead: a call costs the host 90-130 us of Python per forward +
+        # backward (autograd.Function, ctypes), more than the shorter kernels run, and
+        # a loop of nothing but such calls measures Python, not the GPU
+        tq = time_queued(torch, fn, nsets, blocker)
+        qgbps = nbytes / (tq * 1e-3) / 1e9
+        rows.append({
+            "module": name, "cfg": cfg, "MB": round(nbytes / 1e6, 1), "us": round(t[0] * 1e3, 2),
+            "us_med": round(t[1] * 1e3, 2), "us_min": round(t[2] * 1e3, 2), "GBps": round(gbps, 1),
+            "frac": round(gbps / HBM_PEAK_GBPS, 4),
+            "queued_us": round(tq * 1e3, 2), "queued_GBps": round(qgbps, 1),
+            "queued_frac": round(qgbps / HBM_PEAK_GBPS, 4),
+            "c_abi_GBps": None if abi is None else round(abi, 1),
+            "ratio_to_c_abi": None if abi is None else round(gbps / abi, 4),
+            "queued_ratio_to_c_abi": None if abi is None else round(qgbps / abi, 4),
+        })
+        del sets
+        torch.cuda.empty_cache()
+
+    def act(n1, n2):
+        def make(g):
+            x = torch.randn(n1, n2, generator=g, device=dev).to(bf).requires_grad_()
+            return (x,), torch.randn(n1, n2, generator=g, device=dev).to(bf)
+        return make
+
+    # LayerNorm / RMSNorm at cfg2, LayerNorm at cfg5
+    for cfg, n1, n2, kinds in (("cfg2", 16384, 4096, ("ln", "rms")), ("cfg5", 8192, 6144, ("ln",))):
+        T = n1 * n2 * 2
+        for kind in kinds:
+            m = (onn.FusedLayerNorm if kind == "ln" else onn.FusedRMSNorm)(n2, eps=1e-5).to(dev).to(bf)
+            with torch.no_grad():
+                m.weight.normal_(1.0, 0.02)
+                if kind == "ln":
+                    m.bias.normal_(0.0, 0.02)
+            run("FusedLayerNorm" if kind == "ln" else "FusedRMSNorm", cfg, 5 * T, list(m.parameters()), act(n1, n2),
+                m, nsets_for(4 * T), abi_rate(("%s_fwd" % kind, "%s_bwd" % kind), cfg))
+
+    # the four stages of cfg5
+    c = CHAIN
+    n1, hdim, heads, s, ff = c["tokens"], c["hidden"], 64, c["seq"], c["ffn"]
+    f = (s + 1) / (2.0 * s)
+    T = 4 * heads * s * s * 2
+    sm = onn.FusedScaleMaskSoftmax(input_in_bf16=True, attn_mask_type=AttnMaskType.causal, scale=c["scale"])
+
+    def make_scores(g):
+        x = torch.empty(4, heads, s, s, device=dev, dtype=bf).normal_(generator=g).requires_grad_()
+        return (x,), torch.empty(4, heads, s, s, device=dev, dtype=bf).normal_(generator=g)
+
+    run("FusedScaleMaskSoftmax(causal)", "cfg5", (2 + 3 * f) * T, [], make_scores, lambda x: sm(x, None), 1,
+        abi_rate(("softmax_causal_fwd", "softmax_causal_bwd"), "cfg5", exclude="plain allocations"))
+
+    T = n1 * ff * 2
+    bias_ff = (0.02 * torch.randn(ff, device=dev)).to(bf).requires_grad_()
+    run("fused_bias_gelu", "cfg5", 5 * T, [bias_ff], act(n1, ff), lambda x: onn.fused_bias_gelu(x, bias_ff),
+        nsets_for(4 * T), abi_rate(("bias_gelu_fwd", "bias_gelu_bwd"), "cfg5"))
+
+    T = n1 * hdim * 2
+    bias_h = (0.02 * torch.randn(hdim, device=dev)).to(bf).requires_grad_()
+
+    def make_bda(g):
+        x = torch.randn(n1, hdim, generator=g, device=dev).to(bf).requires_grad_()
+        res = torch.randn(n1, hdim, generator=g, device=dev).to(bf)
+        return (x, res), torch.randn(n1, hdim, generator=g, device=dev).to(bf)
+
+    run("fused_bias_dropout_add", "cfg5", 5 * T, [bias_h], make_bda,
+        lambda x, res: onn.fused_bias_dropout_add(x, bias_h, res, c["p"], True), nsets_for(5 * T),
+        abi_rate(("bias_dropout_add_fwd", "bias_dropout_add_bwd"), "cfg5", "p=0.1"))
+    return rows
+
+
 def cpu_model():
+    """Model string of the host CPU with family / model / stepping (a virtual
+    machine may shorten the name) and the number of logical CPUs."""
+    fields = {}
     try:
         for line in open("/proc/cpuinfo"):
-            if line.startswith("model name"):
-                return line.split(":", 1)[1].strip()
+            if ":" in line:
+                k, v = line.split(":", 1)
+                k = k.strip()
+                if k in ("model name", "cpu family", "model", "stepping", "vendor_id") and k not in fields:
+                    fields[k] = v.strip()
     except OSError:
         pass
-    return "unknown"
+    if not fields:
+        return "unknown"
+    return "%s (%s family %s model %s stepping %s), %d logical CPUs" % (
+        fields.get("model name", "?"), fields.get("vendor_id", "?"), fields.get("cpu family", "?"),
+        fields.get("model", "?"), fields.get("stepping", "?"), os.cpu_count() or 0)
 
 
 def cpu_baseline(budget_s=4.0):
@@ -718,37 +934,36 @@ def cpu_baseline(budget_s=4.0):
     stages, measured, runs = [], [0.0], []
     # LayerNorm: the whole [8192, 6144] tensor (a smaller sample would stay in the host caches)
     n1, h = c["tokens"], c["hidden"]
-    x, dy = rnd((n1, h)), rnd((n1, h))
-    gamma, beta = rnd((h,), 0.02, 1.0), rnd((h,), 0.02)
+    x, dy = rnd((n1, h)).requires_grad_(), rnd((n1, h))
+    gamma, beta = rnd((h,), 0.02, 1.0).requires_grad_(), rnd((h,), 0.02).requires_grad_()
 
     def ln():
-        xr = x.clone().requires_grad_()
-        w, b = gamma.clone().requires_grad_(), beta.clone().requires_grad_()
-        tp.layer_norm(xr, w, b, 1e-5).backward(dy)
+        x.grad = gamma.grad = beta.grad = None  # (no copy of an input inside the timed function)
+        tp.layer_norm(x, gamma, beta, 1e-5).backward(dy)
     stages.append(("layer_norm", "[8192,6144] (all)", timed(ln), 1.0))
     # causal softmax: 32 of the 256 attention batches
     s = c["seq"]
-    xs, ds = rnd((32, s, s)), rnd((32, s, s))
+    xs, ds = rnd((32, s, s)).requires_grad_(), rnd((32, s, s))
 
     def sm():
-        xr = xs.clone().requires_grad_()
-        tp.causal_softmax(xr, c["scale"]).backward(ds)
+        xs.grad = None
+        tp.causal_softmax(xs, c["scale"]).backward(ds)
     stages.append(("softmax_causal", "[32,2048,2048] of 256 batches", timed(sm), c["attn_batches"] / 32.0))
     del xs, ds
     # bias-GeLU: 4096 of the 8192 rows
-    xg, dg, bg = rnd((4096, c["ffn"])), rnd((4096, c["ffn"])), rnd((c["ffn"],), 0.02)
+    xg, dg, bg = rnd((4096, c["ffn"])).requires_grad_(), rnd((4096, c["ffn"])), rnd((c["ffn"],), 0.02).requires_grad_()
 
     def ge():
-        xr, br = xg.clone().requires_grad_(), bg.clone().requires_grad_()
-        tp.bias_gelu(xr, br).backward(dg)
+        xg.grad = bg.grad = None
+        tp.bias_gelu(xg, bg).backward(dg)
     stages.append(("bias_gelu", "[4096,24576] of 8192 rows", timed(ge), n1 / 4096.0))
     del xg, dg
     # bias-dropout-add: the whole [8192, 6144] tensor
-    xb, rb, db, bb = rnd((n1, h)), rnd((n1, h)), rnd((n1, h)), rnd((h,), 0.02)
+    xb, rb, db, bb = rnd((n1, h)).requires_grad_(), rnd((n1, h)), rnd((n1, h)), rnd((h,), 0.02).requires_grad_()
 
     def bd():
-        xr, br = xb.clone().requires_grad_(), bb.clone().requires_grad_()
-        tp.bias_dropout_add(xr, br, rb, c["p"], True).backward(db)
+        xb.grad = bb.grad = None
+        tp.bias_dropout_add(xb, bb, rb, c["p"], True).backward(db)
     stages.append(("bias_dropout_add", "[8192,6144] (all)", timed(bd), 1.0))
 
     full_s = sum(t * k for _, _, t, k in stages)
@@ -817,53 +1032,52 @@ def cpu_path_table(gpu_rows, budget_s=3.0):
         })
 
     def causal(cfg, ab, s, dtype, scale, esz):
-        x, dy = rnd((ab, s, s), dtype), rnd((ab, s, s), dtype)
+        x, dy = rnd((ab, s, s), dtype).requires_grad_(), rnd((ab, s, s), dtype)
         f = (s + 1) / (2.0 * s)
 
         def fn():
-            xr = x.clone().requires_grad_()
-            tp.causal_softmax(xr, scale).backward(dy)
+            x.grad = None  # (no copy of an input inside the timed function)
+            tp.causal_softmax(x, scale).backward(dy)
         entry("softmax_causal fwd+bwd", cfg, "[%d,%d,%d] %s" % (ab, s, s, str(dtype).split(".")[-1]),
               (2 + 3 * f) * ab * s * s * esz, fn,
               gpu_rate(("softmax_causal_fwd", "softmax_causal_bwd"), cfg))
 
     def norm_ln(cfg, n1, n2):
-        x, dy = rnd((n1, n2), BF16), rnd((n1, n2), BF16)
-        gamma, beta = rnd((n2,), BF16, 0.02) + 1, rnd((n2,), BF16, 0.02)
+        x, dy = rnd((n1, n2), BF16).requires_grad_(), rnd((n1, n2), BF16)
+        gamma, beta = (rnd((n2,), BF16, 0.02) + 1).requires_grad_(), rnd((n2,), BF16, 0.02).requires_grad_()
 
         def fn():
-            xr = x.clone().requires_grad_()
-            w, b = gamma.clone().requires_grad_(), beta.clone().requires_grad_()
-            tp.layer_norm(xr, w, b, 1e-5).backward(dy)
+            x.grad = gamma.grad = beta.grad = None
+            tp.layer_norm(x, gamma, beta, 1e-5).backward(dy)
         entry("layer_norm fwd+bwd", cfg, "[%d,%d] bf16" % (n1, n2), 5 * n1 * n2 * 2, fn,
               gpu_rate(("ln_fwd", "ln_bwd"), cfg))
 
     def norm_rms(cfg, n1, n2):
-        x, dy = rnd((n1, n2), BF16), rnd((n1, n2), BF16)
-        gamma = rnd((n2,), BF16, 0.02) + 1
+        x, dy = rnd((n1, n2), BF16).requires_grad_(), rnd((n1, n2), BF16)
+        gamma = (rnd((n2,), BF16, 0.02) + 1).requires_grad_()
 
         def fn():
-            xr = x.clone().requires_grad_()
-            w = gamma.clone().requires_grad_()
-            tp.rms_norm(xr, w, 1e-5).backward(dy)
+            x.grad = gamma.grad = None
+            tp.rms_norm(x, gamma, 1e-5).backward(dy)
         entry("rms_norm fwd+bwd", cfg, "[%d,%d] bf16" % (n1, n2), 5 * n1 * n2 * 2, fn,
               gpu_rate(("rms_fwd", "rms_bwd"), cfg))
 
     def gelu(cfg, n1, n2):
-        x, dy, b = rnd((n1, n2), BF16), rnd((n1, n2), BF16), rnd((n2,), BF16, 0.02)
+        x, dy, b = rnd((n1, n2), BF16).requires_grad_(), rnd((n1, n2), BF16), rnd((n2,), BF16, 0.02).requires_grad_()
 
         def fn():
-            xr, br = x.clone().requires_grad_(), b.clone().requires_grad_()
-            tp.bias_gelu(xr, br).backward(dy)
+            x.grad = b.grad = None
+            tp.bias_gelu(x, b).backward(dy)
         entry("bias_gelu fwd+bwd", cfg, "[%d,%d] bf16" % (n1, n2), 5 * n1 * n2 * 2, fn,
               gpu_rate(("bias_gelu_fwd", "bias_gelu_bwd"), cfg))
 
     def bda(cfg, n1, n2):
-        x, res, dy, b = rnd((n1, n2), BF16), rnd((n1, n2), BF16), rnd((n1, n2), BF16), rnd((n2,), BF16, 0.02)
+        x, res, dy = rnd((n1, n2), BF16).requires_grad_(), rnd((n1, n2), BF16), rnd((n1, n2), BF16)
+        b = rnd((n2,), BF16, 0.02).requires_grad_()
 
         def fn():
-            xr, br = x.clone().requires_grad_(), b.clone().requires_grad_()
-            tp.bias_dropout_add(xr, br, res, 0.1, True).backward(dy)
+            x.grad = b.grad = None
+            tp.bias_dropout_add(x, b, res, 0.1, True).backward(dy)
         entry("bias_dropout_add fwd+bwd (p=0.1)", cfg, "[%d,%d] bf16" % (n1, n2), 5 * n1 * n2 * 2, fn,
               gpu_rate(("bias_dropout_add_fwd", "bias_dropout_add_bwd"), cfg, "p=0.1"))
 
@@ -872,14 +1086,14 @@ def cpu_path_table(gpu_rows, budget_s=3.0):
     norm_rms("cfg2", 16384, 4096)
     # cfg3: two of the sixteen batch entries
     b_, h, s = 2, 16, 1024
-    x, dy = rnd((b_, h, s, s), F16, 2.0), rnd((b_, h, s, s), F16)
+    x, dy = rnd((b_, h, s, s), F16, 2.0).requires_grad_(), rnd((b_, h, s, s), F16)
     valid = torch.tensor([1024, 640])
     pad = torch.arange(s)[None, :] >= valid[:, None]
     r = float(valid.double().mean()) / s
 
     def masked():
-        xr = x.clone().requires_grad_()
-        tp.padding_softmax(xr, pad, 0.125).backward(dy)
+        x.grad = None
+        tp.padding_softmax(x, pad, 0.125).backward(dy)
     entry("softmax_masked fwd+bwd", "cfg3", "[2,16,1024,1024] fp16 of batch 16", (2 + 3 * r) * x.numel() * 2,
           masked, gpu_rate(("softmax_masked_fwd", "softmax_masked_bwd"), "cfg3"))
     del x, dy
@@ -1001,6 +1215,16 @@ def main():
                      "graph_us = per launch inside a captured HIP graph; mt_* = multi-tensor optimizer steps over "
                      "192 tensors; copy_probe = a plain copy" % (args.table_iters, BATCHES),
             "rows": rows,
+        }
+        out["modules"] = {
+            "what": "forward + backward through oslo_amd.torch.nn with autograd (out = m(x); out.backward(g) between "
+                    "events on the launch stream, rotating inputs, gradients cleared to None before each call); MB = "
+                    "algorithmic bytes of the pair; c_abi_GBps = the same pair through the raw C ABI on pre-allocated "
+                    "buffers (kernel table); ratio_to_c_abi = GBps / c_abi_GBps; us / GBps = a loop of nothing but "
+                    "these calls (bound by the 90-130 us of Python per call where the kernels are shorter); queued_* "
+                    "= the same eager calls enqueued behind ~5 ms of other GPU work, so that the host runs ahead of "
+                    "the GPU as it does in a training step (events on the stream bracket the calls' GPU time)",
+            "rows": module_table(L, dev, max(20, args.table_iters // 2), rows),
         }
     if not args.no_cpu_baseline:
         cb = cpu_baseline()

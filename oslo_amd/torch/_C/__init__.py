@@ -718,6 +718,39 @@ class _LayerNormKernel:
 # ---------------------------------------------------------------------------
 # scaled masked softmax
 # ---------------------------------------------------------------------------
+# The softmax backward streams three tensors of gigabytes at identical offsets
+# (y, dy -> dx).  torch places large tensors on 2 MiB boundaries; when all three
+# start on the same 2 MiB phase their requests meet in the same memory channels
+# and the kernel measures 1.5-4 % slower on MI355X than with the starts a little
+# over 1 MiB apart.  The tensors this binding allocates for the softmax (the
+# probabilities in forward, the input gradient in backward) are therefore placed
+# on phase k * (1 MiB + 4 KiB) of their own 2 MiB-rounded allocation, k = 1 for
+# forward outputs and k = 2 for backward outputs; operands that torch allocated
+# (the scores, the incoming gradient) sit on phase 0.
+STAGGER_MIN_BYTES = 64 << 20
+STAGGER_STEP = (1 << 20) + 4096
+_STAGGER_ROUND = 2 << 20
+
+
+def empty_staggered(shape, dtype, device, k):
+    """An uninitialised contiguous tensor whose first byte lies k * STAGGER_STEP
+    (modulo 2 MiB) past a 2 MiB boundary; small tensors and k == 0 are plain
+    ``torch.empty``.  Costs 2 MiB of slack per tensor."""
+    n = 1
+    for d in shape:
+        n *= int(d)
+    nbytes = n * torch.empty(0, dtype=dtype).element_size()
+    if k == 0 or nbytes < STAGGER_MIN_BYTES:
+        return torch.empty(tuple(shape), dtype=dtype, device=device)
+    base = torch.empty(nbytes + _STAGGER_ROUND, dtype=torch.uint8, device=device)
+    off = (k * STAGGER_STEP - base.data_ptr()) % _STAGGER_ROUND
+    return base[off:off + nbytes].view(dtype).view(tuple(shape))
+
+
+def _softmax_out(like, k):
+    return empty_staggered(like.shape, like.dtype, like.device, k)
+
+
 class _SoftmaxKernel:
     """The five functions of ``FusedScaleMaskSoftmaxBinder.cpp:111-127``.
 
@@ -751,7 +784,7 @@ class _SoftmaxKernel:
         b, np_, sq, sk, mb, msq = self._masked_dims(input, mask)
         _check_input(input, "input")
         m8 = self._mask_u8(mask, input)
-        out = torch.empty_like(input)
+        out = _softmax_out(input, 1)
         with _device_of(input):
             fn = lib.oslo_softmax_causal_masked_fwd if causal else lib.oslo_softmax_masked_fwd
             rc = fn(
@@ -782,7 +815,7 @@ class _SoftmaxKernel:
             m8 = self._mask_u8(mask, softmax_results)
         # inplace=True overwrites output_grads, as the kernel this shim was
         # written for does
-        grad_input = output_grads if inplace else torch.empty_like(output_grads)
+        grad_input = output_grads if inplace else _softmax_out(output_grads, 2)
         with _device_of(output_grads):
             fn = lib.oslo_softmax_causal_masked_bwd if causal else lib.oslo_softmax_masked_bwd
             rc = fn(
@@ -808,7 +841,7 @@ class _SoftmaxKernel:
             raise RuntimeError("expected 3D tensor")
         _check_input(input, "input")
         ab, sq, sk = input.shape
-        out = torch.empty_like(input)
+        out = _softmax_out(input, 1)
         with _device_of(input):
             rc = lib.oslo_softmax_causal_fwd(
                 _ptr(input), _ptr(out), ab, sq, sk, float(scale_factor),
@@ -830,7 +863,7 @@ class _SoftmaxKernel:
         if output_grads.shape != softmax_results.shape:
             raise RuntimeError("output_grads and softmax_results differ in shape")
         ab, sq, sk = softmax_results.shape
-        grad_input = output_grads if inplace else torch.empty_like(output_grads)
+        grad_input = output_grads if inplace else _softmax_out(output_grads, 2)
         with _device_of(output_grads):
             rc = lib.oslo_softmax_causal_bwd(
                 _ptr(output_grads), _ptr(softmax_results), _ptr(grad_input), ab, sq, sk,
@@ -866,7 +899,7 @@ class _SoftmaxKernel:
         """
         lib = self._lib
         _check_input(input, "input")
-        out = torch.empty_like(input)
+        out = _softmax_out(input, 1)
         rows = input.numel() // input.shape[-1] if input.numel() else 0
         stats = torch.empty((rows, 2), dtype=torch.float32, device=input.device)
         with _device_of(input):
@@ -905,7 +938,7 @@ class _SoftmaxKernel:
         rows = input.numel() // input.shape[-1] if input.numel() else 0
         if stats.dtype != torch.float32 or stats.numel() != 2 * rows:
             raise RuntimeError("stats must be float32 [rows, 2]")
-        grad_input = output_grads if inplace else torch.empty_like(output_grads)
+        grad_input = output_grads if inplace else _softmax_out(output_grads, 2)
         with _device_of(input):
             if mask is None:
                 if input.dim() != 3:
@@ -993,7 +1026,7 @@ class _SoftmaxKernel:
         _check_input(input, "input")
         bias, sb, sh, sq_, bcode = self._bias_operand(bias, input)
         b, np_, sq, sk = input.shape
-        out = torch.empty_like(input)
+        out = _softmax_out(input, 1)
         flags = self._bias_flags(causal, skip_hidden, (sb, sh, sq_))
         with _device_of(input):
             rc = lib.oslo_softmax_bias_fwd(
@@ -1027,7 +1060,7 @@ class _SoftmaxKernel:
             flags = self._bias_flags(causal, skip_hidden, (sb, sh, sq_))
             if not flags & 2:
                 bias = None
-        grad_input = output_grads if inplace else torch.empty_like(output_grads)
+        grad_input = output_grads if inplace else _softmax_out(output_grads, 2)
         with _device_of(output_grads):
             rc = lib.oslo_softmax_bias_bwd(
                 _ptr(output_grads), _ptr(softmax_results), _ptr(bias), _ptr(grad_input),
@@ -1045,7 +1078,7 @@ class _SoftmaxKernel:
         _check_input(input, "input")
         bias, sb, sh, sq_, bcode = self._bias_operand(bias, input)
         b, np_, sq, sk = input.shape
-        out = torch.empty_like(input)
+        out = _softmax_out(input, 1)
         stats = torch.empty((b * np_ * sq, 2), dtype=torch.float32, device=input.device)
         flags = self._bias_flags(causal, skip_hidden, (sb, sh, sq_))
         with _device_of(input):
@@ -1072,7 +1105,7 @@ class _SoftmaxKernel:
         if stats.dtype != torch.float32 or stats.numel() != 2 * b * np_ * sq:
             raise RuntimeError("stats must be float32 [rows, 2]")
         flags = self._bias_flags(causal, skip_hidden, (sb, sh, sq_))
-        grad_input = output_grads if inplace else torch.empty_like(output_grads)
+        grad_input = output_grads if inplace else _softmax_out(output_grads, 2)
         with _device_of(input):
             rc = lib.oslo_softmax_bias_dropout_bwd(
                 _ptr(output_grads), _ptr(input), _ptr(bias), _ptr(stats), _ptr(grad_input),
