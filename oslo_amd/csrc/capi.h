@@ -8,6 +8,7 @@
 #include <stdio.h>
 
 #include "../../include/oslo_hip.h"
+#include "../../include/oslo_hip_testing.h"
 
 namespace oslo {
 

@@ -1,5 +1,5 @@
 """The C-ABI library loads on a machine without a GPU and exports every symbol
-that include/oslo_hip.h declares; argument validation that needs no device is
+that include/oslo_hip.h and include/oslo_hip_testing.h declare; argument validation that needs no device is
 exercised too (no kernel is launched here)."""
 import os
 import re
@@ -11,10 +11,20 @@ from oslo_amd.torch import _C
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
-def declared_symbols():
-    text = open(os.path.join(ROOT, "include", "oslo_hip.h")).read()
-    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
-    return sorted(set(re.findall(r"\b(oslo_[a-z0-9_]+)\s*\(", text)))
+def declared_symbols(header=None):
+    """Symbols declared by the production header, the testing header, or both."""
+    names = []
+    for h in ([header] if header else ["oslo_hip.h", "oslo_hip_testing.h"]):
+        text = open(os.path.join(ROOT, "include", h)).read()
+        text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+        names += re.findall(r"\b(oslo_[a-z0-9_]+)\s*\(", text)
+    return sorted(set(names))
+
+
+def test_test_hooks_live_in_their_own_header():
+    hooks = {"oslo_tune", "oslo_copy_probe", "oslo_philox_words", "oslo_wave_reduce_selftest"}
+    assert set(declared_symbols("oslo_hip_testing.h")) == hooks
+    assert not hooks & set(declared_symbols("oslo_hip.h"))
 
 
 def test_header_and_loader_agree():

@@ -152,6 +152,70 @@ def test_padding_softmax_full_size(device):
     check(dxb, cf.softmax_bwd(f64(gb), f64(yb), scale), "cfg3 bwd rows", atol=1e-7)
 
 
+# --------------------------------------------------------------------------- cfg3 with the mask as an additive term
+@pytest.mark.parametrize("kind", ["m10000", "inf", "position_bias"])
+def test_additive_term_softmax_full_size(device, kind):
+    """Configuration 3 with its mask in the form the reference's models pass
+    it, an additive fp16 term [16, 1, 1, 1024] (-10000 as in
+    oslo/transformers/models/bert/modeling_bert.py:298-306, and -inf), and with
+    a dense position bias [1, 16, 1024, 1024]
+    (oslo/transformers/models/t5/modeling_t5.py:508-514); with the dropout of
+    the probabilities fused in as well."""
+    b, h, s = 16, 16, 1024
+    scale = 0.125
+    x = gpu_randn((b, h, s, s), F16, 3, device, std=2.0)
+    g = gpu_randn((b, h, s, s), F16, 4, device)
+    valid = torch.randint(256, 1025, (b,), generator=torch.Generator().manual_seed(3))
+    pad = torch.arange(s)[None, :] >= valid[:, None]
+    if kind == "position_bias":
+        term = gpu_randn((1, h, s, s), F16, 5, device, std=2.0)
+    else:
+        fill = -10000.0 if kind == "m10000" else float("-inf")
+        term = torch.zeros(b, 1, 1, s, dtype=F16).masked_fill_(pad.view(b, 1, 1, s), fill).to(device)
+    k = _C.get_softmax_kernel()
+    y = k.softmax_bias_forward(x, term, scale)
+    dx = k.softmax_bias_backward(g, y, scale, bias=term)
+    assert torch.equal(dx, k.softmax_bias_backward(g, y, scale))
+    for bi in range(b):
+        yb = y[bi].float()
+        assert (yb.sum(-1) - 1).abs().max().item() <= 2e-3
+        if kind != "position_bias":
+            assert yb[..., int(valid[bi]):].count_nonzero().item() == 0
+            assert dx[bi][..., int(valid[bi]):].count_nonzero().item() == 0
+        gscale = g[bi].float().abs().amax(-1) * scale
+        assert (dx[bi].float().sum(-1).abs() <= 8e-3 * gscale + 1e-6).all()
+    rows = sample_rows(b * h * s)
+    sel = rows.to(device)
+    xb, yb = x.view(-1, s)[sel].cpu(), y.view(-1, s)[sel].cpu()
+    gb, dxb = g.view(-1, s)[sel].cpu(), dx.view(-1, s)[sel].cpu()
+    bi, hi, qi = rows // (h * s), (rows // s) % h, rows % s
+    tb = term.cpu()[0, hi, qi] if kind == "position_bias" else term.cpu()[bi, 0, 0]
+    check(yb, cf.softmax_bias_fwd(f64(xb), f64(tb), scale), kind + " fwd rows", atol=1e-9)
+    check(dxb, cf.softmax_bwd(f64(gb), f64(yb), scale), kind + " bwd rows", atol=1e-7)
+    if kind != "position_bias":
+        # the boolean-mask kernel on the same padding gives the same probabilities
+        # (the two keep their logits in different domains: equal to an ulp)
+        ym = k.fused_scaled_masked_softmax_forward(x, pad.view(b, 1, 1, s).to(device), scale)
+        assert (y.float() - ym.float()).abs().max().item() <= 2.0 ** -10
+        assert torch.equal(y == 0, ym == 0)
+        del ym
+    del dx, y
+    p, seed, offset = 0.1, 321, 12
+    out, stats = k.softmax_bias_dropout_forward(x, term, scale, p, seed, offset)
+    dxd = k.softmax_bias_dropout_backward(g, x, term, stats, scale, p, seed, offset)
+    ob, dxb = out.view(-1, s)[sel].cpu(), dxd.view(-1, s)[sel].cpu()
+    keep_rows = np.stack(
+        [philox.keep_mask(s, p, seed, offset, first_element=int(r) * s) for r in rows]
+    ).astype(bool)
+    check(ob, cf.softmax_bias_dropout_fwd(f64(xb), f64(tb), scale, keep_rows, p), kind + " dropout fwd rows",
+          atol=1e-9)
+    check(dxb, cf.softmax_bias_dropout_bwd(f64(gb), f64(xb), f64(tb), scale, keep_rows, p),
+          kind + " dropout bwd rows", atol=2e-7)
+    keep = _C.get_fused_elementwise_kernel().philox_mask(x.numel(), p, seed, offset, device).view(b, h, s, s)
+    for bi in range(0, b, 4):
+        assert out[bi:bi + 4][~keep[bi:bi + 4].bool()].count_nonzero().item() == 0
+
+
 # --------------------------------------------------------------------------- cfg5 shape, causal + key padding
 def test_causal_padding_softmax_full_size(device):
     """The attention of a causal model on a padded batch

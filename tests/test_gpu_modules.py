@@ -68,6 +68,38 @@ def test_norm_module_cpu_vs_gpu(device, cls, affine, dtype, contiguous):
             check(gpu.bias.grad, f64(cpu.bias.grad), "module dbias", atol=1e-4, min_exact=0.9)
 
 
+@pytest.mark.parametrize("cls", [onn.FusedLayerNorm, onn.FusedRMSNorm])
+@pytest.mark.parametrize("dtype", [F32, BF16])
+def test_norm_module_cpu_vs_gpu_large_batch(device, cls, dtype):
+    """The reference's large case, tests_deprecated/torch/_C/csrc/
+    test_fused_layer_norm.py:104-108: batch 65 536 of normalized_shape [32, 16]
+    (33.5 M elements), the module on the CPU in float64 against the module on
+    the GPU, forward and every gradient."""
+    shape = [32, 16]
+    batch = 65536
+    torch.manual_seed(7)
+    cpu = cls(shape)
+    gpu = cls(shape)
+    with torch.no_grad():
+        cpu.weight.copy_(randn(shape, dtype, 1, std=0.1, mean=1.0))
+        if getattr(cpu, "bias", None) is not None:
+            cpu.bias.copy_(randn(shape, dtype, 2, std=0.1))
+    gpu.load_state_dict(cpu.state_dict())
+    gpu = gpu.to(device=device, dtype=dtype)
+    x = randn([batch] + shape, dtype, 3)
+    dy = randn([batch] + shape, dtype, 4)
+    xc, yc, xg, yg = run_pair(cpu, gpu, x, dy, device)
+    rms16 = cls is onn.FusedRMSNorm and dtype != F32
+    check(yg, f64(yc), "module fwd", atol=2e-6, max_ulp=2 if rms16 else 1, min_exact=0.6 if rms16 else 0.998,
+          l2_tol=4e-3 if rms16 else 2e-3)
+    check(xg.grad, f64(xc.grad), "module dx", atol=4e-6)
+    # column sums over 65 536 rows: float32 accumulation of rounded terms against float64
+    patol = 1e-5 * (batch ** 0.5) + 1e-4
+    check(gpu.weight.grad, f64(cpu.weight.grad), "module dweight", atol=patol, min_exact=0.9)
+    if getattr(gpu, "bias", None) is not None:
+        check(gpu.bias.grad, f64(cpu.bias.grad), "module dbias", atol=patol, min_exact=0.9)
+
+
 @pytest.mark.parametrize("cls", [onn.MixedFusedLayerNorm, onn.MixedFusedRMSNorm])
 def test_mixed_modules_return_parameter_dtype(device, cls):
     m = cls(64).to(device=device, dtype=BF16)
