@@ -499,26 +499,29 @@ def kernel_table(L, dev, iters, graph_column=True):
     # an additive fp16 term [16, 1, 1, 1024] (modeling_bert.py:298-306).  A fill
     # of -10000 obliges the kernel to read every logit (a row whose keys are all
     # filled is the softmax of the logits): forward 2T, backward 3T.  A fill of
-    # -inf hides the key for good: the loads are skipped as with the boolean
-    # mask.  And a dense fp16 position bias [1, 16, 1024, 1024]
+    # -inf hides the key for good: the backward pass skips its loads as with the
+    # boolean mask (the forward pass reads every logit either way, see the
+    # binding).  And a dense fp16 position bias [1, 16, 1024, 1024]
     # (modeling_t5.py:508-514), read once per batch entry: forward 2T + T/16. ----
     pad = (torch.arange(s)[None, :] >= valid[:, None]).view(b, 1, 1, s).to(dev)
     for fill, tag in ((-10000.0, "-10000"), (float("-inf"), "-inf")):
         term = torch.zeros(b, 1, 1, s, dtype=torch.float16, device=dev).masked_fill_(pad, fill)
-        flags = 2  # OSLO_SOFTMAX_SKIP_HIDDEN, what the binding passes for a term shared by heads and queries
+        # what the binding passes for a term shared by heads and queries: the logits of a forward
+        # pass are always read (waiting for the term costs more than the unread logits save), the
+        # backward pass skips hidden chunks (OSLO_SOFTMAX_SKIP_HIDDEN)
         dense = fill == -10000.0
 
         def bfwd(i):
             x, y, dy, dx = bufs[i]
-            L.ok(lib.oslo_softmax_bias_fwd(p(x), p(term), p(y), b, h, s, s, s, 0, 0, F16, flags, 0.125, F16,
+            L.ok(lib.oslo_softmax_bias_fwd(p(x), p(term), p(y), b, h, s, s, s, 0, 0, F16, 0, 0.125, F16,
                                            L.stream()))
 
         def bbwd(i):
             x, y, dy, dx = bufs[i]
-            L.ok(lib.oslo_softmax_bias_bwd(p(dy), p(y), p(term), p(dx), b, h, s, s, s, 0, 0, F16, flags, 0.125,
+            L.ok(lib.oslo_softmax_bias_bwd(p(dy), p(y), p(term), p(dx), b, h, s, s, s, 0, 0, F16, 2, 0.125,
                                            F16, L.stream()))
 
-        rows.append(table_row("softmax_bias_fwd", "cfg3", (2 if dense else r + 1) * T, timed(bfwd, ns),
+        rows.append(table_row("softmax_bias_fwd", "cfg3", 2 * T, timed(bfwd, ns),
                               note="additive [16,1,1,1024] fp16 mask, fill %s" % tag))
         rows.append(table_row("softmax_bias_bwd", "cfg3", (3 if dense else 2 * r + 1) * T, timed(bbwd, ns),
                               note="additive [16,1,1,1024] fp16 mask, fill %s" % tag))

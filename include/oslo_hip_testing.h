@@ -37,7 +37,10 @@ int oslo_wave_reduce_selftest(float *out4, void *stream);
  * "softmax_fwd_elems", "eltwise_unroll", "eltwise_rowgroups",
  * "eltwise_fwd_steps", "eltwise_tile_max", "eltwise_tile_min" (lanes along
  * the columns of an element-wise tile; 64 as the minimum restores whole-wave
- * tiles), "adam_unroll";
+ * tiles), "adam_unroll", "softmax_bias_order" (order of the rows of a
+ * softmax whose additive term is shared by the batch: 1 plain, 2 the batch
+ * entries of a row of the term next to each other, 3 that and every eighth
+ * workgroup on consecutive rows, the default);
  * value 0 restores the default.  Other values must be ones the launch code
  * has a kernel build and a valid workgroup shape for, else
  * OSLO_ERR_INVALID_ARGUMENT: chunks per lane (*_vpl: 1, 2, 4, forward also 8,

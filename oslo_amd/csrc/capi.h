@@ -46,6 +46,7 @@ struct Tuning {
   int norm_bwd_prefetch;
   int norm_fwd_iters;
   int adam_unroll;
+  int softmax_bias_order;
 };
 // oslo_tune() writes a process-wide table under a lock; every entry point
 // copies that table into a per-thread snapshot before it plans a launch

@@ -123,6 +123,7 @@ int oslo_tune(const char *key, int value) {
       {"norm_bwd_prefetch", &shared.norm_bwd_prefetch, kRange, 1, 2},
       {"norm_fwd_iters", &shared.norm_fwd_iters, kRange, 1, 16},
       {"adam_unroll", &shared.adam_unroll, kPow2, 1, 4},
+      {"softmax_bias_order", &shared.softmax_bias_order, kRange, 1, 3},
   };
   for (const Entry &e : table) {
     if (strcmp(e.name, key) == 0) {

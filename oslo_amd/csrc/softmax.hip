@@ -195,6 +195,14 @@ static int bias_geom(const char *what, int64_t b, int64_t np, int64_t sq,
   g->bias_sq = sq_stride;
   g->bias_esize = dtype_size(bias_dtype);
   g->bias_skip = (flags & OSLO_SOFTMAX_SKIP_HIDDEN) ? 1 : 0;
+  // a term with a row per head or query that the whole batch shares (a
+  // position bias): the batch entries of one row of it run next to each other
+  if (bias != nullptr && sb == 0 && b > 1 && b <= 0x7fffffff && (sh != 0 || sq_stride != 0) &&
+      g_tune.softmax_bias_order != 1) {
+    g->batch_inner = 1;
+    g->nb = (int)b;
+    g->hq_rows = np * sq;
+  }
   return OSLO_OK;
 }
 

@@ -53,7 +53,22 @@ struct SoftmaxGeom {
   // terms are all <= kBiasHidden skips the load of its logits
   int64_t bias_sb = 0, bias_sh = 0, bias_sq = 0;
   int bias_esize = 0, bias_skip = 0;
+  // An additive term shared by the batch (a position bias [1, np, sq, sk]): the
+  // rows are visited with the batch index innermost, so that the nb rows that
+  // read one row of the term run next to each other, and workgroup w works on
+  // block (w % 8) * xcd_wpx + w / 8, so that they also run on one of the eight
+  // dies, whose L2 then serves the term's row to all but the first of them.
+  int batch_inner = 0, nb = 1;
+  uint32_t nb_mul = 0, nb_shift = 32;
+  int64_t hq_rows = 0;   // np * sq
+  int64_t xcd_wpx = 0;   // 0: blocks in launch order
 };
+
+// The block of rows a workgroup works on.
+__device__ __forceinline__ int64_t work_block(const SoftmaxGeom &g) {
+  if (g.xcd_wpx != 0) return (int64_t)(blockIdx.x & 7u) * g.xcd_wpx + (int64_t)(blockIdx.x >> 3);
+  return (int64_t)blockIdx.x + g.blk0;
+}
 
 // Division of n < 2^31 by a divisor 1 <= d < 2^31 fixed for the launch: with
 // l = ceil(log2 d) and mul = ceil(2^(31 + l) / d) < 2^32, floor(n / d) equals
@@ -75,6 +90,7 @@ static inline void fast_div_make(uint32_t d, uint32_t *mul, uint32_t *shift) {
 static inline void set_fast_div(SoftmaxGeom &g) {
   fast_div_make((uint32_t)g.sq, &g.sq_mul, &g.sq_shift);
   fast_div_make((uint32_t)g.np, &g.np_mul, &g.np_shift);
+  fast_div_make((uint32_t)g.nb, &g.nb_mul, &g.nb_shift);
   g.inv_sk = 1.0f / (float)g.sk;
 }
 
@@ -194,6 +210,12 @@ __device__ __forceinline__ void row_setup(const SoftmaxGeom &g, int64_t r,
         bi * g.mask_b_stride_rows + (g.mask_per_query ? qi : 0);
     mrow = mask + mr * g.sk;
   } else if constexpr (MODE == kModeBias) {
+    if (g.batch_inner) {
+      const int64_t hq =
+          small ? (int64_t)fast_div((uint32_t)r, g.nb_mul, g.nb_shift) : r / g.nb;
+      r = (r - hq * g.nb) * g.hq_rows + hq;
+      row = r;
+    }
     const int64_t bh =
         small ? (int64_t)fast_div((uint32_t)r, g.sq_mul, g.sq_shift) : r / g.sq;
     int qi = (int)(r - bh * g.sq);
@@ -212,39 +234,51 @@ __device__ __forceinline__ void row_setup(const SoftmaxGeom &g, int64_t r,
   }
 }
 
-// One chunk of the additive term in its storage form: E values of the logits'
-// type T or of float (a launch-uniform choice, so one kernel serves both).
+// One chunk of the additive term, E values of the logits' type T or of float
+// (a launch-uniform choice, so one kernel serves both), converted to float as
+// soon as it arrives: the float form is no wider than a float chunk as loaded.
 template <typename T, int E>
-struct BiasChunk {
-  static constexpr int NV = E / 4;  // vectors of a float chunk
-  u32x4 r[NV];
-  __device__ __forceinline__ void load(const uint8_t *row, int c, bool f32) {
-    if (f32) {
+__device__ __forceinline__ void load_bias_chunk(const uint8_t *row, int c, bool f32, float *f) {
+  if (sizeof(T) == 4 || f32) {
 #pragma unroll
-      for (int v = 0; v < NV; ++v)
-        r[v] = ld16_cached(row + ((int64_t)c * E + 4 * v) * 4);
-    } else {
-      r[0] = ld16_cached(row + (int64_t)c * E * (int64_t)sizeof(T));
-    }
+    for (int v = 0; v < E / 4; ++v)
+      io<float>::unpack(ld16_cached(row + ((int64_t)c * E + 4 * v) * 4), f + 4 * v);
+  } else {
+    io<T>::unpack(ld16_cached(row + (int64_t)c * E * (int64_t)sizeof(T)), f);
   }
-  __device__ __forceinline__ void unpack(float *f, bool f32) const {
-    if (sizeof(T) == 4 || f32) {
+}
+
+// The same in two steps, for code that issues all its loads before it
+// converts any of them: the chunk as loaded (E / 4 vectors, the first one only
+// for a 16-bit term), then its conversion.
+template <typename T, int E>
+__device__ __forceinline__ void load_bias_raw(const uint8_t *row, int c, bool f32, u32x4 *r) {
+  if (sizeof(T) == 4 || f32) {
 #pragma unroll
-      for (int v = 0; v < NV; ++v) io<float>::unpack(r[v], f + 4 * v);
-    } else {
-      io<T>::unpack(r[0], f);
-    }
+    for (int v = 0; v < E / 4; ++v) r[v] = ld16_cached(row + ((int64_t)c * E + 4 * v) * 4);
+  } else {
+    r[0] = ld16_cached(row + (int64_t)c * E * (int64_t)sizeof(T));
   }
-  // every term of the chunk absorbs its logit
-  __device__ __forceinline__ bool all_hidden(bool f32) const {
-    float f[E];
-    unpack(f, f32);
-    float m = f[0];
+}
+template <typename T, int E>
+__device__ __forceinline__ void unpack_bias_raw(const u32x4 *r, bool f32, float *f) {
+  if (sizeof(T) == 4 || f32) {
 #pragma unroll
-    for (int e = 1; e < E; ++e) m = fmaxf(m, f[e]);
-    return m <= kBiasHidden;  // (false for NaN)
+    for (int v = 0; v < E / 4; ++v) io<float>::unpack(r[v], f + 4 * v);
+  } else {
+    io<T>::unpack(r[0], f);
   }
-};
+}
+
+// every term of the chunk absorbs its logit
+template <int E>
+__device__ __forceinline__ bool bias_all_hidden(const float *f) {
+  float m = f[0];
+#pragma unroll
+  for (int e = 1; e + 1 < E; e += 2) m = fmaxf(fmaxf(m, f[e]), f[e + 1]);  // v_max3_f32
+  if constexpr (E % 2 == 0) m = fmaxf(m, f[E - 1]);
+  return m <= kBiasHidden;  // (false for NaN)
+}
 
 // scalar read of element i of an additive-term row (generic kernels)
 template <typename T>
@@ -286,7 +320,7 @@ __global__ __launch_bounds__(1024) void softmax_fwd_kernel(
 
   // first row of this lane: the wave's first row plus the lane group's index
   const int64_t rbase =
-      (((int64_t)blockIdx.x + g.blk0) * g.rpb + rslot) * (RPW * SUB) +
+      (work_block(g) * g.rpb + rslot) * (RPW * SUB) +
       (LPR == kWave ? 0 : lane / LPR);
 
   float v[RPW][VPL][E];
@@ -297,7 +331,9 @@ __global__ __launch_bounds__(1024) void softmax_fwd_kernel(
   // additive term (kModeBias): the chunks as loaded, and whether a chunk's
   // logits were left unread
   constexpr bool kBias = MODE == kModeBias;
-  BiasChunk<T, E> braw[kBias ? RPW : 1][kBias ? VPL : 1];
+  float bv[kBias ? RPW : 1][kBias ? VPL : 1][kBias ? E : 1];
+  u32x4 braw[kBias ? RPW : 1][kBias ? VPL : 1][kBias ? E / 4 : 1];
+  RawChunk<T, E> xraw[kBias ? RPW : 1][kBias ? VPL : 1];
   bool bhid[kBias ? RPW : 1][kBias ? VPL : 1];
   const bool bias_f32 = g.bias_esize == 4;
 
@@ -335,8 +371,10 @@ __global__ __launch_bounds__(1024) void softmax_fwd_kernel(
       if constexpr (MODE == kModeBias) {
         // the additive term of every chunk that has a key below the diagonal
         // (cached loads: its rows are normally shared by many rows of logits)
+        // (all of them requested before any is converted: a conversion
+        //  waits for its load)
         bhid[j][k] = false;
-        if (mb != kAll) braw[j][k].load(mrow, c, bias_f32);
+        if (mb != kAll) load_bias_raw<T, E>(mrow, c, bias_f32, braw[j][k]);
       }
     }
   }
@@ -348,7 +386,10 @@ __global__ __launch_bounds__(1024) void softmax_fwd_kernel(
       for (int j = 0; j < RPW; ++j)
 #pragma unroll
         for (int k = 0; k < VPL; ++k)
-          if (mbits[j][k] != kAll) bhid[j][k] = braw[j][k].all_hidden(bias_f32);
+          if (mbits[j][k] != kAll) {
+            unpack_bias_raw<T, E>(braw[j][k], bias_f32, bv[j][k]);
+            bhid[j][k] = bias_all_hidden<E>(bv[j][k]);
+          }
     }
   }
 #pragma unroll
@@ -360,9 +401,28 @@ __global__ __launch_bounds__(1024) void softmax_fwd_kernel(
       // (a chunk without a visible key is not loaded; its registers are never
       //  used: every select below takes the masked branch for it)
       bool want = mbits[j][k] != (1u << E) - 1u;
-      if constexpr (MODE == kModeBias) want = want && !bhid[j][k];
-      if (want) load_chunk<T, E>(xr + (int64_t)c * E, v[j][k]);
+      if constexpr (MODE == kModeBias) {
+        if (want && !bhid[j][k]) xraw[j][k].load(xr + (int64_t)c * E);
+      } else {
+        if (want) load_chunk<T, E>(xr + (int64_t)c * E, v[j][k]);
+      }
     }
+  }
+  if constexpr (MODE == kModeBias) {
+    // (without the test above the logits were requested together with the
+    //  terms: the terms are converted only now)
+    if (!g.bias_skip) {
+#pragma unroll
+      for (int j = 0; j < RPW; ++j)
+#pragma unroll
+        for (int k = 0; k < VPL; ++k)
+          if (mbits[j][k] != kAll) unpack_bias_raw<T, E>(braw[j][k], bias_f32, bv[j][k]);
+    }
+#pragma unroll
+    for (int j = 0; j < RPW; ++j)
+#pragma unroll
+      for (int k = 0; k < VPL; ++k)
+        if (mbits[j][k] != kAll && !bhid[j][k]) xraw[j][k].unpack(v[j][k]);
   }
 
   // Wave-uniform shortcuts: where no lane of the wave sees a key of chunk
@@ -370,12 +430,18 @@ __global__ __launch_bounds__(1024) void softmax_fwd_kernel(
   // all its keys the per-element mask selects are skipped.  The logits are
   // kept in the log2 domain, t = x * (scale * log2 e), so exp is one exp2.
   bool none_visible[RPW][VPL], all_visible[RPW][VPL];
+  // additive term: no lane of the wave read the logits of the slot (every
+  // chunk of it lies beyond the diagonal or under terms that absorb it)
+  bool slot_unread[kBias ? RPW : 1][kBias ? VPL : 1];
 #pragma unroll
   for (int j = 0; j < RPW; ++j)
 #pragma unroll
     for (int k = 0; k < VPL; ++k) {
       none_visible[j][k] = __builtin_amdgcn_ballot_w64(mbits[j][k] != kAll) == 0;
       all_visible[j][k] = __builtin_amdgcn_ballot_w64(mbits[j][k] != 0u) == 0;
+      if constexpr (kBias)
+        slot_unread[j][k] =
+            __builtin_amdgcn_ballot_w64(mbits[j][k] != kAll && !bhid[j][k]) == 0;
     }
   const float c2 = scale * kLog2e;
 
@@ -390,11 +456,13 @@ __global__ __launch_bounds__(1024) void softmax_fwd_kernel(
         // the sum scale * x + term as one fused multiply-add, kept in the
         // natural domain: a large negative term (-10000) then costs the logit
         // one rounding, as in a float evaluation of the unfused chain
-        float bf[E];
-        braw[j][k].unpack(bf, bias_f32);
+        const float *bf = bv[j][k];
+        // (wave-uniform: no lane of the wave left the logits of this slot unread)
+        const bool no_skip = __builtin_amdgcn_ballot_w64(bhid[j][k]) == 0;
 #pragma unroll
         for (int e = 0; e < E; ++e) {
-          float t = bhid[j][k] ? bf[e] : __builtin_fmaf(v[j][k][e], scale, bf[e]);
+          float t = __builtin_fmaf(v[j][k][e], scale, bf[e]);
+          if (!no_skip) t = bhid[j][k] ? bf[e] : t;
           if (!all_visible[j][k]) t = (mbits[j][k] >> e) & 1u ? ninf : t;
           v[j][k][e] = t;
           m = fmaxf(m, t);
@@ -434,9 +502,21 @@ __global__ __launch_bounds__(1024) void softmax_fwd_kernel(
     // (with an additive term a row of -inf sums is NaN, as torch.softmax
     //  returns it: the maximum is subtracted as it is)
     const float off = mx[j] == ninf && !kBias ? 0.f : mx[j];
+    // (additive term: a slot whose logits were all left unread holds exact
+    //  zeros as soon as every row of the wave has another key: no exponentials)
+    bool hidden_are_zero = false;
+    if constexpr (kBias)
+      hidden_are_zero = __builtin_amdgcn_ballot_w64(!(mx[j] > kBiasHidden)) == 0;
 #pragma unroll
     for (int k = 0; k < VPL; ++k) {
       if (none_visible[j][k]) continue;
+      if constexpr (kBias) {
+        if (slot_unread[j][k] && hidden_are_zero) {
+#pragma unroll
+          for (int e = 0; e < E; ++e) v[j][k][e] = 0.f;
+          continue;
+        }
+      }
 #pragma unroll
       for (int e = 0; e < E; ++e) {
         float d = sub_rn(v[j][k][e], off);
@@ -560,7 +640,7 @@ __global__ __launch_bounds__(1024) void softmax_dropout_bwd_kernel(
   constexpr int SUB = kWave / LPR;
   const int sl = LPR == kWave ? lane : (lane & (LPR - 1));
   const int c0 = (wave - first) * kWave + sl;
-  const int64_t rbase = (((int64_t)blockIdx.x + g.blk0) * g.rpb + rslot) * (RPW * SUB) +
+  const int64_t rbase = (work_block(g) * g.rpb + rslot) * (RPW * SUB) +
                         (LPR == kWave ? 0 : lane / LPR);
   const float c2 = scale * kLog2e;
 
@@ -570,7 +650,7 @@ __global__ __launch_bounds__(1024) void softmax_dropout_bwd_kernel(
   bool rvalid[RPW];
   float rmax[RPW], rinv[RPW];
   constexpr bool kBias = MODE == kModeBias;
-  BiasChunk<T, E> braw[kBias ? RPW : 1][kBias ? VPL : 1];
+  float bv[kBias ? RPW : 1][kBias ? VPL : 1][kBias ? E : 1];
   const bool bias_f32 = g.bias_esize == 4;
 
 #pragma unroll
@@ -606,11 +686,11 @@ __global__ __launch_bounds__(1024) void softmax_dropout_bwd_kernel(
       }
       if constexpr (kBias) {
         if (mb != kAll) {
-          braw[j][k].load(mrow, c, bias_f32);
+          load_bias_chunk<T, E>(mrow, c, bias_f32, bv[j][k]);
           // A chunk whose terms all absorb their logits has probability 0
           // throughout, unless the row's maximum is such a term itself (a
           // row without any other key): skip it altogether
-          if (g.bias_skip && rmax[j] > kBiasHidden && braw[j][k].all_hidden(bias_f32))
+          if (g.bias_skip && rmax[j] > kBiasHidden && bias_all_hidden<E>(bv[j][k]))
             mb = kAll;
         }
       }
@@ -655,8 +735,8 @@ __global__ __launch_bounds__(1024) void softmax_dropout_bwd_kernel(
       // (a chunk without a visible key was not loaded: its gradients are zeros
       //  whatever the draw says)
       const KeepWords<E> keep = chunk_keep_words<E>(row[j], g.sk, c, d);
-      float bf[E];
-      if constexpr (kBias) braw[j][k].unpack(bf, bias_f32);
+      const float *bf = nullptr;
+      if constexpr (kBias) bf = bv[j][k];
 #pragma unroll
       for (int e = 0; e < E; ++e) {
         // the product is rounded before the subtraction, exactly as the
@@ -727,7 +807,7 @@ __global__ __launch_bounds__(1024) void softmax_bwd_kernel(
   const int sl = LPR == kWave ? lane : (lane & (LPR - 1));
   const int c0 = (wave - first) * kWave + sl;
 
-  const int64_t rbase = (((int64_t)blockIdx.x + g.blk0) * g.rpb + rslot) * (RPW * SUB) +
+  const int64_t rbase = (work_block(g) * g.rpb + rslot) * (RPW * SUB) +
                         (LPR == kWave ? 0 : lane / LPR);
 
   float yv[RPW][VPL][E], gv[RPW][VPL][E];
@@ -759,9 +839,9 @@ __global__ __launch_bounds__(1024) void softmax_bwd_kernel(
           // like that, which the test below catches)
           sk_ = visible - c * E <= 0;
           if (!sk_) {
-            BiasChunk<T, E> braw;
-            braw.load(mrow, c, g.bias_esize == 4);
-            sk_ = braw.all_hidden(g.bias_esize == 4);
+            float bf[E];
+            load_bias_chunk<T, E>(mrow, c, g.bias_esize == 4, bf);
+            sk_ = bias_all_hidden<E>(bf);
           }
         } else {
           sk_ = false;
@@ -1484,10 +1564,10 @@ int launch_softmax_fwd(const void *x, const uint8_t *mask, void *y,
   // fit one workgroup
   const int cap = g_tune.softmax_fwd_elems > 0 ? g_tune.softmax_fwd_elems
                                                : (sizeof(T) == 4 ? 16 : 32);
-  // (two row sets per wave where the loads of the logits wait for mask bytes
-  //  or additive terms)
-  const int default_rpw =
-      MODE == kModeMasked || (MODE == kModeBias && g.bias_skip) ? 2 : 1;
+  // (two row sets per wave where the loads of the logits wait for mask bytes;
+  //  with an additive term one measures faster, 186 against 232 us at
+  //  [16,16,1024,1024] fp16, whether or not the loads wait for the term)
+  const int default_rpw = MODE == kModeMasked ? 2 : 1;
   SoftmaxPlan pl = plan_softmax(g.sk, E, cap, default_rpw, 4, true);
   if (!pl.ok && cap < kFwdMaxElems && MODE != kModeBias)
     pl = plan_softmax(g.sk, E, kFwdMaxElems, default_rpw, 4);
@@ -1555,8 +1635,15 @@ int launch_softmax_fwd(const void *x, const uint8_t *mask, void *y,
               (const T *)x, mask, (T *)y, nullptr, g, scale, d);     \
   } else                                                             \
     return fail(OSLO_ERR_UNSUPPORTED, "softmax fwd: no kernel for %d x %d chunks per lane", VPL, RPW)
-  for (g.blk0 = 0; g.blk0 < nblocks; g.blk0 += per_launch) {
-    const int64_t grid = nblocks - g.blk0 < per_launch ? nblocks - g.blk0 : per_launch;
+  // (rows of a term shared by the batch: one die per run of consecutive blocks)
+  int64_t launch_blocks = nblocks;
+  if (MODE == kModeBias && g.batch_inner && g_tune.softmax_bias_order != 2 &&
+      nblocks >= 64 && nblocks + 8 <= per_launch) {
+    g.xcd_wpx = ceil_div(nblocks, 8);
+    launch_blocks = 8 * g.xcd_wpx;
+  }
+  for (g.blk0 = 0; g.blk0 < launch_blocks; g.blk0 += per_launch) {
+    const int64_t grid = launch_blocks - g.blk0 < per_launch ? launch_blocks - g.blk0 : per_launch;
     OSLO_SM_CASES(OSLO_SM_FWD)
     const int rc = check_launch("softmax_fwd_kernel");
     if (rc != OSLO_OK) return rc;
@@ -1695,8 +1782,15 @@ int launch_softmax_dropout_bwd(const void *dy, const void *x,
             scale, d);                                              \
   else                                                              \
     return fail(OSLO_ERR_UNSUPPORTED, "softmax dropout bwd: no kernel for %d x %d chunks per lane", VPL, RPW)
-  for (g.blk0 = 0; g.blk0 < nblocks; g.blk0 += per_launch) {
-    const int64_t grid = nblocks - g.blk0 < per_launch ? nblocks - g.blk0 : per_launch;
+  // (rows of a term shared by the batch: one die per run of consecutive blocks)
+  int64_t launch_blocks = nblocks;
+  if (MODE == kModeBias && g.batch_inner && g_tune.softmax_bias_order != 2 &&
+      nblocks >= 64 && nblocks + 8 <= per_launch) {
+    g.xcd_wpx = ceil_div(nblocks, 8);
+    launch_blocks = 8 * g.xcd_wpx;
+  }
+  for (g.blk0 = 0; g.blk0 < launch_blocks; g.blk0 += per_launch) {
+    const int64_t grid = launch_blocks - g.blk0 < per_launch ? launch_blocks - g.blk0 : per_launch;
     OSLO_SM_CASES(OSLO_SM_DBWD)
     const int rc = check_launch("softmax_dropout_bwd_kernel");
     if (rc != OSLO_OK) return rc;
