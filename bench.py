@@ -69,6 +69,9 @@ def parse_args():
     ap.add_argument("--table-iters", type=int, default=200, help="launches per kernel in the per-kernel table (0 = skip)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-graph-column", action="store_true", help="skip the captured-graph timings of the table")
+    ap.add_argument("--finalize-ab", action="store_true",
+                    help="only the A/B of the column-sum finalize launch (serial against a second stream or a "
+                         "graph branch): prints its own JSON line and exits")
     ap.add_argument("--traffic-optional", action="store_true",
                     help="report roofline.traffic as null when the counter summary has no row for the roofline "
                          "kernel (for the profiling runs that produce that summary); without it a missing row "
@@ -882,6 +885,121 @@ def module_table(L, dev, iters, kernel_rows):
     return rows
 
 
+def finalize_ab(L, dev, iters=200):
+    """A/B of the second launch of the column-sum backwards (their partial rows
+    are reduced by a finalize kernel that cannot start before the main kernel
+    has drained): serial on one stream, as the entry points issue it, against
+    the finalize on a second stream beside the next call's main kernel, eager
+    (events between the streams) and as a parallel branch of a captured graph.
+    Uses the measurement knob "colsum_defer" and oslo_colsum_finalize_probe of
+    include/oslo_hip_testing.h.  Returns rows for the JSON line."""
+    torch = L.torch
+    lib = L.lib
+    _C = L._C
+    main = torch.cuda.current_stream()
+    side = torch.cuda.Stream()
+    out = []
+
+    def ab(name, nbytes, run_main, finalize, nsets):
+        _C.tune("colsum_defer", 0)
+        t_serial = time_launches(torch, lambda i: run_main(i, main.cuda_stream, 0), iters, nsets)[0]
+        _C.tune("colsum_defer", 1)
+        ready = [torch.cuda.Event() for _ in range(2)]
+        free = [torch.cuda.Event() for _ in range(2)]
+        used = [False, False]
+
+        def deferred(i):
+            w = i % 2  # two workspaces: the main kernel of call i + 1 must not overwrite rows finalize(i) reads
+            if used[w]:
+                main.wait_event(free[w])
+            run_main(i % nsets, main.cuda_stream, w)
+            ready[w].record(main)
+            side.wait_event(ready[w])
+            finalize(side.cuda_stream, w)
+            free[w].record(side)
+            used[w] = True
+
+        t_side = time_launches(torch, deferred, iters, max(2, nsets) * 2)[0]
+        torch.cuda.synchronize()
+
+        def graph_time(branch):
+            _C.tune("colsum_defer", 1 if branch else 0)
+            cap, br = torch.cuda.Stream(), torch.cuda.Stream()
+            g = torch.cuda.CUDAGraph()
+            cap.wait_stream(main)
+            reps = 12
+            with torch.cuda.stream(cap):
+                with torch.cuda.graph(g, stream=cap):
+                    for k in range(reps):
+                        run_main(k % nsets, cap.cuda_stream, k % 2)
+                        if branch:
+                            br.wait_stream(cap)
+                            finalize(br.cuda_stream, k % 2)
+                            if k % 2 == 1:
+                                cap.wait_stream(br)  # both workspaces free again
+                    if branch:
+                        cap.wait_stream(br)
+            main.wait_stream(cap)
+            torch.cuda.synchronize()
+            for _ in range(3):
+                g.replay()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(8):
+                g.replay()
+            e1.record()
+            torch.cuda.synchronize()
+            return e0.elapsed_time(e1) / (8 * reps)
+
+        tg_serial, tg_branch = graph_time(False), graph_time(True)
+        _C.tune("colsum_defer", 0)
+        out.append({"kernel": name, "MB": round(nbytes / 1e6, 1),
+                    "serial_us": round(t_serial * 1e3, 2), "side_stream_us": round(t_side * 1e3, 2),
+                    "graph_serial_us": round(tg_serial * 1e3, 2), "graph_branch_us": round(tg_branch * 1e3, 2)})
+
+    for cfg, n1, n2 in (("cfg5", 8192, 6144), ("cfg2", 16384, 4096)):
+        T = n1 * n2 * 2
+        ns = nsets_for(4 * T)
+        sets, gamma, beta, dgamma, dbeta = norm_buffers(torch, dev, n1, n2, ns, 1)
+        wss = [L.ws(_C.OSLO_OP_LN_BWD, n1, n2, dev) for _ in range(2)]
+        for s_ in sets:
+            L.ok(lib.oslo_ln_fwd(p(s_["x"]), p(gamma), p(beta), p(s_["y"]), p(s_["mean"]), p(s_["invvar"]), n1, n2,
+                                 1e-5, BF16, BF16, main.cuda_stream))
+        parts = wss[0][1] // (2 * n2 * 4)
+
+        def run_main(i, st, w):
+            s_ = sets[i]
+            L.ok(lib.oslo_ln_bwd(p(s_["dy"]), p(s_["x"]), p(s_["mean"]), p(s_["invvar"]), p(gamma), p(s_["dx"]),
+                                 p(dgamma), p(dbeta), p(wss[w][0]), wss[w][1], n1, n2, BF16, BF16, st))
+
+        def fin(st, w):
+            L.ok(lib.oslo_colsum_finalize_probe(p(wss[w][0]), parts, n2, p(dgamma), p(dbeta), None, BF16, st))
+
+        ab("ln_bwd " + cfg, 3 * T, run_main, fin, ns)
+        del sets
+        torch.cuda.empty_cache()
+
+    n1, n2 = 8192, 6144
+    T = n1 * n2 * 2
+    ns = nsets_for(5 * T)
+    g = torch.Generator(device=dev).manual_seed(5)
+    gs = [torch.randn(n1, n2, generator=g, device=dev).to(torch.bfloat16) for _ in range(ns)]
+    dxs = [torch.empty_like(t) for t in gs]
+    dbias = torch.empty(n2, device=dev, dtype=torch.bfloat16)
+    wss = [L.ws(_C.OSLO_OP_BIAS_DROPOUT_ADD_BWD, n1, n2, dev) for _ in range(2)]
+    parts = wss[0][1] // (n2 * 4)
+
+    def run_bda(i, st, w):
+        L.ok(lib.oslo_bias_dropout_add_bwd(p(gs[i]), p(dxs[i]), p(dbias), p(wss[w][0]), wss[w][1], n1, n2, 0.1, 1234,
+                                           0, BF16, st))
+
+    def fin_bda(st, w):
+        L.ok(lib.oslo_colsum_finalize_probe(p(wss[w][0]), parts, n2, p(dbias), None, None, BF16, st))
+
+    ab("bias_dropout_add_bwd cfg5", 2 * T, run_bda, fin_bda, ns)
+    return out
+
+
 def cpu_model():
     """Model string of the host CPU with family / model / stepping (a virtual
     machine may shorten the name) and the number of logical CPUs."""
@@ -1128,6 +1246,10 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     L = Lib(torch, _C)
+
+    if args.finalize_ab:
+        print(json.dumps({"finalize_ab": finalize_ab(L, dev, max(20, args.table_iters))}))
+        return
 
     # the counter summary must hold the roofline kernel's row: fail before timing anything
     try:

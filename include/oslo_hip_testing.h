@@ -23,6 +23,17 @@ int oslo_philox_words(uint32_t *out, int64_t ngroups, int64_t first_group,
  * load/store path the kernels use; calibrates bandwidth and HBM counters. */
 int oslo_copy_probe(const void *src, void *dst, int64_t bytes, void *stream);
 
+/* Measurement of a backward pass whose second launch runs beside other work:
+ * with the knob "colsum_defer" set to 1 (oslo_tune) the backward entry points
+ * that end in a column-sum launch (LayerNorm / RMSNorm, bias-GeLU,
+ * bias-dropout-add and its fusion into the norm) stop after their main kernel
+ * and leave the fp32 partial rows in the workspace: `parts` rows of `cols`
+ * values per output, parts = workspace bytes / (outputs * cols * 4).  This
+ * call then reduces them to out0 (and out1, out2) of `dtype`, on any stream. */
+int oslo_colsum_finalize_probe(const void *partial_rows, int64_t parts, int64_t cols,
+                               void *out0, void *out1, void *out2, int dtype,
+                               void *stream);
+
 /* Wavefront reduction self-test: out[0..3] = (sum, max, sum-of-pair a,
  * sum-of-pair b) of lane-dependent values; the expected values are
  * 2016, 63, 2016, 4032.                                                    */
@@ -40,7 +51,8 @@ int oslo_wave_reduce_selftest(float *out4, void *stream);
  * tiles), "adam_unroll", "softmax_bias_order" (order of the rows of a
  * softmax whose additive term is shared by the batch: 1 plain, 2 the batch
  * entries of a row of the term next to each other, 3 that and every eighth
- * workgroup on consecutive rows, the default);
+ * workgroup on consecutive rows, the default), "colsum_defer" (1: see
+ * oslo_colsum_finalize_probe);
  * value 0 restores the default.  Other values must be ones the launch code
  * has a kernel build and a valid workgroup shape for, else
  * OSLO_ERR_INVALID_ARGUMENT: chunks per lane (*_vpl: 1, 2, 4, forward also 8,

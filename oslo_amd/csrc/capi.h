@@ -47,6 +47,7 @@ struct Tuning {
   int norm_fwd_iters;
   int adam_unroll;
   int softmax_bias_order;
+  int colsum_defer;
 };
 // oslo_tune() writes a process-wide table under a lock; every entry point
 // copies that table into a per-thread snapshot before it plans a launch

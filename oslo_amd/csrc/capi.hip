@@ -124,6 +124,7 @@ int oslo_tune(const char *key, int value) {
       {"norm_fwd_iters", &shared.norm_fwd_iters, kRange, 1, 16},
       {"adam_unroll", &shared.adam_unroll, kPow2, 1, 4},
       {"softmax_bias_order", &shared.softmax_bias_order, kRange, 1, 3},
+      {"colsum_defer", &shared.colsum_defer, kRange, 1, 1},
   };
   for (const Entry &e : table) {
     if (strcmp(e.name, key) == 0) {

@@ -690,6 +690,7 @@ static int run_bias_gelu_bwd(const void *gr, const void *x, const void *bias,
   });
   int rc = check_launch("bias_gelu_bwd_kernel");
   if (rc != OSLO_OK || dbias == nullptr) return rc;
+  if (g_tune.colsum_defer) return rc;  // measurement only: see oslo_colsum_finalize_probe
   return launch_colsum_finalize<T>(part, parts, cols, dbias, nullptr, st);
 }
 
@@ -797,6 +798,7 @@ static int run_bda_bwd(const void *gr, void *dx, void *dbias, void *ws,
   });
   int rc = check_launch("bias_dropout_add_bwd_kernel");
   if (rc != OSLO_OK || dbias == nullptr) return rc;
+  if (g_tune.colsum_defer) return rc;  // measurement only: see oslo_colsum_finalize_probe
   return launch_colsum_finalize<T>(part, parts, cols, dbias, nullptr, st);
 }
 
@@ -915,6 +917,20 @@ int oslo_philox_words(uint32_t *out, int64_t ngroups, int64_t first_group,
                         (hipStream_t)stream>>>(out, ngroups, first_group, seed,
                                                offset);
   return check_launch("philox_words_kernel");
+}
+
+int oslo_colsum_finalize_probe(const void *partial_rows, int64_t parts, int64_t cols,
+                               void *out0, void *out1, void *out2, int dtype,
+                               void *stream) {
+  if (!valid_dtype(dtype) || parts < 0 || cols < 4 || cols % 4 != 0 || !partial_rows || !out0)
+    return fail(OSLO_ERR_INVALID_ARGUMENT, "colsum_finalize_probe: bad arguments");
+  const int na = out2 ? 3 : (out1 ? 2 : 1);
+  hipStream_t st = (hipStream_t)stream;
+  if (dtype == OSLO_DTYPE_F32)
+    return launch_colsum_finalize<float>((const float *)partial_rows, parts, cols, out0, out1, st, out2, na);
+  if (dtype == OSLO_DTYPE_F16)
+    return launch_colsum_finalize<_Float16>((const float *)partial_rows, parts, cols, out0, out1, st, out2, na);
+  return launch_colsum_finalize<__bf16>((const float *)partial_rows, parts, cols, out0, out1, st, out2, na);
 }
 
 int oslo_copy_probe(const void *src, void *dst, int64_t bytes, void *stream) {

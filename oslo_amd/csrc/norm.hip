@@ -1446,6 +1446,7 @@ static int launch_norm_bwd(const void *dy, const void *x, const float *mean,
 #undef OSLO_BWD_CASE
   int rc = check_launch("norm_bwd_reg_kernel");
   if (rc != OSLO_OK || !want_params) return rc;
+  if (g_tune.colsum_defer) return rc;  // measurement only: see oslo_colsum_finalize_probe
   // arrays of partial rows: dgamma, dbeta (LayerNorm), bias gradient (fused)
   void *outs[3] = {dgamma, nullptr, nullptr};
   int na = 1;

@@ -47,7 +47,8 @@ _int = ctypes.c_int
 _f32 = ctypes.c_float
 _f64 = ctypes.c_double
 
-# name -> (restype, argtypes); one entry per declaration in include/oslo_hip.h
+# name -> (restype, argtypes); one entry per declaration in include/oslo_hip.h and
+# include/oslo_hip_testing.h
 _SIGNATURES = {
     "oslo_hip_last_error": (ctypes.c_char_p, []),
     "oslo_hip_arch": (ctypes.c_char_p, []),
@@ -190,6 +191,7 @@ _SIGNATURES = {
     "oslo_philox_mask": (_int, [_p, _i64, _f32, _u64, _u64, _p]),
     "oslo_philox_words": (_int, [_p, _i64, _i64, _u64, _u64, _p]),
     "oslo_copy_probe": (_int, [_p, _p, _i64, _p]),
+    "oslo_colsum_finalize_probe": (_int, [_p, _i64, _i64, _p, _p, _p, _int, _p]),
     "oslo_wave_reduce_selftest": (_int, [_p, _p]),
     "oslo_tune": (_int, [ctypes.c_char_p, _int]),
 }

@@ -22,7 +22,8 @@ def declared_symbols(header=None):
 
 
 def test_test_hooks_live_in_their_own_header():
-    hooks = {"oslo_tune", "oslo_copy_probe", "oslo_philox_words", "oslo_wave_reduce_selftest"}
+    hooks = {"oslo_tune", "oslo_copy_probe", "oslo_philox_words", "oslo_wave_reduce_selftest",
+             "oslo_colsum_finalize_probe"}
     assert set(declared_symbols("oslo_hip_testing.h")) == hooks
     assert not hooks & set(declared_symbols("oslo_hip.h"))
 
