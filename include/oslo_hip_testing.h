@@ -28,7 +28,9 @@ int oslo_copy_probe(const void *src, void *dst, int64_t bytes, void *stream);
  * that end in a column-sum launch (LayerNorm / RMSNorm, bias-GeLU,
  * bias-dropout-add and its fusion into the norm) stop after their main kernel
  * and leave the fp32 partial rows in the workspace: `parts` rows of `cols`
- * values per output, parts = workspace bytes / (outputs * cols * 4).  This
+ * values per output; parts = workspace bytes / (outputs * cols * 4) for the
+ * shapes the hook is meant for (long rows and at least as many rows as the
+ * GPU has compute units; other shapes may fill fewer partial rows).  This
  * call then reduces them to out0 (and out1, out2) of `dtype`, on any stream. */
 int oslo_colsum_finalize_probe(const void *partial_rows, int64_t parts, int64_t cols,
                                void *out0, void *out1, void *out2, int dtype,

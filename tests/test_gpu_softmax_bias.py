@@ -379,3 +379,44 @@ def test_module_takes_additive_and_per_head_masks(device):
     torch.softmax(0.25 * xr + br, -1).square().sum().backward()
     assert torch.allclose(bias.grad, br.grad, rtol=1e-4, atol=1e-6)
     assert torch.allclose(xg.grad, xr.grad, rtol=1e-4, atol=1e-6)
+
+
+@pytest.mark.parametrize("b,np_,sq,sk,dtype,causal", [
+    (3, 4, 50, 256, BF16, False),     # 600 rows: workgroups not a multiple of 8, batch of 3
+    (16, 2, 64, 1024, F16, False),    # two row sets ... one per workgroup, 2048 workgroups
+    (5, 3, 7, 64, F32, True),         # rows side by side in a wave, few workgroups
+    (2, 2, 33, 33, BF16, False),      # scalar kernels
+    (4, 2, 8, 4096, BF16, True),      # two waves per row
+])
+def test_row_order_of_a_term_shared_by_the_batch(device, b, np_, sq, sk, dtype, causal):
+    """A position bias [1, np, sq, sk]: the kernels visit the rows with the
+    batch index innermost and spread the workgroups so that one die works on
+    consecutive rows (softmax_bias_order 3, the default), or only the former
+    (2), or in plain order (1).  The order changes no bit of any row."""
+    x = randn((b, np_, sq, sk), dtype, seed=3, std=2.0)
+    g = randn((b, np_, sq, sk), dtype, seed=4)
+    bias = randn((1, np_, sq, sk), dtype, seed=5, std=2.0)
+    k = _C.get_softmax_kernel()
+    want = cf.softmax_bias_fwd(f64(x), f64(bias), 0.25, causal=causal)
+    seed, offset, p = 11, 16, 0.2
+    keep = philox.keep_mask(x.numel(), p, seed, offset).reshape(x.shape).astype(bool)
+    outs = []
+    for order in (1, 2, 3):
+        _C.tune("softmax_bias_order", order)
+        try:
+            y = k.softmax_bias_forward(x.to(device), bias.to(device), 0.25, causal=causal)
+            o, stats = k.softmax_bias_dropout_forward(x.to(device), bias.to(device), 0.25, p, seed, offset,
+                                                      causal=causal)
+            dx = k.softmax_bias_dropout_backward(g.to(device), x.to(device), bias.to(device), stats, 0.25, p,
+                                                 seed, offset, causal=causal)
+        finally:
+            _C.tune("softmax_bias_order", 0)
+        check(y, want, "order %d fwd" % order, atol=1e-9)
+        check(o, cf.softmax_bias_dropout_fwd(f64(x), f64(bias), 0.25, keep, p, causal=causal),
+              "order %d dropout fwd" % order, atol=1e-9)
+        check(dx, cf.softmax_bias_dropout_bwd(f64(g), f64(x), f64(bias), 0.25, keep, p, causal=causal),
+              "order %d dropout bwd" % order, atol=2e-7)
+        outs.append((y.cpu(), o.cpu(), dx.cpu(), stats.cpu()))
+    for other in outs[1:]:
+        for a, c in zip(outs[0], other):
+            assert torch.equal(a, c)

@@ -22,7 +22,7 @@ F32, F16, BF16 = torch.float32, torch.float16, torch.bfloat16
 KEYS = [
     "softmax_rows_per_wave", "softmax_lanes_per_row", "softmax_fwd_elems", "softmax_rows_per_block",
     "eltwise_tile_max", "eltwise_tile_min", "eltwise_unroll", "eltwise_rowgroups", "eltwise_fwd_steps",
-    "adam_unroll",
+    "adam_unroll", "softmax_bias_order", "colsum_defer",
 ]
 
 
@@ -86,3 +86,65 @@ def test_adam_override_keeps_the_result(device, tuned, dtype, unroll):
     _C.tune("adam_unroll", unroll)
     check_adam(device, dtype, 1, 1, 0.01)
     check_adam_views(device)
+
+
+# ------------------------------------------------------------ bias softmax under the launch overrides
+BIAS_OVERRIDES = [
+    ("softmax_rows_per_wave", 2), ("softmax_rows_per_wave", 4), ("softmax_lanes_per_row", 1),
+    ("softmax_lanes_per_row", 64), ("softmax_fwd_elems", 16), ("softmax_fwd_elems", 64),
+    ("softmax_rows_per_block", 3), ("softmax_rows_per_block", 16),
+]
+
+
+@pytest.mark.parametrize("key,value", BIAS_OVERRIDES)
+@pytest.mark.parametrize("sq,sk,dtype", [(40, 128, BF16), (19, 512, F32), (9, 1024, F16), (5, 4096, BF16),
+                                         (7, 2048, F16)])
+def test_bias_softmax_override_keeps_the_result(device, tuned, sq, sk, dtype, key, value):
+    """The softmax with an additive term under every launch-shape override
+    (shapes the defaults never take), with and without the skip of hidden
+    chunks and the fused dropout, against the float64 oracle."""
+    from test_gpu_softmax_bias import test_bias_softmax as check_bias
+    from test_gpu_softmax_bias import test_bias_softmax_dropout as check_bias_dropout
+
+    _C.tune(key, value)
+    check_bias(device, 2, 2, sq, sk, dtype, 0.25, "min" if dtype != F16 else "inf", True)
+    check_bias(device, 2, 2, sq, sk, dtype, 0.25, "t5", False)
+    _C.tune(key, value)  # (check_bias pins and then releases softmax_rows_per_wave)
+    check_bias_dropout(device, 2, 2, sq, sk, dtype, 0.25, "perq", False, 0.1)
+
+
+# ------------------------------------------------------------ the column-sum finalize as a call of its own
+def test_deferred_finalize_probe_equals_the_entry_point(device, tuned):
+    """Measurement hook: with "colsum_defer" the backward entry points stop
+    after their main kernel, and oslo_colsum_finalize_probe reduces the partial
+    rows they left in the workspace.  The pair gives the bits of the plain call."""
+    from helpers import randn
+
+    lib = _C.load_library()
+    ln = _C.get_layernorm_kernel()
+    n1, n2 = 512, 6144   # one row per step and workgroup: every partial row of the workspace is used
+    x = randn((n1, n2), BF16, 1).to(device)
+    dy = randn((n1, n2), BF16, 2).to(device)
+    gamma = randn((n2,), BF16, 3, std=0.1, mean=1.0).to(device)
+    beta = randn((n2,), BF16, 4, std=0.1).to(device)
+    _, mean, invvar = ln.layer_norm_forward_affine(x, (n2,), gamma, beta, 1e-5)
+    dx0, dg0, db0 = ln.layer_norm_backward_affine(dy, mean, invvar, x, (n2,), gamma, beta, 1e-5)
+    nbytes = int(lib.oslo_workspace_bytes(_C.OSLO_OP_LN_BWD, n1, n2))
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=device)
+    dx, dg, db = torch.empty_like(x), torch.full_like(gamma, float("nan")), torch.full_like(beta, float("nan"))
+    st = torch.cuda.current_stream().cuda_stream
+    _C.tune("colsum_defer", 1)
+    try:
+        rc = lib.oslo_ln_bwd(dy.data_ptr(), x.data_ptr(), mean.data_ptr(), invvar.data_ptr(), gamma.data_ptr(),
+                             dx.data_ptr(), dg.data_ptr(), db.data_ptr(), ws.data_ptr(), nbytes, n1, n2, 2, 2, st)
+        assert rc == 0, lib.oslo_hip_last_error()
+    finally:
+        _C.tune("colsum_defer", 0)
+    torch.cuda.synchronize()
+    assert torch.equal(dx, dx0) and torch.isnan(dg.float()).all()   # parameter gradients not written yet
+    parts = nbytes // (2 * n2 * 4)
+    rc = lib.oslo_colsum_finalize_probe(ws.data_ptr(), parts, n2, dg.data_ptr(), db.data_ptr(), None, 2, st)
+    assert rc == 0, lib.oslo_hip_last_error()
+    torch.cuda.synchronize()
+    assert torch.equal(dg, dg0) and torch.equal(db, db0)
+    assert lib.oslo_colsum_finalize_probe(None, parts, n2, dg.data_ptr(), None, None, 2, st) == -1
