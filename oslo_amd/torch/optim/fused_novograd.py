@@ -15,6 +15,12 @@ from oslo_amd.torch._C import get_l2norm_kernel, get_novograd_kernel
 from oslo_amd.torch.optim._common import ZeroGradMixin, checked_params, multi_tensor_applier
 
 
+def _bucket_name(dtype):
+    """Key of a dtype's norms in ``group["exp_avg_sq"]``: a plain string, so
+    that a state dict holds nothing tied to a device index."""
+    return str(dtype).split(".")[-1]
+
+
 class FusedNovograd(ZeroGradMixin, torch.optim.Optimizer):
     """Implements the NovoGrad algorithm on the GPU.
 
@@ -101,28 +107,48 @@ class FusedNovograd(ZeroGradMixin, torch.optim.Optimizer):
             group["step"] = group.get("step", 0) + 1
 
             buckets = {}
+            device = None
             for p in checked_params(group, "FusedNovograd"):
+                if device is None:
+                    device = p.device
+                elif p.device != device:
+                    raise RuntimeError("FusedNovograd: the parameters of a group must live on one device")
                 state = self.state[p]
                 if len(state) == 0:
                     state["exp_avg"] = torch.zeros_like(p.data, memory_format=torch.contiguous_format)
-                g, pd, m = buckets.setdefault((p.dtype, p.device), ([], [], []))
+                g, pd, m = buckets.setdefault(_bucket_name(p.dtype), ([], [], []))
                 g.append(p.grad.data.contiguous())
                 pd.append(p.data)
                 m.append(state["exp_avg"])
 
             # one norm per tensor (the norm, not its square, so that both norm
-            # types blend the same way), kept per bucket
-            norms = group.setdefault("exp_avg_sq", {})
+            # types blend the same way), kept per dtype in the parameter group,
+            # in the order of the parameters that have a gradient
+            norms = group.get("exp_avg_sq")
+            if isinstance(norms, (list, tuple)):
+                # a state dict of the reference: [norms of the 16-bit tensors,
+                # norms of the float32 tensors] (fused_novograd.py:172-226)
+                norms = {
+                    name: norms[1 if name == "float32" else 0].to(device=device, dtype=torch.float32)
+                    for name in buckets
+                    if len(norms) > (1 if name == "float32" else 0)
+                    and norms[1 if name == "float32" else 0].numel() > 0
+                }
+            if norms is None:
+                norms = {}
+            group["exp_avg_sq"] = norms
             for key, (g, pd, m) in buckets.items():
                 if key not in norms:
                     if group["init_zero"]:
-                        norms[key] = torch.zeros(len(g), dtype=torch.float32, device=key[1])
+                        norms[key] = torch.zeros(len(g), dtype=torch.float32, device=device)
                     else:
                         # the first step's own norm: the first blend changes nothing
-                        norms[key] = torch.zeros(len(g), dtype=torch.float32, device=key[1])
+                        norms[key] = torch.zeros(len(g), dtype=torch.float32, device=device)
                         get_l2norm_kernel().multi_tensor_norm_out(
                             0, None, [g], norms[key], 0.0, 1.0, group["norm_type"]
                         )
+                elif norms[key].device != device:
+                    norms[key] = norms[key].to(device)
                 elif norms[key].numel() != len(g):
                     raise RuntimeError(
                         "FusedNovograd: the set of parameters with gradients changed between steps"

@@ -356,6 +356,50 @@ def test_fused_novograd_follows_the_oracle(device, dtype, init_zero, reg_inside,
         FusedNovograd(ps, norm_type=1)
 
 
+@pytest.mark.parametrize("dtype", [F32, F16])
+def test_fused_novograd_state_dict_round_trip_and_reference_layout(device, dtype):
+    """The per-tensor norms live in the parameter group under plain string
+    keys; a state dict written by the reference (a two-element list, norms of
+    the 16-bit tensors then of the float32 tensors, oslo/torch/optim/
+    fused_novograd.py:172-226) is accepted too.  Both continue the trajectory
+    of an optimizer that was never saved."""
+    import copy
+
+    from oslo_amd.torch.optim import FusedNovograd
+
+    def fresh():
+        ps, grads = _param_set(device, dtype)
+        return ps, grads, FusedNovograd(ps, lr=0.01, betas=(0.95, 0.98), weight_decay=0.01)
+
+    def run(ps, grads, opt, steps):
+        for gs in steps:
+            for p, g in zip(ps, gs):
+                p.grad = g.to(device)
+            opt.step()
+
+    ps, grads, opt = fresh()
+    run(ps, grads, opt, grads)                       # never saved
+    want = [p.detach().clone() for p in ps]
+    for layout in ("own", "reference"):
+        ps2, grads2, opt2 = fresh()
+        run(ps2, grads2, opt2, grads2[:1])
+        sd = copy.deepcopy(opt2.state_dict())
+        norms = sd["param_groups"][0]["exp_avg_sq"]
+        assert list(norms) == [str(dtype).split(".")[-1]]
+        if layout == "reference":
+            v = norms[str(dtype).split(".")[-1]]
+            empty = torch.zeros(0, device=device)
+            sd["param_groups"][0]["exp_avg_sq"] = [empty, v] if dtype == F32 else [v, empty]
+        ps3, grads3, opt3 = fresh()
+        with torch.no_grad():
+            for a, b in zip(ps3, ps2):
+                a.copy_(b)
+        opt3.load_state_dict(sd)
+        run(ps3, grads3, opt3, grads3[1:])
+        for a, b in zip(ps3, want):
+            assert torch.equal(a, b), layout
+
+
 @pytest.mark.parametrize("dtype", [F32, BF16])
 @pytest.mark.parametrize("wd,max_grad_norm,nvlamb", [(0.01, 0.0, False), (0.0, 0.5, False), (0.0, 0.0, True)])
 def test_fused_lamb_follows_the_oracle(device, dtype, wd, max_grad_norm, nvlamb):
