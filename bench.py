@@ -69,6 +69,7 @@ def parse_args():
     ap.add_argument("--table-iters", type=int, default=200, help="launches per kernel in the per-kernel table (0 = skip)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-graph-column", action="store_true", help="skip the captured-graph timings of the table")
+    ap.add_argument("--no-modules", action="store_true", help="skip the module-API rows")
     ap.add_argument("--finalize-ab", action="store_true",
                     help="only the A/B of the column-sum finalize launch (serial against a second stream or a "
                          "graph branch): prints its own JSON line and exits")
@@ -1341,6 +1342,7 @@ def main():
                      "192 tensors; copy_probe = a plain copy" % (args.table_iters, BATCHES),
             "rows": rows,
         }
+    if args.table_iters > 0 and not args.no_modules:
         out["modules"] = {
             "what": "forward + backward through oslo_amd.torch.nn with autograd (out = m(x); out.backward(g) between "
                     "events on the launch stream, rotating inputs, gradients cleared to None before each call); MB = "
