@@ -1123,7 +1123,8 @@ def cpu_path_table(gpu_rows, budget_s=3.0):
         return (std * torch.randn(shape, generator=g)).to(dtype)
 
     def gpu_rate(names, cfg, note=None):
-        rows = [r for r in gpu_rows if r[0] in names and r[1] == cfg and (note is None or r[9] == note)]
+        rows = [r for r in gpu_rows if r[0] in names and r[1] == cfg and r[9] != "plain allocations"
+                and (note is None or r[9] == note)]
         if len(rows) != len(names):
             return None
         return sum(r[2] for r in rows) / sum(r[3] for r in rows) * 1e3

@@ -53,7 +53,10 @@ int oslo_wave_reduce_selftest(float *out4, void *stream);
  * tiles), "adam_unroll", "softmax_bias_order" (order of the rows of a
  * softmax whose additive term is shared by the batch: 1 plain, 2 the batch
  * entries of a row of the term next to each other, 3 that and every eighth
- * workgroup on consecutive rows, the default), "colsum_defer" (1: see
+ * workgroup on consecutive rows, the default), "softmax_causal_order" (order
+ * of the queries of an attention matrix under the diagonal: 1 long rows first,
+ * the default for rows of one wave, 2 as stored, the default for longer rows,
+ * 3 long and short rows in turn), "colsum_defer" (1: see
  * oslo_colsum_finalize_probe);
  * value 0 restores the default.  Other values must be ones the launch code
  * has a kernel build and a valid workgroup shape for, else

@@ -48,6 +48,7 @@ struct Tuning {
   int adam_unroll;
   int softmax_bias_order;
   int colsum_defer;
+  int softmax_causal_order;
 };
 // oslo_tune() writes a process-wide table under a lock; every entry point
 // copies that table into a per-thread snapshot before it plans a launch

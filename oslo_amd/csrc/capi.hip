@@ -125,6 +125,7 @@ int oslo_tune(const char *key, int value) {
       {"adam_unroll", &shared.adam_unroll, kPow2, 1, 4},
       {"softmax_bias_order", &shared.softmax_bias_order, kRange, 1, 3},
       {"colsum_defer", &shared.colsum_defer, kRange, 1, 1},
+      {"softmax_causal_order", &shared.softmax_causal_order, kRange, 1, 3},
   };
   for (const Entry &e : table) {
     if (strcmp(e.name, key) == 0) {

@@ -207,6 +207,71 @@ def test_softmax_with_and_without_dropout(device, i, b, np_, sq, sk, dtype, kind
               min_exact=0.98)
 
 
+def draw_term_softmax(seed, count):
+    r = np.random.default_rng(seed + FUZZ_SEED)
+    count = FUZZ_COUNT or count
+    out = []
+    for i in range(count):
+        sk = int(r.choice([1, 5, 8, 16, 24, 31, 64, 96, 100, 128, 192, 256, 257, 384, 512, 768, 1000, 1024, 1536,
+                           2048, 2050, 4096, 8192, 9000, 16384]))
+        sq = int(r.integers(1, 40)) if r.random() < 0.6 else min(sk, 48)
+        b, np_ = int(r.integers(1, 5)), int(r.integers(1, 4))
+        out.append((i, b, np_, sq, sk, DTYPES[int(r.integers(0, 3))], int(r.integers(0, 6))))
+    return out
+
+
+@pytest.mark.parametrize("i,b,np_,sq,sk,dtype,kind", draw_term_softmax(505, 60))
+def test_softmax_with_an_additive_term(device, i, b, np_, sq, sk, dtype, kind):
+    """kind 0: -10000 key mask [b,1,1,sk]; 1: lowest-value key mask; 2: -inf staircase per query
+    [b,1,sq,sk] (key 0 stays visible); 3: dense term shared by the batch [1,np,sq,sk]; 4: dense
+    term per sample and head; 5: per-head vector [np,1,sk].  Each with or without the diagonal,
+    the term in the scores' type or in float32, hidden chunks skipped or not, with or without
+    the fused dropout."""
+    r = np.random.default_rng(2000 + i)
+    scale = float(r.choice([0.125, 0.5, 1.0]))
+    p = float(r.choice([0.0, 0.0, 0.1, 0.3]))
+    causal = bool(r.integers(0, 2)) and sq <= sk
+    skip = bool(r.integers(0, 2))
+    term_f32 = bool(r.integers(0, 2))
+    seed, offset = 70 + i, 4 * i
+    x = randn((b, np_, sq, sk), dtype, 19 * i, std=2.0)
+    g = randn((b, np_, sq, sk), dtype, 19 * i + 1)
+    tdtype = torch.float32 if term_f32 else dtype
+    if kind in (0, 1):
+        valid = r.integers(1, sk + 1, size=b)
+        pad = torch.from_numpy(np.arange(sk)[None, :] >= valid[:, None]).view(b, 1, 1, sk)
+        fill = -10000.0 if kind == 0 else float(torch.finfo(tdtype).min)
+        term = torch.zeros(b, 1, 1, sk).masked_fill(pad, fill).to(tdtype)
+    elif kind == 2:
+        cut = torch.from_numpy(r.integers(1, sk + 1, size=(b, 1, sq, 1)))
+        term = torch.zeros(b, 1, sq, sk).masked_fill(
+            torch.arange(sk).view(1, 1, 1, sk) >= cut, float("-inf")).to(tdtype)
+    elif kind == 3:
+        term = randn((1, np_, sq, sk), tdtype, 19 * i + 2, std=2.0)
+    elif kind == 4:
+        term = randn((b, np_, sq, sk), tdtype, 19 * i + 2, std=2.0)
+    else:
+        term = randn((np_, 1, sk), tdtype, 19 * i + 2, std=2.0)
+    k = _C.get_softmax_kernel()
+    xd, gd, td = x.to(device), g.to(device), term.to(device)
+    xv, gv, tv = f64(x), f64(g), f64(term)
+    if p == 0.0:
+        y = k.softmax_bias_forward(xd, td, scale, causal=causal, skip_hidden=skip)
+        dx = k.softmax_bias_backward(gd, y, scale, bias=td, causal=causal, skip_hidden=skip)
+        check(y, cf.softmax_bias_fwd(xv, tv, scale, causal=causal), "term softmax fwd", atol=1e-9)
+        check(dx, cf.softmax_bwd(gv, f64(y), scale), "term softmax bwd", atol=2e-7)
+    else:
+        out, stats = k.softmax_bias_dropout_forward(xd, td, scale, p, seed, offset, causal=causal,
+                                                    skip_hidden=skip)
+        keep = philox.keep_mask(x.numel(), p, seed, offset).reshape(xv.shape).astype(bool)
+        check(out, cf.softmax_bias_dropout_fwd(xv, tv, scale, keep, p, causal=causal),
+              "term softmax dropout fwd", atol=1e-9)
+        dx = k.softmax_bias_dropout_backward(gd, xd, td, stats, scale, p, seed, offset, causal=causal,
+                                             skip_hidden=skip)
+        check(dx, cf.softmax_bias_dropout_bwd(gv, xv, tv, scale, keep, p, causal=causal),
+              "term softmax dropout bwd", atol=3e-7, min_exact=0.98)
+
+
 @pytest.mark.parametrize("i,n1,n2,dtype,flags", draw_cases(404, 50))
 def test_elementwise(device, i, n1, n2, dtype, flags):
     has_bias, has_res = flags[0], flags[1]

@@ -22,7 +22,7 @@ F32, F16, BF16 = torch.float32, torch.float16, torch.bfloat16
 KEYS = [
     "softmax_rows_per_wave", "softmax_lanes_per_row", "softmax_fwd_elems", "softmax_rows_per_block",
     "eltwise_tile_max", "eltwise_tile_min", "eltwise_unroll", "eltwise_rowgroups", "eltwise_fwd_steps",
-    "adam_unroll", "softmax_bias_order", "colsum_defer",
+    "adam_unroll", "softmax_bias_order", "colsum_defer", "softmax_causal_order",
 ]
 
 
@@ -39,6 +39,7 @@ SOFTMAX_OVERRIDES = [
     ("softmax_fwd_elems", 16), ("softmax_fwd_elems", 32), ("softmax_fwd_elems", 64),
     ("softmax_rows_per_block", 1), ("softmax_rows_per_block", 3), ("softmax_rows_per_block", 4),
     ("softmax_rows_per_block", 16),
+    ("softmax_causal_order", 1), ("softmax_causal_order", 2), ("softmax_causal_order", 3),
 ]
 
 # (sq, sk, dtype): one to eight chunks per lane, one or several waves per row
@@ -93,6 +94,7 @@ BIAS_OVERRIDES = [
     ("softmax_rows_per_wave", 2), ("softmax_rows_per_wave", 4), ("softmax_lanes_per_row", 1),
     ("softmax_lanes_per_row", 64), ("softmax_fwd_elems", 16), ("softmax_fwd_elems", 64),
     ("softmax_rows_per_block", 3), ("softmax_rows_per_block", 16),
+    ("softmax_causal_order", 2), ("softmax_causal_order", 3),
 ]
 
 
@@ -111,6 +113,20 @@ def test_bias_softmax_override_keeps_the_result(device, tuned, sq, sk, dtype, ke
     check_bias(device, 2, 2, sq, sk, dtype, 0.25, "t5", False)
     _C.tune(key, value)  # (check_bias pins and then releases softmax_rows_per_wave)
     check_bias_dropout(device, 2, 2, sq, sk, dtype, 0.25, "perq", False, 0.1)
+
+
+@pytest.mark.parametrize("order", [1, 2, 3])
+@pytest.mark.parametrize("sq,sk,dtype", [(37, 64, F16), (64, 40, BF16), (33, 33, F32), (96, 96, BF16),
+                                         (8, 4096, BF16), (5, 2051, BF16), (64, 1024, F16)])
+def test_causal_order_with_a_key_mask(device, tuned, sq, sk, dtype, order):
+    """Every order of the queries under the diagonal, for the kernels that take
+    the diagonal next to a key mask (odd and even numbers of queries, sq != sk)."""
+    from test_gpu_softmax_causal_masked import test_causal_masked as check_cm
+    from test_gpu_softmax_causal_masked import test_causal_masked_dropout as check_cm_dropout
+
+    _C.tune("softmax_causal_order", order)
+    check_cm(device, 2, 2, sq, sk, dtype, 0.25, "right")
+    check_cm_dropout(device, 2, 2, sq, sk, dtype, 0.25, "holes", 0.1)
 
 
 # ------------------------------------------------------------ the column-sum finalize as a call of its own
