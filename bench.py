@@ -73,6 +73,10 @@ def parse_args():
     ap.add_argument("--finalize-ab", action="store_true",
                     help="only the A/B of the column-sum finalize launch (serial against a second stream or a "
                          "graph branch): prints its own JSON line and exits")
+    ap.add_argument("--tune-ab", metavar="KEY=V1,V2,...",
+                    help="print the kernel table once per value of one launch knob (oslo_tune; 0 = the default) "
+                         "and exit: the A/B behind a default, from committed code")
+    ap.add_argument("--only", default="", help="with --tune-ab: keep the rows whose kernel name contains this")
     ap.add_argument("--traffic-optional", action="store_true",
                     help="report roofline.traffic as null when the counter summary has no row for the roofline "
                          "kernel (for the profiling runs that produce that summary); without it a missing row "
@@ -1251,6 +1255,19 @@ def main():
 
     if args.finalize_ab:
         print(json.dumps({"finalize_ab": finalize_ab(L, dev, max(20, args.table_iters))}))
+        return
+
+    if args.tune_ab:
+        key, _, values = args.tune_ab.partition("=")
+        out = {"knob": key, "only": args.only, "iters": max(20, args.table_iters), "cols": TABLE_COLS, "values": {}}
+        for v in [int(t) for t in values.split(",")]:
+            _C.tune(key, v)
+            try:
+                rows = kernel_table(L, dev, out["iters"], graph_column=False)
+            finally:
+                _C.tune(key, 0)
+            out["values"][str(v)] = [r for r in rows if args.only in r[0]]
+        print(json.dumps({"tune_ab": out}))
         return
 
     # the counter summary must hold the roofline kernel's row: fail before timing anything
