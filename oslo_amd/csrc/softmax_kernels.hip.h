@@ -470,13 +470,22 @@ __global__ __launch_bounds__(1024) void softmax_fwd_kernel(
         const float *bf = bv[j][k];
         // (wave-uniform: no lane of the wave left the logits of this slot unread)
         const bool no_skip = __builtin_amdgcn_ballot_w64(bhid[j][k]) == 0;
+        if (no_skip && all_visible[j][k]) {
+          // (the common slot, as a branch of its own: two instructions a key)
 #pragma unroll
-        for (int e = 0; e < E; ++e) {
-          float t = __builtin_fmaf(v[j][k][e], scale, bf[e]);
-          if (!no_skip) t = bhid[j][k] ? bf[e] : t;
-          if (!all_visible[j][k]) t = (mbits[j][k] >> e) & 1u ? ninf : t;
-          v[j][k][e] = t;
-          m = fmaxf(m, t);
+          for (int e = 0; e < E; ++e) {
+            const float t = __builtin_fmaf(v[j][k][e], scale, bf[e]);
+            v[j][k][e] = t;
+            m = fmaxf(m, t);
+          }
+        } else {
+#pragma unroll
+          for (int e = 0; e < E; ++e) {
+            float t = bhid[j][k] ? bf[e] : __builtin_fmaf(v[j][k][e], scale, bf[e]);
+            t = (mbits[j][k] >> e) & 1u ? ninf : t;
+            v[j][k][e] = t;
+            m = fmaxf(m, t);
+          }
         }
         continue;
       }
@@ -515,19 +524,17 @@ __global__ __launch_bounds__(1024) void softmax_fwd_kernel(
     const float off = mx[j] == ninf && !kBias ? 0.f : mx[j];
     // (additive term: a slot whose logits were all left unread holds exact
     //  zeros as soon as every row of the wave has another key: no exponentials)
-    bool hidden_are_zero = false;
-    if constexpr (kBias)
-      hidden_are_zero = __builtin_amdgcn_ballot_w64(!(mx[j] > kBiasHidden)) == 0;
+    if constexpr (kBias) {
+      const bool hidden_are_zero = __builtin_amdgcn_ballot_w64(!(mx[j] > kBiasHidden)) == 0;
+      // (such a slot is written as zeros below, like one that no lane sees:
+      //  its registers are not touched again)
+#pragma unroll
+      for (int k = 0; k < VPL; ++k)
+        if (slot_unread[j][k] && hidden_are_zero) none_visible[j][k] = true;
+    }
 #pragma unroll
     for (int k = 0; k < VPL; ++k) {
       if (none_visible[j][k]) continue;
-      if constexpr (kBias) {
-        if (slot_unread[j][k] && hidden_are_zero) {
-#pragma unroll
-          for (int e = 0; e < E; ++e) v[j][k][e] = 0.f;
-          continue;
-        }
-      }
 #pragma unroll
       for (int e = 0; e < E; ++e) {
         float d = sub_rn(v[j][k][e], off);
