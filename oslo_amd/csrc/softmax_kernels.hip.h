@@ -755,6 +755,9 @@ __global__ __launch_bounds__(1024) void softmax_dropout_bwd_kernel(
       const KeepWords<E> keep = chunk_keep_words<E>(row[j], g.sk, c, d);
       const float *bf = nullptr;
       if constexpr (kBias) bf = bv[j][k];
+      // (the selects below stay per element: a wave-uniform branch around
+      //  them for slots in which every lane sees all its keys measured 12 %
+      //  slower at [256, 2048, 2048], 690 -> 772 us)
 #pragma unroll
       for (int e = 0; e < E; ++e) {
         // the product is rounded before the subtraction, exactly as the
