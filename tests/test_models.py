@@ -605,6 +605,73 @@ def test_fuse_all_across_architectures_on_gpu(device, name):
         assert (pr.grad - pf.grad).abs().max().item() <= 2e-3 * scale + 1e-6, n
 
 
+def tiny_bart(seed=0):
+    from transformers import BartConfig, BartForConditionalGeneration
+
+    cfg = BartConfig(vocab_size=211, d_model=64, encoder_layers=2, decoder_layers=2, encoder_attention_heads=4,
+                     decoder_attention_heads=4, encoder_ffn_dim=128, decoder_ffn_dim=128,
+                     max_position_embeddings=64, dropout=0.0, attention_dropout=0.0, activation_dropout=0.0)
+    torch.manual_seed(seed)
+    return BartForConditionalGeneration(cfg)
+
+
+def bart_inputs(seed=1):
+    g = torch.Generator().manual_seed(seed)
+    src = torch.randint(3, 211, (3, 24), generator=g)
+    am = torch.ones(3, 24, dtype=torch.long)
+    am[1, 17:] = 0
+    am[2, 9:] = 0
+    return src, am, torch.randint(3, 211, (3, 10), generator=g)
+
+
+def test_bart_swaps_on_cpu_keep_the_model_output():
+    """An encoder-decoder in the layout of oslo/transformers/models/bart/modeling_bart.py:
+    padded encoder self-attention, causal decoder self-attention, cross-attention of 10
+    queries over 24 padded keys."""
+    from oslo_amd.transformers import fuse_all
+
+    m = tiny_bart().eval()
+    src, am, dec = bart_inputs()
+    with torch.no_grad():
+        ref = m(input_ids=src, attention_mask=am, decoder_input_ids=dec).logits
+    changed = fuse_all(m)
+    assert changed["fused_scale_mask_softmax"] and changed["fused_layer_norm"] == 12
+    with torch.no_grad():
+        out = m(input_ids=src, attention_mask=am, decoder_input_ids=dec).logits
+    assert torch.allclose(out, ref, atol=2e-5, rtol=1e-5)
+
+
+@pytest.mark.gpu
+def test_bart_through_the_fused_kernels(device, monkeypatch):
+    """Loss and every parameter gradient, fp32; the three kinds of attention reach
+    the padding-masked, the causal and (cross-attention, sq != sk) the padding-masked
+    kernel again, none of them the unfused chain."""
+    import warnings
+
+    from oslo_amd.transformers import fuse_all
+
+    masked = _spy(monkeypatch, "scaled_masked_softmax_dropout")
+    causal = _spy(monkeypatch, "scaled_upper_triang_masked_softmax_dropout")
+    src, am, dec = (t.to(device) for t in bart_inputs())
+    ref = tiny_bart().to(device).train()
+    fused = tiny_bart().to(device).train()
+    fuse_all(fused)
+    lr = ref(input_ids=src, attention_mask=am, decoder_input_ids=dec, labels=dec).loss
+    with warnings.catch_warnings():
+        warnings.simplefilter("error", RuntimeWarning)   # the unfused chain would warn
+        lf = fused(input_ids=src, attention_mask=am, decoder_input_ids=dec, labels=dec).loss
+    assert abs(lr.item() - lf.item()) <= 1e-4
+    # 2 encoder layers + 2 cross-attentions with the source's padding mask; 2 causal decoder layers
+    assert len(masked) + len(causal) == 6 and len(causal) >= 2, (len(masked), len(causal))
+    lr.backward()
+    lf.backward()
+    for (n, pr), (_, pf) in zip(ref.named_parameters(), fused.named_parameters()):
+        if pr.grad is None:
+            continue
+        scale = pr.grad.abs().max().item() + 1e-8
+        assert (pr.grad - pf.grad).abs().max().item() <= 2e-3 * scale + 1e-6, n
+
+
 def tiny_t5(seed=0):
     from transformers import T5Config, T5ForConditionalGeneration
 
