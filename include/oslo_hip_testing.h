@@ -51,9 +51,11 @@ int oslo_wave_reduce_selftest(float *out4, void *stream);
  * "eltwise_fwd_steps", "eltwise_tile_max", "eltwise_tile_min" (lanes along
  * the columns of an element-wise tile; 64 as the minimum restores whole-wave
  * tiles), "adam_unroll", "softmax_bias_order" (order of the rows of a
- * softmax whose additive term is shared by the batch: 1 plain, 2 the batch
- * entries of a row of the term next to each other, 3 that and every eighth
- * workgroup on consecutive rows, the default), "softmax_causal_order" (order
+ * softmax whose additive term is shared by the batch: 1 as stored, 2 the batch
+ * entries of a run of rows of the term next to each other, the default, 3 that
+ * and every eighth workgroup on consecutive rows), "softmax_bias_group" (rows
+ * in such a run, a power of two up to 256, default 32; lowered to a divisor of
+ * heads * queries), "softmax_causal_order" (order
  * of the queries of an attention matrix under the diagonal: 1 long rows first,
  * the default for rows of one wave, 2 as stored, the default for longer rows,
  * 3 long and short rows in turn), "colsum_defer" (1: see

@@ -49,6 +49,7 @@ struct Tuning {
   int softmax_bias_order;
   int colsum_defer;
   int softmax_causal_order;
+  int softmax_bias_group;
 };
 // oslo_tune() writes a process-wide table under a lock; every entry point
 // copies that table into a per-thread snapshot before it plans a launch

@@ -126,6 +126,7 @@ int oslo_tune(const char *key, int value) {
       {"softmax_bias_order", &shared.softmax_bias_order, kRange, 1, 3},
       {"colsum_defer", &shared.colsum_defer, kRange, 1, 1},
       {"softmax_causal_order", &shared.softmax_causal_order, kRange, 1, 3},
+      {"softmax_bias_group", &shared.softmax_bias_group, kPow2, 1, 256},
   };
   for (const Entry &e : table) {
     if (strcmp(e.name, key) == 0) {

@@ -202,6 +202,11 @@ static int bias_geom(const char *what, int64_t b, int64_t np, int64_t sq,
     g->batch_inner = 1;
     g->nb = (int)b;
     g->hq_rows = np * sq;
+    // (runs of 2^group_shift consecutive rows of one batch entry, then the same
+    //  rows of the next entry)
+    int group = g_tune.softmax_bias_group > 0 ? g_tune.softmax_bias_group : 32;
+    while (group > 1 && g->hq_rows % group != 0) group >>= 1;
+    while ((1 << g->group_shift) < group) ++g->group_shift;
   }
   return OSLO_OK;
 }

@@ -389,10 +389,11 @@ def test_module_takes_additive_and_per_head_masks(device):
     (4, 2, 8, 4096, BF16, True),      # two waves per row
 ])
 def test_row_order_of_a_term_shared_by_the_batch(device, b, np_, sq, sk, dtype, causal):
-    """A position bias [1, np, sq, sk]: the kernels visit the rows with the
-    batch index innermost and spread the workgroups so that one die works on
-    consecutive rows (softmax_bias_order 3, the default), or only the former
-    (2), or in plain order (1).  The order changes no bit of any row."""
+    """A position bias [1, np, sq, sk]: the kernels visit the rows in runs of
+    softmax_bias_group rows of one batch entry followed by the same rows of
+    the next entry (softmax_bias_order 2, the default), also spread the
+    workgroups so that one die works on consecutive rows (3), or keep the
+    stored order (1).  The order changes no bit of any row."""
     x = randn((b, np_, sq, sk), dtype, seed=3, std=2.0)
     g = randn((b, np_, sq, sk), dtype, seed=4)
     bias = randn((1, np_, sq, sk), dtype, seed=5, std=2.0)
@@ -401,8 +402,9 @@ def test_row_order_of_a_term_shared_by_the_batch(device, b, np_, sq, sk, dtype, 
     seed, offset, p = 11, 16, 0.2
     keep = philox.keep_mask(x.numel(), p, seed, offset).reshape(x.shape).astype(bool)
     outs = []
-    for order in (1, 2, 3):
+    for order, group in ((1, 0), (2, 0), (3, 0), (2, 1), (3, 1), (2, 8), (3, 64)):
         _C.tune("softmax_bias_order", order)
+        _C.tune("softmax_bias_group", group)
         try:
             y = k.softmax_bias_forward(x.to(device), bias.to(device), 0.25, causal=causal)
             o, stats = k.softmax_bias_dropout_forward(x.to(device), bias.to(device), 0.25, p, seed, offset,
@@ -411,6 +413,7 @@ def test_row_order_of_a_term_shared_by_the_batch(device, b, np_, sq, sk, dtype, 
                                                  seed, offset, causal=causal)
         finally:
             _C.tune("softmax_bias_order", 0)
+            _C.tune("softmax_bias_group", 0)
         check(y, want, "order %d fwd" % order, atol=1e-9)
         check(o, cf.softmax_bias_dropout_fwd(f64(x), f64(bias), 0.25, keep, p, causal=causal),
               "order %d dropout fwd" % order, atol=1e-9)

@@ -22,7 +22,7 @@ F32, F16, BF16 = torch.float32, torch.float16, torch.bfloat16
 KEYS = [
     "softmax_rows_per_wave", "softmax_lanes_per_row", "softmax_fwd_elems", "softmax_rows_per_block",
     "eltwise_tile_max", "eltwise_tile_min", "eltwise_unroll", "eltwise_rowgroups", "eltwise_fwd_steps",
-    "adam_unroll", "softmax_bias_order", "colsum_defer", "softmax_causal_order",
+    "adam_unroll", "softmax_bias_order", "colsum_defer", "softmax_causal_order", "softmax_bias_group",
 ]
 
 
@@ -95,6 +95,7 @@ BIAS_OVERRIDES = [
     ("softmax_lanes_per_row", 64), ("softmax_fwd_elems", 16), ("softmax_fwd_elems", 64),
     ("softmax_rows_per_block", 3), ("softmax_rows_per_block", 16),
     ("softmax_causal_order", 2), ("softmax_causal_order", 3),
+    ("softmax_bias_group", 1), ("softmax_bias_group", 4), ("softmax_bias_group", 256),
 ]
 
 
