@@ -1018,9 +1018,9 @@ class _SoftmaxKernel:
             # queries): a hidden chunk saves two loads there.  In the forward
             # pass it does not: the loads of the logits then wait for the term,
             # which costs more than the unread logits save (measured at
-            # [16,16,1024,1024] fp16 with 48 % of the keys under -inf: 157 us
-            # with the test, 165 us without; with a -10000 mask, which hides
-            # nothing, 195 us against 165 us).
+            # [16,16,1024,1024] fp16 with 48 % of the keys under -inf: 159 us
+            # with the test, 163 us without; with a -10000 mask, which hides
+            # nothing, 190-210 us against 163 us).
             skip_hidden = (not forward) and (strides[1] == 0 or strides[2] == 0)
         return (1 if causal else 0) | (2 if skip_hidden else 0)
 
