@@ -77,6 +77,8 @@ def parse_args():
                     help="print the kernel table once per value of one launch knob (oslo_tune; 0 = the default) "
                          "and exit: the A/B behind a default, from committed code")
     ap.add_argument("--only", default="", help="with --tune-ab: keep the rows whose kernel name contains this")
+    ap.add_argument("--tune-fixed", default="", metavar="KEY=V[,KEY=V]",
+                    help="with --tune-ab: other knobs held at a value in every column")
     ap.add_argument("--traffic-optional", action="store_true",
                     help="report roofline.traffic as null when the counter summary has no row for the roofline "
                          "kernel (for the profiling runs that produce that summary); without it a missing row "
@@ -1259,13 +1261,19 @@ def main():
 
     if args.tune_ab:
         key, _, values = args.tune_ab.partition("=")
-        out = {"knob": key, "only": args.only, "iters": max(20, args.table_iters), "cols": TABLE_COLS, "values": {}}
+        fixed = [kv.split("=") for kv in args.tune_fixed.split(",") if kv]
+        out = {"knob": key, "fixed": args.tune_fixed, "only": args.only, "iters": max(20, args.table_iters),
+               "cols": TABLE_COLS, "values": {}}
         for v in [int(t) for t in values.split(",")]:
+            for fk, fv in fixed:
+                _C.tune(fk, int(fv))
             _C.tune(key, v)
             try:
                 rows = kernel_table(L, dev, out["iters"], graph_column=False)
             finally:
                 _C.tune(key, 0)
+                for fk, _ in fixed:
+                    _C.tune(fk, 0)
             out["values"][str(v)] = [r for r in rows if args.only in r[0]]
         print(json.dumps({"tune_ab": out}))
         return
