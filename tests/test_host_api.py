@@ -147,6 +147,48 @@ def test_softmax_module_cpu_and_flags():
     assert filled[0, 0, 0, 1] == -10000.0
 
 
+def test_additive_term_operand_and_flags():
+    """How the binding hands an additive term to the kernel: element strides of
+    the batch / head / query dimensions (0 where the term broadcasts, expanded
+    views included), float32 for a term in another type than the scores, and
+    the default of the skip flag (backward passes of a term shared by heads or
+    queries only).  Host logic: no GPU needed."""
+    from oslo_amd.torch._C import _SoftmaxKernel as K
+
+    x = torch.zeros(3, 4, 5, 8, dtype=torch.bfloat16)
+    op = K._bias_operand
+    t, sb, sh, sq, code = op(torch.zeros(3, 1, 1, 8, dtype=torch.bfloat16), x)
+    assert (sb, sh, sq, code) == (8, 0, 0, 2) and t.shape == (3, 1, 1, 8)
+    t, sb, sh, sq, code = op(torch.zeros(4, 5, 8, dtype=torch.bfloat16), x)      # [np, sq, sk]
+    assert (sb, sh, sq) == (0, 40, 8) and t.dim() == 4
+    base = torch.zeros(1, 4, 5, 8, dtype=torch.bfloat16)
+    t, sb, sh, sq, code = op(base.expand(3, 4, 5, 8), x)                          # stride 0 kept
+    assert (sb, sh, sq) == (0, 40, 8) and t.data_ptr() == base.data_ptr()
+    t, sb, sh, sq, code = op(torch.zeros(8, dtype=torch.float16), x)              # another type -> float32
+    assert (sb, sh, sq, code) == (0, 0, 0, 0) and t.dtype == torch.float32
+    t, sb, sh, sq, code = op(torch.zeros(3, 4, 5, 8, dtype=torch.float64), x)
+    assert t.dtype == torch.float32 and (sb, sh, sq) == (160, 40, 8)
+    t, sb, sh, sq, code = op(torch.zeros(5, 1, dtype=torch.bfloat16), x)          # a column: expanded over the keys
+    assert t.shape == (1, 1, 5, 8) and (sb, sh, sq) == (0, 0, 8) and t.stride(3) == 1
+    wide = torch.zeros(5, 16, dtype=torch.bfloat16)
+    t, sb, sh, sq, code = op(wide[:, ::2], x)                                     # keys not contiguous: copied
+    assert t.stride(3) == 1 and sq == 8
+    t, sb, sh, sq, code = op(wide[:, 3:11], x)                                    # rows 32 bytes apart stay a view
+    assert sq == 16 and t.data_ptr() == wide.data_ptr() + 6
+    for bad in (torch.zeros(2, 1, 1, 8), torch.zeros(3, 4, 5, 7), torch.zeros(1, 1, 1, 1, 8)):
+        with pytest.raises(RuntimeError):
+            op(bad, x)
+    with pytest.raises(RuntimeError):
+        op(torch.zeros(3, 1, 1, 8, dtype=torch.bool), x)
+    with pytest.raises(RuntimeError):
+        op(torch.zeros(8), x[0])
+    fl = K._bias_flags
+    assert fl(False, None, (8, 0, 0), True) == 0 and fl(True, None, (8, 0, 0), True) == 1
+    assert fl(False, None, (8, 0, 0), False) == 2 and fl(True, None, (0, 40, 0), False) == 3
+    assert fl(False, None, (160, 40, 8), False) == 0          # a dense term: reading it would cost a third stream
+    assert fl(False, True, (160, 40, 8), True) == 2 and fl(True, False, (8, 0, 0), False) == 1
+
+
 def test_skip_bias_add_producers():
     lin = onn.Linear(8, 12, skip_bias_add=True)
     out, bias = lin(torch.randn(3, 8))
