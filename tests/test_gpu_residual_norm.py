@@ -219,6 +219,71 @@ def test_module_and_autograd(device, rms):
     check(y_eval, oy0, "module eval y", atol=1e-6, max_ulp=2 if rms else 1)
 
 
+@pytest.mark.parametrize("n1,n2,dtype,rms,second", [
+    (48, 16384, BF16, False, True), (40, 14336, F16, False, False), (24, 12288, F32, False, True),
+    (48, 16384, BF16, True, False), (16, 8192, F32, True, True),
+])
+def test_wide_rows_take_the_two_backward_kernels(device, monkeypatch, n1, n2, dtype, rms, second):
+    """Rows beyond 12288 16-bit or 6144 float32 elements: the module's backward
+    runs the norm's backward kernel and then the bias-dropout-add backward
+    kernel (the one-kernel backward spills there).  Gradients against the
+    float64 oracle; the gradient of the sum is rounded to its dtype between
+    the two kernels, as in the chain of unfused modules, so 16-bit results may
+    differ from the one-kernel oracle by an ulp more often."""
+    import oslo_amd.torch.nn as onn
+    from oslo_amd.torch import _C
+
+    p = 0.1
+    x, res, bias, gamma, beta, dy, dh = make_inputs(n1, n2, dtype, 31)
+    kernel = _C.get_layernorm_kernel()
+    fused_calls = []
+    real = kernel.bias_dropout_add_norm_backward
+    monkeypatch.setattr(kernel, "bias_dropout_add_norm_backward",
+                        lambda *a, **k: fused_calls.append(1) or real(*a, **k))
+    leaves = [t.to(device).requires_grad_(True) for t in (x, bias, res)]
+    w = gamma.to(device).requires_grad_(True)
+    b = None if rms else beta.to(device).requires_grad_(True)
+    torch.manual_seed(5)
+    gen = torch.cuda.default_generators[leaves[0].device.index or 0]
+    seed, offset = gen.initial_seed(), gen.get_offset()
+    if rms:
+        y, h = onn.fused_bias_dropout_add_rms_norm(*leaves, w, (n2,), 1e-5, p, True, return_sum=True)
+    else:
+        y, h = onn.fused_bias_dropout_add_layer_norm(*leaves, w, b, (n2,), 1e-5, p, True, return_sum=True)
+    loss = (y * dy.to(device)).sum()
+    if second:
+        loss = loss + (h * dh.to(device)).sum()
+    loss.backward()
+    assert not fused_calls, "the one-kernel backward ran"
+    keep = philox.keep_mask(n1 * n2, p, seed, offset).reshape(n1, n2).astype(bool)
+    name = NP_NAME[dtype]
+    hk = f64(h)
+    if rms:
+        _, oinv = cf.rms_norm_fwd(hk, f64(gamma), 1e-5, name)
+        omean = None
+    else:
+        _, omean, oinv = cf.layer_norm_fwd(hk, f64(gamma), f64(beta), 1e-5, name)
+    odres, odx, odg, odb, _ = cf.bias_dropout_add_norm_bwd(
+        f64(dy), f64(dh) if second else None, hk, omean, oinv, f64(gamma), keep, p, rms, name)
+    lowp = dict(max_ulp=2, min_exact=0.9) if dtype != F32 else {}
+    # (the norm's gradient is rounded before the second consumer's gradient is added:
+    #  half an ulp of that operand is the absolute error of a sum that cancels)
+    floor = 4e-6
+    if second and dtype != F32:
+        floor = 0.5 * float(torch.finfo(dtype).eps) * float(np.abs(odres).max() + np.abs(f64(dh)).max())
+    check(leaves[2].grad, odres, "wide dres", atol=floor, **lowp)
+    # (dx = keep * round(dres) / (1 - p) is rounded twice: a quarter of the 16-bit values land an ulp
+    #  beside the once-rounded oracle)
+    if dtype != F32:
+        lowp = dict(max_ulp=2, min_exact=0.7, l2_tol=4e-3)
+    check(leaves[0].grad, odx, "wide dx", atol=floor / (1 - p), **lowp)
+    col = 1e-5 * np.sqrt(n1) + 1e-6
+    check(leaves[1].grad, f64(leaves[0].grad).sum(0), "wide dbias", atol=3 * col, max_ulp=2, min_exact=0.97)
+    check(w.grad, odg, "wide dgamma", atol=3 * col, max_ulp=2, min_exact=0.97)
+    if not rms:
+        check(b.grad, odb, "wide dbeta", atol=col, max_ulp=2, min_exact=0.97)
+
+
 def test_unused_outputs_get_no_materialised_gradient(device, monkeypatch):
     """A post-LN block uses y only: backward must hand the kernel no dh_extra
     (not a zero-filled tensor, which costs a fill and a full read).  A caller
