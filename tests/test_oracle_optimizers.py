@@ -1,7 +1,8 @@
 """Pins the optimizer steps of oracle/closed_form.py (SGD, Adagrad, NovoGrad, LAMB,
 tensor norms) without a GPU: against torch.optim where torch has the algorithm,
-and for the rest against special cases that reduce to a pinned routine, hand
-arithmetic on tiny inputs and invariants of the update."""
+and for the rest (NovoGrad, LAMB) against reductions to torch.optim.SGD /
+torch.optim.Adam plus torch's vector norms, special cases that reduce to a
+pinned routine, hand arithmetic on tiny inputs and invariants of the update."""
 import numpy as np
 import pytest
 import torch
@@ -183,3 +184,78 @@ def test_lamb_gradient_scale_and_update_type():
                        out_update="bf16")
     assert np.array_equal(c[0], cf.round_bf16(b[0].astype(np.float32)))
     assert np.array_equal(c[1], b[1].astype(np.float32))
+
+
+@pytest.mark.parametrize("moment_mode", [0, 1])
+@pytest.mark.parametrize("grad_averaging", [True, False])
+def test_novograd_is_momentum_sgd_on_the_normalised_gradient(moment_mode, grad_averaging):
+    """NovoGrad keeps one second moment per tensor (a scalar), so its
+    element-wise part is torch.optim.SGD with momentum: in mode 0 on the
+    gradient g / (norm + eps) + decay * p with dampening beta1 (gradient
+    averaging) or 0, in mode 1 on the raw gradient with the step divided by
+    norm + eps and the decay applied to the old weight.  Five steps, the norm
+    following blend_norm (pinned against torch.linalg.vector_norm above), no
+    bias correction (its two scalars are pinned by hand above)."""
+    r = np.random.default_rng(11)
+    beta2, eps = 0.75, 2.0 ** -10
+    p0 = r.standard_normal((5, 8))
+    p_t = torch.nn.Parameter(torch.from_numpy(p0.copy()))
+    p, m, norm = p0.copy(), np.zeros_like(p0), 0.0
+    buf = None
+    for step in range(1, 6):
+        g = r.standard_normal((5, 8))
+        # the first step stores the plain norm, later ones blend (fused_novograd.py:199-207 of the reference)
+        norm = float(torch.linalg.vector_norm(torch.from_numpy(g))) if step == 1 else float(
+            np.sqrt(beta2 * norm ** 2 + (1 - beta2) * float(torch.linalg.vector_norm(torch.from_numpy(g))) ** 2))
+        denom = norm + eps
+        old = p_t.detach().clone()
+        if moment_mode == 0:
+            lr_t, grad = LR, torch.from_numpy(g) / denom + WD * old
+        else:
+            lr_t, grad = LR / denom, torch.from_numpy(g.copy())
+        opt = torch.optim.SGD([p_t], lr=lr_t, momentum=MU, dampening=MU if grad_averaging else 0.0)
+        # (a zero buffer instead of torch's first-step copy of the gradient: the kernel's moment starts at zero)
+        opt.state[p_t]["momentum_buffer"] = torch.zeros_like(p_t) if buf is None else buf
+        p_t.grad = grad
+        opt.step()
+        buf = opt.state[p_t]["momentum_buffer"]
+        if moment_mode == 1:
+            with torch.no_grad():
+                p_t -= LR * WD * old
+        p, m = cf.novograd_step(g, p, m, norm, LR, MU, beta2, eps, step, False, WD, grad_averaging, moment_mode)
+        assert np.allclose(p, p_t.detach().numpy(), rtol=1e-12, atol=1e-14), step
+        assert np.allclose(m, buf.numpy(), rtol=1e-12, atol=1e-14), step
+
+
+@pytest.mark.parametrize("mode", [0, 1])
+def test_lamb_is_the_adam_direction_under_a_trust_ratio(mode):
+    """Five LAMB steps assembled from library pieces: torch.optim.Adam with
+    lr = 1 and no decay gives the direction a = m_hat / (sqrt(v_hat) + eps) (on
+    g + decay * p in mode 0), the update is u = a (+ decay * p in mode 1), and
+    the weight moves by lr * |p| / |u| * u with torch's vector norms; the
+    gradient is first divided by max(1, global norm / threshold)."""
+    r = np.random.default_rng(12)
+    beta2, eps, max_norm = 0.75, 2.0 ** -20, 4.0
+    p0 = r.standard_normal((6, 7))
+    shadow = torch.nn.Parameter(torch.from_numpy(p0.copy()))
+    adam = torch.optim.Adam([shadow], lr=1.0, betas=(MU, beta2), eps=eps, weight_decay=0.0)
+    p, m, v = p0.copy(), np.zeros_like(p0), np.zeros_like(p0)
+    p_t = torch.from_numpy(p0.copy())
+    for step in range(1, 6):
+        g = (3.0 if step % 2 else 0.3) * r.standard_normal((6, 7))   # some steps are clipped, some not
+        gn = float(torch.linalg.vector_norm(torch.from_numpy(g)))
+        clipped = torch.from_numpy(g) / max(1.0, gn / max_norm)
+        with torch.no_grad():
+            shadow.copy_(p_t)
+        shadow.grad = clipped + WD * p_t if mode == 0 else clipped
+        adam.step()
+        a = p_t - shadow.detach()                       # the Adam direction (lr = 1)
+        u = a + WD * p_t if mode == 1 else a
+        ratio = LR * float(torch.linalg.vector_norm(p_t)) / float(torch.linalg.vector_norm(u))
+        p_t = p_t - ratio * u
+        upd, m, v = cf.lamb_stage1(g, p, m, v, MU, beta2, eps, step, True, WD, True, mode, gn, max_norm)
+        assert np.allclose(upd, u.numpy(), rtol=1e-11, atol=1e-13), step
+        p = cf.lamb_stage2(upd, p, cf.tensor_norm(p), cf.tensor_norm(upd), LR, WD, False)
+        assert np.allclose(p, p_t.numpy(), rtol=1e-11, atol=1e-13), step
+        st = adam.state[shadow]
+        assert np.allclose(m, st["exp_avg"].numpy(), rtol=1e-12) and np.allclose(v, st["exp_avg_sq"].numpy(), rtol=1e-12)
