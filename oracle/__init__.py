@@ -25,7 +25,22 @@ How each function is pinned (tests/test_oracle_*.py, no GPU needed)
                     rounding order against manual_rms_norm in bf16.
   bias-GeLU         torch.nn.functional.gelu(approximate="tanh") + autograd in
                     fp64; gelu(0)=0, gelu'(0)=0.5, gelu(u)-gelu(-u)=u.
+  softmax with an additive term
+                    torch.softmax(scale * x + M) + autograd in fp64 for key
+                    masks, per-query masks and shared biases, with the diagonal;
+                    the rows without a visible key for each fill value;
+                    committed torch-float64 vectors (tests/golden).
   bias-dropout-add  p=0 identity; mask scale; autograd with an explicit mask.
+  softmax + dropout, bias-dropout-add + norm
+                    torch autograd in fp64 through the unfused chain with an
+                    explicit keep mask.
+  optimizer steps   Adam / AdamW, SGD, Adagrad against torch.optim over five
+                    steps; NovoGrad as torch.optim.SGD with momentum on the
+                    normalised gradient; LAMB as torch.optim.Adam's direction
+                    under the trust ratio with torch's vector norms.  The
+                    mixed-precision LAMB's overflow flag and master copies are
+                    behaviours of the optimizer class: parity unpinned beyond
+                    the reduction to the plain LAMB step.
   Philox            the three Random123 known-answer vectors; an independent
                     pure-Python big-integer implementation; the C++ engine of
                     ATen (PhiloxRNGEngine.h) where torch exposes it.
