@@ -945,11 +945,19 @@ static int launch_norm_fwd(const void *x, const void *gamma, const void *beta,
     const int64_t nch = n2 / E;
     int cap = (!RMS && nch <= kWave * 2 * 4 && nch % (kWave * 4) != 0) ? 2 : 4;
     if (E == 8 && nch == 1536) cap = 2;
+    // rows of 8200 ... 12288 16-bit elements: two chunks per lane over up to
+    // twelve waves measure 5-13 % faster than four over five or six
+    // (LayerNorm bf16 [8192, 9216] 67 -> 58 us, [8192, 11264] 70 -> 66 us);
+    // RMSNorm gains up to 16384 elements together with two row groups per
+    // workgroup (below): [8192, 11264] 68 -> 61 us, [8192, 15360] 86 -> 84.5 us
+    if (E == 8 && nch > kWave * 4 * 4 && (RMS || nch <= kWave * 2 * 12)) cap = 2;
     // fp32 rows of 3072 and 4096 elements: 3 % faster over twice the waves
     if (E == 4 && (nch == 768 || nch == 1024)) cap = 2;
     // fp16 LayerNorm: four chunks per lane spill in the builds for more than
     // four waves (128 VGPRs), 20 % slower at 10240 elements than two per lane
-    if (!RMS && std::is_same<T, _Float16>::value && nch > kWave * 4 * 4 && nch <= kWave * 2 * 16)
+    // (beyond twelve waves of two the four-chunk build wins again: 13312
+    //  elements 95 -> 80 us, 15360 elements 101 -> 89 us)
+    if (!RMS && std::is_same<T, _Float16>::value && nch > kWave * 4 * 4 && nch <= kWave * 2 * 12)
       cap = 2;
     // LayerNorm rows of 768 eight-element chunks (6144 elements): four waves of
     // three chunks measure 1.3 % faster than three waves of four (35.7 against
@@ -1009,7 +1017,7 @@ static int launch_norm_fwd(const void *x, const void *gamma, const void *beta,
   // (LayerNorm: two groups, the second one prefetched; RMSNorm is fastest
   // with short-lived workgroups)
   int iters = g_tune.norm_fwd_iters > 0 ? g_tune.norm_fwd_iters
-              : (RMS && !(E == 8 && n2 / E == 1536)) ? 1 : 2;
+              : (RMS && !(E == 8 && n2 / E > kWave * 4 * 4)) ? 1 : 2;
   int64_t grid = ceil_div(ceil_div(n1, sp.rpb), iters);
   const int64_t maxgrid = (int64_t)device_cu_count() * 64;
   if (grid > maxgrid) grid = maxgrid;
