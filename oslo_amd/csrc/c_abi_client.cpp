@@ -183,6 +183,65 @@ static void causal_softmax_f32(hipStream_t st) {
   HIP_OK(hipFree(y));
 }
 
+// softmax(scale * x + M) with the additive key mask [b, 1, 1, sk] of
+// oslo/transformers/models/bert/modeling_bert.py:298-306 (-10000 on the
+// padded keys) under the diagonal, forward and backward, float32
+static void additive_mask_softmax_f32(hipStream_t st) {
+  const int64_t b = 3, np = 2, sq = 24, sk = 32;
+  const float scale = 0.5f;
+  uint32_t seed = 23;
+  std::vector<float> x(b * np * sq * sk), g(x.size()), m(b * sk, 0.f);
+  for (auto &v : x) v = 4.0f * next_value(seed);
+  for (auto &v : g) v = next_value(seed);
+  const int64_t valid[3] = {32, 20, 9};
+  for (int64_t i = 0; i < b; ++i)
+    for (int64_t j = valid[i]; j < sk; ++j) m[i * sk + j] = -10000.f;
+  float *dx_ = to_device(x), *dg = to_device(g), *dm = to_device(m), *y = nullptr, *dxo = nullptr;
+  HIP_OK(hipMalloc(&y, x.size() * 4));
+  HIP_OK(hipMalloc(&dxo, x.size() * 4));
+  // the mask broadcasts over heads and queries: their strides are 0
+  OSLO_CHECK(oslo_softmax_bias_fwd(dx_, dm, y, b, np, sq, sk, sk, 0, 0, OSLO_DTYPE_F32,
+                                   OSLO_SOFTMAX_CAUSAL, scale, OSLO_DTYPE_F32, st));
+  OSLO_CHECK(oslo_softmax_bias_bwd(dg, y, dm, dxo, b, np, sq, sk, sk, 0, 0, OSLO_DTYPE_F32,
+                                   OSLO_SOFTMAX_CAUSAL | OSLO_SOFTMAX_SKIP_HIDDEN, scale,
+                                   OSLO_DTYPE_F32, st));
+  HIP_OK(hipStreamSynchronize(st));
+  const auto hy = to_host(y, x.size());
+  const auto hdx = to_host(dxo, x.size());
+  for (int64_t r = 0; r < b * np * sq; ++r) {
+    const int64_t bi = r / (np * sq), i = r % sq;
+    const int64_t visible = i + 1 + (sk - sq);
+    const float *xr = &x[r * sk];
+    std::vector<double> u(sk), p(sk);
+    double mx = -1e300, s = 0, dot = 0;
+    for (int64_t j = 0; j < visible; ++j) {
+      // the kernel forms the sum in float32 with one multiply-add
+      u[j] = (double)std::fmaf(xr[j], scale, m[bi * sk + j]);
+      mx = std::fmax(mx, u[j]);
+    }
+    for (int64_t j = 0; j < visible; ++j) s += std::exp(u[j] - mx);
+    for (int64_t j = 0; j < sk; ++j) p[j] = j < visible ? std::exp(u[j] - mx) / s : 0.0;
+    for (int64_t j = 0; j < sk; ++j) dot += p[j] * g[r * sk + j];
+    for (int64_t j = 0; j < sk; ++j) {
+      expect_close("additive-mask softmax y", hy[r * sk + j], p[j], 1e-5, 1e-9);
+      if (j >= visible && hy[r * sk + j] != 0.0f) {
+        std::fprintf(stderr, "additive-mask softmax: a key beyond the diagonal is not an exact zero\n");
+        ++fails;
+      }
+      expect_close("additive-mask softmax dx", hdx[r * sk + j], scale * p[j] * (g[r * sk + j] - dot),
+                   1e-5, 2e-7);
+    }
+  }
+  // a term in a type the kernel does not add is refused with a message
+  if (oslo_softmax_bias_fwd(dx_, dm, y, b, np, sq, sk, sk, 0, 0, OSLO_DTYPE_F16, 0, scale,
+                            OSLO_DTYPE_F32, st) == OSLO_OK ||
+      std::strlen(oslo_hip_last_error()) == 0) {
+    std::fprintf(stderr, "a float16 term next to float32 scores was not refused\n");
+    ++fails;
+  }
+  for (void *q : {(void *)dx_, (void *)dg, (void *)dm, (void *)y, (void *)dxo}) HIP_OK(hipFree(q));
+}
+
 int main() {
   int ndev = 0;
   HIP_OK(hipGetDeviceCount(&ndev));
@@ -196,6 +255,7 @@ int main() {
   std::printf("liboslo_hip.so built for %s\n", oslo_hip_arch());
   layer_norm_bf16(st);
   causal_softmax_f32(st);
+  additive_mask_softmax_f32(st);
   HIP_OK(hipStreamDestroy(st));
   if (fails) {
     std::fprintf(stderr, "%d mismatches\n", fails);
