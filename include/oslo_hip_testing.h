@@ -59,7 +59,10 @@ int oslo_wave_reduce_selftest(float *out4, void *stream);
  * of the queries of an attention matrix under the diagonal: 1 long rows first,
  * the default for rows of one wave, 2 as stored, the default for longer rows,
  * 3 long and short rows in turn), "colsum_defer" (1: see
- * oslo_colsum_finalize_probe);
+ * oslo_colsum_finalize_probe), "colsum_slices" (slices of the partial rows
+ * that a workgroup of the column-sum reduction adds side by side: 64 or 128,
+ * the default, with eight lanes per slice and 32 columns per workgroup, or
+ * 256 with four lanes per slice and 16 columns);
  * value 0 restores the default.  Other values must be ones the launch code
  * has a kernel build and a valid workgroup shape for, else
  * OSLO_ERR_INVALID_ARGUMENT: chunks per lane (*_vpl: 1, 2, 4, forward also 8,

@@ -50,6 +50,7 @@ struct Tuning {
   int colsum_defer;
   int softmax_causal_order;
   int softmax_bias_group;
+  int colsum_slices;
 };
 // oslo_tune() writes a process-wide table under a lock; every entry point
 // copies that table into a per-thread snapshot before it plans a launch

@@ -127,6 +127,7 @@ int oslo_tune(const char *key, int value) {
       {"colsum_defer", &shared.colsum_defer, kRange, 1, 1},
       {"softmax_causal_order", &shared.softmax_causal_order, kRange, 1, 3},
       {"softmax_bias_group", &shared.softmax_bias_group, kPow2, 1, 256},
+      {"colsum_slices", &shared.colsum_slices, kPow2, 64, 256},
   };
   for (const Entry &e : table) {
     if (strcmp(e.name, key) == 0) {

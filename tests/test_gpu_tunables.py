@@ -23,6 +23,7 @@ KEYS = [
     "softmax_rows_per_wave", "softmax_lanes_per_row", "softmax_fwd_elems", "softmax_rows_per_block",
     "eltwise_tile_max", "eltwise_tile_min", "eltwise_unroll", "eltwise_rowgroups", "eltwise_fwd_steps",
     "adam_unroll", "softmax_bias_order", "colsum_defer", "softmax_causal_order", "softmax_bias_group",
+    "colsum_slices",
 ]
 
 
@@ -165,3 +166,29 @@ def test_deferred_finalize_probe_equals_the_entry_point(device, tuned):
     torch.cuda.synchronize()
     assert torch.equal(dg, dg0) and torch.equal(db, db0)
     assert lib.oslo_colsum_finalize_probe(None, parts, n2, dg.data_ptr(), None, None, 2, st) == -1
+
+
+@pytest.mark.parametrize("slices", [64, 128, 256])
+@pytest.mark.parametrize("parts,cols,dtype", [(256, 6144, BF16), (300, 1024, F32), (7, 36, F16), (1, 4, F32)])
+def test_finalize_slices_keep_the_column_sums(device, tuned, parts, cols, dtype, slices):
+    """The reduction of the partial rows under every workgroup shape
+    ("colsum_slices": 64 or 128 slices of the rows over 32 columns, 256 over
+    16 columns), against a float64 sum of the same rows: the shape changes the
+    order of the additions, not the addends."""
+    lib = _C.load_library()
+    g = torch.Generator().manual_seed(parts * 131 + cols)
+    part = torch.randn(2, parts, cols, generator=g, dtype=torch.float32)
+    want = part.double().sum(dim=1)
+    part_d = part.to(device)
+    out = torch.full((2, cols), float("nan"), dtype=dtype, device=device)
+    st = torch.cuda.current_stream().cuda_stream
+    code = {F32: 0, F16: 1, BF16: 2}[dtype]
+    _C.tune("colsum_slices", slices)
+    rc = lib.oslo_colsum_finalize_probe(part_d.data_ptr(), parts, cols, out[0].data_ptr(), out[1].data_ptr(),
+                                        None, code, st)
+    assert rc == 0, lib.oslo_hip_last_error()
+    torch.cuda.synchronize()
+    # fp32 accumulation of `parts` addends of unit variance, then one rounding to dtype
+    scale = float(want.abs().max()) + 1.0
+    tol = scale * (parts * 2.0 ** -24 + {F32: 2.0 ** -24, F16: 2.0 ** -11, BF16: 2.0 ** -8}[dtype])
+    assert (out.double().cpu() - want).abs().max().item() <= tol
