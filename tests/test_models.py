@@ -672,6 +672,111 @@ def test_bart_through_the_fused_kernels(device, monkeypatch):
         assert (pr.grad - pf.grad).abs().max().item() <= 2e-3 * scale + 1e-6, n
 
 
+# The encoder families the reference ships next to BERT, GPT-2, BART and T5
+# (oslo/transformers/models/{distilbert,roberta,albert,electra,mbart,mt5}), as Hugging Face builds them today.
+def _reference_family(name, seed=0):
+    import transformers as tf
+
+    kw = dict(vocab_size=211, max_position_embeddings=64)
+    enc = dict(hidden_size=64, intermediate_size=128, num_hidden_layers=2, num_attention_heads=4,
+               hidden_dropout_prob=0.0, attention_probs_dropout_prob=0.0)
+    torch.manual_seed(seed)
+    if name == "distilbert":   # masked_fill(mask == 0, -inf): modeling_distilbert.py:225-234
+        return tf.DistilBertForMaskedLM(tf.DistilBertConfig(dim=64, hidden_dim=128, n_layers=2, n_heads=4,
+                                                            dropout=0.0, attention_dropout=0.0, **kw))
+    if name == "roberta":
+        return tf.RobertaForMaskedLM(tf.RobertaConfig(**enc, **kw))
+    if name == "albert":
+        return tf.AlbertForMaskedLM(tf.AlbertConfig(embedding_size=32, **enc, **kw))
+    if name == "electra":
+        return tf.ElectraForMaskedLM(tf.ElectraConfig(embedding_size=32, **enc, **kw))
+    if name == "mbart":
+        return tf.MBartForConditionalGeneration(tf.MBartConfig(
+            d_model=64, encoder_layers=2, decoder_layers=2, encoder_attention_heads=4, decoder_attention_heads=4,
+            encoder_ffn_dim=128, decoder_ffn_dim=128, dropout=0.0, attention_dropout=0.0, activation_dropout=0.0,
+            **kw))
+    if name == "mt5":
+        return tf.MT5ForConditionalGeneration(tf.MT5Config(vocab_size=211, d_model=64, d_kv=16, d_ff=128,
+                                                           num_layers=2, num_decoder_layers=2, num_heads=4,
+                                                           dropout_rate=0.0, decoder_start_token_id=0,
+                                                           pad_token_id=0))
+    raise ValueError(name)
+
+
+# (layer norms, rms norms, post-LN output blocks, softmax kernel launches of one forward pass)
+REFERENCE_FAMILIES = {
+    "distilbert": (6, 0, 0, 2),
+    "roberta": (6, 0, 4, 2),
+    "albert": (4, 0, 0, 2),     # one shared layer, run twice
+    "electra": (6, 0, 4, 2),
+    "mbart": (14, 0, 0, 6),     # encoder, decoder self- and cross-attention
+    "mt5": (0, 12, 0, 6),
+}
+
+
+def _family_call(name, m, src, am, dec, labels=False):
+    kw = dict(input_ids=src, attention_mask=am)
+    if name in ("mbart", "mt5"):
+        kw["decoder_input_ids"] = dec
+        if labels:
+            kw["labels"] = dec
+    elif labels:
+        kw["labels"] = src
+    return m(**kw)
+
+
+@pytest.mark.parametrize("name", sorted(REFERENCE_FAMILIES))
+def test_reference_families_on_cpu(name):
+    from oslo_amd.transformers import fuse_all
+
+    m = _reference_family(name).eval()
+    src, am, dec = bart_inputs()
+    with torch.no_grad():
+        ref = _family_call(name, m, src, am, dec).logits
+    changed = fuse_all(m)
+    ln, rms, post_ln, _ = REFERENCE_FAMILIES[name]
+    assert (changed["fused_layer_norm"], changed["fused_rms_norm"],
+            changed["fused_bias_dropout_add_layer_norm"], changed["fused_scale_mask_softmax"]) == \
+        (ln, rms, post_ln, True), changed
+    with torch.no_grad():
+        out = _family_call(name, m, src, am, dec).logits
+    if name not in ("mbart", "mt5"):   # (the rows of padding tokens attend to nothing meaningful)
+        out, ref = out[am.bool()], ref[am.bool()]
+    assert torch.allclose(out, ref, atol=5e-5, rtol=1e-5)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", sorted(REFERENCE_FAMILIES))
+def test_reference_families_through_the_fused_kernels(device, monkeypatch, name):
+    """Loss and every parameter gradient of the swapped model against the model
+    as Hugging Face builds it, fp32, on a right-padded batch; every attention
+    of the forward pass reaches a softmax kernel and none the unfused chain."""
+    import warnings
+
+    from oslo_amd.transformers import fuse_all
+
+    spies = [_spy(monkeypatch, fn) for fn in ("scaled_masked_softmax_dropout",
+                                              "scaled_upper_triang_masked_softmax_dropout",
+                                              "scaled_bias_softmax_dropout")]
+    src, am, dec = (t.to(device) for t in bart_inputs())
+    ref = _reference_family(name).to(device).train()
+    fused = _reference_family(name).to(device).train()
+    fuse_all(fused)
+    lr = _family_call(name, ref, src, am, dec, labels=True).loss
+    with warnings.catch_warnings():
+        warnings.simplefilter("error", RuntimeWarning)   # the unfused chain would warn
+        lf = _family_call(name, fused, src, am, dec, labels=True).loss
+    assert abs(lr.item() - lf.item()) <= 1e-4 * max(1.0, abs(lr.item()))
+    assert sum(len(s) for s in spies) == REFERENCE_FAMILIES[name][3], [len(s) for s in spies]
+    lr.backward()
+    lf.backward()
+    for (n, pr), (_, pf) in zip(ref.named_parameters(), fused.named_parameters()):
+        if pr.grad is None:
+            continue
+        scale = pr.grad.abs().max().item() + 1e-8
+        assert (pr.grad - pf.grad).abs().max().item() <= 2e-3 * scale + 1e-6, n
+
+
 def tiny_t5(seed=0):
     from transformers import T5Config, T5ForConditionalGeneration
 
