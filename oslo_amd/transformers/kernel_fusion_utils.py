@@ -136,6 +136,22 @@ def _is_tanh_gelu(act):
     )
 
 
+def _is_erf_gelu(act):
+    """True when ``act`` computes the exact form x * Phi(x) ("gelu" in Hugging
+    Face's table), decided by its values."""
+    probe = torch.linspace(-6.0, 6.0, 97)
+    try:
+        out = act(probe)
+    except Exception:
+        return False
+    want = 0.5 * probe * (1.0 + torch.erf(probe * 0.7071067811865476))
+    return (
+        isinstance(out, torch.Tensor)
+        and out.shape == probe.shape
+        and torch.allclose(out.float(), want, atol=2e-6, rtol=0.0)
+    )
+
+
 def _is_projection(layer):
     # nn.Linear, or transformers' Conv1D (weight stored [in, out], ``nf`` outputs)
     return isinstance(layer, nn.Linear) or (
@@ -163,7 +179,7 @@ _MLP_SHAPES = (
 )
 
 
-def _mlp_shape(module):
+def _mlp_shape(module, tanh_for_erf=False):
     try:
         names = list(inspect.signature(type(module).forward).parameters)
     except (TypeError, ValueError):
@@ -181,7 +197,7 @@ def _mlp_shape(module):
         if "dropout" in children and not isinstance(children["dropout"], nn.Dropout):
             continue
         fn = getattr(module, act, None)
-        if callable(fn) and _is_tanh_gelu(fn):
+        if callable(fn) and (_is_tanh_gelu(fn) or (tanh_for_erf and _is_erf_gelu(fn))):
             return up, down
     return None
 
@@ -199,19 +215,27 @@ def _mlp_forward(self, hidden_states):
 _MLP_CLASSES = {}
 
 
-def fused_bias_gelu(model):
+def fused_bias_gelu(model, tanh_for_erf=False):
     """Gives every MLP (or BERT-style intermediate) block of ``model`` whose
     activation is the tanh form of GeLU a forward that adds the up projection's
     bias inside the GeLU kernel (the reference's ``fused_bias_gelu`` over a
     ``skip_bias_add`` linear, linear.py:31-35).  A block is changed only if its
     new forward reproduces the old one on a probe input.  Returns the number
-    of blocks changed."""
+    of blocks changed.
+
+    ``tanh_for_erf=True`` also changes the blocks whose activation is the
+    exact form x * Phi(x): the reference's models evaluate the tanh form
+    whatever the configuration names (``intermediate_act_fn =
+    onn.fused_bias_gelu``, modeling_bert.py:426; modeling_electra.py:469-484;
+    modeling_albert.py:333-336), which differs from the exact form by at most
+    4.8e-4 in absolute value (4.73e-4 near |x| = 2.3).  Off by default: the swap then changes no
+    result of the model beyond rounding."""
     n = 0
     for module in model.modules():
         cls = type(module)
         if cls in _MLP_CLASSES.values():
             continue
-        shape = _mlp_shape(module)
+        shape = _mlp_shape(module, tanh_for_erf)
         if shape is None:
             continue
         if cls not in _MLP_CLASSES:
@@ -229,6 +253,8 @@ def fused_bias_gelu(model):
             got = module(probe)
         module.train(was_training)
         tol = 1e-4 if want.dtype == torch.float32 else 3e-2
+        if tanh_for_erf:
+            tol += 2e-3  # the two forms of GeLU differ by up to 4.8e-4 before the down projection
         scale = want.float().abs().max().item() + 1e-6
         if (got.float() - want.float()).abs().max().item() > tol * scale:
             module.__class__ = cls  # not the chain it looked like: leave it alone
@@ -645,14 +671,15 @@ def fused_scale_mask_softmax(model, name=ATTENTION_NAME):
     return model
 
 
-def fuse_all(model, attention=True):
+def fuse_all(model, attention=True, tanh_for_erf=False):
     """Applies every swap of this module that fits ``model``; returns how many
     modules each one changed (``attention`` is True/False: the attention
-    function is a property of the whole model)."""
+    function is a property of the whole model; ``tanh_for_erf``: see
+    ``fused_bias_gelu``)."""
     changed = {
         "fused_pre_ln_block": fused_pre_ln_block(model),
         "fused_bias_dropout_add_layer_norm": fused_bias_dropout_add_layer_norm(model),
-        "fused_bias_gelu": fused_bias_gelu(model),
+        "fused_bias_gelu": fused_bias_gelu(model, tanh_for_erf),
         "fused_layer_norm": fused_layer_norm(model),
         "fused_rms_norm": fused_rms_norm(model),
         "fused_scale_mask_softmax": False,

@@ -318,6 +318,30 @@ def test_bias_gelu_swap_on_cpu_keeps_the_model_output():
     assert torch.allclose(b(ids, attention_mask=am).last_hidden_state, ref, atol=1e-5, rtol=1e-5)
 
 
+def test_bias_gelu_swap_with_the_tanh_form_for_the_exact_one():
+    """The reference's models evaluate the tanh form whatever the configuration
+    names (modeling_bert.py:426): the swap does the same on request, and the
+    output then moves by what the two forms differ by (4.7e-4 at most per
+    activation), no more."""
+    from oslo_amd.transformers import fuse_all, fused_bias_gelu
+
+    ids, am = inputs()
+    b = tiny_bert().eval()   # "gelu": x * Phi(x)
+    with torch.no_grad():
+        ref = b(ids, attention_mask=am).last_hidden_state
+    assert fused_bias_gelu(b) == 0
+    assert fused_bias_gelu(b, tanh_for_erf=True) == 2 and fused_bias_gelu(b, tanh_for_erf=True) == 0
+    with torch.no_grad():
+        out = b(ids, attention_mask=am).last_hidden_state
+    err = (out - ref).abs().max().item()
+    assert 1e-6 < err < 2e-2, err   # another function, close to the first
+    # a relu block is neither form
+    import transformers as tf
+    opt = tf.OPTForCausalLM(tf.OPTConfig(hidden_size=64, ffn_dim=128, num_hidden_layers=1, num_attention_heads=4,
+                                         word_embed_proj_dim=64, vocab_size=211, max_position_embeddings=64))
+    assert fuse_all(opt, attention=False, tanh_for_erf=True)["fused_bias_gelu"] == 0
+
+
 @pytest.mark.gpu
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_gpt2_with_every_swap_outputs_and_gradients(device, dtype, monkeypatch):
