@@ -609,6 +609,15 @@ static inline int64_t flat_grid(int64_t n) {
     }                        \
   } while (0)
 
+// (the forward of bias-dropout-add: one or two steps in flight)
+#define OSLO_ELT_U2(U_, ...)  \
+  do {                        \
+    switch (U_) {             \
+      case 1: { constexpr int U = 1; __VA_ARGS__; } break; \
+      default: { constexpr int U = 2; __VA_ARGS__; } break; \
+    }                         \
+  } while (0)
+
 #define OSLO_ELT_U8(U_, ...)  \
   do {                        \
     switch (U_) {             \
@@ -685,12 +694,15 @@ static int run_bias_gelu_bwd(const void *gr, const void *x, const void *bias,
     part = (float *)ws;
   }
   OSLO_ELT_U8(unroll, {
-    if (bias)
-      bias_gelu_bwd_kernel<T, U, true><<<grid, 256, 0, st>>>(
-          (const T *)gr, (const T *)x, (const T *)bias, (T *)dx, part, g);
-    else
-      bias_gelu_bwd_kernel<T, U, false><<<grid, 256, 0, st>>>(
-          (const T *)gr, (const T *)x, nullptr, (T *)dx, part, g);
+    // (eight steps in flight are built for the 16-bit types, whose default it is)
+    if constexpr (U < 8 || sizeof(T) == 2) {
+      if (bias)
+        bias_gelu_bwd_kernel<T, U, true><<<grid, 256, 0, st>>>(
+            (const T *)gr, (const T *)x, (const T *)bias, (T *)dx, part, g);
+      else
+        bias_gelu_bwd_kernel<T, U, false><<<grid, 256, 0, st>>>(
+            (const T *)gr, (const T *)x, nullptr, (T *)dx, part, g);
+    }
   });
   int rc = check_launch("bias_gelu_bwd_kernel");
   if (rc != OSLO_OK || dbias == nullptr) return rc;
@@ -727,7 +739,7 @@ static int run_bda_fwd(const void *x, const void *bias, const void *res,
       (const T *)x, (const T *)bias, (const T *)res, (T *)out, mask_out, g, d)
   for (g.blk0 = 0; g.blk0 < nblocks; g.blk0 += per_launch) {
     const dim3 grid((unsigned)(nblocks - g.blk0 < per_launch ? nblocks - g.blk0 : per_launch));
-    OSLO_ELT_U(unroll, {
+    OSLO_ELT_U2(unroll, {
       const int key = (bias ? 4 : 0) | (res ? 2 : 0) | (drop ? 1 : 0);
       switch (key) {
         case 0: OSLO_BDA_FWD(false, false, false); break;
@@ -926,6 +938,7 @@ int oslo_philox_words(uint32_t *out, int64_t ngroups, int64_t first_group,
 int oslo_colsum_finalize_probe(const void *partial_rows, int64_t parts, int64_t cols,
                                void *out0, void *out1, void *out2, int dtype,
                                void *stream) {
+  oslo::tune_snapshot();
   if (!valid_dtype(dtype) || parts < 0 || cols < 4 || cols % 4 != 0 || !partial_rows || !out0)
     return fail(OSLO_ERR_INVALID_ARGUMENT, "colsum_finalize_probe: bad arguments");
   const int na = out2 ? 3 : (out1 ? 2 : 1);

@@ -1571,6 +1571,19 @@ constexpr int kBwdMaxElems = 32;  // two operands resident
     LAUNCH(8, 1, kWave);                   \
   }
 
+// The (chunks per lane, row sets per wave, lanes per row) triples that the
+// plan of a backward pass can come out with: at most 32 resident elements of
+// each operand per lane in a 16-bit type and 16 in fp32 (32 only for rows that
+// need eight chunks per lane, which take one row set), and two chunks per lane
+// in a lane group only in the forward pass.  Other triples are not built.
+template <typename T>
+constexpr bool bwd_plan_reaches(int vpl, int rpw, int lpr) {
+  constexpr int E = io<T>::EPV;
+  if (vpl == 2 && lpr < kWave) return false;
+  if (sizeof(T) == 4) return vpl * rpw * E <= 16 || (vpl == 8 && rpw == 1);
+  return vpl * rpw * E <= kBwdMaxElems;
+}
+
 // The register kernels read the additive term in 16-byte vectors: its base
 // address and the byte offsets of its rows must be multiples of 16.
 static inline bool bias_vec_ok(const SoftmaxGeom &g, const uint8_t *bias) {
@@ -1741,7 +1754,7 @@ int launch_softmax_bwd(const void *dy, const void *y,
       ceil_div(g.rows, (int64_t)pl.rpb * pl.rpw * (kWave / pl.lpr));
   const int64_t per_launch = max_workgroups(threads);
 #define OSLO_SM_BWD(VPL, RPW, LPR_)                        \
-  if constexpr (VPL * RPW * E <= kBwdMaxElems)             \
+  if constexpr (bwd_plan_reaches<T>(VPL, RPW, LPR_))       \
     softmax_bwd_kernel<T, VPL, RPW, MODE, LPR_>            \
         <<<dim3((unsigned)grid), threads, 0, st>>>(        \
             (const T *)dy, (const T *)y, mask, (T *)dx, g, scale); \
@@ -1815,7 +1828,7 @@ int launch_softmax_dropout_bwd(const void *dy, const void *x,
       ceil_div(g.rows, (int64_t)pl.rpb * pl.rpw * (kWave / pl.lpr));
   const int64_t per_launch = max_workgroups(threads);
 #define OSLO_SM_DBWD(VPL, RPW, LPR_)                                \
-  if constexpr (VPL * RPW * E <= kBwdMaxElems && (MODE != kModeBias || RPW <= 2)) \
+  if constexpr (bwd_plan_reaches<T>(VPL, RPW, LPR_) && (MODE != kModeBias || RPW <= 2)) \
     softmax_dropout_bwd_kernel<T, VPL, RPW, MODE, LPR_>             \
         <<<dim3((unsigned)grid), threads, 0, st>>>(                 \
             (const T *)dy, (const T *)x, stats, mask, (T *)dx, g,   \

@@ -48,7 +48,8 @@ def unrounded(dtype):
 
 @pytest.mark.parametrize("gdtype,wdtype,copy", [(F32, F32, None), (F16, F16, None), (BF16, BF16, None),
                                                 (F16, F32, F16), (BF16, F32, BF16), (F32, F32, BF16),
-                                                (BF16, F32, None)])
+                                                (BF16, F32, None), (F16, F32, None), (F16, F32, BF16),
+                                                (BF16, F32, F16), (F32, F32, F16)])
 @pytest.mark.parametrize("momentum,dampening,nesterov,wd,after", [
     (0.0, 0.0, False, 0.0, False), (0.9, 0.0, False, 0.01, False), (0.9, 0.1, False, 0.01, True),
     (0.9, 0.0, True, 0.01, False)])
@@ -133,6 +134,18 @@ def test_multi_tensor_l2norm(device, dtype):
     devl[0][4][17] = float("inf")
     total3, _ = k.multi_tensor_l2norm(2048 * 32, flag, devl, False)
     assert torch.isinf(total3).all() and flag.item() == 1
+
+
+def test_largest_magnitude_over_all_tensors(device):
+    """norm_type 0 with a result over all tensors (the C entry point takes it;
+    the reference's bindings only ask for it per tensor)."""
+    host, devl = make_lists([F16], 60, device)
+    k = _C.get_l2norm_kernel()
+    total = torch.empty(1, dtype=torch.float32, device=device)
+    per = torch.empty(len(SIZES), dtype=torch.float32, device=device)
+    k._run(devl[0], total, per, 0, 0, 0.0, 0.0, None)
+    want = [float(np.abs(f64(t)).max()) if t.numel() else 0.0 for t in host[0]]
+    assert np.array_equal(f64(per), np.array(want)) and total.item() == max(want)
 
 
 @pytest.mark.parametrize("norm_type", [2, 0])
@@ -443,7 +456,8 @@ def _scalars(device, lr, step, max_norm, inv_scale):
     return f(lr), f(step, torch.int32), f(max_norm), f(inv_scale)
 
 
-@pytest.mark.parametrize("gdtype,master", [(F32, False), (BF16, False), (F16, True), (BF16, True)])
+@pytest.mark.parametrize("gdtype,master", [(F32, False), (BF16, False), (F16, True), (BF16, True), (F16, False),
+                                           (F32, True)])
 @pytest.mark.parametrize("mode,wd,nvlamb", [(1, 0.01, False), (0, 0.01, False), (1, 0.0, True)])
 def test_multi_tensor_lamb_mp_vs_oracle(device, gdtype, master, mode, wd, nvlamb):
     pdtype = F32 if master else gdtype

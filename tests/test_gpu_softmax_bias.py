@@ -100,7 +100,8 @@ def run_pair(k, x, dy, bias, scale, causal, device, skip):
 
 
 @pytest.mark.parametrize("b,np_,sq,sk,dtype,scale,kind,causal", CASES)
-def test_bias_softmax(device, b, np_, sq, sk, dtype, scale, kind, causal):
+def test_bias_softmax(device, b, np_, sq, sk, dtype, scale, kind, causal, rows_per_wave=(1, 0)):
+    # rows_per_wave: the override both launches below run under, and the value put back afterwards
     x = randn((b, np_, sq, sk), dtype, seed=sq + sk, std=2.0)
     dy = randn((b, np_, sq, sk), dtype, seed=sq + sk + 1)
     bias = make_bias(kind, b, np_, sq, sk, dtype, seed=sk)
@@ -117,11 +118,11 @@ def test_bias_softmax(device, b, np_, sq, sk, dtype, scale, kind, causal):
     for skip in (False, True):
         # (the same launch shape for both: two builds of a kernel may round a 16-bit
         #  output once or twice, which differs on ties)
-        _C.tune("softmax_rows_per_wave", 1)
+        _C.tune("softmax_rows_per_wave", rows_per_wave[0])
         try:
             y, dx = run_pair(k, x, dy, bias, scale, causal, device, skip)
         finally:
-            _C.tune("softmax_rows_per_wave", 0)
+            _C.tune("softmax_rows_per_wave", rows_per_wave[1])
         ycpu = y.cpu()
         fr = torch.from_numpy(finite_rows)
         assert (ycpu[~fr] == 0).all() and (dx.cpu()[~fr] == 0).all()

@@ -83,7 +83,7 @@ def test_eltwise_override_keeps_the_result(device, tuned, rows, cols, dtype, key
 
 
 @pytest.mark.parametrize("unroll", [1, 2, 4])
-@pytest.mark.parametrize("dtype", [F32, BF16])
+@pytest.mark.parametrize("dtype", [F32, F16, BF16])
 def test_adam_override_keeps_the_result(device, tuned, dtype, unroll):
     _C.tune("adam_unroll", unroll)
     check_adam(device, dtype, 1, 1, 0.01)
