@@ -9,7 +9,7 @@ select another build, each against the float64 oracle through the checks of
 the per-op test files.  An override that a shape has no build for is refused
 by the library (RuntimeError) and skipped.
 
-The full sweep (2200 runs of a shape under a setting, eight minutes) runs with
+The full sweep (2200 runs of a shape under a setting, four minutes) runs with
 OSLO_LAUNCH_TABLE=full.  By default each shape runs only the settings that
 golden/launch_table_cover.json lists for it: a smallest set of (shape, setting)
 pairs that between them launch every kernel build the full sweep launches,
