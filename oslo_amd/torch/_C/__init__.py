@@ -1433,6 +1433,9 @@ class _AdagradKernel:
         tables, sizes, n, ref = _tensor_tables(tensor_lists, ("grad", "param", "sum"), [d] * 3)
         if n == 0:
             return
+        # (an int32 tensor on the GPU, which multi_tensor_apply.cuh:100 takes the pointer
+        #  of; the update itself does not read it, multi_tensor_adagrad.cu:26-80)
+        _flag_ptr(noop_flag, ref)
         with _device_of(ref):
             rc = lib.oslo_multi_tensor_adagrad(
                 tables[0], tables[1], tables[2], sizes, n, float(lr), float(epsilon), int(mode),
