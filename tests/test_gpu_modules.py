@@ -259,6 +259,29 @@ def test_fused_scale_mask_softmax_adds_a_floating_point_mask(device):
     assert not m.is_kernel_available(torch.zeros(b, 1, 1, sk + 1, device=device), b, h, sq, sk, input=x)
 
 
+def test_fused_scale_mask_softmax_without_a_mask_and_with_an_integer_mask(device):
+    """A padding-type module called without a mask is a plain scaled softmax; a
+    mask of integers counts as its non-zero pattern; both on the kernels (the
+    torch chain would warn)."""
+    import warnings
+
+    x = randn((2, 3, 9, 64), torch.bfloat16, 5).to(device)
+    m = onn.FusedScaleMaskSoftmax(input_in_bf16=True, attn_mask_type=onn.AttnMaskType.padding, scale=0.25)
+    pad = torch.zeros(2, 1, 1, 64, dtype=torch.int32, device=device)
+    pad[1, ..., 50:] = 7
+    with warnings.catch_warnings():
+        warnings.simplefilter("error", RuntimeWarning)
+        y0 = m(x, None)
+        y1 = m(x, pad)
+    ref0 = torch.softmax(x.float() * 0.25, dim=-1)
+    ref1 = torch.softmax((x.float() * 0.25).masked_fill(pad.bool(), float("-inf")), dim=-1)
+    assert (y0.float() - ref0).abs().max().item() <= 4e-3 and (y1.float() - ref1).abs().max().item() <= 4e-3
+    assert (y1[1, ..., 50:] == 0).all()
+    # rows per workgroup of the masked kernel, as the reference's shim reports it
+    # (FusedScaleMaskSoftmaxBinder.cpp:122-127)
+    assert onn.FusedScaleMaskSoftmax.get_batch_per_block(9, 64, 2, 3) >= 1
+
+
 def test_skip_bias_add_producers_feed_the_fused_ops(device):
     lin = onn.Linear(32, 64, skip_bias_add=True).to(device)
     conv = onn.Conv1D(64, 32, skip_bias_add=True).to(device)

@@ -145,6 +145,30 @@ def test_softmax_module_cpu_and_flags():
         causal(x[0], None)
     filled = onn.attention_mask_func(torch.zeros(1, 1, 2, 2), torch.tensor([[[[False, True], [False, False]]]]))
     assert filled[0, 0, 0, 1] == -10000.0
+    with pytest.raises(ValueError, match="between 0 and 1"):
+        onn.FusedScaleMaskSoftmax(attn_dropout=1.5)
+    # why a call would not reach the kernels, as the module reports it
+    assert "does not broadcast" in padding._unfused_reason(torch.zeros(1, 1, 1, 1, 8, dtype=torch.bool), 2, 3, 8, 8)
+    assert padding._unfused_reason(None, 0, 3, 8, 8) == "empty input"
+    assert padding(torch.zeros(0, 3, 8, 8), None).shape == (0, 3, 8, 8)
+    # the torch chain applies the module's own dropout: off in eval mode, in training mode zeros and 1 / (1 - p)
+    drop = onn.FusedScaleMaskSoftmax(attn_mask_type=onn.AttnMaskType.causal, scale=0.5, attn_dropout=0.5)
+    assert torch.equal(drop.eval()(x, None), y * 0 + causal(x, None))
+    torch.manual_seed(0)
+    yd = drop.train()(x, None)
+    ref = causal(x, None)
+    kept = yd != 0
+    assert 0.2 < kept.float().mean().item() / (ref != 0).float().mean().item() < 0.8
+    assert torch.allclose(yd[kept], 2.0 * ref[kept])
+
+
+def test_residual_norm_module_without_parameters():
+    m = onn.FusedBiasDropoutAddLayerNorm(16, p=0.0, elementwise_affine=False)
+    assert m.weight is None and m.bias is None and "elementwise_affine=False" in repr(m)
+    x, b, r = torch.randn(3, 16), torch.randn(16), torch.randn(3, 16)
+    out = m(x, b, r)
+    out = out[0] if isinstance(out, tuple) else out
+    assert torch.allclose(out, torch.nn.functional.layer_norm(x + b + r, (16,), eps=m.eps), atol=1e-6)
 
 
 def test_additive_term_operand_and_flags():
