@@ -126,3 +126,46 @@ def test_fused_adam_optimizer_tracks_torch_optim(device, adam_w_mode):
         oa.step(grads=[1])
     oa.zero_grad()
     assert all(p.grad is None for p in a.parameters())
+
+
+def test_fused_adam_step_details(device):
+    """What `step` does around the launch (fused_adam.py:86-184 of the
+    reference): a closure is evaluated with gradients enabled and its loss
+    returned, parameters without a gradient are left alone, a group without any
+    gradient costs nothing, and what the kernel cannot take is refused."""
+    from oslo_amd.torch.optim import FusedAdam
+
+    w = torch.nn.Parameter(randn((33,), F32, 1).to(device))
+    idle = torch.nn.Parameter(randn((5,), F32, 2).to(device))
+    opt = FusedAdam([{"params": [w, idle]}, {"params": [torch.nn.Parameter(torch.zeros(3, device=device))]}],
+                    lr=0.1, set_grad_none=False)
+
+    def closure():
+        assert torch.is_grad_enabled()
+        opt.zero_grad()
+        loss = (w * w).sum()
+        loss.backward()
+        return loss
+
+    before, idle_before = w.detach().clone(), idle.detach().clone()
+    with torch.no_grad():
+        loss = opt.step(closure)
+    assert loss.item() == pytest.approx(float((before * before).sum()))
+    assert not torch.equal(w.detach(), before) and torch.equal(idle.detach(), idle_before)
+    opt.zero_grad()                      # set_grad_none=False: gradients are zeroed, not dropped
+    assert w.grad is not None and not w.grad.any()
+    opt.zero_grad(set_to_none=True)
+    assert w.grad is None
+    with pytest.raises(RuntimeError, match="AMSGrad"):
+        FusedAdam([w], amsgrad=True)
+    for bad, what in ((torch.nn.Parameter(torch.zeros(4)), "GPU-only"),
+                      (torch.nn.Parameter(torch.zeros(4, dtype=torch.float64, device=device)), "fp16, bf16 and fp32"),
+                      (torch.nn.Parameter(torch.zeros(4, 6, device=device).t()), "contiguous")):
+        o = FusedAdam([bad])
+        bad.grad = torch.zeros_like(bad)
+        with pytest.raises(RuntimeError, match=what):
+            o.step()
+    sparse = torch.nn.Parameter(torch.zeros(4, 3, device=device))
+    sparse.grad = torch.zeros(4, 3, device=device).to_sparse()
+    with pytest.raises(RuntimeError, match="sparse"):
+        FusedAdam([sparse]).step()

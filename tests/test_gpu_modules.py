@@ -141,6 +141,28 @@ def test_functional_defaults_and_shapes(device):
     check(y, f64(ref), "functional rms", atol=2e-6)
 
 
+def test_fused_bias_dropout_in_place(device):
+    """inplace=True (functional.py:295-298 hands it to F.dropout): the result
+    overwrites the input's memory, autograd is told so, and values and
+    gradients equal those of the out-of-place call under the same seed."""
+    x = randn((64, 256), BF16, 1).to(device).requires_grad_()
+    b = randn((256,), BF16, 2, std=0.1).to(device).requires_grad_()
+    g = randn((64, 256), BF16, 3).to(device)
+    torch.manual_seed(7)
+    ref = onn.fused_bias_dropout(x * 1, b, 0.25, True, False)
+    ref.backward(g)
+    gx, gb = x.grad.clone(), b.grad.clone()
+    x.grad = b.grad = None
+    h = x * 1
+    torch.manual_seed(7)
+    out = onn.fused_bias_dropout(h, b, 0.25, True, True)
+    assert out.data_ptr() == h.data_ptr() and torch.equal(out, ref)
+    out.backward(g)
+    assert torch.equal(x.grad, gx) and torch.equal(b.grad, gb)
+    with pytest.raises(RuntimeError):   # a leaf that requires a gradient cannot be overwritten
+        onn.fused_bias_dropout(x, b, 0.25, True, True)
+
+
 @pytest.mark.parametrize("dtype", [F32, BF16])
 def test_fused_bias_gelu_autograd(device, dtype):
     x = randn((64, 256), dtype, 1)

@@ -162,6 +162,22 @@ def test_softmax_module_cpu_and_flags():
     assert torch.allclose(yd[kept], 2.0 * ref[kept])
 
 
+def test_operands_without_a_kernel_take_the_torch_formulas():
+    """float64 has no element-wise kernel: the functions evaluate the reference's formulas with torch."""
+    x = torch.randn(5, 16, dtype=torch.float64)
+    b, r = torch.randn(16, dtype=torch.float64), torch.randn(5, 16, dtype=torch.float64)
+    assert torch.allclose(onn.fused_gelu(x), torch.nn.functional.gelu(x, approximate="tanh"), atol=1e-7)
+    assert torch.equal(onn.fused_bias_dropout_add(x, b, r, 0.0, True), x + b + r)
+    assert torch.equal(onn.fused_bias_dropout_add(x, None, None, 0.5, False), x)
+    # the CPU chain of the residual RMSNorm: the reference's manual_rms_norm (layer_norm.py:17-30) on the sum
+    w = torch.rand(16) + 0.5
+    xf, bf, rf = x.float(), b.float(), r.float()
+    y, h = onn.fused_bias_dropout_add_rms_norm(xf, bf, rf, w, (16,), 1e-6, 0.0, False, True)
+    assert torch.equal(h, xf + bf + rf)
+    want = w * (h * torch.rsqrt(h.pow(2).mean(-1, keepdim=True) + 1e-6))
+    assert torch.allclose(y, want, atol=1e-6)
+
+
 def test_residual_norm_module_without_parameters():
     m = onn.FusedBiasDropoutAddLayerNorm(16, p=0.0, elementwise_affine=False)
     assert m.weight is None and m.bias is None and "elementwise_affine=False" in repr(m)
