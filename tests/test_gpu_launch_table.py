@@ -14,8 +14,8 @@ OSLO_LAUNCH_TABLE=full.  By default each shape runs only the settings that
 golden/launch_table_cover.json lists for it: a smallest set of (shape, setting)
 pairs that between them launch every kernel build the full sweep launches,
 taken from a kernel trace of the full sweep (rocprofv3 --kernel-trace, the
-runs told apart by marker launches).  After a change of a launch rule the
-table is made again from such a trace."""
+runs told apart by marker launches) by golden/make_launch_table_cover.py.
+After a change of a launch rule the table is made again from such a trace."""
 import json
 import os
 
