@@ -702,6 +702,8 @@ static int run_bias_gelu_bwd(const void *gr, const void *x, const void *bias,
       else
         bias_gelu_bwd_kernel<T, U, false><<<grid, 256, 0, st>>>(
             (const T *)gr, (const T *)x, nullptr, (T *)dx, part, g);
+    } else {
+      return fail(OSLO_ERR_UNSUPPORTED, "bias_gelu bwd: no kernel for %d steps in flight in float32", U);
     }
   });
   int rc = check_launch("bias_gelu_bwd_kernel");
