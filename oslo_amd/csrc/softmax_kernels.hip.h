@@ -347,6 +347,10 @@ __global__ __launch_bounds__(1024) void softmax_fwd_kernel(
   uint32_t mbits[RPW][VPL];  // bit e set: key masked out
   int64_t row[RPW];
   bool rvalid[RPW];
+  // additive term: a query that the diagonal leaves without any key (sq > sk)
+  // gets zeros (its neighbours in the wave may well see keys, so the
+  // wave-uniform shortcuts below do not catch it)
+  bool nokey[RPW];
   const uint8_t *mrow0 = nullptr;
   // additive term (kModeBias): the chunks as loaded, and whether a chunk's
   // logits were left unread
@@ -365,6 +369,7 @@ __global__ __launch_bounds__(1024) void softmax_fwd_kernel(
     const uint8_t *mrow = nullptr;
     row[j] = 0;
     if (rvalid[j]) row_setup<MODE>(g, r, mask, row[j], visible, mrow);
+    nokey[j] = MODE == kModeBias && rvalid[j] && visible <= 0;
     // consecutive rows of a wave normally share their mask row (a key-padding
     // mask [b, 1, 1, sk]): its bits are then read and unpacked once
     bool shared = false;
@@ -534,7 +539,7 @@ __global__ __launch_bounds__(1024) void softmax_fwd_kernel(
     float s = 0.f;
     // (with an additive term a row of -inf sums is NaN, as torch.softmax
     //  returns it: the maximum is subtracted as it is)
-    const float off = mx[j] == ninf && !kBias ? 0.f : mx[j];
+    const float off = (mx[j] == ninf && !kBias) || nokey[j] ? 0.f : mx[j];
     // (additive term: a slot whose logits were all left unread holds exact
     //  zeros as soon as every row of the wave has another key: no exponentials)
     if constexpr (kBias) {
@@ -569,12 +574,12 @@ __global__ __launch_bounds__(1024) void softmax_fwd_kernel(
     // a row without any visible key: uniform distribution, as softmax of a
     // constant fill value gives
     const bool empty = mx[j] == ninf && !kBias;
-    const float inv = empty ? 0.f : row_recip(sm[j]);
+    const float inv = empty || nokey[j] ? 0.f : row_recip(sm[j]);
     const float fill = empty ? g.inv_sk : 0.f;
     T *yr = y + row[j] * g.sk;
     if constexpr (DROP) {
       if (c0 == 0) {
-        stats[2 * row[j]] = empty ? 0.f : mx[j];
+        stats[2 * row[j]] = empty || nokey[j] ? 0.f : mx[j];
         stats[2 * row[j] + 1] = empty ? -fill : inv;
       }
     }

@@ -79,6 +79,12 @@ CASES = [
     (2, 2, 256, 2048, BF16, 0.10206207, "min", True),  # sq != sk with the diagonal
     (2, 2, 37, 64, F16, 0.5, "inf", True),
     (2, 2, 64, 40, BF16, 0.5, "t5", True),             # sq > sk: the diagonal hides whole rows
+    # the same where rows lie side by side in a wave: a row without any key next to rows that see keys
+    (2, 2, 37, 20, F32, 0.5, "t5", True),
+    (2, 2, 40, 64, BF16, 0.5, "perq", True),
+    (2, 3, 70, 128, F16, 0.25, "m10000", True),
+    (2, 1, 300, 256, BF16, 0.25, "t5", True),
+    (1, 2, 600, 512, BF16, 0.25, "min", True),         # and with a wave per row
     (1, 2, 8, 4096, BF16, 1.0, "min", False),          # two waves per row
     (2, 1, 4, 16384, F16, 1.0, "t5", False),
     (2, 2, 33, 33, F32, 0.7, "m10000", False),         # odd length: scalar kernels
@@ -248,6 +254,11 @@ DROPOUT_CASES = [
     (2, 1, 5, 2051, BF16, 0.25, "t5", False, 0.1),
     (2, 2, 20, 1004, F16, 0.25, "perq", False, 0.1),
     (1, 2, 8, 4096, BF16, 1.0, "min", False, 0.1),
+    # sq > sk under the diagonal: rows without any key, side by side with rows that see keys and alone in a wave
+    (2, 2, 37, 20, F32, 0.5, "perq", True, 0.1),
+    (2, 2, 40, 64, BF16, 0.5, "t5", True, 0.1),
+    (2, 2, 300, 256, F16, 0.25, "min", True, 0.1),
+    (1, 2, 600, 512, BF16, 0.25, "t5", True, 0.1),
 ]
 
 
@@ -263,20 +274,26 @@ def test_bias_softmax_dropout(device, b, np_, sq, sk, dtype, scale, kind, causal
     oo = cf.softmax_bias_dropout_fwd(f64(x), f64(bias), scale, keep, p, causal=causal)
     odx = cf.softmax_bias_dropout_bwd(f64(g), f64(x), f64(bias), scale, keep, p, causal=causal)
     plain = k.softmax_bias_forward(x.to(device), bias.to(device), scale, causal=causal).cpu()
+    # queries that the diagonal leaves without any key (sq > sk; NaN in the oracle as in torch): zeros here
+    fr = np.isfinite(oo).all(-1)
+    assert fr.all() or (causal and sq > sk and not fr[..., : sq - sk].any() and fr[..., sq - sk:].all())
+    frt = torch.from_numpy(fr)
     outs = []
     for skip in (False, True):
         out, stats = k.softmax_bias_dropout_forward(x.to(device), bias.to(device), scale, p, seed,
                                                     offset, causal=causal, skip_hidden=skip)
         plain = k.softmax_bias_forward(x.to(device), bias.to(device), scale, causal=causal,
                                        skip_hidden=skip).cpu()
-        check(out, oo, "bias softmax dropout fwd", atol=1e-9)
+        assert (out.cpu()[~frt] == 0).all() and torch.isfinite(stats).all()
+        check(out.cpu()[frt], oo[fr], "bias softmax dropout fwd", atol=1e-9)
         ocpu = out.cpu()
         # the keep decisions are the Philox stream over the flattened output, bit for bit
         assert (ocpu[torch.from_numpy(~keep)] == 0).all(), "dropped elements must be exactly 0"
         assert (ocpu[torch.from_numpy(keep) & (plain != 0)] != 0).all(), "kept elements must survive"
         dx = k.softmax_bias_dropout_backward(g.to(device), x.to(device), bias.to(device), stats, scale,
                                              p, seed, offset, causal=causal, skip_hidden=skip)
-        check(dx, odx, "bias softmax dropout bwd", atol=2e-7)
+        assert (dx.cpu()[~frt] == 0).all()
+        check(dx.cpu()[frt], odx[fr], "bias softmax dropout bwd", atol=2e-7)
         outs.append((ocpu, dx.cpu()))
         # p = 0 reproduces the plain kernel bit for bit
         out0, _ = k.softmax_bias_dropout_forward(x.to(device), bias.to(device), scale, 0.0, seed,
