@@ -1038,8 +1038,11 @@ __global__ __launch_bounds__(256) void softmax_fwd_generic_kernel(
     }
     if constexpr (DROP) {
       if (threadIdx.x == 0) {
-        stats[2 * row] = empty ? 0.f : m;
-        stats[2 * row + 1] = empty ? -fill : inv;
+        // (a query that the diagonal leaves without any key: zeros above, and
+        //  finite statistics for the backward pass)
+        const bool nokey = kBias && visible <= 0;
+        stats[2 * row] = empty || nokey ? 0.f : m;
+        stats[2 * row + 1] = empty ? -fill : (nokey ? 0.f : inv);
       }
     }
   }
@@ -1275,8 +1278,11 @@ __global__ __launch_bounds__(256) void softmax_fwd_wave_kernel(
     }
     if constexpr (DROP) {
       if (lane == 0) {
-        stats[2 * row] = empty ? 0.f : m;
-        stats[2 * row + 1] = empty ? -fill : inv;
+        // (a query that the diagonal leaves without any key: zeros above, and
+        //  finite statistics for the backward pass)
+        const bool nokey = kBias && visible <= 0;
+        stats[2 * row] = empty || nokey ? 0.f : m;
+        stats[2 * row + 1] = empty ? -fill : (nokey ? 0.f : inv);
       }
     }
   }

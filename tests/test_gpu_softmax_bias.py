@@ -85,6 +85,7 @@ CASES = [
     (2, 3, 70, 128, F16, 0.25, "m10000", True),
     (2, 1, 300, 256, BF16, 0.25, "t5", True),
     (1, 2, 600, 512, BF16, 0.25, "min", True),         # and with a wave per row
+    (1, 1, 2060, 2052, F16, 0.25, "t5", True),         # one workgroup per row
     (1, 2, 8, 4096, BF16, 1.0, "min", False),          # two waves per row
     (2, 1, 4, 16384, F16, 1.0, "t5", False),
     (2, 2, 33, 33, F32, 0.7, "m10000", False),         # odd length: scalar kernels
@@ -259,6 +260,8 @@ DROPOUT_CASES = [
     (2, 2, 40, 64, BF16, 0.5, "t5", True, 0.1),
     (2, 2, 300, 256, F16, 0.25, "min", True, 0.1),
     (1, 2, 600, 512, BF16, 0.25, "t5", True, 0.1),
+    (2, 2, 50, 44, BF16, 0.5, "t5", True, 0.1),        # one wave per row, scalar accesses
+    (1, 1, 2060, 2052, F16, 0.25, "min", True, 0.1),   # one workgroup per row
 ]
 
 
