@@ -68,6 +68,11 @@ CASES = [
     (2, 2, 192, 192, BF16, 0.25, "right"),              # three chunks per lane
     (2, 2, 100, 768, F16, 0.125, "holes"),
     (3, 1, 1, 8, F32, 2.0, "right"),
+    # sq > sk where rows lie side by side in a wave: queries without any key next to queries that see keys
+    (2, 2, 73, 64, BF16, 0.25, "right"),
+    (2, 2, 137, 128, F16, 0.25, "holes"),
+    (2, 2, 41, 32, F32, 0.25, "left"),
+    (2, 2, 300, 256, BF16, 0.25, "right"),
 ]
 
 
@@ -137,6 +142,10 @@ DROPOUT_CASES = [
     (2, 2, 37, 64, F16, 0.5, "right", 0.1),
     (2, 2, 33, 33, F32, 0.7, "right", 0.1),
     (2, 1, 5, 2051, BF16, 0.25, "right", 0.1),
+    # sq > sk where rows lie side by side in a wave: queries without any key next to queries that see keys
+    (2, 2, 73, 64, BF16, 0.25, "right", 0.1),
+    (2, 2, 137, 128, F16, 0.25, "holes", 0.1),
+    (2, 2, 41, 32, F32, 0.25, "left", 0.1),
 ]
 
 
