@@ -230,7 +230,7 @@ def test_softmax_with_an_additive_term(device, i, b, np_, sq, sk, dtype, kind):
     r = np.random.default_rng(2000 + i)
     scale = float(r.choice([0.125, 0.5, 1.0]))
     p = float(r.choice([0.0, 0.0, 0.1, 0.3]))
-    causal = bool(r.integers(0, 2)) and sq <= sk
+    causal = bool(r.integers(0, 2))   # (with sq > sk the first sq - sk queries see no key at all)
     skip = bool(r.integers(0, 2))
     term_f32 = bool(r.integers(0, 2))
     seed, offset = 70 + i, 4 * i
@@ -255,24 +255,37 @@ def test_softmax_with_an_additive_term(device, i, b, np_, sq, sk, dtype, kind):
     k = _C.get_softmax_kernel()
     xd, gd, td = x.to(device), g.to(device), term.to(device)
     xv, gv, tv = f64(x), f64(g), f64(term)
+    # a query that the diagonal leaves without any key is NaN in the oracle (as in torch) and zeros here
+    seen = np.ones((b, np_, sq), dtype=bool)
+    if causal and sq > sk:
+        seen[..., : sq - sk] = False
+    st = torch.from_numpy(seen)
+
+    def compare(actual, truth, what, **kw):
+        a = actual.cpu()
+        assert (a[~st] == 0).all(), what + ": a query without any key must come out as zeros"
+        if seen.any():
+            check(a[st], truth[seen], what, **kw)
+
     if p == 0.0:
         y = k.softmax_bias_forward(xd, td, scale, causal=causal, skip_hidden=skip)
         dx = k.softmax_bias_backward(gd, y, scale, bias=td, causal=causal, skip_hidden=skip)
-        check(y, cf.softmax_bias_fwd(xv, tv, scale, causal=causal), "term softmax fwd", atol=1e-9)
-        check(dx, cf.softmax_bwd(gv, f64(y), scale), "term softmax bwd", atol=2e-7)
+        compare(y, cf.softmax_bias_fwd(xv, tv, scale, causal=causal), "term softmax fwd", atol=1e-9)
+        compare(dx, cf.softmax_bwd(gv, f64(y), scale), "term softmax bwd", atol=2e-7)
     else:
         out, stats = k.softmax_bias_dropout_forward(xd, td, scale, p, seed, offset, causal=causal,
                                                     skip_hidden=skip)
+        assert torch.isfinite(stats).all()
         keep = philox.keep_mask(x.numel(), p, seed, offset).reshape(xv.shape).astype(bool)
-        check(out, cf.softmax_bias_dropout_fwd(xv, tv, scale, keep, p, causal=causal),
-              "term softmax dropout fwd", atol=1e-9)
+        compare(out, cf.softmax_bias_dropout_fwd(xv, tv, scale, keep, p, causal=causal),
+                "term softmax dropout fwd", atol=1e-9)
         dx = k.softmax_bias_dropout_backward(gd, xd, td, stats, scale, p, seed, offset, causal=causal,
                                              skip_hidden=skip)
         # dx = scale * y * (dp - sum(dp * y)) cancels: the absolute floor is two float32 roundings of the
         # largest product scale * y * dp that can enter it (y <= 1)
         floor = max(3e-7, 2 * 2.0 ** -23 * scale * float(np.abs(gv).max()) / (1.0 - p))
-        check(dx, cf.softmax_bias_dropout_bwd(gv, xv, tv, scale, keep, p, causal=causal),
-              "term softmax dropout bwd", atol=floor, min_exact=0.98)
+        compare(dx, cf.softmax_bias_dropout_bwd(gv, xv, tv, scale, keep, p, causal=causal),
+                "term softmax dropout bwd", atol=floor, min_exact=0.98)
 
 
 @pytest.mark.parametrize("i,n1,n2,dtype,flags", draw_cases(404, 50))
