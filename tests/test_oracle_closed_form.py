@@ -367,6 +367,28 @@ def test_bias_dropout_add_identity_and_scaling():
     assert np.allclose(cf.bias_dropout_add_fwd(x, b, res, keep, 0.3), ref.numpy(), rtol=3e-7, atol=3e-7)
 
 
+def test_share_of_bf16_results_an_fp32_evaluation_rounds_the_other_way():
+    """Where the 99.8 % of the 16-bit parity bar comes from: the same formula
+    evaluated in float32 (every product and sum rounded, as a kernel does) and
+    in float64, both then rounded to bfloat16, differ in one to three results
+    in a thousand for bfloat16 operands with a dropout scale that is no power
+    of two -- sums of short operands land next to rounding ties often -- and
+    in none for p = 0.5, whose scale is exact."""
+    r = rng(52)
+    rows, cols = 64, 4096
+    x = cf.round_to(r.standard_normal((rows, cols)), "bf16")
+    res = cf.round_to(r.standard_normal((rows, cols)), "bf16")
+    keep = np.ones((rows, cols), dtype=bool)
+    for bias_std, p, low, high in ((0.02, 0.1, 5e-4, 2e-3), (0.1, 0.1, 1e-3, 4e-3), (0.1, 0.5, 0.0, 0.0)):
+        b = cf.round_to(bias_std * r.standard_normal(cols), "bf16")
+        exact = cf.bias_dropout_add_fwd(x, b, res, keep, p, out="bf16")
+        single = cf.bias_dropout_add_fwd(x, b, res, keep, p, out="bf16", acc=np.float32)
+        share = float(np.mean(exact != single))
+        assert low <= share <= high, (bias_std, p, share)
+        # one step of bfloat16 at most (sums that cancel carry float32's absolute error instead)
+        assert np.all(np.abs(exact - single) <= np.maximum(2.0 ** -7 * np.abs(exact), 1e-6))
+
+
 def test_bias_dropout_add_bwd_vs_autograd():
     r = rng(51)
     x = torch.from_numpy(r.standard_normal((5, 8))).requires_grad_()
